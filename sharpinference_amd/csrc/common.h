@@ -1,0 +1,80 @@
+// Shared device helpers for the gfx950 kernels: storage types, conversions, wave reductions.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define SHARPI_OK 0
+#define SHARPI_ERR_ARG 1001   // a size or option the kernel does not take
+#define SHARPI_ERR_LAUNCH 1002
+
+#define SHARPI_CHECK_LAUNCH()                                   \
+  do {                                                          \
+    hipError_t e__ = hipGetLastError();                         \
+    if (e__ != hipSuccess) return (int)e__;                     \
+  } while (0)
+
+#define SHARPI_EXPORT extern "C" __attribute__((visibility("default")))
+
+constexpr int kWave = 64;
+
+// bfloat16 as raw bits; conversions are round-to-nearest-even, NaN kept quiet.
+struct bf16_t {
+  uint16_t bits;
+};
+
+__device__ __forceinline__ float bf16_to_f32(bf16_t v) {
+  return __uint_as_float(((uint32_t)v.bits) << 16);
+}
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits16) {
+  return __uint_as_float(bits16 << 16);
+}
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  bf16_t r;
+  if ((u & 0x7fffffffu) > 0x7f800000u) {  // NaN
+    r.bits = (uint16_t)((u >> 16) | 0x0040u);
+    return r;
+  }
+  u += 0x7fffu + ((u >> 16) & 1u);
+  r.bits = (uint16_t)(u >> 16);
+  return r;
+}
+
+template <typename T> __device__ __forceinline__ float to_f32(T v);
+template <> __device__ __forceinline__ float to_f32<float>(float v) { return v; }
+template <> __device__ __forceinline__ float to_f32<bf16_t>(bf16_t v) { return bf16_to_f32(v); }
+
+template <typename T> __device__ __forceinline__ T from_f32(float v);
+template <> __device__ __forceinline__ float from_f32<float>(float v) { return v; }
+template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float v) { return f32_to_bf16(v); }
+
+// dtype codes shared with the Python side
+enum : int { DT_F32 = 0, DT_BF16 = 1 };
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+  return v;
+}
+
+// Block-wide sum for blocks of up to 1024 threads; `red` is LDS of >= 16 floats.
+// The result is the same in every thread; the order of additions is fixed.
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wid = threadIdx.x >> 6;
+  const int nw = (blockDim.x + kWave - 1) >> 6;
+  v = wave_sum(v);
+  __syncthreads();
+  if (lane == 0) red[wid] = v;
+  __syncthreads();
+  float t = 0.f;
+  for (int i = 0; i < nw; ++i) t += red[i];
+  return t;
+}
+
+static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }

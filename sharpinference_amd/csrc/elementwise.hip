@@ -1,0 +1,207 @@
+// Row-wise kernels: embedding gather, residual add + RMSNorm, SiLU*up, MoE combine, casts.
+// All statistics and sums are float; storage may be float or bfloat16.
+#include "common.h"
+
+// ---------------------------------------------------------------------------
+// embedding gather: out[t, :] = table[ids[t], :]   (out is the float residual stream)
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ void embed_gather_kernel(const int* __restrict__ ids, const T* __restrict__ table,
+                                    float* __restrict__ out, int hidden) {
+  const int t = blockIdx.x;
+  const T* row = table + (size_t)ids[t] * hidden;
+  float* o = out + (size_t)t * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) o[i] = to_f32<T>(row[i]);
+}
+
+SHARPI_EXPORT int sharpi_embed_gather(const int* ids, const void* table, int table_dtype, float* out,
+                                      int n_tokens, int hidden, hipStream_t stream) {
+  if (n_tokens <= 0) return SHARPI_OK;
+  if (hidden <= 0) return SHARPI_ERR_ARG;
+  dim3 grid(n_tokens), block(256);
+  if (table_dtype == DT_F32)
+    embed_gather_kernel<float><<<grid, block, 0, stream>>>(ids, (const float*)table, out, hidden);
+  else if (table_dtype == DT_BF16)
+    embed_gather_kernel<bf16_t><<<grid, block, 0, stream>>>(ids, (const bf16_t*)table, out, hidden);
+  else
+    return SHARPI_ERR_ARG;
+  SHARPI_CHECK_LAUNCH();
+  return SHARPI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// residual add + RMSNorm.
+//   r = rows ? rows[i] : i
+//   x = h[r, :] (+ delta[r, :])           float sum
+//   if write_back: h[r, :] = x
+//   out[i, :] = (x * rsqrt(mean(x^2) + eps)) * w     (w may be absent)
+// One block per output row; the order of the additions depends on `hidden` only.
+// ---------------------------------------------------------------------------
+template <typename TD, typename TW, typename TO>
+__global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__ delta,
+                                   const TW* __restrict__ w, TO* __restrict__ out,
+                                   const int* __restrict__ rows, int hidden, float eps, int write_back) {
+  __shared__ float red[16];
+  const int i = blockIdx.x;
+  const int r = rows ? rows[i] : i;
+  float* hr = h + (size_t)r * hidden;
+  const TD* dr = delta ? delta + (size_t)r * hidden : nullptr;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < hidden; c += blockDim.x) {
+    float x = hr[c];
+    if (dr) {
+      x += to_f32<TD>(dr[c]);
+      if (write_back) hr[c] = x;
+    }
+    ss += x * x;
+  }
+  const float total = block_sum(ss, red);
+  const float s = 1.0f / sqrtf(total / (float)hidden + eps);
+  TO* o = out + (size_t)i * hidden;
+  for (int c = threadIdx.x; c < hidden; c += blockDim.x) {
+    float x = hr[c];
+    if (dr && !write_back) x += to_f32<TD>(dr[c]);
+    float y = x * s;
+    if (w) y *= to_f32<TW>(w[c]);
+    o[c] = from_f32<TO>(y);
+  }
+}
+
+template <typename TD, typename TW>
+static int launch_add_rmsnorm_o(float* h, const void* delta, const void* w, void* out, int out_dtype,
+                                const int* rows, int n_out, int hidden, float eps, int write_back,
+                                hipStream_t stream) {
+  dim3 grid(n_out), block(hidden >= 2048 ? 512 : 256);
+  if (out_dtype == DT_F32)
+    add_rmsnorm_kernel<TD, TW, float><<<grid, block, 0, stream>>>(h, (const TD*)delta, (const TW*)w,
+                                                                 (float*)out, rows, hidden, eps, write_back);
+  else if (out_dtype == DT_BF16)
+    add_rmsnorm_kernel<TD, TW, bf16_t><<<grid, block, 0, stream>>>(h, (const TD*)delta, (const TW*)w,
+                                                                  (bf16_t*)out, rows, hidden, eps, write_back);
+  else
+    return SHARPI_ERR_ARG;
+  SHARPI_CHECK_LAUNCH();
+  return SHARPI_OK;
+}
+
+template <typename TD>
+static int launch_add_rmsnorm_w(float* h, const void* delta, const void* w, int w_dtype, void* out,
+                                int out_dtype, const int* rows, int n_out, int hidden, float eps,
+                                int write_back, hipStream_t stream) {
+  if (w_dtype == DT_F32 || w == nullptr)
+    return launch_add_rmsnorm_o<TD, float>(h, delta, w, out, out_dtype, rows, n_out, hidden, eps, write_back, stream);
+  if (w_dtype == DT_BF16)
+    return launch_add_rmsnorm_o<TD, bf16_t>(h, delta, w, out, out_dtype, rows, n_out, hidden, eps, write_back, stream);
+  return SHARPI_ERR_ARG;
+}
+
+SHARPI_EXPORT int sharpi_add_rmsnorm(float* h, const void* delta, int delta_dtype, const void* w, int w_dtype,
+                                     void* out, int out_dtype, const int* rows, int n_out, int hidden,
+                                     float eps, int write_back, hipStream_t stream) {
+  if (n_out <= 0) return SHARPI_OK;
+  if (hidden <= 0 || !(eps > 0.f)) return SHARPI_ERR_ARG;
+  if (rows && write_back) return SHARPI_ERR_ARG;  // gathered rows never write the stream back
+  if (delta == nullptr || delta_dtype == DT_F32)
+    return launch_add_rmsnorm_w<float>(h, delta, w, w_dtype, out, out_dtype, rows, n_out, hidden, eps, write_back, stream);
+  if (delta_dtype == DT_BF16)
+    return launch_add_rmsnorm_w<bf16_t>(h, delta, w, w_dtype, out, out_dtype, rows, n_out, hidden, eps, write_back, stream);
+  return SHARPI_ERR_ARG;
+}
+
+// ---------------------------------------------------------------------------
+// SwiGLU activation on a fused [M, 2*I] buffer (gate columns first, up columns second):
+//   out[m, i] = silu(s_m * g) * (s_m * u),  silu(x) = x / (1 + exp(-x)),  s_m = scale ? scale[m] : 1
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ gu, const float* __restrict__ scale,
+                                T* __restrict__ out, int inter) {
+  const int m = blockIdx.x;
+  const int i = blockIdx.y * blockDim.x + threadIdx.x;
+  if (i >= inter) return;
+  const T* row = gu + (size_t)m * 2 * inter;
+  float g = to_f32<T>(row[i]);
+  float u = to_f32<T>(row[inter + i]);
+  if (scale) {
+    const float s = scale[m];
+    g *= s;
+    u *= s;
+  }
+  const float a = g / (1.0f + expf(-g));
+  out[(size_t)m * inter + i] = from_f32<T>(a * u);
+}
+
+SHARPI_EXPORT int sharpi_silu_mul(const void* gu, const float* scale, void* out, int dtype, int rows, int inter,
+                                  hipStream_t stream) {
+  if (rows <= 0) return SHARPI_OK;
+  if (inter <= 0 || ceil_div(inter, 256) > 65535) return SHARPI_ERR_ARG;
+  dim3 block(256), grid(rows, ceil_div(inter, 256));
+  if (dtype == DT_F32)
+    silu_mul_kernel<float><<<grid, block, 0, stream>>>((const float*)gu, scale, (float*)out, inter);
+  else if (dtype == DT_BF16)
+    silu_mul_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)gu, scale, (bf16_t*)out, inter);
+  else
+    return SHARPI_ERR_ARG;
+  SHARPI_CHECK_LAUNCH();
+  return SHARPI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// MoE combine: out[t, :] = sum_j y[inv_pos[t*k + j], :] (+ shared[t, :]); float sums, j ascending.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ void moe_combine_kernel(const T* __restrict__ y, const int* __restrict__ inv_pos,
+                                   const T* __restrict__ shared, T* __restrict__ out, int hidden, int k) {
+  const int t = blockIdx.x;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= hidden) return;
+  float acc = 0.f;
+  for (int j = 0; j < k; ++j) acc += to_f32<T>(y[(size_t)inv_pos[t * k + j] * hidden + c]);
+  if (shared) acc += to_f32<T>(shared[(size_t)t * hidden + c]);
+  out[(size_t)t * hidden + c] = from_f32<T>(acc);
+}
+
+SHARPI_EXPORT int sharpi_moe_combine(const void* y, const int* inv_pos, const void* shared, void* out, int dtype,
+                                     int n_tokens, int hidden, int k, hipStream_t stream) {
+  if (n_tokens <= 0) return SHARPI_OK;
+  if (hidden <= 0 || k <= 0 || ceil_div(hidden, 256) > 65535) return SHARPI_ERR_ARG;
+  dim3 block(256), grid(n_tokens, ceil_div(hidden, 256));
+  if (dtype == DT_F32)
+    moe_combine_kernel<float><<<grid, block, 0, stream>>>((const float*)y, inv_pos, (const float*)shared,
+                                                         (float*)out, hidden, k);
+  else if (dtype == DT_BF16)
+    moe_combine_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)y, inv_pos, (const bf16_t*)shared,
+                                                          (bf16_t*)out, hidden, k);
+  else
+    return SHARPI_ERR_ARG;
+  SHARPI_CHECK_LAUNCH();
+  return SHARPI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// casts between the two storage types
+// ---------------------------------------------------------------------------
+template <typename TI, typename TO>
+__global__ void cast_kernel(const TI* __restrict__ in, TO* __restrict__ out, size_t n) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) out[i] = from_f32<TO>(to_f32<TI>(in[i]));
+}
+
+SHARPI_EXPORT int sharpi_cast(const void* in, int in_dtype, void* out, int out_dtype, long long n,
+                              hipStream_t stream) {
+  if (n <= 0) return SHARPI_OK;
+  long long nb = (n + 255) / 256;
+  dim3 block(256), grid((unsigned)(nb > 65536 ? 65536 : nb));
+  if (in_dtype == DT_F32 && out_dtype == DT_BF16)
+    cast_kernel<float, bf16_t><<<grid, block, 0, stream>>>((const float*)in, (bf16_t*)out, (size_t)n);
+  else if (in_dtype == DT_BF16 && out_dtype == DT_F32)
+    cast_kernel<bf16_t, float><<<grid, block, 0, stream>>>((const bf16_t*)in, (float*)out, (size_t)n);
+  else if (in_dtype == DT_F32 && out_dtype == DT_F32)
+    cast_kernel<float, float><<<grid, block, 0, stream>>>((const float*)in, (float*)out, (size_t)n);
+  else if (in_dtype == DT_BF16 && out_dtype == DT_BF16)
+    cast_kernel<bf16_t, bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)in, (bf16_t*)out, (size_t)n);
+  else
+    return SHARPI_ERR_ARG;
+  SHARPI_CHECK_LAUNCH();
+  return SHARPI_OK;
+}

@@ -1,0 +1,120 @@
+// Position encoding, weightless per-head norm, query temperature and the cache write, one kernel.
+//
+// Input  qkv [T, (nh + 2*nkv) * hd]: q heads, then k heads, then v heads of each token.
+// q head : rotate (if inv_freq) -> norm (if qk_norm) -> * temperature (if temp_tuning) -> q_out
+// k head : rotate (if inv_freq) -> norm (if qk_norm) -> cache K at slot_mapping[t]
+// v head : cache V at slot_mapping[t]
+// Rotation is on interleaved pairs (2i, 2i+1) with angle = float(pos) * inv_freq[i], all in float.
+// Cache layout of one layer: [page][kv head][page_size][hd]; slot = page * page_size + offset;
+// a negative slot means "do not store" (the layer reads another layer's cache).
+#include "common.h"
+
+template <typename T>
+__global__ void rope_kv_kernel(const T* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_cache,
+                               T* __restrict__ v_cache, const int* __restrict__ slot_mapping,
+                               const int* __restrict__ positions, const float* __restrict__ inv_freq,
+                               int qk_norm, float eps, int temp_tuning, float floor_scale, float attn_scale,
+                               int nh, int nkv, int hd, int page_size) {
+  const int t = blockIdx.x;
+  const int head = blockIdx.y;            // 0..nh-1 q, nh..nh+nkv-1 k, then v
+  const int lane = threadIdx.x;           // one wave
+  const int half = hd >> 1;
+  const T* src = qkv + ((size_t)t * (nh + 2 * nkv) + head) * hd;
+  const int pos = positions[t];
+  const bool is_q = head < nh;
+  const bool is_k = !is_q && head < nh + nkv;
+  const int slot = slot_mapping[t];
+
+  if (!is_q && !is_k) {  // v: plain copy into the cache
+    if (slot < 0) return;
+    const int kvh = head - nh - nkv;
+    T* dst = v_cache + (((size_t)(slot / page_size) * nkv + kvh) * page_size + (slot % page_size)) * hd;
+    for (int d = lane; d < hd; d += kWave) dst[d] = src[d];
+    return;
+  }
+  if (is_k && slot < 0) return;
+
+  // pairs handled by this lane: i = lane, lane + 64, ... (hd <= 512)
+  float x0[4], x1[4];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int i = lane + j * kWave;
+    x0[j] = 0.f;
+    x1[j] = 0.f;
+    if (i < half) {
+      float a = to_f32<T>(src[2 * i]);
+      float b = to_f32<T>(src[2 * i + 1]);
+      if (inv_freq) {
+        const float ang = (float)pos * inv_freq[i];
+        const float c = cosf(ang);
+        const float s = sinf(ang);
+        const float ra = a * c - b * s;
+        const float rb = a * s + b * c;
+        a = ra;
+        b = rb;
+      }
+      x0[j] = a;
+      x1[j] = b;
+      ss += a * a + b * b;
+    }
+  }
+  float mul = 1.0f;
+  if (qk_norm) {
+    const float total = wave_sum(ss);
+    mul = 1.0f / sqrtf(total / (float)hd + eps);
+  }
+  float post = 1.0f;
+  if (is_q && temp_tuning) {
+    post = 1.0f + attn_scale * logf(floorf(((float)pos + 1.0f) / floor_scale) + 1.0f);
+  }
+  T* dst;
+  if (is_q) {
+    dst = q_out + ((size_t)t * nh + head) * hd;
+  } else {
+    const int kvh = head - nh;
+    dst = k_cache + (((size_t)(slot / page_size) * nkv + kvh) * page_size + (slot % page_size)) * hd;
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int i = lane + j * kWave;
+    if (i < half) {
+      float a = x0[j], b = x1[j];
+      if (qk_norm) {
+        a *= mul;
+        b *= mul;
+      }
+      if (is_q && temp_tuning) {
+        a *= post;
+        b *= post;
+      }
+      dst[2 * i] = from_f32<T>(a);
+      dst[2 * i + 1] = from_f32<T>(b);
+    }
+  }
+}
+
+SHARPI_EXPORT int sharpi_rope_kv(const void* qkv, void* q_out, void* k_cache, void* v_cache, int dtype,
+                                 const int* slot_mapping, const int* positions, const float* inv_freq,
+                                 int qk_norm, float eps, int temp_tuning, float floor_scale, float attn_scale,
+                                 int n_tokens, int nh, int nkv, int hd, int page_size, hipStream_t stream) {
+  if (n_tokens <= 0) return SHARPI_OK;
+  if (hd <= 0 || (hd & 1) || hd > 512 || nh <= 0 || nkv <= 0 || page_size <= 0) return SHARPI_ERR_ARG;
+  if (nh + 2 * nkv > 65535) return SHARPI_ERR_ARG;
+  if (temp_tuning && !(floor_scale > 0.f)) return SHARPI_ERR_ARG;
+  dim3 grid(n_tokens, nh + 2 * nkv), block(kWave);
+  if (dtype == DT_F32)
+    rope_kv_kernel<float><<<grid, block, 0, stream>>>((const float*)qkv, (float*)q_out, (float*)k_cache,
+                                                     (float*)v_cache, slot_mapping, positions, inv_freq, qk_norm,
+                                                     eps, temp_tuning, floor_scale, attn_scale, nh, nkv, hd,
+                                                     page_size);
+  else if (dtype == DT_BF16)
+    rope_kv_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)qkv, (bf16_t*)q_out, (bf16_t*)k_cache,
+                                                      (bf16_t*)v_cache, slot_mapping, positions, inv_freq,
+                                                      qk_norm, eps, temp_tuning, floor_scale, attn_scale, nh, nkv,
+                                                      hd, page_size);
+  else
+    return SHARPI_ERR_ARG;
+  SHARPI_CHECK_LAUNCH();
+  return SHARPI_OK;
+}

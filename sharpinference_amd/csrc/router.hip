@@ -1,0 +1,134 @@
+// MoE routing on the device: router logits, gate, top-k, and the expert-sorted row list.
+//
+// router_topk: one block per token. logits[e] = Wr[e, :] . x[t, :] in float (each wave owns
+// experts e = wave, wave + nwaves, ...; lanes stride over the hidden width, so the order of
+// the additions depends on the width only).  gate 0 = sigmoid over every expert, gate 1 =
+// softmax over every expert.  The k picks scan ascending with a strict >, so the lowest index
+// wins a tie; the weight of a pick is its gate value; renorm divides the k weights by their sum.
+//
+// moe_permute: one block. Counts rows per expert, prefix-sums them into offsets[E + 1] and
+// writes, in expert order, the token and weight of every (token, pick) pair plus the inverse
+// map inv_pos[t * k + j] = row in that order.
+#include "common.h"
+
+constexpr int kMaxExperts = 1024;
+
+template <typename T, typename TW>
+__global__ __launch_bounds__(256) void router_topk_kernel(const T* __restrict__ x, const TW* __restrict__ wr,
+                                                          int* __restrict__ topk_ids,
+                                                          float* __restrict__ topk_w,
+                                                          float* __restrict__ gate_out, int hidden,
+                                                          int n_experts, int k, int gate, int renorm) {
+  __shared__ float g[kMaxExperts];
+  const int t = blockIdx.x;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int w = threadIdx.x >> 6;
+  const int nw = blockDim.x >> 6;
+  const T* xr = x + (size_t)t * hidden;
+  for (int e = w; e < n_experts; e += nw) {
+    const TW* wrow = wr + (size_t)e * hidden;
+    float s = 0.f;
+    for (int c = lane; c < hidden; c += kWave) s = fmaf(to_f32<T>(xr[c]), to_f32<TW>(wrow[c]), s);
+    s = wave_sum(s);
+    if (lane == 0) g[e] = s;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    if (gate == 0) {
+      for (int e = 0; e < n_experts; ++e) g[e] = 1.0f / (1.0f + expf(-g[e]));
+    } else {
+      float mx = g[0];
+      for (int e = 1; e < n_experts; ++e) mx = fmaxf(mx, g[e]);
+      float sum = 0.f;
+      for (int e = 0; e < n_experts; ++e) {
+        g[e] = expf(g[e] - mx);
+        sum += g[e];
+      }
+      const float inv = 1.0f / sum;
+      for (int e = 0; e < n_experts; ++e) g[e] *= inv;
+    }
+    if (gate_out)
+      for (int e = 0; e < n_experts; ++e) gate_out[(size_t)t * n_experts + e] = g[e];
+    float wsum = 0.f;
+    for (int j = 0; j < k; ++j) {
+      int best = -1;
+      float bv = -INFINITY;
+      for (int e = 0; e < n_experts; ++e) {
+        bool taken = false;
+        for (int i = 0; i < j; ++i) taken |= (topk_ids[t * k + i] == e);
+        if (!taken && (best < 0 || g[e] > bv)) {
+          bv = g[e];
+          best = e;
+        }
+      }
+      topk_ids[t * k + j] = best;
+      topk_w[t * k + j] = bv;
+      wsum += bv;
+    }
+    if (renorm && k > 1 && wsum > 0.f)
+      for (int j = 0; j < k; ++j) topk_w[t * k + j] /= wsum;
+  }
+}
+
+SHARPI_EXPORT int sharpi_router_topk(const void* x, int x_dtype, const void* wr, int w_dtype, int* topk_ids,
+                                     float* topk_w, float* gate_out, int n_tokens, int hidden, int n_experts,
+                                     int k, int gate, int renorm, hipStream_t stream) {
+  if (n_tokens <= 0) return SHARPI_OK;
+  if (hidden <= 0 || n_experts <= 0 || n_experts > kMaxExperts || k <= 0 || k > n_experts) return SHARPI_ERR_ARG;
+  if (gate < 0 || gate > 1) return SHARPI_ERR_ARG;
+  dim3 grid(n_tokens), block(256);
+#define ROUTER_LAUNCH(TX, TWT)                                                                              \
+  router_topk_kernel<TX, TWT><<<grid, block, 0, stream>>>((const TX*)x, (const TWT*)wr, topk_ids, topk_w,   \
+                                                          gate_out, hidden, n_experts, k, gate, renorm)
+  if (x_dtype == DT_F32 && w_dtype == DT_F32) ROUTER_LAUNCH(float, float);
+  else if (x_dtype == DT_BF16 && w_dtype == DT_BF16) ROUTER_LAUNCH(bf16_t, bf16_t);
+  else if (x_dtype == DT_BF16 && w_dtype == DT_F32) ROUTER_LAUNCH(bf16_t, float);
+  else if (x_dtype == DT_F32 && w_dtype == DT_BF16) ROUTER_LAUNCH(float, bf16_t);
+  else return SHARPI_ERR_ARG;
+#undef ROUTER_LAUNCH
+  SHARPI_CHECK_LAUNCH();
+  return SHARPI_OK;
+}
+
+__global__ __launch_bounds__(1024) void moe_permute_kernel(const int* __restrict__ topk_ids,
+                                                           const float* __restrict__ topk_w,
+                                                           int* __restrict__ offsets,
+                                                           int* __restrict__ sorted_token,
+                                                           float* __restrict__ sorted_w,
+                                                           int* __restrict__ inv_pos, int n_pairs, int k,
+                                                           int n_experts) {
+  __shared__ int count[kMaxExperts];
+  __shared__ int cursor[kMaxExperts];
+  for (int e = threadIdx.x; e < n_experts; e += blockDim.x) count[e] = 0;
+  __syncthreads();
+  for (int i = threadIdx.x; i < n_pairs; i += blockDim.x) atomicAdd(&count[topk_ids[i]], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0;
+    for (int e = 0; e < n_experts; ++e) {
+      offsets[e] = run;
+      cursor[e] = run;
+      run += count[e];
+    }
+    offsets[n_experts] = run;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < n_pairs; i += blockDim.x) {
+    const int e = topk_ids[i];
+    const int r = atomicAdd(&cursor[e], 1);
+    sorted_token[r] = i / k;
+    sorted_w[r] = topk_w[i];
+    inv_pos[i] = r;
+  }
+}
+
+SHARPI_EXPORT int sharpi_moe_permute(const int* topk_ids, const float* topk_w, int* offsets, int* sorted_token,
+                                     float* sorted_w, int* inv_pos, int n_tokens, int k, int n_experts,
+                                     hipStream_t stream) {
+  if (n_experts <= 0 || n_experts > kMaxExperts || k <= 0) return SHARPI_ERR_ARG;
+  if (n_tokens < 0) return SHARPI_ERR_ARG;
+  moe_permute_kernel<<<1, 1024, 0, stream>>>(topk_ids, topk_w, offsets, sorted_token, sorted_w, inv_pos,
+                                             n_tokens * k, k, n_experts);
+  SHARPI_CHECK_LAUNCH();
+  return SHARPI_OK;
+}

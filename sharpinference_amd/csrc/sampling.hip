@@ -1,0 +1,261 @@
+// Token selection from float logits [rows, vocab]: argmax, and temperature sampling with the
+// top-k / min-p / top-p filters, one block per row.
+//
+// argmax: the lowest index among equal maxima wins.
+// sample: p = softmax(logits / T); top-k keeps every p >= the k-th largest value and
+// renormalises; min-p zeroes p < min_p * max p; top-p keeps every p >= the value at which the
+// descending running sum first reaches top_p (equal values at that cut are all kept); after a
+// last renormalisation the token is the first index whose ascending running sum reaches u, or
+// vocab - 1 if rounding leaves none.  `probs` is a [rows, vocab] float workspace.
+#include "common.h"
+
+constexpr int kSampThreads = 1024;
+
+__device__ __forceinline__ float block_max(float v, float* red) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wid = threadIdx.x >> 6;
+  const int nw = (blockDim.x + kWave - 1) >> 6;
+  v = wave_max(v);
+  __syncthreads();
+  if (lane == 0) red[wid] = v;
+  __syncthreads();
+  float t = red[0];
+  for (int i = 1; i < nw; ++i) t = fmaxf(t, red[i]);
+  return t;
+}
+
+__global__ __launch_bounds__(kSampThreads) void argmax_rows_kernel(const float* __restrict__ logits,
+                                                                  int* __restrict__ out, int vocab) {
+  __shared__ float bv[kSampThreads / kWave];
+  __shared__ int bi[kSampThreads / kWave];
+  const float* x = logits + (size_t)blockIdx.x * vocab;
+  float best = -INFINITY;
+  int idx = 0x7fffffff;
+  for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
+    const float v = x[i];
+    if (v > best || idx == 0x7fffffff) {  // ascending i per thread: strict > keeps the lowest index
+      best = v;
+      idx = i;
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(best, off, kWave);
+    const int oi = __shfl_xor(idx, off, kWave);
+    if (oi != 0x7fffffff && (idx == 0x7fffffff || ov > best || (ov == best && oi < idx))) {
+      best = ov;
+      idx = oi;
+    }
+  }
+  const int lane = threadIdx.x & (kWave - 1), wid = threadIdx.x >> 6;
+  if (lane == 0) {
+    bv[wid] = best;
+    bi[wid] = idx;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int i = 1; i < (int)(blockDim.x >> 6); ++i) {
+      if (bi[i] != 0x7fffffff && (idx == 0x7fffffff || bv[i] > best || (bv[i] == best && bi[i] < idx))) {
+        best = bv[i];
+        idx = bi[i];
+      }
+    }
+    out[blockIdx.x] = idx == 0x7fffffff ? 0 : idx;
+  }
+}
+
+SHARPI_EXPORT int sharpi_argmax_rows(const float* logits, int* out, int rows, int vocab, hipStream_t stream) {
+  if (rows <= 0) return SHARPI_OK;
+  if (vocab <= 0) return SHARPI_ERR_ARG;
+  argmax_rows_kernel<<<rows, kSampThreads, 0, stream>>>(logits, out, vocab);
+  SHARPI_CHECK_LAUNCH();
+  return SHARPI_OK;
+}
+
+// count and sum of the entries of p with bits >= thr_bits (p >= 0, so float order == uint order)
+__device__ __forceinline__ void count_sum_ge(const float* p, int vocab, uint32_t thr_bits, float* red,
+                                             int* red_i, int& count, float& sum) {
+  int c = 0;
+  float s = 0.f;
+  for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
+    const float v = p[i];
+    if (__float_as_uint(v) >= thr_bits) {
+      ++c;
+      s += v;
+    }
+  }
+  sum = block_sum(s, red);
+  // integer block sum
+  const int lane = threadIdx.x & (kWave - 1), wid = threadIdx.x >> 6;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) c += __shfl_xor(c, off, kWave);
+  __syncthreads();
+  if (lane == 0) red_i[wid] = c;
+  __syncthreads();
+  int t = 0;
+  for (int i = 0; i < (int)(blockDim.x >> 6); ++i) t += red_i[i];
+  count = t;
+}
+
+__device__ __forceinline__ void renormalise(float* p, int vocab, float* red) {
+  float s = 0.f;
+  for (int i = threadIdx.x; i < vocab; i += blockDim.x) s += p[i];
+  const float total = block_sum(s, red);
+  if (total > 0.f && total != 1.0f) {
+    const float inv = 1.0f / total;
+    for (int i = threadIdx.x; i < vocab; i += blockDim.x) p[i] *= inv;
+  }
+  __syncthreads();
+}
+
+__global__ __launch_bounds__(kSampThreads) void sample_rows_kernel(
+    const float* __restrict__ logits, float* __restrict__ probs, const float* __restrict__ temperature,
+    const float* __restrict__ uniform, const int* __restrict__ top_k, const float* __restrict__ top_p,
+    const float* __restrict__ min_p, int* __restrict__ out, int vocab) {
+  __shared__ float red[16];
+  __shared__ int red_i[16];
+  __shared__ float chunk_prefix[kSampThreads];
+  __shared__ int winner;
+  const int r = blockIdx.x;
+  const float* x = logits + (size_t)r * vocab;
+  float* p = probs + (size_t)r * vocab;
+  const float T = temperature[r];
+  const float invT = 1.0f / T;
+
+  // softmax(logits / T)
+  float mx = -INFINITY;
+  for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
+    const float v = (T != 1.0f) ? x[i] * invT : x[i];
+    p[i] = v;
+    mx = fmaxf(mx, v);
+  }
+  mx = block_max(mx, red);
+  float s = 0.f;
+  for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
+    const float e = expf(p[i] - mx);
+    p[i] = e;
+    s += e;
+  }
+  const float inv_sum = 1.0f / block_sum(s, red);
+  for (int i = threadIdx.x; i < vocab; i += blockDim.x) p[i] *= inv_sum;
+  __syncthreads();
+
+  // top-k: largest threshold whose count of p >= threshold is still >= k
+  const int k = top_k ? top_k[r] : 0;
+  if (k > 0 && k < vocab) {
+    uint32_t lo = 0u, hi = 0x7f800000u;  // invariant: count(>= lo) >= k, count(>= hi + 1) < k
+    while (lo < hi) {
+      const uint32_t mid = lo + (hi - lo + 1) / 2;
+      int c;
+      float sm;
+      count_sum_ge(p, vocab, mid, red, red_i, c, sm);
+      if (c >= k) lo = mid; else hi = mid - 1;
+    }
+    for (int i = threadIdx.x; i < vocab; i += blockDim.x)
+      if (__float_as_uint(p[i]) < lo) p[i] = 0.f;
+    __syncthreads();
+    renormalise(p, vocab, red);
+  }
+  // min-p
+  const float mp = min_p ? min_p[r] : 0.f;
+  if (mp > 0.f) {
+    float pm = 0.f;
+    for (int i = threadIdx.x; i < vocab; i += blockDim.x) pm = fmaxf(pm, p[i]);
+    pm = block_max(pm, red);
+    const float thr = mp * pm;
+    for (int i = threadIdx.x; i < vocab; i += blockDim.x)
+      if (p[i] < thr) p[i] = 0.f;
+    __syncthreads();
+  }
+  // top-p: largest threshold whose sum of p >= threshold still reaches top_p
+  const float tp = top_p ? top_p[r] : 1.0f;
+  if (tp > 0.f && tp < 1.0f) {
+    uint32_t lo = 1u, hi = 0x7f800000u;  // bits 1 = smallest positive: keeps every non-zero entry
+    while (lo < hi) {
+      const uint32_t mid = lo + (hi - lo + 1) / 2;
+      int c;
+      float sm;
+      count_sum_ge(p, vocab, mid, red, red_i, c, sm);
+      if (sm >= tp) lo = mid; else hi = mid - 1;
+    }
+    for (int i = threadIdx.x; i < vocab; i += blockDim.x)
+      if (__float_as_uint(p[i]) < lo) p[i] = 0.f;
+    __syncthreads();
+  }
+  renormalise(p, vocab, red);
+
+  // inverse CDF: contiguous chunk per thread, ascending index
+  const int chunk = (vocab + blockDim.x - 1) / blockDim.x;
+  const int b = threadIdx.x * chunk;
+  const int e = min(b + chunk, vocab);
+  float cs = 0.f;
+  for (int i = b; i < e; ++i) cs += p[i];
+  chunk_prefix[threadIdx.x] = cs;
+  if (threadIdx.x == 0) winner = 0x7fffffff;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float run = 0.f;
+    for (int i = 0; i < (int)blockDim.x; ++i) {
+      const float c = chunk_prefix[i];
+      chunk_prefix[i] = run;
+      run += c;
+    }
+  }
+  __syncthreads();
+  const float u = uniform[r];
+  float run = chunk_prefix[threadIdx.x];
+  for (int i = b; i < e; ++i) {
+    run += p[i];
+    if (u <= run) {
+      atomicMin(&winner, i);
+      break;
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) out[r] = winner == 0x7fffffff ? vocab - 1 : winner;
+}
+
+SHARPI_EXPORT int sharpi_sample_rows(const float* logits, float* probs, const float* temperature,
+                                     const float* uniform, const int* top_k, const float* top_p,
+                                     const float* min_p, int* out, int rows, int vocab, hipStream_t stream) {
+  if (rows <= 0) return SHARPI_OK;
+  if (vocab <= 0) return SHARPI_ERR_ARG;
+  sample_rows_kernel<<<rows, kSampThreads, 0, stream>>>(logits, probs, temperature, uniform, top_k, top_p, min_p,
+                                                        out, vocab);
+  SHARPI_CHECK_LAUNCH();
+  return SHARPI_OK;
+}
+
+// Sparse logit edits before sampling (repetition / frequency / presence penalties, additive bias):
+// for entry i of row r (entries [row_offsets[r], row_offsets[r+1])): id = ids[i]
+//   x = logits[r, id]; if rep != 1: x = x > 0 ? x / rep : x * rep; x -= counts[i] * freq + pres (if count > 0);
+//   x += bias[i]
+__global__ void edit_logits_kernel(float* __restrict__ logits, const int* __restrict__ row_offsets,
+                                   const int* __restrict__ ids, const int* __restrict__ counts,
+                                   const float* __restrict__ bias, const float* __restrict__ rep,
+                                   const float* __restrict__ freq, const float* __restrict__ pres, int vocab) {
+  const int r = blockIdx.x;
+  float* x = logits + (size_t)r * vocab;
+  for (int i = row_offsets[r] + threadIdx.x; i < row_offsets[r + 1]; i += blockDim.x) {
+    const int id = ids[i];
+    if (id < 0 || id >= vocab) continue;
+    float v = x[id] + bias[i];
+    const int c = counts[i];
+    if (c > 0) {
+      const float rp = rep[r];
+      if (rp != 1.0f) v = v > 0.f ? v / rp : v * rp;
+      v -= (float)c * freq[r] + pres[r];
+    }
+    x[id] = v;
+  }
+}
+
+SHARPI_EXPORT int sharpi_edit_logits(float* logits, const int* row_offsets, const int* ids, const int* counts,
+                                     const float* bias, const float* rep, const float* freq, const float* pres,
+                                     int rows, int vocab, hipStream_t stream) {
+  if (rows <= 0) return SHARPI_OK;
+  if (vocab <= 0) return SHARPI_ERR_ARG;
+  edit_logits_kernel<<<rows, 256, 0, stream>>>(logits, row_offsets, ids, counts, bias, rep, freq, pres, vocab);
+  SHARPI_CHECK_LAUNCH();
+  return SHARPI_OK;
+}

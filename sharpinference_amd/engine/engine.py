@@ -1,0 +1,180 @@
+"""The engine: a model folder (or a configuration and a seed) turned into something that steps
+and generates.  This is the Python entry point; the command line and trace replay are thin
+layers over it.
+
+The reference's library API streams chunks from ``GenerateChunksAsync(prompt, SamplingParams)``
+(reference: src/SharpInference.Engine/IInferenceEngine.cs:60-64); there is no tokenizer here, so
+prompts are lists of token ids and results are lists of token ids.
+"""
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass, field
+from typing import Dict, Hashable, List, Optional, Sequence, Union
+
+import torch
+
+from ..cache.manager import CacheManager
+from ..config.base import ModelConfig, load_config
+from ..registry import build_model
+from ..sampling.params import SamplingParams
+from ..sampling.sampler import Sampler, penalty_window
+from ..weights.loader import RandomSource, SafetensorsSource, load_model_weights
+from .runner import ModelRunner, StepEntry
+from .scheduler import Request, Scheduler
+
+_DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
+           torch.bfloat16: torch.bfloat16, torch.float32: torch.float32}
+
+
+def parse_dtype(dtype) -> torch.dtype:
+    try:
+        return _DTYPES[dtype]
+    except KeyError:
+        raise ValueError(f"dtype {dtype!r} is not supported (bfloat16 or float32)") from None
+
+
+@dataclass
+class GenerationResult:
+    token_ids: List[int]
+    finish_reason: str
+    prompt_tokens: int
+
+
+@dataclass
+class GenerationStats:
+    prefill_tokens: int = 0
+    decode_tokens: int = 0
+    prefill_seconds: float = 0.0
+    decode_seconds: float = 0.0
+    steps: int = 0
+
+
+class Engine:
+    def __init__(self, model_dir: Optional[str] = None, *, config: Union[ModelConfig, dict, None] = None,
+                 weight_seed: Optional[int] = None, dtype="bfloat16", device="cuda:0",
+                 max_model_len: Optional[int] = None, max_num_seqs: int = 8, max_tokens_per_step: int = 2048,
+                 kv_tokens: Optional[int] = None, page_size: int = 16, weight_std: float = 0.02,
+                 weight_std_by_suffix: Optional[Dict[str, float]] = None, verbose: bool = False):
+        self.dtype = parse_dtype(dtype)
+        self.device = torch.device(device)
+        if self.device.type != "cuda":
+            raise RuntimeError("the engine runs on the GPU only (device must be cuda:N)")
+        if not torch.cuda.is_available():
+            raise RuntimeError("no GPU is visible: the engine has no CPU path")
+        from ..ops import lib as _kernel_lib
+
+        _kernel_lib.load(verbose=True)                      # fails loudly if the kernels are missing
+        torch.cuda.set_device(self.device)
+        if model_dir is not None:
+            self.config = load_config(model_dir)
+        elif isinstance(config, dict):
+            self.config = load_config(config)
+        elif config is not None:
+            self.config = config
+            self.config.validate()
+        else:
+            raise ValueError("give a model folder or a configuration")
+        self.model = build_model(self.config)
+        if model_dir is not None:
+            source = SafetensorsSource(model_dir, self.dtype, self.device)
+        else:
+            if weight_seed is None:
+                raise ValueError("a configuration without a model folder needs weight_seed (random weights)")
+            source = RandomSource(self.model.param_specs(), weight_seed, self.dtype, self.device,
+                                  stored_dtype=torch.bfloat16, std=weight_std, std_by_suffix=weight_std_by_suffix,
+                                  generate_on_device=True)
+        t0 = time.time()
+        load_model_weights(self.model, source)
+        if verbose:
+            print(f"[engine] weights ready in {time.time() - t0:.1f}s", flush=True)
+        limit = getattr(self.config, "max_position_embeddings", 0) or 0
+        self.max_model_len = int(max_model_len or limit or 4096)
+        if limit and self.max_model_len > limit:
+            raise ValueError(f"max_model_len {self.max_model_len} exceeds the model's max_position_embeddings {limit}")
+        self.max_num_seqs = int(max_num_seqs)
+        self.max_tokens_per_step = int(max_tokens_per_step)
+        self.page_size = int(page_size)
+        if kv_tokens is None:
+            kv_tokens = self.max_num_seqs * ((self.max_model_len + page_size - 1) // page_size * page_size)
+        num_pages = max(1, (int(kv_tokens) + page_size - 1) // page_size)
+        self.cache = CacheManager(self.model.cache_specs(), page_size, num_pages, self.max_num_seqs, self.dtype,
+                                  self.device)
+        self.runner = ModelRunner(self.model, self.cache, self.dtype, self.device)
+        self.sampler = Sampler(self.device)
+        self.last_stats = GenerationStats()
+
+    # -- the low level: requests and steps ------------------------------------
+    def add_request(self, req_id: Hashable) -> None:
+        self.cache.add_request(req_id)
+
+    def free_request(self, req_id: Hashable) -> None:
+        self.cache.free_request(req_id)
+
+    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        return self.runner.step(entries)
+
+    # -- generation -------------------------------------------------------------
+    def generate(self, prompts: Sequence[Sequence[int]], params: Union[SamplingParams, Sequence[SamplingParams], None] = None,
+                 *, max_new_tokens: Optional[int] = None, temperature: Optional[float] = None,
+                 seeds: Optional[Sequence[int]] = None, stop_token_ids: Sequence[int] = ()) -> List[GenerationResult]:
+        """Generate for a list of prompts (token ids) under continuous batching."""
+        plist: List[SamplingParams] = []
+        for i in range(len(prompts)):
+            if isinstance(params, SamplingParams):
+                p = SamplingParams(**{**params.__dict__})
+            elif params is not None:
+                p = params[i]
+            else:
+                p = SamplingParams(temperature=0.0)
+            if max_new_tokens is not None:
+                p.max_new_tokens = int(max_new_tokens)
+            if temperature is not None:
+                p.temperature = float(temperature)
+            if seeds is not None:
+                p.seed = int(seeds[i])
+            if stop_token_ids:
+                p.stop_token_ids = tuple(int(t) for t in stop_token_ids)
+            plist.append(p)
+        sched = Scheduler(self.cache, self.max_num_seqs, self.max_tokens_per_step, self.max_model_len)
+        reqs = [Request(("gen", i), [int(t) for t in prompt], plist[i]) for i, prompt in enumerate(prompts)]
+        for r in reqs:
+            sched.add(r)
+        stats = GenerationStats()
+        try:
+            while sched.has_work():
+                batch = sched.schedule()
+                if not batch:
+                    if sched.has_work():
+                        raise RuntimeError("scheduler has work but nothing can run")
+                    break
+                t0 = time.perf_counter()
+                entries = [StepEntry(s.request.req_id, s.tokens, (len(s.tokens) - 1,) if s.samples else ())
+                           for s in batch]
+                logits = self.runner.step(entries)
+                sampling = [s for s in batch if s.samples]
+                tokens: List[Optional[int]] = [None] * len(batch)
+                if sampling:
+                    hist = [penalty_window(s.request.params, s.request.prompt, s.request.output)
+                            if s.request.params.edits_logits else () for s in sampling]
+                    picked = self.sampler.sample(logits, [s.request.params for s in sampling],
+                                                 [s.request.draws for s in sampling], hist)
+                    it = iter(picked)
+                    tokens = [next(it) if s.samples else None for s in batch]
+                dt = time.perf_counter() - t0
+                n_prefill = sum(len(s.tokens) for s in batch if s.request.in_prefill)
+                n_decode = sum(1 for s in batch if not s.request.in_prefill)
+                if n_prefill:
+                    stats.prefill_tokens += n_prefill
+                    stats.prefill_seconds += dt * n_prefill / (n_prefill + n_decode)
+                if n_decode:
+                    stats.decode_tokens += n_decode
+                    stats.decode_seconds += dt * n_decode / (n_prefill + n_decode)
+                stats.steps += 1
+                sched.update(batch, tokens)
+        finally:
+            for r in list(sched.running):                  # an error mid-way: give everything back
+                if self.cache.has_request(r.req_id):
+                    self.cache.free_request(r.req_id)
+        self.last_stats = stats
+        return [GenerationResult(r.output, r.finish_reason or "abort", len(r.prompt)) for r in reqs]

@@ -1,0 +1,153 @@
+"""The step function: one batch of (request, its next tokens) through the model, from the cache.
+
+The reference has three batched entry points that never mix prompt portions with decoded
+tokens (reference: src/SharpInference.Engine/IBatchedForwardPass.cs:27-69;
+src/SharpInference.Engine/ContinuousBatchingEngine.cs:306-347).  Here there is one: a step takes
+any number of entries, each a request with one or more next tokens, runs exactly those tokens
+as one flat batch against what earlier steps left in the cache, and returns float32 logits at
+the wanted places.  Lengths advance only when the step has run (the reference is transactional
+in the same way, src/SharpInference.Engine/CudaForwardPass.cs:4894, 4985-4986).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Hashable, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache.manager import CacheError, CacheManager
+from ..parts.base import GroupView, LayerCache, StepContext
+
+
+class CacheExhausted(CacheError):
+    """A step needed more pages than the pools hold; nothing was changed."""
+
+
+@dataclass
+class StepEntry:
+    req_id: Hashable
+    tokens: Sequence[int]
+    want: Sequence[int] = field(default_factory=tuple)   # places among `tokens` whose logits are asked for
+
+
+class ModelRunner:
+    def __init__(self, model, cache: CacheManager, act_dtype: torch.dtype, device):
+        self.model = model
+        self.cache = cache
+        self.act_dtype = act_dtype
+        self.device = torch.device(device)
+        self.steps_run = 0
+
+    # ------------------------------------------------------------------
+    def _validate(self, entries: Sequence[StepEntry]) -> None:
+        seen = set()
+        vocab = self.model.vocab_size
+        for e in entries:
+            if e.req_id in seen:
+                raise ValueError(f"request {e.req_id!r} appears twice in one step")
+            seen.add(e.req_id)
+            if not self.cache.has_request(e.req_id):
+                raise ValueError(f"request {e.req_id!r} is not in the cache (add_request first)")
+            if len(e.tokens) == 0:
+                raise ValueError(f"request {e.req_id!r} brings no tokens")
+            for t in e.tokens:
+                if not 0 <= int(t) < vocab:
+                    raise ValueError(f"request {e.req_id!r}: token id {t} outside the vocabulary of {vocab}")
+            for w in e.want:
+                if not 0 <= int(w) < len(e.tokens):
+                    raise ValueError(f"request {e.req_id!r}: wanted place {w} outside its {len(e.tokens)} tokens")
+
+    def build_context(self, entries: Sequence[StepEntry]):
+        """Host side of a step: lay the batch out flat and pack all index arrays into one upload."""
+        cache = self.cache
+        ps = cache.page_size
+        n = len(entries)
+        lens = [len(e.tokens) for e in entries]
+        starts = [cache.length(e.req_id) for e in entries]
+        T = sum(lens)
+        token_ids = np.empty(T, dtype=np.int32)
+        positions = np.empty(T, dtype=np.int32)
+        entry_of = np.empty(T, dtype=np.int32)
+        cu = np.zeros(n + 1, dtype=np.int32)
+        rows: List[int] = []
+        o = 0
+        for i, e in enumerate(entries):
+            L = lens[i]
+            token_ids[o:o + L] = np.asarray(e.tokens, dtype=np.int32)
+            positions[o:o + L] = np.arange(starts[i], starts[i] + L, dtype=np.int32)
+            entry_of[o:o + L] = i
+            rows.extend(o + int(w) for w in e.want)
+            o += L
+            cu[i + 1] = o
+        state_slots = np.asarray([cache.requests[e.req_id].state_slot for e in entries], dtype=np.int32)
+        group_tables, group_slots = [], []
+        for g in range(len(cache.groups)):
+            tables = [cache.block_table(e.req_id, g) for e in entries]
+            maxb = max(1, max(len(t) for t in tables))
+            maxb = (maxb + 3) // 4 * 4
+            bt = np.full((n, maxb), -1, dtype=np.int32)
+            for i, t in enumerate(tables):
+                bt[i, :len(t)] = t
+            sm = np.empty(T, dtype=np.int32)
+            for i in range(n):
+                pos = positions[cu[i]:cu[i + 1]]
+                pages = bt[i, pos // ps]
+                if (pages < 0).any():
+                    raise CacheError(f"request {entries[i].req_id!r}: a new position has no page in group {g}")
+                sm[cu[i]:cu[i + 1]] = pages * ps + pos % ps
+            group_tables.append(bt)
+            group_slots.append(sm)
+        rows_np = np.asarray(rows, dtype=np.int32)
+        pieces = [token_ids, positions, entry_of, cu, state_slots, np.full(T, -1, dtype=np.int32), rows_np]
+        for bt, sm in zip(group_tables, group_slots):
+            pieces += [bt.reshape(-1), sm]
+        flat = np.concatenate(pieces) if pieces else np.zeros(0, dtype=np.int32)
+        dev = torch.from_numpy(flat).to(self.device)
+        views, off = [], 0
+        for p in pieces:
+            views.append(dev[off:off + p.size])
+            off += p.size
+        d_tok, d_pos, d_ent, d_cu, d_state, d_nostore, d_rows = views[:7]
+        groups = []
+        for g in range(len(cache.groups)):
+            bt = views[7 + 2 * g].view(n, group_tables[g].shape[1])
+            groups.append(GroupView(bt, views[8 + 2 * g], ps, max_context=int(positions.max()) + 1 if T else 0))
+        ctx = StepContext(n_tokens=T, n_entries=n, token_ids=d_tok, positions=d_pos, entry_of_token=d_ent,
+                          cu_tokens=d_cu, state_slots=d_state, groups=groups, act_dtype=self.act_dtype,
+                          no_store_slots=d_nostore, entry_lens=lens, entry_starts=starts,
+                          max_entry_len=max(lens) if lens else 1)
+        return ctx, (d_rows if rows else None)
+
+    def layer_caches(self, ctx: StepContext) -> List[LayerCache]:
+        cache = self.cache
+        out = []
+        for i in range(len(cache.slot_specs)):
+            g = cache.group_of_slot[i]
+            out.append(LayerCache(group=ctx.groups[g] if g >= 0 else None, k=cache.k[i], v=cache.v[i],
+                                  state=cache.state[i], write=True))
+        return out
+
+    # ------------------------------------------------------------------
+    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        """Run one batch.  Returns float32 logits [wanted, vocab] in the order of the entries and
+        of their ``want`` lists, or None when nothing is wanted."""
+        if not entries:
+            return None
+        self._validate(entries)
+        appended = []
+        try:
+            for e in entries:
+                if not self.cache.append(e.req_id, len(e.tokens)):
+                    raise CacheExhausted(f"no pages left for request {e.req_id!r} ({len(e.tokens)} more tokens)")
+                appended.append(e.req_id)
+            ctx, rows = self.build_context(entries)
+            logits = self.model.forward(ctx, self.layer_caches(ctx), rows)
+        except BaseException:
+            for r in appended:
+                self.cache.rollback(r)
+            raise
+        for e in entries:
+            self.cache.commit(e.req_id)
+        self.steps_run += 1
+        return logits

@@ -1,0 +1,329 @@
+"""Python faces of the HIP kernels.
+
+Every function checks on the host that shapes, dtypes and devices are what the kernel and its
+grid assume, then launches on torch's current stream.  Tensors are only memory here: no torch
+arithmetic runs on the product path except the library matrix product in :func:`linear`.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import lib as _lib
+
+_DT = {torch.float32: 0, torch.bfloat16: 1}
+
+WINDOW_NONE, WINDOW_CHUNK, WINDOW_SLIDING = 0, 1, 2
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _code(dtype: torch.dtype) -> int:
+    try:
+        return _DT[dtype]
+    except KeyError:
+        raise KernelError(f"dtype {dtype} is not taken by the kernels (float32 or bfloat16)") from None
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelError(msg)
+
+
+def _dev(*ts) -> None:
+    for t in ts:
+        if t is not None:
+            _need(t.is_cuda, "kernel operands must live on the GPU")
+            _need(t.is_contiguous(), "kernel operands must be contiguous")
+
+
+def _i32(t: Optional[torch.Tensor], name: str) -> None:
+    if t is not None:
+        _need(t.dtype == torch.int32, f"{name} must be int32")
+
+
+def _run(name: str, *args) -> None:
+    rc = getattr(_lib.load(), name)(*args)
+    if rc != 0:
+        what = {1001: "a size or option the kernel does not take", 1002: "launch failed"}.get(rc, f"HIP error {rc}")
+        raise KernelError(f"{name}: {what}")
+
+
+# ---------------------------------------------------------------------------
+def embed_gather(ids: torch.Tensor, table: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[t] = table[ids[t]] as float32 (the residual stream)."""
+    _dev(ids, table, out)
+    _i32(ids, "ids")
+    _need(ids.dim() == 1 and table.dim() == 2, "embed_gather: ids [T], table [V, H]")
+    T, H = ids.shape[0], table.shape[1]
+    if out is None:
+        out = torch.empty(T, H, dtype=torch.float32, device=table.device)
+    _need(out.shape == (T, H) and out.dtype == torch.float32, "embed_gather: out must be float32 [T, H]")
+    _run("sharpi_embed_gather", _ptr(ids), _ptr(table), _code(table.dtype), _ptr(out), T, H, _stream())
+    return out
+
+
+def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: Optional[torch.Tensor], eps: float,
+                out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None, write_back: bool = True,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """(h + delta) -> RMSNorm -> out; the sum goes back into h unless rows are gathered."""
+    _dev(h, delta, weight, rows, out)
+    _i32(rows, "rows")
+    _need(h.dim() == 2 and h.dtype == torch.float32, "add_rmsnorm: h must be float32 [T, H]")
+    T, H = h.shape
+    if delta is not None:
+        _need(delta.shape == h.shape, f"add_rmsnorm: delta {tuple(delta.shape)} vs h {tuple(h.shape)}")
+    if weight is not None:
+        _need(weight.shape == (H,), f"add_rmsnorm: weight {tuple(weight.shape)} vs width {H}")
+    n_out = T if rows is None else rows.shape[0]
+    if rows is not None:
+        write_back = False
+    if out is None:
+        out = torch.empty(n_out, H, dtype=out_dtype, device=h.device)
+    _need(out.shape == (n_out, H) and out.dtype == out_dtype, "add_rmsnorm: out has the wrong shape or dtype")
+    _run("sharpi_add_rmsnorm", _ptr(h), _ptr(delta), _code(delta.dtype) if delta is not None else 0,
+         _ptr(weight), _code(weight.dtype) if weight is not None else 0, _ptr(out), _code(out_dtype), _ptr(rows),
+         n_out, H, float(eps), 1 if write_back else 0, _stream())
+    return out
+
+
+def silu_mul(gate_up: torch.Tensor, scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """[M, 2I] (gate columns, then up columns) -> silu(s*g) * (s*u) [M, I]."""
+    _dev(gate_up, scale)
+    _need(gate_up.dim() == 2 and gate_up.shape[1] % 2 == 0, "silu_mul: input must be [M, 2I]")
+    M, I2 = gate_up.shape
+    if scale is not None:
+        _need(scale.dtype == torch.float32 and scale.shape == (M,), "silu_mul: scale must be float32 [M]")
+    out = torch.empty(M, I2 // 2, dtype=gate_up.dtype, device=gate_up.device)
+    _run("sharpi_silu_mul", _ptr(gate_up), _ptr(scale), _ptr(out), _code(gate_up.dtype), M, I2 // 2, _stream())
+    return out
+
+
+def moe_combine(y: torch.Tensor, inv_pos: torch.Tensor, shared: Optional[torch.Tensor], n_tokens: int,
+                k: int) -> torch.Tensor:
+    """out[t] = sum_j y[inv_pos[t*k+j]] (+ shared[t])."""
+    _dev(y, inv_pos, shared)
+    _i32(inv_pos, "inv_pos")
+    _need(y.dim() == 2 and y.shape[0] == n_tokens * k and inv_pos.numel() == n_tokens * k,
+          "moe_combine: y must be [T*k, H] and inv_pos [T*k]")
+    H = y.shape[1]
+    if shared is not None:
+        _need(shared.shape == (n_tokens, H) and shared.dtype == y.dtype, "moe_combine: shared must be [T, H]")
+    out = torch.empty(n_tokens, H, dtype=y.dtype, device=y.device)
+    _run("sharpi_moe_combine", _ptr(y), _ptr(inv_pos), _ptr(shared), _ptr(out), _code(y.dtype), n_tokens, H, k,
+         _stream())
+    return out
+
+
+def cast(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    _dev(x)
+    out = torch.empty(x.shape, dtype=dtype, device=x.device)
+    _run("sharpi_cast", _ptr(x), _code(x.dtype), _ptr(out), _code(dtype), x.numel(), _stream())
+    return out
+
+
+# ---------------------------------------------------------------------------
+def rope_kv(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, slot_mapping: torch.Tensor,
+            positions: torch.Tensor, inv_freq: Optional[torch.Tensor], qk_norm: bool, eps: float,
+            temperature: Optional[Tuple[float, float]], nh: int, nkv: int, hd: int) -> torch.Tensor:
+    """Rotate / norm / scale the heads of qkv [T, (nh+2nkv)*hd]; K and V go into the layer's
+    cache [pages, nkv, page_size, hd] at slot_mapping; returns q [T, nh*hd]."""
+    _dev(qkv, k_cache, v_cache, slot_mapping, positions, inv_freq)
+    _i32(slot_mapping, "slot_mapping")
+    _i32(positions, "positions")
+    T = qkv.shape[0]
+    _need(qkv.dim() == 2 and qkv.shape[1] == (nh + 2 * nkv) * hd, "rope_kv: qkv must be [T, (nh+2nkv)*hd]")
+    _need(k_cache.dim() == 4 and k_cache.shape[1] == nkv and k_cache.shape[3] == hd and
+          v_cache.shape == k_cache.shape, "rope_kv: cache must be [pages, nkv, page_size, hd]")
+    _need(k_cache.dtype == qkv.dtype and v_cache.dtype == qkv.dtype, "rope_kv: cache dtype differs from qkv's")
+    _need(slot_mapping.shape == (T,) and positions.shape == (T,), "rope_kv: slot_mapping / positions must be [T]")
+    if inv_freq is not None:
+        _need(inv_freq.dtype == torch.float32 and inv_freq.shape == (hd // 2,), "rope_kv: inv_freq must be float32 [hd/2]")
+    page_size = k_cache.shape[2]
+    q_out = torch.empty(T, nh * hd, dtype=qkv.dtype, device=qkv.device)
+    fs, asc = temperature if temperature is not None else (1.0, 0.0)
+    _run("sharpi_rope_kv", _ptr(qkv), _ptr(q_out), _ptr(k_cache), _ptr(v_cache), _code(qkv.dtype),
+         _ptr(slot_mapping), _ptr(positions), _ptr(inv_freq), 1 if qk_norm else 0, float(eps),
+         1 if temperature is not None else 0, float(fs), float(asc), T, nh, nkv, hd, page_size, _stream())
+    return q_out
+
+
+def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
+                      entry_of_token: torch.Tensor, positions: torch.Tensor, window_kind: int, window: int,
+                      scale: float, nh: int, nkv: int, hd: int) -> torch.Tensor:
+    """Attention of every token of the batch over its request's pages; float arithmetic."""
+    _dev(q, k_cache, v_cache, block_table, entry_of_token, positions)
+    _i32(block_table, "block_table")
+    _i32(entry_of_token, "entry_of_token")
+    _i32(positions, "positions")
+    T = q.shape[0]
+    _need(q.shape == (T, nh * hd), "attention: q must be [T, nh*hd]")
+    _need(k_cache.dim() == 4 and k_cache.shape[1] == nkv and k_cache.shape[3] == hd and
+          v_cache.shape == k_cache.shape and k_cache.dtype == q.dtype, "attention: cache must be [pages, nkv, page_size, hd] of q's dtype")
+    _need(block_table.dim() == 2, "attention: block_table must be [entries, max_blocks]")
+    _need(entry_of_token.shape == (T,) and positions.shape == (T,), "attention: per-token arrays must be [T]")
+    out = torch.empty_like(q)
+    _run("sharpi_attention_generic", _ptr(q), _ptr(k_cache), _ptr(v_cache), _code(q.dtype), _ptr(block_table),
+         _ptr(entry_of_token), _ptr(positions), _ptr(out), int(window_kind), int(window), float(scale), T, nh, nkv,
+         hd, k_cache.shape[2], block_table.shape[1], k_cache.shape[0], _stream())
+    return out
+
+
+# ---------------------------------------------------------------------------
+def gemm_tiled(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """x [M, K] @ w [N, K]^T with float FMA chains (batch-invariant)."""
+    _dev(x, w)
+    _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], f"gemm: x {tuple(x.shape)} vs w {tuple(w.shape)}")
+    _need(x.dtype == w.dtype, "gemm: x and w must share a dtype")
+    out_dtype = out_dtype or x.dtype
+    M, K = x.shape
+    N = w.shape[0]
+    out = torch.empty(M, N, dtype=out_dtype, device=x.device)
+    _run("sharpi_gemm_tiled", _ptr(x), _ptr(w), _ptr(out), _code(x.dtype), _code(out_dtype), M, N, K, None, None, 0,
+         _stream())
+    return out
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """y = x W^T.  float32 weights: the float FMA kernel (true 32-bit, whatever x was stored
+    as).  bfloat16 weights: the library's matrix product with float accumulation."""
+    out_dtype = out_dtype or x.dtype
+    if w.dtype == torch.float32:
+        xf = x if x.dtype == torch.float32 else cast(x, torch.float32)
+        y = gemm_tiled(xf, w, torch.float32)
+        return y if out_dtype == torch.float32 else cast(y, out_dtype)
+    _dev(x, w)
+    xb = x if x.dtype == torch.bfloat16 else cast(x, torch.bfloat16)
+    _need(xb.shape[1] == w.shape[1], f"linear: x {tuple(x.shape)} vs w {tuple(w.shape)}")
+    if out_dtype == torch.bfloat16:
+        return torch.mm(xb, w.t())
+    return torch.mm(xb, w.t(), out_dtype=torch.float32)
+
+
+def grouped_gemm(x: torch.Tensor, w: torch.Tensor, offsets: torch.Tensor, a_rows: Optional[torch.Tensor],
+                 n_rows: int) -> torch.Tensor:
+    """Rows [offsets[e], offsets[e+1]) of the expert-sorted list times w[e]^T.
+    x rows are read through a_rows when given; w is [E, N, K]; returns [n_rows, N]."""
+    _dev(x, w, offsets, a_rows)
+    _i32(offsets, "offsets")
+    _i32(a_rows, "a_rows")
+    _need(w.dim() == 3 and x.dim() == 2 and x.shape[1] == w.shape[2] and x.dtype == w.dtype,
+          f"grouped_gemm: x {tuple(x.shape)} vs w {tuple(w.shape)}")
+    E, N, K = w.shape
+    _need(offsets.shape == (E + 1,), "grouped_gemm: offsets must be [E + 1]")
+    if a_rows is not None:
+        _need(a_rows.shape == (n_rows,), "grouped_gemm: a_rows must be [n_rows]")
+    else:
+        _need(x.shape[0] == n_rows, "grouped_gemm: x must have n_rows rows when not gathered")
+    out = torch.empty(n_rows, N, dtype=x.dtype, device=x.device)
+    _run("sharpi_gemm_tiled", _ptr(x), _ptr(w), _ptr(out), _code(x.dtype), _code(x.dtype), n_rows, N, K, _ptr(a_rows),
+         _ptr(offsets), E, _stream())
+    return out
+
+
+# ---------------------------------------------------------------------------
+GATE_SIGMOID, GATE_SOFTMAX = 0, 1
+
+
+def router_topk(x: torch.Tensor, wr: torch.Tensor, k: int, gate: int = GATE_SIGMOID, renorm: bool = False,
+                want_gates: bool = False):
+    """Router logits in float, gate, k picks (lowest index wins a tie).
+    Returns ids int32 [T, k], weights float32 [T, k] (and the gate values [T, E] if asked)."""
+    _dev(x, wr)
+    _need(x.dim() == 2 and wr.dim() == 2 and x.shape[1] == wr.shape[1], "router: x [T, H], wr [E, H]")
+    T, H = x.shape
+    E = wr.shape[0]
+    ids = torch.empty(T, k, dtype=torch.int32, device=x.device)
+    wts = torch.empty(T, k, dtype=torch.float32, device=x.device)
+    gates = torch.empty(T, E, dtype=torch.float32, device=x.device) if want_gates else None
+    _run("sharpi_router_topk", _ptr(x), _code(x.dtype), _ptr(wr), _code(wr.dtype), _ptr(ids), _ptr(wts), _ptr(gates),
+         T, H, E, k, gate, 1 if renorm else 0, _stream())
+    return (ids, wts, gates) if want_gates else (ids, wts)
+
+
+def moe_permute(ids: torch.Tensor, wts: torch.Tensor, n_experts: int):
+    """(token, pick) pairs sorted by expert: offsets [E+1], sorted_token, sorted_w, inv_pos."""
+    _dev(ids, wts)
+    _i32(ids, "ids")
+    _need(ids.shape == wts.shape and wts.dtype == torch.float32 and ids.dim() == 2, "moe_permute: ids/wts [T, k]")
+    T, k = ids.shape
+    dev = ids.device
+    offsets = torch.empty(n_experts + 1, dtype=torch.int32, device=dev)
+    sorted_token = torch.empty(T * k, dtype=torch.int32, device=dev)
+    sorted_w = torch.empty(T * k, dtype=torch.float32, device=dev)
+    inv_pos = torch.empty(T * k, dtype=torch.int32, device=dev)
+    _run("sharpi_moe_permute", _ptr(ids), _ptr(wts), _ptr(offsets), _ptr(sorted_token), _ptr(sorted_w), _ptr(inv_pos),
+         T, k, n_experts, _stream())
+    return offsets, sorted_token, sorted_w, inv_pos
+
+
+# ---------------------------------------------------------------------------
+def argmax_rows(logits: torch.Tensor) -> torch.Tensor:
+    _dev(logits)
+    _need(logits.dim() == 2 and logits.dtype == torch.float32, "argmax: logits must be float32 [rows, vocab]")
+    out = torch.empty(logits.shape[0], dtype=torch.int32, device=logits.device)
+    _run("sharpi_argmax_rows", _ptr(logits), _ptr(out), logits.shape[0], logits.shape[1], _stream())
+    return out
+
+
+def sample_rows(logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tensor,
+                top_k: Optional[torch.Tensor] = None, top_p: Optional[torch.Tensor] = None,
+                min_p: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _dev(logits, temperature, uniform, top_k, top_p, min_p)
+    _need(logits.dim() == 2 and logits.dtype == torch.float32, "sample: logits must be float32 [rows, vocab]")
+    R = logits.shape[0]
+    for name, t, dt in (("temperature", temperature, torch.float32), ("uniform", uniform, torch.float32),
+                        ("top_k", top_k, torch.int32), ("top_p", top_p, torch.float32), ("min_p", min_p, torch.float32)):
+        if t is not None:
+            _need(t.shape == (R,) and t.dtype == dt, f"sample: {name} must be {dt} [rows]")
+    probs = torch.empty_like(logits)
+    out = torch.empty(R, dtype=torch.int32, device=logits.device)
+    _run("sharpi_sample_rows", _ptr(logits), _ptr(probs), _ptr(temperature), _ptr(uniform), _ptr(top_k), _ptr(top_p),
+         _ptr(min_p), _ptr(out), R, logits.shape[1], _stream())
+    return out
+
+
+def edit_logits(logits: torch.Tensor, row_offsets: torch.Tensor, ids: torch.Tensor, counts: torch.Tensor,
+                bias: torch.Tensor, rep: torch.Tensor, freq: torch.Tensor, pres: torch.Tensor) -> None:
+    _dev(logits, row_offsets, ids, counts, bias, rep, freq, pres)
+    _need(logits.dim() == 2 and logits.dtype == torch.float32, "edit_logits: logits must be float32 [rows, vocab]")
+    R = logits.shape[0]
+    _i32(row_offsets, "row_offsets"); _i32(ids, "ids"); _i32(counts, "counts")
+    _need(row_offsets.shape == (R + 1,), "edit_logits: row_offsets must be [rows + 1]")
+    n = ids.shape[0]
+    _need(counts.shape == (n,) and bias.shape == (n,) and bias.dtype == torch.float32, "edit_logits: per-entry arrays")
+    for t in (rep, freq, pres):
+        _need(t.shape == (R,) and t.dtype == torch.float32, "edit_logits: per-row arrays must be float32 [rows]")
+    _run("sharpi_edit_logits", _ptr(logits), _ptr(row_offsets), _ptr(ids), _ptr(counts), _ptr(bias), _ptr(rep),
+         _ptr(freq), _ptr(pres), R, logits.shape[1], _stream())
+
+
+# ---------------------------------------------------------------------------
+# dispatchers used by the parts
+# ---------------------------------------------------------------------------
+def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, group, ctx, window_kind: int,
+              window: int, scale: float, nh: int, nkv: int, hd: int) -> torch.Tensor:
+    """Attention of the step's tokens over their requests' pages (`group`: the cache group's
+    block tables, `ctx`: the step)."""
+    return attention_generic(q, k_cache, v_cache, group.block_table, ctx.entry_of_token, ctx.positions, window_kind,
+                             window, scale, nh, nkv, hd)
+
+
+def grouped_linear(x: torch.Tensor, w: torch.Tensor, offsets: torch.Tensor, a_rows: Optional[torch.Tensor],
+                   n_rows: int, out_dtype: torch.dtype) -> torch.Tensor:
+    """Per-expert products over the expert-sorted row list (see grouped_gemm)."""
+    if x.dtype != w.dtype:
+        x = cast(x, w.dtype)
+    y = grouped_gemm(x, w, offsets, a_rows, n_rows)
+    return y if y.dtype == out_dtype else cast(y, out_dtype)

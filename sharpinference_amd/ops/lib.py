@@ -1,0 +1,81 @@
+"""Loads the HIP kernel library and declares its entry points for ctypes.
+
+There is no fallback: without the library (and without a way to build it) importing an op
+raises, so a GPU run can never silently use something else.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_longlong, c_void_p
+from typing import Optional
+
+_lib: Optional[ctypes.CDLL] = None
+_lib_path: Optional[str] = None
+
+P = c_void_p
+I = c_int
+F = c_float
+
+_SIGNATURES = {
+    "sharpi_embed_gather": [P, P, I, P, I, I, P],
+    "sharpi_add_rmsnorm": [P, P, I, P, I, P, I, P, I, I, F, I, P],
+    "sharpi_silu_mul": [P, P, P, I, I, I, P],
+    "sharpi_moe_combine": [P, P, P, P, I, I, I, I, P],
+    "sharpi_cast": [P, I, P, I, c_longlong, P],
+    "sharpi_rope_kv": [P, P, P, P, I, P, P, P, I, F, I, F, F, I, I, I, I, I, P],
+    "sharpi_attention_generic": [P, P, P, I, P, P, P, P, I, I, F, I, I, I, I, I, I, I, P],
+    "sharpi_gemm_tiled": [P, P, P, I, I, I, I, I, P, P, I, P],
+    "sharpi_router_topk": [P, I, P, I, P, P, P, I, I, I, I, I, I, P],
+    "sharpi_moe_permute": [P, P, P, P, P, P, I, I, I, P],
+    "sharpi_argmax_rows": [P, P, I, I, P],
+    "sharpi_sample_rows": [P, P, P, P, P, P, P, P, I, I, P],
+    "sharpi_edit_logits": [P, P, P, P, P, P, P, P, I, I, P],
+}
+
+# entry points that newer sources add; bound when present
+_OPTIONAL_SIGNATURES: dict = {}
+
+
+class KernelLibraryError(RuntimeError):
+    pass
+
+
+def library_path() -> Optional[str]:
+    return _lib_path
+
+
+def load(verbose: bool = True) -> ctypes.CDLL:
+    """The kernel library, built first if no up-to-date build exists."""
+    global _lib, _lib_path
+    if _lib is not None:
+        return _lib
+    from ..csrc import build as _build
+
+    try:
+        path = _build.ensure_built(verbose=verbose)
+    except Exception as e:  # noqa: BLE001
+        raise KernelLibraryError(f"the HIP kernel library is missing and could not be built: {e}") from e
+    try:
+        lib = ctypes.CDLL(path)
+    except OSError as e:
+        raise KernelLibraryError(f"cannot load {path}: {e}") from e
+    for name, args in {**_SIGNATURES, **_OPTIONAL_SIGNATURES}.items():
+        try:
+            fn = getattr(lib, name)
+        except AttributeError:
+            if name in _SIGNATURES:
+                raise KernelLibraryError(f"{path} lacks entry point {name}: rebuild the kernels") from None
+            continue
+        fn.argtypes = args
+        fn.restype = c_int
+    _lib, _lib_path = lib, path
+    return lib
+
+
+def register_signature(name: str, argtypes) -> None:
+    """Used by op modules that bind further entry points of the library."""
+    _SIGNATURES[name] = list(argtypes)
+    if _lib is not None:
+        fn = getattr(_lib, name)
+        fn.argtypes = list(argtypes)
+        fn.restype = c_int

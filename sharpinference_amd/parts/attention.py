@@ -1,0 +1,79 @@
+"""The attention mixer: grouped-query attention over the paged cache."""
+from __future__ import annotations
+
+import math
+from typing import Dict, Optional, Tuple
+
+import torch
+
+from .. import ops
+from ..cache.spec import KVSpec, WINDOW_CHUNK, WINDOW_NONE, WINDOW_SLIDING  # noqa: F401
+from .base import LayerCache, ParamSpec, Part, StepContext, TensorSource
+from .position import RotaryInterleaved
+
+
+class Attention(Part):
+    """q/k/v projections without bias -> position encoding -> optional weightless per-head norm
+    -> optional query temperature -> keys and values into the cache -> softmax(q k^T * scale) v
+    over the keys the window admits -> output projection
+    (reference: src/SharpInference.Engine/ForwardPass.cs:1576-1690, 1838-1912; the norm comes
+    after the rotation, 1643-1648).
+
+    Everything that differs between layers is an argument: ``rotary`` (None = no position
+    encoding), ``qk_norm_eps`` (None = no norm), ``q_temperature`` = (floor_scale, attn_scale)
+    multiplying queries by 1 + attn_scale * ln(floor((pos + 1) / floor_scale) + 1), and the
+    window: all keys, the chunk [floor(pos/W)*W, pos], or the last W keys."""
+
+    def __init__(self, hidden: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                 rotary: Optional[RotaryInterleaved] = None, qk_norm_eps: Optional[float] = None,
+                 q_temperature: Optional[Tuple[float, float]] = None, window_kind: int = WINDOW_NONE,
+                 window: int = 0, scale: Optional[float] = None):
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} heads cannot share {num_kv_heads} kv heads")
+        if head_dim % 16 or not 16 <= head_dim <= 256:
+            raise ValueError(f"head_dim {head_dim} is not taken: multiples of 16 from 16 to 256")
+        if rotary is not None and rotary.head_dim != head_dim:
+            raise ValueError("the rotary table's head_dim differs from the mixer's")
+        self.hidden, self.nh, self.nkv, self.hd = int(hidden), int(num_heads), int(num_kv_heads), int(head_dim)
+        self.rotary, self.qk_norm_eps, self.q_temperature = rotary, qk_norm_eps, q_temperature
+        self.window_kind, self.window = int(window_kind), int(window)
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
+        self.w_qkv: Optional[torch.Tensor] = None
+        self.w_o: Optional[torch.Tensor] = None
+
+    # -- what it needs --------------------------------------------------------
+    def cache_spec(self) -> KVSpec:
+        return KVSpec(self.nkv, self.hd, self.window_kind, self.window)
+
+    def param_specs(self, prefix: str) -> Dict[str, ParamSpec]:
+        q, kv = self.nh * self.hd, self.nkv * self.hd
+        return {
+            prefix + "q_proj.weight": ParamSpec((q, self.hidden)),
+            prefix + "k_proj.weight": ParamSpec((kv, self.hidden)),
+            prefix + "v_proj.weight": ParamSpec((kv, self.hidden)),
+            prefix + "o_proj.weight": ParamSpec((self.hidden, q)),
+        }
+
+    def load(self, prefix: str, source: TensorSource) -> None:
+        q, kv = self.nh * self.hd, self.nkv * self.hd
+        parts = [source.get(prefix + n + "_proj.weight") for n in ("q", "k", "v")]
+        dt = torch.float32 if any(p.dtype == torch.float32 for p in parts) else parts[0].dtype
+        fused = torch.empty(q + 2 * kv, self.hidden, dtype=dt, device=parts[0].device)
+        o = 0
+        for p in parts:
+            fused[o:o + p.shape[0]].copy_(p)
+            o += p.shape[0]
+        self.w_qkv = fused
+        self.w_o = source.get(prefix + "o_proj.weight")
+
+    # -- compute --------------------------------------------------------------
+    def forward(self, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> torch.Tensor:
+        g = cache.group
+        qkv = ops.linear(x, self.w_qkv, ctx.act_dtype)
+        slots = g.slot_mapping if cache.write else ctx.no_store_slots
+        inv_freq = self.rotary.table(x.device) if self.rotary is not None else None
+        q = ops.rope_kv(qkv, cache.k, cache.v, slots, ctx.positions, inv_freq, self.qk_norm_eps is not None,
+                        self.qk_norm_eps or 1e-6, self.q_temperature, self.nh, self.nkv, self.hd)
+        o = ops.attention(q, cache.k, cache.v, g, ctx, self.window_kind, self.window, self.scale, self.nh, self.nkv,
+                          self.hd)
+        return ops.linear(o, self.w_o, ctx.act_dtype)

@@ -1,0 +1,79 @@
+"""What every part of a model has in common, and what a part sees of a step.
+
+A *part* (norm, position encoding, mixer, feed-forward, block) takes its sizes and constants
+as constructor arguments, says which tensors it needs (``param_specs``), takes them from a
+source (``load``) and computes (``forward``).  No part knows which model it sits in.
+
+A step hands the parts a :class:`StepContext`: the flat batch of tokens (several requests,
+prompt portions beside single decoded tokens) with per-token positions and, for each cache
+group, the block tables and the slots where this step's keys and values go.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional
+
+import torch
+
+from ..weights.loader import INIT_INT, INIT_NORM_WEIGHT, INIT_NORMAL, ParamSpec, TensorSource  # noqa: F401
+
+
+class Part:
+    """Base of all parts.  Children are parts held in attributes listed by ``children()``."""
+
+    def param_specs(self, prefix: str) -> Dict[str, ParamSpec]:
+        return {}
+
+    def load(self, prefix: str, source: TensorSource) -> None:
+        pass
+
+
+@dataclass
+class GroupView:
+    """One cache group as a step sees it."""
+
+    block_table: torch.Tensor          # int32 [entries, max_blocks], -1 where no page
+    slot_mapping: torch.Tensor         # int32 [tokens]: page * page_size + offset for this step's tokens
+    page_size: int
+    max_context: int = 0               # longest context (position + 1) of any token in the step
+
+
+@dataclass
+class StepContext:
+    n_tokens: int
+    n_entries: int
+    token_ids: torch.Tensor            # int32 [tokens]
+    positions: torch.Tensor            # int32 [tokens]
+    entry_of_token: torch.Tensor       # int32 [tokens]
+    cu_tokens: torch.Tensor            # int32 [entries + 1]
+    state_slots: torch.Tensor          # int32 [entries]: the state slot of each entry's request
+    groups: List[GroupView]
+    act_dtype: torch.dtype
+    no_store_slots: Optional[torch.Tensor] = None   # int32 [tokens] of -1: "store nothing" for cache readers
+    # host copies for parts that plan launches
+    entry_lens: List[int] = field(default_factory=list)
+    entry_starts: List[int] = field(default_factory=list)
+    max_entry_len: int = 1
+    extras: Dict[str, object] = field(default_factory=dict)
+
+
+@dataclass
+class LayerCache:
+    """The cache of one execution of one layer."""
+
+    group: Optional[GroupView] = None
+    k: Optional[torch.Tensor] = None   # [pages, kv heads, page_size, head_dim]
+    v: Optional[torch.Tensor] = None
+    state: Optional[torch.Tensor] = None   # [state slots, ...]
+    write: bool = True                 # False: read another layer's cache, store nothing
+
+
+class ResidualStream:
+    """The float32 residual sum ``h`` and the branch output still to be added to it.
+
+    A branch (mixer, feed-forward) leaves its output in ``pending``; the next norm adds it into
+    ``h`` in the same kernel that normalises, so the sum is formed once, in float."""
+
+    def __init__(self, h: torch.Tensor):
+        self.h = h
+        self.pending: Optional[torch.Tensor] = None

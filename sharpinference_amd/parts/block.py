@@ -1,0 +1,44 @@
+"""How a layer's parts are arranged."""
+from __future__ import annotations
+
+from typing import Dict
+
+from .base import LayerCache, ParamSpec, Part, ResidualStream, StepContext, TensorSource
+
+
+class PreNormBlock(Part):
+    """h += mixer(norm1(h)); h += ffn(norm2(h))
+    (reference: src/SharpInference.Engine/ForwardPass.cs:1557-1561, 1690-1714).
+
+    The additions are folded into the norm that follows them (see ResidualStream), so a block
+    leaves its feed-forward output pending for the next block's first norm.  Names of the four
+    parts in the weight file are arguments."""
+
+    def __init__(self, norm1: Part, mixer: Part, norm2: Part, ffn: Part, names=None):
+        self.norm1, self.mixer, self.norm2, self.ffn = norm1, mixer, norm2, ffn
+        self.names = dict(names or {"norm1": "input_layernorm.", "mixer": "self_attn.",
+                                    "norm2": "post_attention_layernorm.", "ffn": "feed_forward."})
+
+    def _children(self):
+        return ((self.names["norm1"], self.norm1), (self.names["mixer"], self.mixer),
+                (self.names["norm2"], self.norm2), (self.names["ffn"], self.ffn))
+
+    def param_specs(self, prefix: str) -> Dict[str, ParamSpec]:
+        out: Dict[str, ParamSpec] = {}
+        for name, part in self._children():
+            out.update(part.param_specs(prefix + name))
+        return out
+
+    def load(self, prefix: str, source: TensorSource) -> None:
+        for name, part in self._children():
+            part.load(prefix + name, source)
+
+    def cache_spec(self):
+        spec = getattr(self.mixer, "cache_spec", None)
+        return spec() if spec else None
+
+    def forward(self, stream: ResidualStream, ctx: StepContext, cache: LayerCache) -> None:
+        n = self.norm1.forward(stream, ctx.act_dtype)
+        stream.pending = self.mixer.forward(n, ctx, cache)
+        n = self.norm2.forward(stream, ctx.act_dtype)
+        stream.pending = self.ffn.forward(n, ctx)

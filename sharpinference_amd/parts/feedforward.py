@@ -1,0 +1,109 @@
+"""Feed-forward parts: the dense SwiGLU and the routed mixture of SwiGLU experts."""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from .. import ops
+from .base import ParamSpec, Part, StepContext, TensorSource
+
+
+def _fuse_rows(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """[.., Ia, H] and [.., Ib, H] -> [.., Ia + Ib, H] (gate rows first, up rows second)."""
+    dt = torch.float32 if torch.float32 in (a.dtype, b.dtype) else a.dtype
+    shape = list(a.shape)
+    shape[-2] = a.shape[-2] + b.shape[-2]
+    out = torch.empty(shape, dtype=dt, device=a.device)
+    out[..., : a.shape[-2], :].copy_(a)
+    out[..., a.shape[-2]:, :].copy_(b)
+    return out
+
+
+class DenseSwiGLU(Part):
+    """down( silu(gate x) * (up x) ) (reference: src/SharpInference.Engine/ForwardPass.cs:2006-2015;
+    silu(g) = g / (1 + exp(-g)), src/SharpInference.Cpu/SimdKernels.cs:4377-4408)."""
+
+    def __init__(self, hidden: int, intermediate: int):
+        self.hidden, self.inter = int(hidden), int(intermediate)
+        self.w_gate_up: Optional[torch.Tensor] = None
+        self.w_down: Optional[torch.Tensor] = None
+
+    def param_specs(self, prefix: str) -> Dict[str, ParamSpec]:
+        return {
+            prefix + "gate_proj.weight": ParamSpec((self.inter, self.hidden)),
+            prefix + "up_proj.weight": ParamSpec((self.inter, self.hidden)),
+            prefix + "down_proj.weight": ParamSpec((self.hidden, self.inter)),
+        }
+
+    def load(self, prefix: str, source: TensorSource) -> None:
+        g = source.get(prefix + "gate_proj.weight")
+        u = source.get(prefix + "up_proj.weight")
+        self.w_gate_up = _fuse_rows(g, u)
+        del g, u
+        self.w_down = source.get(prefix + "down_proj.weight")
+
+    def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        gu = ops.linear(x, self.w_gate_up, ctx.act_dtype)
+        act = ops.silu_mul(gu)
+        return ops.linear(act, self.w_down, ctx.act_dtype)
+
+
+class MoESwiGLU(Part):
+    """Router -> top-k experts (+ an always-on shared expert)
+    (reference: src/SharpInference.Engine/ForwardPass.cs:2021-2098).
+
+    The router's logits, gate and picks are float and stay on the device.  With
+    ``score_on_input`` the gate and up products of a chosen expert are multiplied by its score
+    before the SiLU (ForwardPass.cs:2083-2089); the shared expert sees the unscaled input
+    (2060-2066); the outputs are summed (2096-2097).  ``gate`` is "sigmoid" or "softmax"
+    (2031-2034); ``renormalise`` divides the k scores by their sum (2156-2162)."""
+
+    def __init__(self, hidden: int, num_experts: int, top_k: int, expert_intermediate: int,
+                 shared_intermediate: Optional[int] = None, gate: str = "sigmoid", renormalise: bool = False,
+                 score_on_input: bool = True):
+        if not 1 <= top_k <= num_experts:
+            raise ValueError(f"top_k {top_k} must lie in 1..{num_experts}")
+        if gate not in ("sigmoid", "softmax"):
+            raise ValueError(f"router gate {gate!r} is not known (sigmoid, softmax)")
+        if not score_on_input:
+            raise NotImplementedError("expert scores applied to the output are not built; only score_on_input=True")
+        self.hidden, self.E, self.k = int(hidden), int(num_experts), int(top_k)
+        self.inter = int(expert_intermediate)
+        self.shared = DenseSwiGLU(hidden, shared_intermediate) if shared_intermediate else None
+        self.gate = ops.GATE_SIGMOID if gate == "sigmoid" else ops.GATE_SOFTMAX
+        self.renormalise = bool(renormalise)
+        self.w_router: Optional[torch.Tensor] = None
+        self.w_gate_up: Optional[torch.Tensor] = None     # [E, 2*I, H]
+        self.w_down: Optional[torch.Tensor] = None        # [E, H, I]
+
+    def param_specs(self, prefix: str) -> Dict[str, ParamSpec]:
+        out = {
+            prefix + "router.weight": ParamSpec((self.E, self.hidden)),
+            prefix + "experts.gate_proj": ParamSpec((self.E, self.inter, self.hidden)),
+            prefix + "experts.up_proj": ParamSpec((self.E, self.inter, self.hidden)),
+            prefix + "experts.down_proj": ParamSpec((self.E, self.hidden, self.inter)),
+        }
+        if self.shared is not None:
+            out.update(self.shared.param_specs(prefix + "shared_expert."))
+        return out
+
+    def load(self, prefix: str, source: TensorSource) -> None:
+        self.w_router = source.get(prefix + "router.weight")
+        g = source.get(prefix + "experts.gate_proj")
+        u = source.get(prefix + "experts.up_proj")
+        self.w_gate_up = _fuse_rows(g, u)
+        del g, u
+        self.w_down = source.get(prefix + "experts.down_proj")
+        if self.shared is not None:
+            self.shared.load(prefix + "shared_expert.", source)
+
+    def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        T = x.shape[0]
+        ids, wts = ops.router_topk(x, self.w_router, self.k, self.gate, self.renormalise)
+        offsets, sorted_token, sorted_w, inv_pos = ops.moe_permute(ids, wts, self.E)
+        shared = self.shared.forward(x, ctx) if self.shared is not None else None
+        gu = ops.grouped_linear(x, self.w_gate_up, offsets, sorted_token, T * self.k, ctx.act_dtype)
+        act = ops.silu_mul(gu, sorted_w)
+        y = ops.grouped_linear(act, self.w_down, offsets, None, T * self.k, ctx.act_dtype)
+        return ops.moe_combine(y, inv_pos, shared, T, self.k)

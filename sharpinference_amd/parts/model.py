@@ -1,0 +1,108 @@
+"""The whole decoder: embedding, a list of blocks, the order they run in, final norm, head."""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Sequence
+
+import torch
+
+from .. import ops
+from .base import LayerCache, ParamSpec, Part, ResidualStream, StepContext, TensorSource
+from .norm import RMSNorm
+
+
+@dataclass(frozen=True)
+class Run:
+    """One entry of the execution order: run `layer` with cache slot `cache`.
+
+    A layer may appear in several entries (its weights are used again; give each entry its own
+    cache slot unless sharing is meant).  ``write=False`` makes the entry read the keys and
+    values that the slot's owner stored earlier in the same step and store nothing."""
+
+    layer: int
+    cache: int
+    write: bool = True
+
+
+class DecoderModel(Part):
+    """tokens -> embedding rows (no scaling; reference: src/SharpInference.Engine/ForwardPass.cs:1478-1483)
+    -> blocks in the order of ``schedule`` -> final norm -> logits through the head, which is the
+    embedding table when tied (ForwardPass.cs:1741-1747, 410-413)."""
+
+    def __init__(self, vocab_size: int, hidden: int, blocks: Sequence[Part], final_norm: RMSNorm,
+                 schedule: Optional[Sequence[Run]] = None, tie_embeddings: bool = False, config=None,
+                 layer_prefix: str = "model.layers.", embed_name: str = "model.embed_tokens.weight",
+                 norm_prefix: str = "model.norm.", head_name: str = "lm_head.weight"):
+        self.vocab_size, self.hidden = int(vocab_size), int(hidden)
+        self.blocks = list(blocks)
+        self.final_norm = final_norm
+        self.schedule: List[Run] = list(schedule) if schedule is not None else [Run(i, i) for i in range(len(self.blocks))]
+        self.tie_embeddings = bool(tie_embeddings)
+        self.config = config
+        self.layer_prefix, self.embed_name, self.norm_prefix, self.head_name = layer_prefix, embed_name, norm_prefix, head_name
+        self.embed: Optional[torch.Tensor] = None
+        self.head: Optional[torch.Tensor] = None
+        self._check_schedule()
+
+    def _check_schedule(self) -> None:
+        n_slots = self.num_cache_slots()
+        owner: Dict[int, int] = {}
+        for r in self.schedule:
+            if not 0 <= r.layer < len(self.blocks):
+                raise ValueError(f"schedule names layer {r.layer}; the model has {len(self.blocks)}")
+            if not 0 <= r.cache < n_slots:
+                raise ValueError(f"schedule names cache slot {r.cache} out of range")
+            spec = self.blocks[r.layer].cache_spec()
+            if r.write:
+                if r.cache in owner:
+                    raise ValueError(f"cache slot {r.cache} is written by two entries of the schedule")
+                owner[r.cache] = r.layer
+            else:
+                if r.cache not in owner:
+                    raise ValueError(f"cache slot {r.cache} is read before any entry has written it")
+                if self.blocks[owner[r.cache]].cache_spec() != spec:
+                    raise ValueError(f"layer {r.layer} reads the cache of layer {owner[r.cache]}, whose shape differs")
+
+    # -- cache ------------------------------------------------------------------
+    def num_cache_slots(self) -> int:
+        return 1 + max((r.cache for r in self.schedule), default=-1)
+
+    def cache_specs(self) -> list:
+        """Per cache slot, what its owner asks of the cache manager."""
+        specs = [None] * self.num_cache_slots()
+        for r in self.schedule:
+            if r.write:
+                specs[r.cache] = self.blocks[r.layer].cache_spec()
+        return specs
+
+    # -- weights ------------------------------------------------------------------
+    def param_specs(self, prefix: str = "") -> Dict[str, ParamSpec]:
+        out = {self.embed_name: ParamSpec((self.vocab_size, self.hidden))}
+        for i, b in enumerate(self.blocks):
+            out.update(b.param_specs(f"{self.layer_prefix}{i}."))
+        out.update(self.final_norm.param_specs(self.norm_prefix))
+        if not self.tie_embeddings:
+            out[self.head_name] = ParamSpec((self.vocab_size, self.hidden))
+        return out
+
+    def load_weights(self, source: TensorSource) -> None:
+        self.embed = source.get(self.embed_name)
+        for i, b in enumerate(self.blocks):
+            b.load(f"{self.layer_prefix}{i}.", source)
+        self.final_norm.load(self.norm_prefix, source)
+        self.head = self.embed if self.tie_embeddings else source.get(self.head_name)
+
+    # -- compute ------------------------------------------------------------------
+    def forward(self, ctx: StepContext, caches: Sequence[LayerCache], logit_rows: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+        """Run the step's tokens through every entry of the schedule.  Returns float32 logits
+        [len(logit_rows), vocab], or None if no row is wanted."""
+        stream = ResidualStream(ops.embed_gather(ctx.token_ids, self.embed))
+        for r in self.schedule:
+            c = caches[r.cache]
+            if not r.write:
+                c = LayerCache(c.group, c.k, c.v, c.state, write=False)
+            self.blocks[r.layer].forward(stream, ctx, c)
+        if logit_rows is None or logit_rows.numel() == 0:
+            return None
+        n = self.final_norm.forward(stream, ctx.act_dtype, rows=logit_rows)
+        return ops.linear(n, self.head, torch.float32)

@@ -1,0 +1,215 @@
+"""Weights by tensor name: checking a file against what the model asks for, then loading.
+
+A model says what it needs as ``{name: ParamSpec}``.  A *source* hands tensors out by name;
+:class:`SafetensorsSource` reads a model folder, :class:`RandomSource` draws them from a seed.
+Before anything is loaded the whole request is checked, and every fault (missing tensors,
+tensors nobody asked for, wrong shapes, wrong kinds) comes back in ONE :class:`WeightError`;
+the reference stops at the first missing name
+(reference: src/SharpInference.Engine/ForwardPass.cs:2301-2306).
+
+Storage policy: 16-bit floats are kept as bfloat16; a tensor stored in 32-bit floats stays
+float32; integer tables become int32.  In float32 mode every float tensor is widened to
+float32 (exact for bfloat16 values).
+"""
+from __future__ import annotations
+
+import hashlib
+import os
+from dataclasses import dataclass
+from typing import Dict, Iterable, List, Optional, Tuple
+
+import torch
+
+from . import safetensors_io as st
+
+INIT_NORMAL, INIT_NORM_WEIGHT, INIT_INT = "normal", "norm_weight", "int"
+
+
+@dataclass(frozen=True)
+class ParamSpec:
+    shape: Tuple[int, ...]
+    init: str = INIT_NORMAL      # how random mode fills it: N(0, std) | U(0.9, 1.1) | integers
+    kind: str = "float"          # "float" or "int"
+
+
+class WeightError(ValueError):
+    """All faults of a weight file at once."""
+
+    def __init__(self, missing: List[str], unexpected: List[str], wrong_shape: List[str], wrong_kind: List[str],
+                 where: str = ""):
+        self.missing, self.unexpected = list(missing), list(unexpected)
+        self.wrong_shape, self.wrong_kind = list(wrong_shape), list(wrong_kind)
+        lines = [f"weights{' in ' + where if where else ''} do not fit the model:"]
+        if missing:
+            lines.append(f"  missing ({len(missing)}): " + ", ".join(missing))
+        if unexpected:
+            lines.append(f"  unexpected ({len(unexpected)}): " + ", ".join(unexpected))
+        if wrong_shape:
+            lines.append(f"  wrong shape ({len(wrong_shape)}): " + "; ".join(wrong_shape))
+        if wrong_kind:
+            lines.append(f"  wrong kind ({len(wrong_kind)}): " + "; ".join(wrong_kind))
+        super().__init__("\n".join(lines))
+
+
+def check_specs(specs: Dict[str, ParamSpec], available: Dict[str, Tuple[Tuple[int, ...], torch.dtype]],
+                where: str = "") -> None:
+    missing = sorted(n for n in specs if n not in available)
+    unexpected = sorted(n for n in available if n not in specs)
+    wrong_shape, wrong_kind = [], []
+    for n, spec in sorted(specs.items()):
+        if n not in available:
+            continue
+        shape, dtype = available[n]
+        if tuple(shape) != tuple(spec.shape):
+            wrong_shape.append(f"{n}: expected {list(spec.shape)}, found {list(shape)}")
+        is_float = dtype.is_floating_point
+        if (spec.kind == "float") != is_float:
+            wrong_kind.append(f"{n}: expected {spec.kind}, found {dtype}")
+    if missing or unexpected or wrong_shape or wrong_kind:
+        raise WeightError(missing, unexpected, wrong_shape, wrong_kind, where)
+
+
+def storage_dtype(stored: torch.dtype, compute: torch.dtype) -> torch.dtype:
+    """What a tensor stored as `stored` becomes in a model computing in `compute`."""
+    if not stored.is_floating_point:
+        return torch.int32
+    if compute == torch.float32:
+        return torch.float32
+    if stored in (torch.float32, torch.float64):
+        return torch.float32
+    return torch.bfloat16
+
+
+# ---------------------------------------------------------------------------
+class TensorSource:
+    """Hands tensors out by name, already on `device` and in their storage dtype."""
+
+    def available(self) -> Dict[str, Tuple[Tuple[int, ...], torch.dtype]]:
+        raise NotImplementedError
+
+    def get(self, name: str) -> torch.Tensor:
+        raise NotImplementedError
+
+    where = ""
+
+
+class SafetensorsSource(TensorSource):
+    def __init__(self, model_dir: str, compute_dtype: torch.dtype, device):
+        self.where = model_dir
+        self.entries = st.index_folder(model_dir)
+        self.compute_dtype = compute_dtype
+        self.device = torch.device(device)
+
+    def available(self):
+        return {n: (e.shape, e.dtype) for n, e in self.entries.items()}
+
+    def get(self, name: str) -> torch.Tensor:
+        e = self.entries[name]
+        host = st.read_tensor(e)
+        want = storage_dtype(e.dtype, self.compute_dtype)
+        if host.dtype != want:
+            host = host.to(want)
+        return host.to(self.device)
+
+
+def _name_seed(seed: int, name: str) -> int:
+    h = hashlib.sha256(f"{seed}:{name}".encode()).digest()
+    return int.from_bytes(h[:8], "little") & ((1 << 63) - 1)
+
+
+class RandomSource(TensorSource):
+    """Seeded random tensors: matrices N(0, std), norm weights U(0.9, 1.1).
+
+    Each tensor's generator is keyed by (seed, name), so the values do not depend on the
+    order of the requests.  ``stored_dtype`` is what a file written from this source holds
+    (values are rounded to it first); ``float32_names`` keeps tensors whose name ends with one
+    of the given suffixes in float32."""
+
+    def __init__(self, specs: Dict[str, ParamSpec], seed: int, compute_dtype: torch.dtype, device,
+                 stored_dtype: torch.dtype = torch.bfloat16, std: float = 0.02,
+                 float32_names: Iterable[str] = (), std_by_suffix: Optional[Dict[str, float]] = None,
+                 generate_on_device: bool = False):
+        self.specs = dict(specs)
+        self.seed = int(seed)
+        self.compute_dtype = compute_dtype
+        self.device = torch.device(device)
+        self.stored_dtype = stored_dtype
+        self.std = float(std)
+        self.float32_names = tuple(float32_names)
+        self.std_by_suffix = dict(std_by_suffix or {})
+        self.generate_on_device = generate_on_device and self.device.type == "cuda"
+        self.where = f"random(seed={seed})"
+
+    def stored_dtype_of(self, name: str) -> torch.dtype:
+        spec = self.specs[name]
+        if spec.kind == "int":
+            return torch.int32
+        if any(name.endswith(s) for s in self.float32_names):
+            return torch.float32
+        return self.stored_dtype
+
+    def available(self):
+        return {n: (s.shape, self.stored_dtype_of(n)) for n, s in self.specs.items()}
+
+    def stored(self, name: str) -> torch.Tensor:
+        """The tensor as a file would hold it (host unless generating on the device)."""
+        spec = self.specs[name]
+        dev = self.device if self.generate_on_device else torch.device("cpu")
+        g = torch.Generator(device=dev)
+        g.manual_seed(_name_seed(self.seed, name))
+        sd = self.stored_dtype_of(name)
+        if spec.kind == "int":
+            return torch.randint(0, 2 ** 15, spec.shape, generator=g, device=dev, dtype=torch.int32)
+        if self.generate_on_device:
+            t = torch.empty(spec.shape, dtype=sd, device=dev)
+            if spec.init == INIT_NORM_WEIGHT:
+                t.uniform_(0.9, 1.1, generator=g)
+            else:
+                t.normal_(0.0, self._std_of(name), generator=g)
+            return t
+        t = torch.empty(spec.shape, dtype=torch.float32)
+        if spec.init == INIT_NORM_WEIGHT:
+            t.uniform_(0.9, 1.1, generator=g)
+        else:
+            t.normal_(0.0, self._std_of(name), generator=g)
+        return t.to(sd)
+
+    def _std_of(self, name: str) -> float:
+        for suffix, s in self.std_by_suffix.items():
+            if name.endswith(suffix):
+                return float(s)
+        return self.std
+
+    def get(self, name: str) -> torch.Tensor:
+        t = self.stored(name)
+        want = storage_dtype(t.dtype, self.compute_dtype)
+        if t.dtype != want:
+            t = t.to(want)
+        return t.to(self.device)
+
+
+# ---------------------------------------------------------------------------
+def load_model_weights(model, source: TensorSource) -> None:
+    """Check the source against the model's request, then let the parts take their tensors."""
+    specs = model.param_specs()
+    check_specs(specs, source.available(), source.where)
+    model.load_weights(source)
+
+
+def write_random_model(config, out_dir: str, seed: int, stored_dtype: torch.dtype = torch.bfloat16,
+                       std: float = 0.02, float32_names: Iterable[str] = (),
+                       std_by_suffix: Optional[Dict[str, float]] = None) -> str:
+    """Random-weights mode: a model folder (config.json, model.safetensors) from a
+    configuration and a seed."""
+    from ..config.base import save_config
+    from ..registry import build_model
+
+    model = build_model(config)
+    specs = model.param_specs()
+    src = RandomSource(specs, seed, torch.float32, "cpu", stored_dtype=stored_dtype, std=std,
+                       float32_names=float32_names, std_by_suffix=std_by_suffix)
+    os.makedirs(out_dir, exist_ok=True)
+    save_config(config, out_dir)
+    st.write_file(os.path.join(out_dir, "model.safetensors"), ((n, src.stored(n)) for n in sorted(specs)),
+                  metadata={"format": "pt", "seed": str(seed)})
+    return out_dir

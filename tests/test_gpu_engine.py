@@ -1,0 +1,75 @@
+"""The engine against the plain implementation: every way of cutting a request into steps."""
+import pytest
+import torch
+
+import helpers as H
+from tiny_configs import CONFIGS, make_model_dir
+
+pytestmark = pytest.mark.gpu
+
+PROMPTS = {"A": [5, 23, 40 + 16], "B": [1, 17, 50, 77 + 24], "C": [3, 64, 95]}
+
+
+@pytest.fixture(scope="module", params=[("A", 0.02), ("B", 0.02), ("C", 0.02), ("A", 0.15), ("B", 0.12), ("C", 0.1)],
+                ids=lambda p: f"{p[0]}-std{p[1]}")
+def model_dir(request, tmp_path_factory):
+    which, std = request.param
+    return which, make_model_dir(tmp_path_factory.mktemp(f"m{which}"), which, std=std)
+
+
+@pytest.fixture(scope="module", params=["float32", "bfloat16"])
+def engine(request, model_dir):
+    which, d = model_dir
+    return which, d, request.param, H.make_engine(d, request.param)
+
+
+def _check(dtype, got, ref, what):
+    if dtype == "float32":
+        H.assert_close_fp32(got, ref, what)
+    else:
+        H.assert_close_bf16(got, ref, what)
+
+
+def _requests(which):
+    vocab = CONFIGS[which]["vocab_size"]
+    return [H.random_tokens(n, vocab, 100 + i) for i, n in enumerate(PROMPTS[which])]
+
+
+def test_whole(engine):
+    which, d, dtype, eng = engine
+    for i, toks in enumerate(_requests(which)):
+        got = H.run_cut(eng, f"w{i}", toks, H.whole(len(toks)))
+        _check(dtype, got, H.plain_logits(d, toks), f"{which} {dtype} whole request {i}")
+
+
+def test_last_tokens_decoded(engine):
+    which, d, dtype, eng = engine
+    for i, toks in enumerate(_requests(which)):
+        got = H.run_cut(eng, f"d{i}", toks, H.last_decoded(len(toks)))
+        _check(dtype, got, H.plain_logits(d, toks), f"{which} {dtype} last-32-decoded request {i}")
+
+
+def test_changing_portions(engine):
+    which, d, dtype, eng = engine
+    for i, toks in enumerate(_requests(which)):
+        for seed in (0, 1):
+            got = H.run_cut(eng, f"p{i}", toks, H.changing_portions(len(toks), seed))
+            _check(dtype, got, H.plain_logits(d, toks), f"{which} {dtype} portions(seed {seed}) request {i}")
+
+
+def test_token_by_token(engine):
+    which, d, dtype, eng = engine
+    toks = _requests(which)[-1]
+    got = H.run_cut(eng, "t", toks, [1] * len(toks))
+    _check(dtype, got, H.plain_logits(d, toks), f"{which} {dtype} token by token")
+
+
+def test_cuts_agree_fp32(engine):
+    """In 32-bit the cut must not change a logit beyond rounding: far below the tolerance."""
+    which, d, dtype, eng = engine
+    if dtype != "float32":
+        pytest.skip("32-bit only")
+    toks = _requests(which)[-1]
+    a = H.run_cut(eng, "x", toks, H.whole(len(toks)))
+    b = H.run_cut(eng, "y", toks, H.changing_portions(len(toks), 3))
+    assert float((a - b).abs().max()) <= 1e-5 * max(1.0, float(a.abs().max()))

@@ -1,0 +1,57 @@
+"""Two tiny Llama 4 configurations that differ in every size and option, as raw config.json dicts."""
+
+TINY_A = {
+    "architectures": ["Llama4ForCausalLM"],
+    "hidden_size": 64, "num_hidden_layers": 2, "num_attention_heads": 4, "num_key_value_heads": 2,
+    "head_dim": 16, "vocab_size": 256,
+    "intermediate_size": 128, "intermediate_size_mlp": 256,
+    "num_local_experts": 4, "num_experts_per_tok": 1, "interleave_moe_layer_step": 1,
+    "no_rope_layers": [1, 0], "attention_chunk_size": 16,
+    "use_qk_norm": True, "attn_temperature_tuning": True, "floor_scale": 8, "attn_scale": 0.1,
+    "rms_norm_eps": 1e-5, "rope_theta": 10000.0, "rope_scaling": None,
+    "tie_word_embeddings": False, "max_position_embeddings": 512, "torch_dtype": "bfloat16",
+}
+
+TINY_B = {
+    "architectures": ["Llama4ForCausalLM"],
+    "hidden_size": 96, "num_hidden_layers": 5, "num_attention_heads": 6, "num_key_value_heads": 3,
+    "head_dim": 32, "vocab_size": 384,
+    "intermediate_size": 64, "intermediate_size_mlp": 160,
+    "num_local_experts": 8, "num_experts_per_tok": 2, "interleave_moe_layer_step": 2,
+    "no_rope_layers": [1, 1, 1, 0, 1], "attention_chunk_size": 24,
+    "use_qk_norm": False, "attn_temperature_tuning": True, "floor_scale": 32, "attn_scale": 0.2,
+    "rms_norm_eps": 1e-6, "rope_theta": 500000.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 32},
+    "tie_word_embeddings": False, "max_position_embeddings": 1024, "torch_dtype": "bfloat16",
+}
+
+# a third one: tied head, one kv head per head, odd-ish sizes, every layer dense but one
+TINY_C = {
+    "architectures": ["Llama4ForCausalLM"],
+    "hidden_size": 80, "num_hidden_layers": 3, "num_attention_heads": 5, "num_key_value_heads": 5,
+    "head_dim": 48, "vocab_size": 203,
+    "intermediate_size": 48, "intermediate_size_mlp": 112,
+    "num_local_experts": 3, "num_experts_per_tok": 3, "interleave_moe_layer_step": 3,
+    "no_rope_layers": [0, 1, 1], "attention_chunk_size": 40,
+    "use_qk_norm": True, "attn_temperature_tuning": False, "floor_scale": 4, "attn_scale": 0.5,
+    "rms_norm_eps": 1e-4, "rope_theta": 1000.0, "rope_scaling": None,
+    "tie_word_embeddings": True, "max_position_embeddings": 512, "torch_dtype": "bfloat16",
+}
+
+SEEDS = {"A": 0, "B": 1, "C": 5}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+# tensors kept in float32 in B's file: shows that 32-bit tensors stay 32-bit in a bfloat16 run
+FLOAT32_NAMES = {"A": (), "B": ("layernorm.weight", "model.norm.weight", "router.weight"), "C": ()}
+
+
+def make_model_dir(tmp_path, which: str, std: float = 0.02, **overrides) -> str:
+    from sharpinference_amd.config.base import load_config
+    from sharpinference_amd.weights.loader import write_random_model
+
+    d = dict(CONFIGS[which])
+    d.update(overrides)
+    cfg = load_config(d)
+    out = str(tmp_path / f"tiny_{which}")
+    write_random_model(cfg, out, SEEDS[which], std=std, float32_names=FLOAT32_NAMES[which])
+    return out
