@@ -111,8 +111,8 @@ class Engine:
     def free_request(self, req_id: Hashable) -> None:
         self.cache.free_request(req_id)
 
-    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
-        return self.runner.step(entries)
+    def step(self, entries: Sequence[StepEntry], router_trace: Optional[list] = None) -> Optional[torch.Tensor]:
+        return self.runner.step(entries, router_trace)
 
     # -- generation -------------------------------------------------------------
     def generate(self, prompts: Sequence[Sequence[int]], params: Union[SamplingParams, Sequence[SamplingParams], None] = None,

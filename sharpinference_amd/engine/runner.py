@@ -129,9 +129,11 @@ class ModelRunner:
         return out
 
     # ------------------------------------------------------------------
-    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+    def step(self, entries: Sequence[StepEntry], router_trace: Optional[list] = None) -> Optional[torch.Tensor]:
         """Run one batch.  Returns float32 logits [wanted, vocab] in the order of the entries and
-        of their ``want`` lists, or None when nothing is wanted."""
+        of their ``want`` lists, or None when nothing is wanted.  A list given as ``router_trace``
+        receives, per routed layer run, the (expert ids, weights) of the step's tokens, as the
+        reference can print its router picks (src/SharpInference.Engine/ForwardPass.cs:2042-2056)."""
         if not entries:
             return None
         self._validate(entries)
@@ -142,6 +144,8 @@ class ModelRunner:
                     raise CacheExhausted(f"no pages left for request {e.req_id!r} ({len(e.tokens)} more tokens)")
                 appended.append(e.req_id)
             ctx, rows = self.build_context(entries)
+            if router_trace is not None:
+                ctx.extras["router_trace"] = router_trace
             logits = self.model.forward(ctx, self.layer_caches(ctx), rows)
         except BaseException:
             for r in appended:

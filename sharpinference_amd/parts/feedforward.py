@@ -101,6 +101,9 @@ class MoESwiGLU(Part):
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         T = x.shape[0]
         ids, wts = ops.router_topk(x, self.w_router, self.k, self.gate, self.renormalise)
+        trace = ctx.extras.get("router_trace")
+        if trace is not None:      # the picks of this step, layer by layer (reference: ForwardPass.cs:2042-2056)
+            trace.append((ids, wts))
         offsets, sorted_token, sorted_w, inv_pos = ops.moe_permute(ids, wts, self.E)
         shared = self.shared.forward(x, ctx) if self.shared is not None else None
         gu = ops.grouped_linear(x, self.w_gate_up, offsets, sorted_token, T * self.k, ctx.act_dtype)

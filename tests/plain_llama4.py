@@ -157,17 +157,29 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: torch.Ten
     return out
 
 
+def _same(t: torch.Tensor) -> torch.Tensor:
+    return t
+
+
+def store_bf16(t: torch.Tensor) -> torch.Tensor:
+    """Round to bfloat16 and back: what the engine's bfloat16 path does wherever a tensor is
+    handed from one kernel to the next or kept in the cache.  The residual sum, norm
+    statistics, angles, scores and router values stay in float there and are not rounded here."""
+    return t.to(torch.bfloat16).to(t.dtype)
+
+
 def attention_layer(c: dict, W: Dict[str, torch.Tensor], layer: int, n: torch.Tensor,
-                    positions: torch.Tensor) -> torch.Tensor:
+                    positions: torch.Tensor, store=_same) -> torch.Tensor:
     """ForwardPass.cs:1576-1690 for one layer on normed input n [T, H]: projections
     without bias, rotary then weightless norm on rotary layers (1635-1648), temperature
-    on the others, attention, output projection."""
+    on the others, attention, output projection.  `store` marks where the engine stores a
+    tensor (identity in the 32-bit case)."""
     p = f"model.layers.{layer}.self_attn."
     nh, nkv, hd = c["num_attention_heads"], c.get("num_key_value_heads", c["num_attention_heads"]), head_dim_of(c)
     T = n.shape[0]
-    q = (n @ W[p + "q_proj.weight"].T).view(T, nh, hd)
-    k = (n @ W[p + "k_proj.weight"].T).view(T, nkv, hd)
-    v = (n @ W[p + "v_proj.weight"].T).view(T, nkv, hd)
+    q = store(n @ W[p + "q_proj.weight"].T).view(T, nh, hd)
+    k = store(n @ W[p + "k_proj.weight"].T).view(T, nkv, hd)
+    v = store(n @ W[p + "v_proj.weight"].T).view(T, nkv, hd)
     eps = float(c.get("rms_norm_eps", 1e-5))
     if layer_uses_rope(c, layer):
         inv = rope_inv_freq(hd, float(c.get("rope_theta", 500000.0)), c.get("rope_scaling"))
@@ -182,8 +194,9 @@ def attention_layer(c: dict, W: Dict[str, torch.Tensor], layer: int, n: torch.Te
             t = query_temperature(positions, float(c.get("floor_scale", 8192)), float(c.get("attn_scale", 0.1)))
             q = q * t.to(q.dtype)[:, None, None]
         mask = attention_mask(positions, None)
-    o = attention(q, k, v, mask).reshape(T, nh * hd)
-    return o @ W[p + "o_proj.weight"].T
+    q, k = store(q), store(k)
+    o = store(attention(q, k, v, mask)).reshape(T, nh * hd)
+    return store(o @ W[p + "o_proj.weight"].T)
 
 
 # ----------------------------------------------------------------------------
@@ -194,17 +207,21 @@ def silu(x: torch.Tensor) -> torch.Tensor:
     return x / (1.0 + torch.exp(-x))
 
 
-def swiglu(n: torch.Tensor, wg: torch.Tensor, wu: torch.Tensor, wd: torch.Tensor) -> torch.Tensor:
+def swiglu(n: torch.Tensor, wg: torch.Tensor, wu: torch.Tensor, wd: torch.Tensor, store=_same) -> torch.Tensor:
     """ForwardPass.cs:2006-2015: down( silu(gate n) * (up n) )."""
-    return (silu(n @ wg.T) * (n @ wu.T)) @ wd.T
+    return store(store(silu(store(n @ wg.T)) * store(n @ wu.T)) @ wd.T)
+
+
+def router_gates(n: torch.Tensor, wr: torch.Tensor) -> torch.Tensor:
+    """ForwardPass.cs:2028-2032: logits = Wr n, then a sigmoid over every expert."""
+    return 1.0 / (1.0 + torch.exp(-(n @ wr.T)))
 
 
 def router_topk(n: torch.Tensor, wr: torch.Tensor, k: int):
-    """ForwardPass.cs:2028-2040 and 2132-2150: logits = Wr n; sigmoid over all experts;
-    k picks by value, strict > so the lowest index wins a tie; weight = that sigmoid.
-    No renormalisation of the k weights (the reference would renormalise for k > 1,
-    2156-2162; this engine does not, by decision)."""
-    sig = 1.0 / (1.0 + torch.exp(-(n @ wr.T)))          # [T, E]
+    """ForwardPass.cs:2028-2040 and 2132-2150: k picks by gate value, strict > so the lowest
+    index wins a tie; weight = that gate value.  No renormalisation of the k weights (the
+    reference would renormalise for k > 1, 2156-2162; this engine does not, by decision)."""
+    sig = router_gates(n, wr)                            # [T, E]
     T, E = sig.shape
     ids = torch.zeros(T, k, dtype=torch.long)
     wts = torch.zeros(T, k, dtype=sig.dtype)
@@ -223,41 +240,74 @@ def router_topk(n: torch.Tensor, wr: torch.Tensor, k: int):
     return ids, wts
 
 
-def moe_layer(c: dict, W: Dict[str, torch.Tensor], layer: int, n: torch.Tensor) -> torch.Tensor:
+def router_margin(n: torch.Tensor, wr: torch.Tensor, k: int) -> torch.Tensor:
+    """Per token: router logit of the k-th pick minus that of the best expert left out,
+    relative to the rms of the token's logits (inf if no expert is left out).  Where it is
+    tiny, rounding decides the route; tests use it to tell which positions of a
+    reduced-precision run can be compared with a 32-bit one."""
+    r = n @ wr.T
+    srt = torch.sort(r, dim=-1, descending=True).values
+    if srt.shape[1] <= k:
+        return torch.full((n.shape[0],), float("inf"))
+    return (srt[:, k - 1] - srt[:, k]) / r.pow(2).mean(dim=-1).sqrt().clamp_min(1e-30)
+
+
+def moe_layer(c: dict, W: Dict[str, torch.Tensor], layer: int, n: torch.Tensor, trace: Optional[dict] = None,
+              store=_same, routes: Optional[dict] = None) -> torch.Tensor:
     """ForwardPass.cs:2021-2098: shared expert on the unscaled input (2060-2066); each chosen
     expert's gate and up products are multiplied by its score before the SiLU (2083-2089);
     sum of experts plus shared (2096-2097)."""
     p = f"model.layers.{layer}.feed_forward."
     k = int(c.get("num_experts_per_tok", 1))
     ids, wts = router_topk(n, W[p + "router.weight"], k)
+    if routes is not None:
+        # Picks given from outside (a reduced-precision run's own): take them, with this
+        # implementation's gate values as weights, and record how far each lies below the
+        # pick made here, relative to the rms of the token's router logits.
+        r = n @ W[p + "router.weight"].T
+        forced = routes[layer].to(torch.long)
+        own = torch.gather(r, 1, ids)
+        got = torch.gather(r, 1, forced)
+        regret = (own.sort(dim=1).values - got.sort(dim=1).values).abs().max(dim=1).values
+        regret = regret / r.pow(2).mean(dim=-1).sqrt().clamp_min(1e-30)
+        if trace is not None:
+            trace["route_regret"] = max(float(regret.max()), trace.get("route_regret", 0.0))
+        ids = forced
+        wts = torch.gather(router_gates(n, W[p + "router.weight"]), 1, forced)
+    if trace is not None:
+        m = router_margin(n, W[p + "router.weight"], k)
+        trace["router_margin"] = torch.minimum(trace["router_margin"], m) if "router_margin" in trace else m
     out = swiglu(n, W[p + "shared_expert.gate_proj.weight"], W[p + "shared_expert.up_proj.weight"],
-                 W[p + "shared_expert.down_proj.weight"])
+                 W[p + "shared_expert.down_proj.weight"], store)
     Wg, Wu, Wd = W[p + "experts.gate_proj"], W[p + "experts.up_proj"], W[p + "experts.down_proj"]
     routed = torch.zeros_like(out)
     for t in range(n.shape[0]):
         for j in range(k):
             e = int(ids[t, j])
             w = wts[t, j]
-            g = (Wg[e] @ n[t]) * w
-            u = (Wu[e] @ n[t]) * w
-            routed[t] += Wd[e] @ (silu(g) * u)
-    return routed + out
+            g = store(Wg[e] @ n[t]) * w
+            u = store(Wu[e] @ n[t]) * w
+            routed[t] += store(Wd[e] @ store(silu(g) * u))
+    return store(routed + out)
 
 
-def dense_layer(c: dict, W: Dict[str, torch.Tensor], layer: int, n: torch.Tensor) -> torch.Tensor:
+def dense_layer(c: dict, W: Dict[str, torch.Tensor], layer: int, n: torch.Tensor, store=_same) -> torch.Tensor:
     p = f"model.layers.{layer}.feed_forward."
-    return swiglu(n, W[p + "gate_proj.weight"], W[p + "up_proj.weight"], W[p + "down_proj.weight"])
+    return swiglu(n, W[p + "gate_proj.weight"], W[p + "up_proj.weight"], W[p + "down_proj.weight"], store)
 
 
 # ----------------------------------------------------------------------------
 # whole model
 # ----------------------------------------------------------------------------
 def forward(c: dict, W: Dict[str, torch.Tensor], tokens: Sequence[int], start_pos: int = 0,
-            dtype: torch.dtype = torch.float32) -> torch.Tensor:
+            dtype: torch.dtype = torch.float32, trace: Optional[dict] = None, store=_same,
+            routes: Optional[dict] = None) -> torch.Tensor:
     """ForwardPass.cs:1474-1757 (Forward / RunTrunk) for a whole sequence at once:
     embed (no scale, 1478-1483); per layer norm -> attention -> +residual (1557-1690),
     norm -> feed-forward -> +residual (1695-1714); final norm and head (1741-1747).
-    Returns logits [T, vocab]."""
+    Returns logits [T, vocab].  With store=store_bf16 every tensor the engine's bfloat16 path
+    stores is rounded as it is there; the arithmetic stays float.  `routes` ({layer: ids [T, k]})
+    replaces the router's picks (see moe_layer)."""
     W = {k: v.to(dtype) if v.is_floating_point() else v for k, v in W.items()}
     eps = float(c.get("rms_norm_eps", 1e-5))
     ids = torch.tensor(list(tokens), dtype=torch.long)
@@ -265,11 +315,11 @@ def forward(c: dict, W: Dict[str, torch.Tensor], tokens: Sequence[int], start_po
     h = W["model.embed_tokens.weight"][ids]
     for l in range(int(c["num_hidden_layers"])):
         p = f"model.layers.{l}."
-        n = rms_norm(h, W[p + "input_layernorm.weight"], eps)
-        h = h + attention_layer(c, W, l, n, positions)
-        n = rms_norm(h, W[p + "post_attention_layernorm.weight"], eps)
-        h = h + (moe_layer(c, W, l, n) if layer_is_moe(c, l) else dense_layer(c, W, l, n))
-    h = rms_norm(h, W["model.norm.weight"], eps)
+        n = store(rms_norm(h, W[p + "input_layernorm.weight"], eps))
+        h = h + attention_layer(c, W, l, n, positions, store)
+        n = store(rms_norm(h, W[p + "post_attention_layernorm.weight"], eps))
+        h = h + (moe_layer(c, W, l, n, trace, store, routes) if layer_is_moe(c, l) else dense_layer(c, W, l, n, store))
+    h = store(rms_norm(h, W["model.norm.weight"], eps))
     head = W["model.embed_tokens.weight"] if c.get("tie_word_embeddings", False) else W["lm_head.weight"]
     return h @ head.T
 

@@ -23,13 +23,6 @@ def engine(request, model_dir):
     return which, d, request.param, H.make_engine(d, request.param)
 
 
-def _check(dtype, got, ref, what):
-    if dtype == "float32":
-        H.assert_close_fp32(got, ref, what)
-    else:
-        H.assert_close_bf16(got, ref, what)
-
-
 def _requests(which):
     vocab = CONFIGS[which]["vocab_size"]
     return [H.random_tokens(n, vocab, 100 + i) for i, n in enumerate(PROMPTS[which])]
@@ -38,30 +31,28 @@ def _requests(which):
 def test_whole(engine):
     which, d, dtype, eng = engine
     for i, toks in enumerate(_requests(which)):
-        got = H.run_cut(eng, f"w{i}", toks, H.whole(len(toks)))
-        _check(dtype, got, H.plain_logits(d, toks), f"{which} {dtype} whole request {i}")
+        H.check_against_plain(eng, d, dtype, f"w{i}", toks, H.whole(len(toks)), f"{which} {dtype} whole request {i}")
 
 
 def test_last_tokens_decoded(engine):
     which, d, dtype, eng = engine
     for i, toks in enumerate(_requests(which)):
-        got = H.run_cut(eng, f"d{i}", toks, H.last_decoded(len(toks)))
-        _check(dtype, got, H.plain_logits(d, toks), f"{which} {dtype} last-32-decoded request {i}")
+        H.check_against_plain(eng, d, dtype, f"d{i}", toks, H.last_decoded(len(toks)),
+                              f"{which} {dtype} last-32-decoded request {i}")
 
 
 def test_changing_portions(engine):
     which, d, dtype, eng = engine
     for i, toks in enumerate(_requests(which)):
         for seed in (0, 1):
-            got = H.run_cut(eng, f"p{i}", toks, H.changing_portions(len(toks), seed))
-            _check(dtype, got, H.plain_logits(d, toks), f"{which} {dtype} portions(seed {seed}) request {i}")
+            H.check_against_plain(eng, d, dtype, f"p{i}", toks, H.changing_portions(len(toks), seed),
+                                  f"{which} {dtype} portions(seed {seed}) request {i}")
 
 
 def test_token_by_token(engine):
     which, d, dtype, eng = engine
     toks = _requests(which)[-1]
-    got = H.run_cut(eng, "t", toks, [1] * len(toks))
-    _check(dtype, got, H.plain_logits(d, toks), f"{which} {dtype} token by token")
+    H.check_against_plain(eng, d, dtype, "t", toks, [1] * len(toks), f"{which} {dtype} token by token")
 
 
 def test_cuts_agree_fp32(engine):
