@@ -155,3 +155,108 @@ def assert_close_bf16(got: torch.Tensor, ref: torch.Tensor, what: str = "", tol_
         first = int(bad.nonzero()[0])
         raise AssertionError(f"{what}: max |diff| / row rms = {float(e_max.max()):.3f} (tol {tol_max}), "
                              f"rms diff / row rms = {float(e_rms.max()):.3f} (tol {tol_rms}); first wrong row {first}")
+
+
+# ---------------------------------------------------------------------------
+# traces: the same requests replayed step by step, several live at a time
+# ---------------------------------------------------------------------------
+def mixed_trace(requests: Dict[str, Sequence[int]], seed: int, max_live: int = 4, tail: int = 32) -> List[dict]:
+    """Steps in the format of bin/trace_run.  Up to `max_live` requests are live; each reads its
+    prompt in portions of changing size (down to two tokens) and its last `tail` tokens one by
+    one; a live request is sometimes left out of a step; logits are wanted everywhere."""
+    rng = random.Random(seed)
+    waiting = list(requests.items())
+    live: Dict[str, int] = {}              # id -> tokens done
+    steps: List[dict] = []
+    while waiting or live:
+        while waiting and len(live) < max_live and (not live or rng.random() < 0.6):
+            rid, _ = waiting.pop(0)
+            live[rid] = 0
+        entries, end = [], []
+        for rid in list(live):
+            toks = requests[rid]
+            done = live[rid]
+            if len(live) > 1 and rng.random() < 0.2:
+                continue                               # sits this step out
+            left = len(toks) - done
+            if left <= tail:
+                take = 1
+            else:
+                take = min(left - tail, rng.choice([2, 2, 3, 5, 7, 13, 21]))
+            entries.append({"id": rid, "tokens": list(toks[done:done + take]), "want": list(range(take))})
+            live[rid] = done + take
+            if live[rid] == len(toks):
+                end.append(rid)
+                del live[rid]
+        if entries:
+            steps.append({"step": len(steps), "entries": entries, "end": end})
+    return steps
+
+
+def tokens_held(steps: List[dict], round_to: int = 64) -> int:
+    """The most tokens that live requests hold at any time, each rounded up to `round_to`."""
+    held: Dict[str, int] = {}
+    worst = 0
+    for st in steps:
+        for e in st["entries"]:
+            held[e["id"]] = held.get(e["id"], 0) + len(e["tokens"])
+        worst = max(worst, sum((n + round_to - 1) // round_to * round_to for n in held.values()))
+        for rid in st["end"]:
+            held.pop(rid, None)
+    return worst
+
+
+def replay(engine, steps: List[dict], with_routes: bool = False):
+    """Feed a trace through the engine's step function.  Returns {id: logits [len, vocab]} for
+    the wanted places in order (and {id: [ids per routed layer]} if asked)."""
+    from sharpinference_amd.engine import StepEntry
+
+    logits: Dict[str, List[torch.Tensor]] = {}
+    picks: Dict[str, List[List[torch.Tensor]]] = {}
+    live = set()
+    for st in steps:
+        entries = []
+        for e in st["entries"]:
+            if e["id"] not in live:
+                engine.add_request(e["id"])
+                live.add(e["id"])
+            entries.append(StepEntry(e["id"], e["tokens"], e["want"]))
+        trace: list = []
+        lg = engine.step(entries, router_trace=trace if with_routes else None)
+        lg = lg.float().cpu() if lg is not None else None
+        row, tok = 0, 0
+        for e in st["entries"]:
+            n = len(e["want"])
+            if n:
+                logits.setdefault(e["id"], []).append(lg[row:row + n])
+                row += n
+            if with_routes:
+                picks.setdefault(e["id"], []).append([ids[tok:tok + len(e["tokens"])].cpu() for ids, _ in trace])
+            tok += len(e["tokens"])
+        for rid in st["end"]:
+            engine.free_request(rid)
+            live.discard(rid)
+        engine.cache.check_invariants()
+    out = {rid: torch.cat(v, 0) for rid, v in logits.items()}
+    if not with_routes:
+        return out
+    routes = {}
+    for rid, per_step in picks.items():
+        n_moe = len(per_step[0])
+        routes[rid] = [torch.cat([p[i] for p in per_step], 0) for i in range(n_moe)]
+    return out, routes
+
+
+def check_trace_against_plain(engine, model_dir: str, dtype: str, requests: Dict[str, Sequence[int]],
+                              steps: List[dict], what: str) -> None:
+    if dtype == "float32":
+        got = replay(engine, steps)
+        for rid, toks in requests.items():
+            assert_close_fp32(got[rid], plain_logits(model_dir, toks), f"{what} request {rid}")
+        return
+    got, picks = replay(engine, steps, with_routes=True)
+    layers = moe_layers_of(model_dir)
+    for rid, toks in requests.items():
+        ref, regret = plain_logits_routed(model_dir, toks, dict(zip(layers, picks[rid])))
+        assert regret <= ROUTE_REGRET, f"{what} request {rid}: expert pick {regret:.3f} (relative) below the best"
+        assert_close_bf16(got[rid], ref, f"{what} request {rid}")

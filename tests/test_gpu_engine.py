@@ -64,3 +64,24 @@ def test_cuts_agree_fp32(engine):
     a = H.run_cut(eng, "x", toks, H.whole(len(toks)))
     b = H.run_cut(eng, "y", toks, H.changing_portions(len(toks), 3))
     assert float((a - b).abs().max()) <= 1e-5 * max(1.0, float(a.abs().max()))
+
+
+@pytest.mark.parametrize("seed", [0, 1])
+def test_mixed_batches_with_page_reuse(model_dir, seed):
+    """Up to four live requests, portions of some beside decoded tokens of others, in a pool so
+    small that pages of finished requests are used again."""
+    which, d = model_dir
+    vocab = CONFIGS[which]["vocab_size"]
+    lens = [37, 70, 5, 101, 64, 49, 83]
+    reqs = {f"r{i}": H.random_tokens(n, vocab, 300 + 10 * seed + i) for i, n in enumerate(lens)}
+    steps = H.mixed_trace(reqs, seed)
+    assert max(len(s["entries"]) for s in steps) >= 3
+    assert any(len(e["tokens"]) == 1 for s in steps for e in s["entries"]) and \
+        any(len(e["tokens"]) > 1 for s in steps for e in s["entries"])
+    held = H.tokens_held(steps)
+    for dtype in ("float32", "bfloat16"):
+        eng = H.make_engine(d, dtype, kv_tokens=held, max_num_seqs=4)
+        H.check_trace_against_plain(eng, d, dtype, reqs, steps, f"{which} {dtype} mixed(seed {seed})")
+        for g in eng.cache.groups:
+            assert g.pool.total_allocs > g.pool.num_pages, "the pool was large enough to never reuse a page"
+            assert g.pool.num_free == g.pool.num_pages
