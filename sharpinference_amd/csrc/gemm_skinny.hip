@@ -1,0 +1,174 @@
+// Weight-streaming matrix product for few rows (decode): out[M, N] = x[M, K] * W[N, K]^T, bfloat16
+// inputs, float accumulation on the matrix cores (v_mfma_f32_16x16x32_bf16), M <= 64.
+//
+// The weights are read from HBM exactly once; everything else is arranged around that.
+//  * A block owns R tiles of 16 weight rows; its NW waves split K into contiguous slices.  Per
+//    128-wide K unit a lane loads 64 contiguous bytes of each of its weight rows and of each of
+//    its x rows and feeds 4 MFMAs per (tile, row block): W is the A operand (rows = n), x the
+//    B operand.  Both operands take element (group g, index i) of a lane from the same k, so
+//    the order of k inside a unit is free: lanes read 64-byte runs, not 16-byte ones.
+//  * The waves' partial sums meet in LDS and are added in wave order.  R and NW are chosen from
+//    the weight's shape alone and the x rows never mix, so a row's result does not depend on
+//    the batch around it.
+//  * Grouped form (routed experts): block (tile, expert e) handles rows
+//    [offsets[e], offsets[e + 1]) of the expert-sorted row list with W[e], sixteen at a time;
+//    x rows are gathered through a_rows.  Experts without rows return at once.
+//
+// Limits (the caller falls back to other kernels otherwise): K % 128 == 0, N % 4 == 0, M <= 64.
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+template <typename TO> __device__ __forceinline__ void store4(TO* p, f32x4 v);
+template <> __device__ __forceinline__ void store4<float>(float* p, f32x4 v) {
+  *reinterpret_cast<f32x4*>(p) = v;
+}
+template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, f32x4 v) {
+  uint2 packed;
+  packed.x = (uint32_t)f32_to_bf16(v[0]).bits | ((uint32_t)f32_to_bf16(v[1]).bits << 16);
+  packed.y = (uint32_t)f32_to_bf16(v[2]).bits | ((uint32_t)f32_to_bf16(v[3]).bits << 16);
+  *reinterpret_cast<uint2*>(p) = packed;
+}
+
+constexpr int kRedTiles = 2;  // (tile, row block) pairs summed per LDS round
+
+template <int R, int MB, int NW, typename TO>
+__global__ __launch_bounds__(NW* kWave) void skinny_gemm_kernel(
+    const bf16_t* __restrict__ x, const bf16_t* __restrict__ W, TO* __restrict__ out, int M, int N, int K,
+    const int* __restrict__ a_rows, const int* __restrict__ group_offsets) {
+  __shared__ f32x4 red[NW][kRedTiles][kWave];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int w = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int nb = blockIdx.x;
+  const int e = blockIdx.y;
+  int row_begin = 0, row_end = M;
+  if (group_offsets) {
+    row_begin = group_offsets[e];
+    row_end = group_offsets[e + 1];
+    W += (size_t)e * N * K;
+  }
+  const int n_rows = row_end - row_begin;
+  if (n_rows <= 0) return;
+  const int n_base = nb * 16 * R;
+
+  // this wave's K units
+  const int U = K >> 7;
+  const int u_begin = (U * w) / NW;
+  const int u_end = (U * (w + 1)) / NW;
+
+  const bf16_t* wrow[R];
+#pragma unroll
+  for (int t = 0; t < R; ++t) {
+    int n = n_base + t * 16 + r;
+    if (n >= N) n = N - 1;  // loaded, never stored
+    wrow[t] = W + (size_t)n * K + g * 32;
+  }
+
+  for (int rb0 = 0; rb0 * 16 < n_rows; rb0 += MB) {
+    const bf16_t* xrow[MB];
+    bool xvalid[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      const int m = row_begin + (rb0 + mb) * 16 + r;
+      xvalid[mb] = m < row_end;
+      const int src = xvalid[mb] ? (a_rows ? a_rows[m] : m) : 0;
+      xrow[mb] = x + (size_t)src * K + g * 32;
+    }
+    f32x4 acc[R][MB];
+#pragma unroll
+    for (int t = 0; t < R; ++t)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) acc[t][mb] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    for (int u = u_begin; u < u_end; ++u) {
+      const int k0 = u << 7;
+      bf16x8 wf[R][4], xf[MB][4];
+#pragma unroll
+      for (int t = 0; t < R; ++t)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) wf[t][j] = *reinterpret_cast<const bf16x8*>(wrow[t] + k0 + j * 8);
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          if (xvalid[mb]) xf[mb][j] = *reinterpret_cast<const bf16x8*>(xrow[mb] + k0 + j * 8);
+          else xf[mb][j] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+        }
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int t = 0; t < R; ++t)
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb)
+            acc[t][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[t][j], xf[mb][j], acc[t][mb], 0, 0, 0);
+    }
+
+    // add the waves' K slices in wave order, kRedTiles (tile, row block) pairs per round;
+    // pair p of a round is summed and stored by wave p
+#pragma unroll
+    for (int p0 = 0; p0 < R * MB; p0 += kRedTiles) {
+      __syncthreads();
+#pragma unroll
+      for (int p = 0; p < kRedTiles; ++p)
+        if (p0 + p < R * MB) red[w][p][lane] = acc[(p0 + p) / MB][(p0 + p) % MB];
+      __syncthreads();
+      if (w < kRedTiles && p0 + w < R * MB) {
+        const int t = (p0 + w) / MB, mb = (p0 + w) % MB;
+        f32x4 v = red[0][w][lane];
+#pragma unroll
+        for (int ww = 1; ww < NW; ++ww) v += red[ww][w][lane];
+        // lane holds out[row = ... + r][n = n_base + t*16 + g*4 + 0..3]
+        const int row = row_begin + (rb0 + mb) * 16 + r;
+        const int n = n_base + t * 16 + g * 4;
+        if (row < row_end && n < N) store4<TO>(out + (size_t)row * N + n, v);
+      }
+    }
+  }
+}
+
+template <int R, int MB, int NW>
+static int launch_skinny(const void* x, const void* W, void* out, int out_dtype, int M, int N, int K,
+                         const int* a_rows, const int* group_offsets, int groups, hipStream_t stream) {
+  dim3 grid(ceil_div(N, 16 * R), groups > 0 ? groups : 1), block(NW * kWave);
+  const int* go = groups > 0 ? group_offsets : nullptr;
+  if (out_dtype == DT_F32)
+    skinny_gemm_kernel<R, MB, NW, float><<<grid, block, 0, stream>>>((const bf16_t*)x, (const bf16_t*)W,
+                                                                    (float*)out, M, N, K, a_rows, go);
+  else
+    skinny_gemm_kernel<R, MB, NW, bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)x, (const bf16_t*)W,
+                                                                     (bf16_t*)out, M, N, K, a_rows, go);
+  SHARPI_CHECK_LAUNCH();
+  return SHARPI_OK;
+}
+
+template <int R, int NW>
+static int dispatch_mb(int MB, const void* x, const void* W, void* out, int out_dtype, int M, int N, int K,
+                       const int* a_rows, const int* group_offsets, int groups, hipStream_t stream) {
+  if (MB == 1) return launch_skinny<R, 1, NW>(x, W, out, out_dtype, M, N, K, a_rows, group_offsets, groups, stream);
+  if (MB == 2) return launch_skinny<R, 2, NW>(x, W, out, out_dtype, M, N, K, a_rows, group_offsets, groups, stream);
+  return launch_skinny<R, 4, NW>(x, W, out, out_dtype, M, N, K, a_rows, group_offsets, groups, stream);
+}
+
+// x [M, K] bf16 (rows gathered through a_rows if given), W [N, K] or [groups, N, K] bf16,
+// out [M, N] (out_dtype float or bf16).  groups == 0: plain.  groups > 0: rows are the
+// expert-sorted list, group_offsets [groups + 1].  R in {1, 2, 4}: 16-row weight tiles per block;
+// NW in {4, 8, 16}: waves per block splitting K.
+SHARPI_EXPORT int sharpi_gemm_skinny(const void* x, const void* W, void* out, int out_dtype, int M, int N, int K,
+                                     const int* a_rows, const int* group_offsets, int groups, int R, int NW,
+                                     hipStream_t stream) {
+  if (M <= 0) return SHARPI_OK;
+  if (M > 64 || N <= 0 || (N & 3) || K <= 0 || (K & 127) || groups < 0 || groups > 65535) return SHARPI_ERR_ARG;
+  if (groups > 0 && group_offsets == nullptr) return SHARPI_ERR_ARG;
+  if (out_dtype != DT_F32 && out_dtype != DT_BF16) return SHARPI_ERR_ARG;
+  // grouped rows are spread over experts: one row block at a time; plain: all row blocks at once
+  const int MB = groups > 0 ? 1 : ceil_div(M, 16);
+#define SK(RR, WW) \
+  if (R == RR && NW == WW) return dispatch_mb<RR, WW>(MB, x, W, out, out_dtype, M, N, K, a_rows, group_offsets, groups, stream)
+  SK(1, 4); SK(1, 8); SK(1, 16);
+  SK(2, 4); SK(2, 8); SK(2, 16);
+  SK(4, 4); SK(4, 8); SK(4, 16);
+#undef SK
+  return SHARPI_ERR_ARG;
+}

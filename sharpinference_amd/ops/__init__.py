@@ -195,6 +195,55 @@ def gemm_tiled(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype
     return out
 
 
+# ---------------------------------------------------------------------------
+# the weight-streaming product for few rows (decode)
+# ---------------------------------------------------------------------------
+SKINNY_MAX_ROWS = 64          # grouped form: rows of all experts together
+SKINNY_MAX_ROWS_PLAIN = 16    # plain form: beyond one row block the library's product is faster
+
+
+def skinny_ok(M: int, N: int, K: int, grouped: bool = False) -> bool:
+    return 0 < M <= (SKINNY_MAX_ROWS if grouped else SKINNY_MAX_ROWS_PLAIN) and K % 128 == 0 and N % 4 == 0
+
+
+def skinny_plan(N: int, K: int):
+    """(R, NW): 16-row weight tiles per block and waves per block splitting K (measured on
+    MI355X over the projection shapes of the model).  Both depend on the weight's shape only,
+    so the order of a row's sums does not change with the batch."""
+    return (4 if N >= 12288 else 2), 8
+
+
+def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, a_rows: Optional[torch.Tensor] = None,
+                offsets: Optional[torch.Tensor] = None, n_rows: Optional[int] = None, R: Optional[int] = None,
+                NW: Optional[int] = None) -> torch.Tensor:
+    """x [M, K] @ w[N, K]^T (or per expert with w [E, N, K]) for M <= 64 on the matrix cores."""
+    _dev(x, w, a_rows, offsets)
+    _i32(a_rows, "a_rows")
+    _i32(offsets, "offsets")
+    _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_skinny: bfloat16 operands only")
+    grouped = offsets is not None
+    if grouped:
+        _need(w.dim() == 3 and offsets.shape == (w.shape[0] + 1,), "gemm_skinny: grouped needs w [E, N, K], offsets [E+1]")
+        E, N, K = w.shape
+        M = int(n_rows)
+        if a_rows is not None:
+            _need(a_rows.shape == (M,), "gemm_skinny: a_rows must be [n_rows]")
+        else:
+            _need(x.shape[0] == M, "gemm_skinny: x must have n_rows rows when not gathered")
+    else:
+        _need(w.dim() == 2 and a_rows is None, "gemm_skinny: plain needs w [N, K]")
+        E, (N, K) = 0, w.shape
+        M = x.shape[0]
+    _need(x.dim() == 2 and x.shape[1] == K, f"gemm_skinny: x {tuple(x.shape)} vs w {tuple(w.shape)}")
+    _need(0 < M <= SKINNY_MAX_ROWS and K % 128 == 0 and N % 4 == 0,
+          f"gemm_skinny: shape M={M} N={N} K={K} is not taken (M <= 64, K % 128 == 0, N % 4 == 0)")
+    pr, pw = skinny_plan(N, K)
+    out = torch.empty(M, N, dtype=out_dtype, device=x.device)
+    _run("sharpi_gemm_skinny", _ptr(x), _ptr(w), _ptr(out), _code(out_dtype), M, N, K, _ptr(a_rows), _ptr(offsets), E,
+         R or pr, NW or pw, _stream())
+    return out
+
+
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """y = x W^T.  float32 weights: the float FMA kernel (true 32-bit, whatever x was stored
     as).  bfloat16 weights: the library's matrix product with float accumulation."""
@@ -206,6 +255,8 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     _dev(x, w)
     xb = x if x.dtype == torch.bfloat16 else cast(x, torch.bfloat16)
     _need(xb.shape[1] == w.shape[1], f"linear: x {tuple(x.shape)} vs w {tuple(w.shape)}")
+    if skinny_ok(xb.shape[0], w.shape[0], w.shape[1]):
+        return gemm_skinny(xb, w, out_dtype)
     if out_dtype == torch.bfloat16:
         return torch.mm(xb, w.t())
     return torch.mm(xb, w.t(), out_dtype=torch.float32)
@@ -325,5 +376,7 @@ def grouped_linear(x: torch.Tensor, w: torch.Tensor, offsets: torch.Tensor, a_ro
     """Per-expert products over the expert-sorted row list (see grouped_gemm)."""
     if x.dtype != w.dtype:
         x = cast(x, w.dtype)
+    if w.dtype == torch.bfloat16 and skinny_ok(n_rows, w.shape[1], w.shape[2], grouped=True):
+        return gemm_skinny(x, w, out_dtype, a_rows=a_rows, offsets=offsets, n_rows=n_rows)
     y = grouped_gemm(x, w, offsets, a_rows, n_rows)
     return y if y.dtype == out_dtype else cast(y, out_dtype)
