@@ -118,9 +118,12 @@ class CacheManager:
             for i, spec in enumerate(self.slot_specs):
                 if isinstance(spec, KVSpec):
                     n = self.groups[self.group_of_slot[i]].pool.num_pages
-                    shape = (n, spec.num_kv_heads, page_size, spec.head_dim)
-                    self.k[i] = torch.zeros(shape, dtype=dtype, device=self.device)
-                    self.v[i] = torch.zeros(shape, dtype=dtype, device=self.device)
+                    # keys [page, kv head, position, head_dim]; values transposed inside the page,
+                    # [page, kv head, head_dim, position], the layout the matrix-core kernels read
+                    self.k[i] = torch.zeros((n, spec.num_kv_heads, page_size, spec.head_dim), dtype=dtype,
+                                            device=self.device)
+                    self.v[i] = torch.zeros((n, spec.num_kv_heads, spec.head_dim, page_size), dtype=dtype,
+                                            device=self.device)
                 elif isinstance(spec, StateSpec):
                     self.state[i] = torch.zeros((max_requests, *spec.shape), dtype=spec.dtype, device=self.device)
 

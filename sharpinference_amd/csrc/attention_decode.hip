@@ -1,0 +1,261 @@
+// Attention for single-token entries (decode): split-K flash-decode on the matrix cores.
+//
+// One block = (a run of SPLIT_KEYS keys, one token, one kv head with up to 16 of its query
+// heads).  Everything is computed transposed, so that no operand ever has to be re-laid-out:
+//   S^T[key, head] = K[key, :] . Q[head, :]      A = K block (16 keys x 32 d), B = Q^T
+//   O^T[d, head]  += V^T[d, key] * P^T[key, head] A = V^T block (16 d x 32 keys), B = P^T
+// The S^T accumulator of a lane (4 keys of each of two 16-key blocks, one head) is exactly
+// the B operand the second product wants, once exponentiated and split into a bfloat16 pair
+// (hi + lo, two products, so the probabilities keep ~16 bits); the
+// value cache is stored transposed inside a page for the A operand of the second product.
+// Keys are walked in 16-key blocks aligned to absolute positions (a block never straddles a
+// page); keys before the window's start or after the query are masked.  The four waves take
+// 32-key chunks round-robin and meet in LDS; the block leaves (max, sum, unnormalised O) per
+// head, and a second kernel merges the runs of a token.  The run length is fixed, so the sums
+// of a query depend on (start, position) only, not on the batch.
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+constexpr int kDecWaves = 4;
+constexpr int kSplitBlocks = 16;  // 16-key blocks per run: 256 keys
+
+__device__ __forceinline__ __bf16 to_bf16_rne(float f) {
+  bf16_t b = f32_to_bf16(f);
+  return __builtin_bit_cast(__bf16, b.bits);
+}
+
+template <int HD>
+__global__ __launch_bounds__(kDecWaves* kWave) void attn_decode_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    const int* __restrict__ block_table, const int* __restrict__ entry_of_token,
+    const int* __restrict__ positions, const int* __restrict__ token_list, float* __restrict__ part_o,
+    float* __restrict__ part_ml, int window_kind, int window, float scale, int nh, int nkv, int page_size,
+    int max_blocks, int num_pages, int max_splits) {
+  constexpr int NJ = HD / 32;  // 32-wide d chunks of the first product
+  constexpr int ND = HD / 16;  // 16-row d tiles of the second product
+  __shared__ f32x4 acc_s[kDecWaves][ND][kWave];
+  __shared__ float m_s[kDecWaves][16];
+  __shared__ float l_s[kDecWaves][kWave];
+
+  const int lane = threadIdx.x & (kWave - 1);
+  const int w = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int sp = blockIdx.x;
+  const int li = blockIdx.y;
+  const int t = token_list ? token_list[li] : li;
+  const int G = nh / nkv;
+  const int hgroups = (G + 15) / 16;
+  const int kvh = blockIdx.z / hgroups;
+  const int h0 = kvh * G + (blockIdx.z % hgroups) * 16;
+  const int hcount = min(16, kvh * G + G - h0);
+
+  const int p = positions[t];
+  int start = 0;
+  if (window_kind == 1) start = (p / window) * window;
+  else if (window_kind == 2) start = p - window + 1 > 0 ? p - window + 1 : 0;
+  const int b_first = (start >> 4) + sp * kSplitBlocks;
+  const int b_last = min(p >> 4, b_first + kSplitBlocks - 1);
+  if (b_first > (p >> 4)) return;  // this run lies beyond the query
+  const int* bt = block_table + (size_t)entry_of_token[t] * max_blocks;
+
+  // Q^T fragments: lane (head r, group g) holds q[head][j*32 + g*8 .. +8]
+  bf16x8 qf[NJ];
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) {
+    if (r < hcount) qf[j] = *reinterpret_cast<const bf16x8*>(q + ((size_t)t * nh + h0 + r) * HD + j * 32 + g * 8);
+    else qf[j] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+  }
+
+  float m = -INFINITY, l = 0.f;   // for head r: m identical in the 4 lanes of a column, l a partial sum
+  f32x4 acc[ND];
+#pragma unroll
+  for (int d = 0; d < ND; ++d) acc[d] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  for (int b = b_first + 2 * w; b <= b_last; b += 2 * kDecWaves) {
+    // two 16-key blocks: b and b + 1 (the second may lie beyond the range)
+    f32x4 s[2];
+    long long kbase[2], vbase[2];
+    bool have[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int bb = b + u;
+      have[u] = bb <= b_last;
+      int page = -1;
+      if (have[u]) {
+        const int pi = (bb << 4) / page_size;
+        page = pi < max_blocks ? bt[pi] : -1;
+        if (page < 0 || page >= num_pages) have[u] = false;
+      }
+      const int off = (bb << 4) % page_size;
+      kbase[u] = have[u] ? (((long long)page * nkv + kvh) * page_size + off) * HD : 0;
+      vbase[u] = have[u] ? ((long long)page * nkv + kvh) * HD * page_size + off : 0;
+      s[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (have[u]) {
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+          const bf16x8 kf = *reinterpret_cast<const bf16x8*>(k_cache + kbase[u] + (size_t)r * HD + j * 32 + g * 8);
+          s[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[j], s[u], 0, 0, 0);
+        }
+      }
+    }
+    // lane holds S^T[key = 16*(b+u) + 4g + i][head r]
+    float cm = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = ((b + u) << 4) + 4 * g + i;
+        const bool ok = have[u] && key >= start && key <= p;
+        s[u][i] = ok ? s[u][i] * scale : -INFINITY;
+        cm = fmaxf(cm, s[u][i]);
+      }
+    cm = fmaxf(cm, __shfl_xor(cm, 16, kWave));
+    cm = fmaxf(cm, __shfl_xor(cm, 32, kWave));
+    const float m_new = fmaxf(m, cm);
+    float corr = 1.0f;
+    bf16x8 pf, pf_lo;   // probabilities as a bfloat16 pair hi + lo: ~16 bits survive the product
+    if (m_new == -INFINITY) {
+      pf = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      pf_lo = pf;
+    } else {
+      corr = expf(m - m_new);  // m = -inf gives 0
+      float ls = 0.f;
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float e = expf(s[u][i] - m_new);  // masked: exp(-inf) = 0
+          ls += e;
+          const bf16_t hi = f32_to_bf16(e);
+          pf[u * 4 + i] = __builtin_bit_cast(__bf16, hi.bits);
+          pf_lo[u * 4 + i] = to_bf16_rne(e - bf16_to_f32(hi));
+        }
+      l = l * corr + ls;
+      m = m_new;
+    }
+#pragma unroll
+    for (int d = 0; d < ND; ++d) {
+      // V^T fragment: lane (d row r, group g) holds keys 4g..4g+3 of block b, then of block b + 1
+      bf16x4 va = bf16x4{0, 0, 0, 0}, vb = bf16x4{0, 0, 0, 0};
+      if (have[0]) va = *reinterpret_cast<const bf16x4*>(v_cache + vbase[0] + (size_t)(d * 16 + r) * page_size + 4 * g);
+      if (have[1]) vb = *reinterpret_cast<const bf16x4*>(v_cache + vbase[1] + (size_t)(d * 16 + r) * page_size + 4 * g);
+      const bf16x8 vf = __builtin_shufflevector(va, vb, 0, 1, 2, 3, 4, 5, 6, 7);
+      acc[d] *= corr;   // corr belongs to head r = the accumulator's column
+      acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, acc[d], 0, 0, 0);
+      acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf_lo, acc[d], 0, 0, 0);
+    }
+  }
+
+  // meet in LDS: per head, the four waves' (m, l, O)
+  if (g == 0) m_s[w][r] = m;
+  l_s[w][lane] = l;
+#pragma unroll
+  for (int d = 0; d < ND; ++d) acc_s[w][d][lane] = acc[d];
+  __syncthreads();
+  if (w != 0) return;
+  float M = m_s[0][r];
+#pragma unroll
+  for (int ww = 1; ww < kDecWaves; ++ww) M = fmaxf(M, m_s[ww][r]);
+  float f[kDecWaves];
+  float L = 0.f;
+#pragma unroll
+  for (int ww = 0; ww < kDecWaves; ++ww) {
+    f[ww] = m_s[ww][r] == -INFINITY ? 0.f : expf(m_s[ww][r] - M);
+    const float lw = l_s[ww][r] + l_s[ww][r + 16] + l_s[ww][r + 32] + l_s[ww][r + 48];
+    L += f[ww] * lw;
+  }
+  if (r >= hcount) return;
+  const size_t slot = ((size_t)li * nh + h0 + r) * max_splits + sp;
+  if (g == 0) {
+    part_ml[slot * 2] = M;
+    part_ml[slot * 2 + 1] = L;
+  }
+#pragma unroll
+  for (int d = 0; d < ND; ++d) {
+    f32x4 o = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ww = 0; ww < kDecWaves; ++ww) o += acc_s[ww][d][lane] * f[ww];
+    // lane holds O^T[d*16 + 4g + i][head r]
+    *reinterpret_cast<f32x4*>(part_o + slot * HD + d * 16 + 4 * g) = o;
+  }
+}
+
+// merge the runs of one (token, head): out = sum_s O_s e^(m_s - M) / sum_s l_s e^(m_s - M)
+__global__ void attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                         const int* __restrict__ positions, const int* __restrict__ token_list,
+                                         bf16_t* __restrict__ out, int window_kind, int window, int nh, int hd,
+                                         int max_splits) {
+  const int li = blockIdx.x;
+  const int h = blockIdx.y;
+  const int t = token_list ? token_list[li] : li;
+  const int p = positions[t];
+  int start = 0;
+  if (window_kind == 1) start = (p / window) * window;
+  else if (window_kind == 2) start = p - window + 1 > 0 ? p - window + 1 : 0;
+  const int n_runs = ((p >> 4) - (start >> 4)) / kSplitBlocks + 1;
+  const size_t base = ((size_t)li * nh + h) * max_splits;
+  float M = -INFINITY;
+  for (int s = 0; s < n_runs; ++s) M = fmaxf(M, part_ml[(base + s) * 2]);
+  float L = 0.f;
+  for (int s = 0; s < n_runs; ++s) {
+    const float ms = part_ml[(base + s) * 2];
+    L += ms == -INFINITY ? 0.f : part_ml[(base + s) * 2 + 1] * expf(ms - M);
+  }
+  for (int d = threadIdx.x; d < hd; d += blockDim.x) {
+    float o = 0.f;
+    for (int s = 0; s < n_runs; ++s) {
+      const float ms = part_ml[(base + s) * 2];
+      if (ms != -INFINITY) o += part_o[(base + s) * hd + d] * expf(ms - M);
+    }
+    out[((size_t)t * nh + h) * hd + d] = f32_to_bf16(L > 0.f ? o / L : 0.f);
+  }
+}
+
+template <int HD>
+static int launch_decode(const void* q, const void* k_cache, const void* v_cache, const int* block_table,
+                         const int* entry_of_token, const int* positions, const int* token_list, float* part_o,
+                         float* part_ml, void* out, int window_kind, int window, float scale, int n_list, int nh,
+                         int nkv, int page_size, int max_blocks, int num_pages, int max_splits, hipStream_t stream) {
+  const int G = nh / nkv;
+  dim3 grid(max_splits, n_list, nkv * ((G + 15) / 16)), block(kDecWaves * kWave);
+  attn_decode_kernel<HD><<<grid, block, 0, stream>>>((const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache,
+                                                    block_table, entry_of_token, positions, token_list, part_o,
+                                                    part_ml, window_kind, window, scale, nh, nkv, page_size,
+                                                    max_blocks, num_pages, max_splits);
+  SHARPI_CHECK_LAUNCH();
+  dim3 mgrid(n_list, nh), mblock(HD >= 128 ? 128 : 64);
+  attn_decode_merge_kernel<<<mgrid, mblock, 0, stream>>>(part_o, part_ml, positions, token_list, (bf16_t*)out,
+                                                         window_kind, window, nh, HD, max_splits);
+  SHARPI_CHECK_LAUNCH();
+  return SHARPI_OK;
+}
+
+// q [T, nh, hd] bf16; caches K [pages, nkv, page_size, hd], V [pages, nkv, hd, page_size] bf16;
+// token_list [n_list] (or null: tokens 0..n_list-1); part_o float [n_list, nh, max_splits, hd];
+// part_ml float [n_list, nh, max_splits, 2]; out [T, nh, hd] bf16 (rows of the listed tokens).
+// max_splits must cover every listed token: ceil over 256-key runs of its visible keys.
+SHARPI_EXPORT int sharpi_attention_decode(const void* q, const void* k_cache, const void* v_cache,
+                                          const int* block_table, const int* entry_of_token, const int* positions,
+                                          const int* token_list, float* part_o, float* part_ml, void* out,
+                                          int window_kind, int window, float scale, int n_list, int nh, int nkv,
+                                          int hd, int page_size, int max_blocks, int num_pages, int max_splits,
+                                          hipStream_t stream) {
+  if (n_list <= 0) return SHARPI_OK;
+  if (nh <= 0 || nkv <= 0 || nh % nkv != 0 || nh > 65535 || n_list > 65535) return SHARPI_ERR_ARG;
+  if (page_size <= 0 || page_size % 16 != 0 || max_blocks <= 0 || num_pages <= 0 || max_splits <= 0) return SHARPI_ERR_ARG;
+  if (window_kind < 0 || window_kind > 2 || (window_kind != 0 && window <= 0)) return SHARPI_ERR_ARG;
+  if (nkv * ((nh / nkv + 15) / 16) > 65535) return SHARPI_ERR_ARG;
+#define DEC(HDV)                                                                                                  \
+  if (hd == HDV)                                                                                                  \
+  return launch_decode<HDV>(q, k_cache, v_cache, block_table, entry_of_token, positions, token_list, part_o,      \
+                            part_ml, out, window_kind, window, scale, n_list, nh, nkv, page_size, max_blocks,     \
+                            num_pages, max_splits, stream)
+  DEC(32); DEC(64); DEC(96); DEC(128); DEC(192); DEC(256);
+#undef DEC
+  return SHARPI_ERR_ARG;  // head sizes that are no multiple of 32 go to the generic kernel
+}
+
+SHARPI_EXPORT int sharpi_attention_decode_split_keys() { return kSplitBlocks * 16; }

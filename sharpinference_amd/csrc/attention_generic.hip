@@ -82,11 +82,12 @@ __global__ __launch_bounds__(kAttnWaves* kWave) void attn_generic_kernel(
         const int r = vrow[w][j];
         if (r < 0) continue;
         const float pj = pw[w][j];
-        const T* vr = v_cache + (size_t)r * hd;
+        // values are stored transposed inside a page: [page][kv head][hd][page_size]
+        const T* vr = v_cache + (size_t)(r / page_size) * hd * page_size + (r % page_size);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int d = lane + i * kWave;
-          if (d < hd) acc[i] = fmaf(pj, to_f32<T>(vr[d]), acc[i]);
+          if (d < hd) acc[i] = fmaf(pj, to_f32<T>(vr[(size_t)d * page_size]), acc[i]);
         }
       }
     }

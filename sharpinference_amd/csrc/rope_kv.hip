@@ -5,7 +5,9 @@
 // k head : rotate (if inv_freq) -> norm (if qk_norm) -> cache K at slot_mapping[t]
 // v head : cache V at slot_mapping[t]
 // Rotation is on interleaved pairs (2i, 2i+1) with angle = float(pos) * inv_freq[i], all in float.
-// Cache layout of one layer: [page][kv head][page_size][hd]; slot = page * page_size + offset;
+// Cache layout of one layer: keys [page][kv head][page_size][hd], values transposed inside the page,
+// [page][kv head][hd][page_size] (so that the matrix-core kernels read runs of keys for one
+// value column); slot = page * page_size + offset;
 // a negative slot means "do not store" (the layer reads another layer's cache).
 #include "common.h"
 
@@ -28,8 +30,8 @@ __global__ void rope_kv_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
   if (!is_q && !is_k) {  // v: plain copy into the cache
     if (slot < 0) return;
     const int kvh = head - nh - nkv;
-    T* dst = v_cache + (((size_t)(slot / page_size) * nkv + kvh) * page_size + (slot % page_size)) * hd;
-    for (int d = lane; d < hd; d += kWave) dst[d] = src[d];
+    T* dst = v_cache + ((size_t)(slot / page_size) * nkv + kvh) * hd * page_size + (slot % page_size);
+    for (int d = lane; d < hd; d += kWave) dst[(size_t)d * page_size] = src[d];
     return;
   }
   if (is_k && slot < 0) return;

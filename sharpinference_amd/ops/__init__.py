@@ -134,6 +134,11 @@ def cast(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
 
 
 # ---------------------------------------------------------------------------
+def _cache_shapes_ok(k_cache: torch.Tensor, v_cache: torch.Tensor, nkv: int, hd: int) -> bool:
+    return (k_cache.dim() == 4 and v_cache.dim() == 4 and k_cache.shape[1] == nkv and k_cache.shape[3] == hd
+            and v_cache.shape == (k_cache.shape[0], nkv, hd, k_cache.shape[2]))
+
+
 def rope_kv(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, slot_mapping: torch.Tensor,
             positions: torch.Tensor, inv_freq: Optional[torch.Tensor], qk_norm: bool, eps: float,
             temperature: Optional[Tuple[float, float]], nh: int, nkv: int, hd: int) -> torch.Tensor:
@@ -144,8 +149,7 @@ def rope_kv(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, slo
     _i32(positions, "positions")
     T = qkv.shape[0]
     _need(qkv.dim() == 2 and qkv.shape[1] == (nh + 2 * nkv) * hd, "rope_kv: qkv must be [T, (nh+2nkv)*hd]")
-    _need(k_cache.dim() == 4 and k_cache.shape[1] == nkv and k_cache.shape[3] == hd and
-          v_cache.shape == k_cache.shape, "rope_kv: cache must be [pages, nkv, page_size, hd]")
+    _need(_cache_shapes_ok(k_cache, v_cache, nkv, hd), "rope_kv: caches must be K [pages, nkv, page_size, hd], V [pages, nkv, hd, page_size]")
     _need(k_cache.dtype == qkv.dtype and v_cache.dtype == qkv.dtype, "rope_kv: cache dtype differs from qkv's")
     _need(slot_mapping.shape == (T,) and positions.shape == (T,), "rope_kv: slot_mapping / positions must be [T]")
     if inv_freq is not None:
@@ -169,14 +173,52 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     _i32(positions, "positions")
     T = q.shape[0]
     _need(q.shape == (T, nh * hd), "attention: q must be [T, nh*hd]")
-    _need(k_cache.dim() == 4 and k_cache.shape[1] == nkv and k_cache.shape[3] == hd and
-          v_cache.shape == k_cache.shape and k_cache.dtype == q.dtype, "attention: cache must be [pages, nkv, page_size, hd] of q's dtype")
+    _need(_cache_shapes_ok(k_cache, v_cache, nkv, hd) and k_cache.dtype == q.dtype and v_cache.dtype == q.dtype,
+          "attention: caches must be K [pages, nkv, page_size, hd], V [pages, nkv, hd, page_size] of q's dtype")
     _need(block_table.dim() == 2, "attention: block_table must be [entries, max_blocks]")
     _need(entry_of_token.shape == (T,) and positions.shape == (T,), "attention: per-token arrays must be [T]")
     out = torch.empty_like(q)
     _run("sharpi_attention_generic", _ptr(q), _ptr(k_cache), _ptr(v_cache), _code(q.dtype), _ptr(block_table),
          _ptr(entry_of_token), _ptr(positions), _ptr(out), int(window_kind), int(window), float(scale), T, nh, nkv,
          hd, k_cache.shape[2], block_table.shape[1], k_cache.shape[0], _stream())
+    return out
+
+
+DECODE_RUN_KEYS = 256   # keys per block of the decode kernel (fixed: sums must not depend on the batch)
+
+
+def decode_attention_ok(dtype: torch.dtype, hd: int) -> bool:
+    return dtype == torch.bfloat16 and hd % 32 == 0 and 32 <= hd <= 256
+
+
+def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
+                     entry_of_token: torch.Tensor, positions: torch.Tensor, token_list: Optional[torch.Tensor],
+                     max_context: int, window_kind: int, window: int, scale: float, nh: int, nkv: int, hd: int,
+                     out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Split-K flash-decode for the listed tokens (all tokens if token_list is None), each a
+    single query over its request's pages.  `max_context` bounds position + 1 of every token."""
+    _dev(q, k_cache, v_cache, block_table, entry_of_token, positions, token_list, out)
+    _i32(block_table, "block_table")
+    _i32(entry_of_token, "entry_of_token")
+    _i32(positions, "positions")
+    _i32(token_list, "token_list")
+    T = q.shape[0]
+    _need(q.shape == (T, nh * hd) and decode_attention_ok(q.dtype, hd), "attention_decode: q must be bfloat16 [T, nh*hd], hd a multiple of 32")
+    _need(_cache_shapes_ok(k_cache, v_cache, nkv, hd) and k_cache.dtype == q.dtype and v_cache.dtype == q.dtype,
+          "attention_decode: caches must be K [pages, nkv, page_size, hd], V [pages, nkv, hd, page_size] bfloat16")
+    _need(block_table.dim() == 2 and entry_of_token.shape == (T,) and positions.shape == (T,),
+          "attention_decode: block_table [entries, max_blocks], per-token arrays [T]")
+    n_list = T if token_list is None else token_list.shape[0]
+    if out is None:
+        out = torch.empty_like(q)
+    _need(out.shape == q.shape and out.dtype == q.dtype, "attention_decode: out must match q")
+    max_splits = ((max(1, int(max_context)) - 1) >> 4) // (DECODE_RUN_KEYS // 16) + 1
+    part_o = torch.empty(n_list * nh * max_splits * hd, dtype=torch.float32, device=q.device)
+    part_ml = torch.empty(n_list * nh * max_splits * 2, dtype=torch.float32, device=q.device)
+    _run("sharpi_attention_decode", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), _ptr(entry_of_token),
+         _ptr(positions), _ptr(token_list), _ptr(part_o), _ptr(part_ml), _ptr(out), int(window_kind), int(window),
+         float(scale), n_list, nh, nkv, hd, k_cache.shape[2], block_table.shape[1], k_cache.shape[0], max_splits,
+         _stream())
     return out
 
 
@@ -367,6 +409,9 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, gro
               window: int, scale: float, nh: int, nkv: int, hd: int) -> torch.Tensor:
     """Attention of the step's tokens over their requests' pages (`group`: the cache group's
     block tables, `ctx`: the step)."""
+    if decode_attention_ok(q.dtype, hd) and ctx.max_entry_len == 1:
+        return attention_decode(q, k_cache, v_cache, group.block_table, ctx.entry_of_token, ctx.positions, None,
+                                group.max_context, window_kind, window, scale, nh, nkv, hd)
     return attention_generic(q, k_cache, v_cache, group.block_table, ctx.entry_of_token, ctx.positions, window_kind,
                              window, scale, nh, nkv, hd)
 

@@ -24,6 +24,7 @@ _SIGNATURES = {
     "sharpi_cast": [P, I, P, I, c_longlong, P],
     "sharpi_rope_kv": [P, P, P, P, I, P, P, P, I, F, I, F, F, I, I, I, I, I, P],
     "sharpi_attention_generic": [P, P, P, I, P, P, P, P, I, I, F, I, I, I, I, I, I, I, P],
+    "sharpi_attention_decode": [P, P, P, P, P, P, P, P, P, P, I, I, F, I, I, I, I, I, I, I, I, P],
     "sharpi_gemm_tiled": [P, P, P, I, I, I, I, I, P, P, I, P],
     "sharpi_gemm_skinny": [P, P, P, I, I, I, I, P, P, I, I, I, P],
     "sharpi_router_topk": [P, I, P, I, P, P, P, I, I, I, I, I, I, P],

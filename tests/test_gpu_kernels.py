@@ -61,3 +61,81 @@ def test_gemm_skinny_grouped(rows, E):
     for R, NW in ((1, 16), (2, 8), (4, 4)):
         got = ops.gemm_skinny(x, w, torch.float32, a_rows=a_rows.to(DEV), offsets=offsets.to(DEV), n_rows=rows, R=R, NW=NW)
         assert float((got - ref).abs().max()) <= 1e-3 * float(ref.abs().max()), (R, NW)
+
+
+# ---------------------------------------------------------------------------
+# attention over a paged cache
+# ---------------------------------------------------------------------------
+def _paged_case(lens, nh, nkv, hd, ps, dtype, seed, strong_key=None):
+    """Random q/k/v for requests of the given context lengths, scattered over shuffled pages.
+    Returns what the kernels need plus dense per-request k, v for the reference."""
+    g = torch.Generator().manual_seed(seed)
+    n = len(lens)
+    blocks = [(L + ps - 1) // ps for L in lens]
+    n_pages = sum(blocks) + 3
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    maxb = max(blocks)
+    bt = torch.full((n, maxb), -1, dtype=torch.int32)
+    kc = torch.zeros(n_pages, nkv, ps, hd)
+    vc = torch.zeros(n_pages, nkv, hd, ps)
+    ks, vs = [], []
+    it = iter(perm)
+    for i, L in enumerate(lens):
+        k = torch.randn(L, nkv, hd, generator=g)
+        v = torch.randn(L, nkv, hd, generator=g)
+        if strong_key is not None and L > strong_key:
+            k[strong_key] *= 6.0                       # one far key that must not be missed
+        ks.append(k.to(dtype).float())
+        vs.append(v.to(dtype).float())
+        for b in range(blocks[i]):
+            page = next(it)
+            bt[i, b] = page
+            seg = slice(b * ps, min(L, (b + 1) * ps))
+            m = seg.stop - seg.start
+            kc[page, :, :m, :] = ks[i][seg].permute(1, 0, 2)
+            vc[page, :, :, :m] = vs[i][seg].permute(1, 2, 0)
+    return bt, kc.to(dtype), vc.to(dtype), ks, vs
+
+
+def _ref_attention(q, k, v, p, start, scale):
+    """q [nh, hd]; k, v [L, nkv, hd]: softmax over keys start..p."""
+    nh, hd = q.shape
+    nkv = k.shape[1]
+    out = torch.empty(nh, hd)
+    for h in range(nh):
+        kh, vh = k[start:p + 1, h // (nh // nkv)], v[start:p + 1, h // (nh // nkv)]
+        w = torch.softmax((kh @ q[h]) * scale, dim=0)
+        out[h] = w @ vh
+    return out
+
+
+def _start(p, kind, window):
+    return (p // window) * window if kind == 1 else max(0, p - window + 1) if kind == 2 else 0
+
+
+@pytest.mark.parametrize("nh,nkv,hd", [(8, 2, 64), (5, 5, 32), (40, 8, 128), (3, 1, 96), (34, 2, 32)])
+@pytest.mark.parametrize("kind,window", [(0, 0), (1, 24), (1, 300), (2, 50)])
+@pytest.mark.parametrize("ps", [16, 64])
+def test_attention_decode_kernel(nh, nkv, hd, kind, window, ps):
+    ops = _ops()
+    lens = [1, 17, 300, 1000, 257, 512]
+    bt, kc, vc, ks, vs = _paged_case(lens, nh, nkv, hd, ps, torch.bfloat16, seed=nh * 7 + hd, strong_key=3)
+    n = len(lens)
+    g = torch.Generator().manual_seed(5)
+    q = torch.randn(n, nh, hd, generator=g).to(torch.bfloat16)
+    positions = torch.tensor([L - 1 for L in lens], dtype=torch.int32)
+    scale = 1.0 / math.sqrt(hd)
+    ref = torch.stack([_ref_attention(q[i].float(), ks[i], vs[i], lens[i] - 1, _start(lens[i] - 1, kind, window), scale)
+                       for i in range(n)])
+    args = (q.reshape(n, nh * hd).to(DEV), kc.to(DEV), vc.to(DEV), bt.to(DEV), torch.arange(n, dtype=torch.int32, device=DEV),
+            positions.to(DEV))
+    got = ops.attention_decode(*args, None, max(lens), kind, window, scale, nh, nkv, hd).float().cpu().view(n, nh, hd)
+    assert float((got - ref).abs().max()) <= 2e-2, float((got - ref).abs().max())
+    gen = ops.attention_generic(*args, kind, window, scale, nh, nkv, hd).float().cpu().view(n, nh, hd)
+    assert float((gen - ref).abs().max()) <= 1e-2
+    # a subset through the token list leaves the other rows alone
+    sel = torch.tensor([4, 1, 3], dtype=torch.int32, device=DEV)
+    out = torch.zeros(n, nh * hd, dtype=torch.bfloat16, device=DEV)
+    ops.attention_decode(*args, sel, max(lens), kind, window, scale, nh, nkv, hd, out=out)
+    out = out.float().cpu().view(n, nh, hd)
+    assert torch.equal(out[[4, 1, 3]], got[[4, 1, 3]]) and float(out[[0, 2, 5]].abs().max()) == 0.0
