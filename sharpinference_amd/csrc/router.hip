@@ -8,27 +8,53 @@
 //
 // moe_permute: one block. Counts rows per expert, prefix-sums them into offsets[E + 1] and
 // writes, in expert order, the token and weight of every (token, pick) pair plus the inverse
-// map inv_pos[t * k + j] = row in that order.
+// map inv_pos[t * k + j] = row in that order, and the list of (expert, first row) tiles of
+// tile_rows rows that the grouped product of many rows walks.
 #include "common.h"
 
 constexpr int kMaxExperts = 1024;
 
+// eight consecutive elements as floats
+__device__ __forceinline__ void load8(const float* p, float* v) {
+  const float4 a = *reinterpret_cast<const float4*>(p);
+  const float4 b = *reinterpret_cast<const float4*>(p + 4);
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+__device__ __forceinline__ void load8(const bf16_t* p, float* v) {
+  const uint4 a = *reinterpret_cast<const uint4*>(p);
+  v[0] = bf16_bits_to_f32(a.x & 0xffffu); v[1] = bf16_bits_to_f32(a.x >> 16);
+  v[2] = bf16_bits_to_f32(a.y & 0xffffu); v[3] = bf16_bits_to_f32(a.y >> 16);
+  v[4] = bf16_bits_to_f32(a.z & 0xffffu); v[5] = bf16_bits_to_f32(a.z >> 16);
+  v[6] = bf16_bits_to_f32(a.w & 0xffffu); v[7] = bf16_bits_to_f32(a.w >> 16);
+}
+
 template <typename T, typename TW>
-__global__ __launch_bounds__(256) void router_topk_kernel(const T* __restrict__ x, const TW* __restrict__ wr,
-                                                          int* __restrict__ topk_ids,
-                                                          float* __restrict__ topk_w,
-                                                          float* __restrict__ gate_out, int hidden,
-                                                          int n_experts, int k, int gate, int renorm) {
+__global__ __launch_bounds__(1024) void router_topk_kernel(const T* __restrict__ x, const TW* __restrict__ wr,
+                                                           int* __restrict__ topk_ids,
+                                                           float* __restrict__ topk_w,
+                                                           float* __restrict__ gate_out, int hidden,
+                                                           int n_experts, int k, int gate, int renorm) {
   __shared__ float g[kMaxExperts];
   const int t = blockIdx.x;
   const int lane = threadIdx.x & (kWave - 1);
   const int w = threadIdx.x >> 6;
   const int nw = blockDim.x >> 6;
   const T* xr = x + (size_t)t * hidden;
+  const bool vec = (hidden & 7) == 0;
   for (int e = w; e < n_experts; e += nw) {
     const TW* wrow = wr + (size_t)e * hidden;
     float s = 0.f;
-    for (int c = lane; c < hidden; c += kWave) s = fmaf(to_f32<T>(xr[c]), to_f32<TW>(wrow[c]), s);
+    if (vec) {  // lane-strided runs of 8: the order of the additions depends on the width only
+      for (int c = lane * 8; c < hidden; c += kWave * 8) {
+        float a[8], b[8];
+        load8(xr + c, a);
+        load8(wrow + c, b);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) s = fmaf(a[i], b[i], s);
+      }
+    } else {
+      for (int c = lane; c < hidden; c += kWave) s = fmaf(to_f32<T>(xr[c]), to_f32<TW>(wrow[c]), s);
+    }
     s = wave_sum(s);
     if (lane == 0) g[e] = s;
   }
@@ -76,7 +102,8 @@ SHARPI_EXPORT int sharpi_router_topk(const void* x, int x_dtype, const void* wr,
   if (n_tokens <= 0) return SHARPI_OK;
   if (hidden <= 0 || n_experts <= 0 || n_experts > kMaxExperts || k <= 0 || k > n_experts) return SHARPI_ERR_ARG;
   if (gate < 0 || gate > 1) return SHARPI_ERR_ARG;
-  dim3 grid(n_tokens), block(256);
+  // one wave per expert at a time: enough waves for the experts, at most 16
+  dim3 grid(n_tokens), block(kWave * (n_experts >= 16 ? 16 : n_experts >= 8 ? 8 : 4));
 #define ROUTER_LAUNCH(TX, TWT)                                                                              \
   router_topk_kernel<TX, TWT><<<grid, block, 0, stream>>>((const TX*)x, (const TWT*)wr, topk_ids, topk_w,   \
                                                           gate_out, hidden, n_experts, k, gate, renorm)
@@ -95,8 +122,11 @@ __global__ __launch_bounds__(1024) void moe_permute_kernel(const int* __restrict
                                                            int* __restrict__ offsets,
                                                            int* __restrict__ sorted_token,
                                                            float* __restrict__ sorted_w,
-                                                           int* __restrict__ inv_pos, int n_pairs, int k,
-                                                           int n_experts) {
+                                                           int* __restrict__ inv_pos,
+                                                           int* __restrict__ tile_expert,
+                                                           int* __restrict__ tile_row0,
+                                                           int* __restrict__ n_tiles, int n_pairs, int k,
+                                                           int n_experts, int tile_rows, int max_tiles) {
   __shared__ int count[kMaxExperts];
   __shared__ int cursor[kMaxExperts];
   for (int e = threadIdx.x; e < n_experts; e += blockDim.x) count[e] = 0;
@@ -111,6 +141,17 @@ __global__ __launch_bounds__(1024) void moe_permute_kernel(const int* __restrict
       run += count[e];
     }
     offsets[n_experts] = run;
+    // row tiles of the experts that have rows, for the grouped product of many rows
+    int nt = 0;
+    for (int e = 0; e < n_experts; ++e)
+      for (int r0 = offsets[e]; r0 < offsets[e] + count[e]; r0 += tile_rows) {
+        if (nt < max_tiles) {
+          tile_expert[nt] = e;
+          tile_row0[nt] = r0;
+          ++nt;
+        }
+      }
+    n_tiles[0] = nt;
   }
   __syncthreads();
   for (int i = threadIdx.x; i < n_pairs; i += blockDim.x) {
@@ -123,12 +164,15 @@ __global__ __launch_bounds__(1024) void moe_permute_kernel(const int* __restrict
 }
 
 SHARPI_EXPORT int sharpi_moe_permute(const int* topk_ids, const float* topk_w, int* offsets, int* sorted_token,
-                                     float* sorted_w, int* inv_pos, int n_tokens, int k, int n_experts,
-                                     hipStream_t stream) {
+                                     float* sorted_w, int* inv_pos, int* tile_expert, int* tile_row0,
+                                     int* n_tiles, int n_tokens, int k, int n_experts, int tile_rows,
+                                     int max_tiles, hipStream_t stream) {
   if (n_experts <= 0 || n_experts > kMaxExperts || k <= 0) return SHARPI_ERR_ARG;
-  if (n_tokens < 0) return SHARPI_ERR_ARG;
+  if (n_tokens < 0 || tile_rows <= 0) return SHARPI_ERR_ARG;
+  if (max_tiles < (n_tokens * k + tile_rows - 1) / tile_rows + n_experts) return SHARPI_ERR_ARG;
   moe_permute_kernel<<<1, 1024, 0, stream>>>(topk_ids, topk_w, offsets, sorted_token, sorted_w, inv_pos,
-                                             n_tokens * k, k, n_experts);
+                                             tile_expert, tile_row0, n_tiles, n_tokens * k, k, n_experts,
+                                             tile_rows, max_tiles);
   SHARPI_CHECK_LAUNCH();
   return SHARPI_OK;
 }

@@ -20,6 +20,9 @@ from ..cache.manager import CacheError, CacheManager
 from ..parts.base import GroupView, LayerCache, StepContext
 
 
+TILE = 32   # tokens per attention tile of multi-token entries (ops.PREFILL_TILE_TOKENS)
+
+
 class CacheExhausted(CacheError):
     """A step needed more pages than the pools hold; nothing was changed."""
 
@@ -99,7 +102,14 @@ class ModelRunner:
             group_tables.append(bt)
             group_slots.append(sm)
         rows_np = np.asarray(rows, dtype=np.int32)
-        pieces = [token_ids, positions, entry_of, cu, state_slots, np.full(T, -1, dtype=np.int32), rows_np]
+        # attention work lists: single-token entries, and tiles of the longer ones
+        dec = [int(cu[i]) for i in range(n) if lens[i] == 1]
+        tiles = [(i, int(cu[i]) + o, min(TILE, lens[i] - o)) for i in range(n) if lens[i] > 1
+                 for o in range(0, lens[i], TILE)]
+        dec_np = np.asarray(dec, dtype=np.int32)
+        tiles_np = np.asarray(tiles, dtype=np.int32).reshape(-1)
+        pieces = [token_ids, positions, entry_of, cu, state_slots, np.full(T, -1, dtype=np.int32), rows_np,
+                  dec_np, tiles_np]
         for bt, sm in zip(group_tables, group_slots):
             pieces += [bt.reshape(-1), sm]
         flat = np.concatenate(pieces) if pieces else np.zeros(0, dtype=np.int32)
@@ -108,15 +118,17 @@ class ModelRunner:
         for p in pieces:
             views.append(dev[off:off + p.size])
             off += p.size
-        d_tok, d_pos, d_ent, d_cu, d_state, d_nostore, d_rows = views[:7]
+        d_tok, d_pos, d_ent, d_cu, d_state, d_nostore, d_rows, d_dec, d_tiles = views[:9]
         groups = []
         for g in range(len(cache.groups)):
-            bt = views[7 + 2 * g].view(n, group_tables[g].shape[1])
-            groups.append(GroupView(bt, views[8 + 2 * g], ps, max_context=int(positions.max()) + 1 if T else 0))
+            bt = views[9 + 2 * g].view(n, group_tables[g].shape[1])
+            groups.append(GroupView(bt, views[10 + 2 * g], ps, max_context=int(positions.max()) + 1 if T else 0))
         ctx = StepContext(n_tokens=T, n_entries=n, token_ids=d_tok, positions=d_pos, entry_of_token=d_ent,
                           cu_tokens=d_cu, state_slots=d_state, groups=groups, act_dtype=self.act_dtype,
                           no_store_slots=d_nostore, entry_lens=lens, entry_starts=starts,
-                          max_entry_len=max(lens) if lens else 1)
+                          max_entry_len=max(lens) if lens else 1, n_decode=len(dec),
+                          decode_tokens=None if len(dec) == T else d_dec, n_prefill_tiles=len(tiles),
+                          prefill_tiles=d_tiles.view(-1, 3) if tiles else None)
         return ctx, (d_rows if rows else None)
 
     def layer_caches(self, ctx: StepContext) -> List[LayerCache]:

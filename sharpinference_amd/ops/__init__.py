@@ -222,6 +222,33 @@ def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     return out
 
 
+PREFILL_TILE_TOKENS = 32   # tokens per wave of the prefill kernel
+
+
+def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
+                      positions: torch.Tensor, tiles: torch.Tensor, window_kind: int, window: int, scale: float,
+                      nh: int, nkv: int, hd: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Flash attention for the listed tiles: tiles int32 [n, 3] = (entry, first token, rows <= 32),
+    the tokens of a tile consecutive in one entry."""
+    _dev(q, k_cache, v_cache, block_table, positions, tiles, out)
+    _i32(block_table, "block_table")
+    _i32(positions, "positions")
+    _i32(tiles, "tiles")
+    T = q.shape[0]
+    _need(q.shape == (T, nh * hd) and decode_attention_ok(q.dtype, hd), "attention_prefill: q must be bfloat16 [T, nh*hd], hd a multiple of 32")
+    _need(_cache_shapes_ok(k_cache, v_cache, nkv, hd) and k_cache.dtype == q.dtype and v_cache.dtype == q.dtype,
+          "attention_prefill: caches must be K [pages, nkv, page_size, hd], V [pages, nkv, hd, page_size] bfloat16")
+    _need(block_table.dim() == 2 and positions.shape == (T,) and tiles.dim() == 2 and tiles.shape[1] == 3,
+          "attention_prefill: block_table [entries, max_blocks], positions [T], tiles [n, 3]")
+    if out is None:
+        out = torch.empty_like(q)
+    _need(out.shape == q.shape and out.dtype == q.dtype, "attention_prefill: out must match q")
+    _run("sharpi_attention_prefill", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), _ptr(positions),
+         _ptr(tiles), _ptr(out), tiles.shape[0], int(window_kind), int(window), float(scale), nh, nkv, hd,
+         k_cache.shape[2], block_table.shape[1], k_cache.shape[0], _stream())
+    return out
+
+
 # ---------------------------------------------------------------------------
 def gemm_tiled(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """x [M, K] @ w [N, K]^T with float FMA chains (batch-invariant)."""
@@ -345,20 +372,61 @@ def router_topk(x: torch.Tensor, wr: torch.Tensor, k: int, gate: int = GATE_SIGM
     return (ids, wts, gates) if want_gates else (ids, wts)
 
 
-def moe_permute(ids: torch.Tensor, wts: torch.Tensor, n_experts: int):
-    """(token, pick) pairs sorted by expert: offsets [E+1], sorted_token, sorted_w, inv_pos."""
+GROUPED_TILE_ROWS = 64
+
+
+class Routing:
+    """The expert-sorted view of a step's (token, pick) pairs, all on the device."""
+
+    __slots__ = ("n_tokens", "k", "n_experts", "offsets", "sorted_token", "sorted_w", "inv_pos", "tile_expert",
+                 "tile_row0", "n_tiles", "max_tiles")
+
+    @property
+    def n_rows(self) -> int:
+        return self.n_tokens * self.k
+
+
+def moe_permute(ids: torch.Tensor, wts: torch.Tensor, n_experts: int) -> Routing:
+    """(token, pick) pairs sorted by expert: offsets [E+1], sorted_token, sorted_w, inv_pos, and
+    the list of 64-row tiles of the experts that have rows."""
     _dev(ids, wts)
     _i32(ids, "ids")
     _need(ids.shape == wts.shape and wts.dtype == torch.float32 and ids.dim() == 2, "moe_permute: ids/wts [T, k]")
     T, k = ids.shape
     dev = ids.device
-    offsets = torch.empty(n_experts + 1, dtype=torch.int32, device=dev)
-    sorted_token = torch.empty(T * k, dtype=torch.int32, device=dev)
-    sorted_w = torch.empty(T * k, dtype=torch.float32, device=dev)
-    inv_pos = torch.empty(T * k, dtype=torch.int32, device=dev)
-    _run("sharpi_moe_permute", _ptr(ids), _ptr(wts), _ptr(offsets), _ptr(sorted_token), _ptr(sorted_w), _ptr(inv_pos),
-         T, k, n_experts, _stream())
-    return offsets, sorted_token, sorted_w, inv_pos
+    rt = Routing()
+    rt.n_tokens, rt.k, rt.n_experts = T, k, n_experts
+    rt.max_tiles = (T * k + GROUPED_TILE_ROWS - 1) // GROUPED_TILE_ROWS + n_experts
+    ints = torch.empty(n_experts + 1 + 2 * T * k + 2 * rt.max_tiles + 1, dtype=torch.int32, device=dev)
+    o = 0
+    rt.offsets = ints[o:o + n_experts + 1]; o += n_experts + 1
+    rt.sorted_token = ints[o:o + T * k]; o += T * k
+    rt.inv_pos = ints[o:o + T * k]; o += T * k
+    rt.tile_expert = ints[o:o + rt.max_tiles]; o += rt.max_tiles
+    rt.tile_row0 = ints[o:o + rt.max_tiles]; o += rt.max_tiles
+    rt.n_tiles = ints[o:o + 1]
+    rt.sorted_w = torch.empty(T * k, dtype=torch.float32, device=dev)
+    _run("sharpi_moe_permute", _ptr(ids), _ptr(wts), _ptr(rt.offsets), _ptr(rt.sorted_token), _ptr(rt.sorted_w),
+         _ptr(rt.inv_pos), _ptr(rt.tile_expert), _ptr(rt.tile_row0), _ptr(rt.n_tiles), T, k, n_experts,
+         GROUPED_TILE_ROWS, rt.max_tiles, _stream())
+    return rt
+
+
+def gemm_grouped(x: torch.Tensor, w: torch.Tensor, rt: Routing, gather: bool, out_dtype: torch.dtype) -> torch.Tensor:
+    """Per-expert products for many rows on the matrix cores (bfloat16).  gather: x rows are read
+    through the routing's token list; otherwise x is already in expert-sorted order."""
+    _dev(x, w)
+    _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_grouped: bfloat16 operands only")
+    _need(w.dim() == 3 and w.shape[0] == rt.n_experts and x.dim() == 2 and x.shape[1] == w.shape[2],
+          f"gemm_grouped: x {tuple(x.shape)} vs w {tuple(w.shape)}")
+    E, N, K = w.shape
+    _need(K % 128 == 0 and N % 4 == 0, "gemm_grouped: K % 128 == 0 and N % 4 == 0 wanted")
+    _need(x.shape[0] == (rt.n_tokens if gather else rt.n_rows), "gemm_grouped: x has the wrong number of rows")
+    out = torch.empty(rt.n_rows, N, dtype=out_dtype, device=x.device)
+    _run("sharpi_gemm_grouped", _ptr(x), _ptr(w), _ptr(out), _code(out_dtype), rt.n_rows, N, K,
+         _ptr(rt.sorted_token) if gather else None, _ptr(rt.offsets), _ptr(rt.tile_expert), _ptr(rt.tile_row0),
+         _ptr(rt.n_tiles), rt.max_tiles, _stream())
+    return out
 
 
 # ---------------------------------------------------------------------------
@@ -409,19 +477,30 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, gro
               window: int, scale: float, nh: int, nkv: int, hd: int) -> torch.Tensor:
     """Attention of the step's tokens over their requests' pages (`group`: the cache group's
     block tables, `ctx`: the step)."""
-    if decode_attention_ok(q.dtype, hd) and ctx.max_entry_len == 1:
-        return attention_decode(q, k_cache, v_cache, group.block_table, ctx.entry_of_token, ctx.positions, None,
-                                group.max_context, window_kind, window, scale, nh, nkv, hd)
+    if decode_attention_ok(q.dtype, hd):
+        # entries of one token: split-K decode kernel; longer entries: flash kernel, 32 tokens a wave
+        out = torch.empty_like(q)
+        if ctx.n_prefill_tiles:
+            attention_prefill(q, k_cache, v_cache, group.block_table, ctx.positions, ctx.prefill_tiles, window_kind,
+                              window, scale, nh, nkv, hd, out=out)
+        if ctx.n_decode:
+            attention_decode(q, k_cache, v_cache, group.block_table, ctx.entry_of_token, ctx.positions,
+                             ctx.decode_tokens, group.max_context, window_kind, window, scale, nh, nkv, hd, out=out)
+        return out
     return attention_generic(q, k_cache, v_cache, group.block_table, ctx.entry_of_token, ctx.positions, window_kind,
                              window, scale, nh, nkv, hd)
 
 
-def grouped_linear(x: torch.Tensor, w: torch.Tensor, offsets: torch.Tensor, a_rows: Optional[torch.Tensor],
-                   n_rows: int, out_dtype: torch.dtype) -> torch.Tensor:
-    """Per-expert products over the expert-sorted row list (see grouped_gemm)."""
+def grouped_linear(x: torch.Tensor, w: torch.Tensor, rt: Routing, gather: bool, out_dtype: torch.dtype) -> torch.Tensor:
+    """Per-expert products over the routing's expert-sorted row list: w [E, N, K]; x rows are read
+    through the token list (gather) or are already in sorted order.  Returns [n_rows, N]."""
     if x.dtype != w.dtype:
         x = cast(x, w.dtype)
-    if w.dtype == torch.bfloat16 and skinny_ok(n_rows, w.shape[1], w.shape[2], grouped=True):
-        return gemm_skinny(x, w, out_dtype, a_rows=a_rows, offsets=offsets, n_rows=n_rows)
-    y = grouped_gemm(x, w, offsets, a_rows, n_rows)
+    N, K = w.shape[1], w.shape[2]
+    a_rows = rt.sorted_token if gather else None
+    if w.dtype == torch.bfloat16 and K % 128 == 0 and N % 4 == 0:
+        if rt.n_rows <= SKINNY_MAX_ROWS:
+            return gemm_skinny(x, w, out_dtype, a_rows=a_rows, offsets=rt.offsets, n_rows=rt.n_rows)
+        return gemm_grouped(x, w, rt, gather, out_dtype)
+    y = grouped_gemm(x, w, rt.offsets, a_rows, rt.n_rows)
     return y if y.dtype == out_dtype else cast(y, out_dtype)

@@ -104,9 +104,9 @@ class MoESwiGLU(Part):
         trace = ctx.extras.get("router_trace")
         if trace is not None:      # the picks of this step, layer by layer (reference: ForwardPass.cs:2042-2056)
             trace.append((ids, wts))
-        offsets, sorted_token, sorted_w, inv_pos = ops.moe_permute(ids, wts, self.E)
+        rt = ops.moe_permute(ids, wts, self.E)
         shared = self.shared.forward(x, ctx) if self.shared is not None else None
-        gu = ops.grouped_linear(x, self.w_gate_up, offsets, sorted_token, T * self.k, ctx.act_dtype)
-        act = ops.silu_mul(gu, sorted_w)
-        y = ops.grouped_linear(act, self.w_down, offsets, None, T * self.k, ctx.act_dtype)
-        return ops.moe_combine(y, inv_pos, shared, T, self.k)
+        gu = ops.grouped_linear(x, self.w_gate_up, rt, True, ctx.act_dtype)
+        act = ops.silu_mul(gu, rt.sorted_w)
+        y = ops.grouped_linear(act, self.w_down, rt, False, ctx.act_dtype)
+        return ops.moe_combine(y, rt.inv_pos, shared, T, self.k)

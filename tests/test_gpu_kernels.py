@@ -139,3 +139,102 @@ def test_attention_decode_kernel(nh, nkv, hd, kind, window, ps):
     ops.attention_decode(*args, sel, max(lens), kind, window, scale, nh, nkv, hd, out=out)
     out = out.float().cpu().view(n, nh, hd)
     assert torch.equal(out[[4, 1, 3]], got[[4, 1, 3]]) and float(out[[0, 2, 5]].abs().max()) == 0.0
+
+
+# ---------------------------------------------------------------------------
+# routing and the grouped product for many rows
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("T,E,k,H", [(300, 16, 1, 256), (70, 5, 2, 136), (1, 3, 3, 64), (513, 128, 1, 128)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_router_and_permute(T, E, k, H, dtype):
+    ops = _ops()
+    x = _rand(T, H, dtype=dtype, seed=T)
+    wr = _rand(E, H, dtype=dtype, scale=0.3, seed=E)
+    ids, wts, gates = ops.router_topk(x, wr, k, want_gates=True)
+    sig = torch.sigmoid(x.float() @ wr.float().T)
+    assert float((gates - sig).abs().max()) <= 2e-5
+    # picks: descending by the kernel's own gate values, lowest index on ties
+    order = torch.sort(gates, dim=1, descending=True, stable=True)
+    assert torch.equal(ids.long(), order.indices[:, :k])
+    assert torch.equal(wts, order.values[:, :k])
+    rt = ops.moe_permute(ids, wts, E)
+    off = rt.offsets.cpu().tolist()
+    flat = ids.flatten().cpu()
+    assert off[0] == 0 and off[-1] == T * k
+    counts = torch.bincount(flat.long(), minlength=E).tolist()
+    assert [off[e + 1] - off[e] for e in range(E)] == counts
+    st, inv, sw = rt.sorted_token.cpu(), rt.inv_pos.cpu().long(), rt.sorted_w.cpu()
+    assert sorted(inv.tolist()) == list(range(T * k))
+    for e in range(E):
+        assert all(int(flat[i]) == e for i in (inv >= off[e]).logical_and(inv < off[e + 1]).nonzero().flatten().tolist())
+    assert torch.equal(st[inv].long(), torch.arange(T * k) // k)
+    assert torch.equal(sw[inv], wts.flatten().cpu())
+    nt = int(rt.n_tiles.cpu())
+    tiles = list(zip(rt.tile_expert.cpu().tolist()[:nt], rt.tile_row0.cpu().tolist()[:nt]))
+    want = [(e, r0) for e in range(E) for r0 in range(off[e], off[e + 1], ops.GROUPED_TILE_ROWS)]
+    assert tiles == want
+
+
+def test_router_ties_pick_the_lowest_index():
+    ops = _ops()
+    x = _rand(4, 64)
+    wr = torch.zeros(6, 64, device=DEV)
+    ids, wts = ops.router_topk(x, wr, 2)
+    assert ids.cpu().tolist() == [[0, 1]] * 4 and float((wts - 0.5).abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("T,E,k,N,K", [(300, 4, 1, 264, 256), (700, 16, 2, 512, 128), (65, 3, 1, 20, 384)])
+def test_gemm_grouped(T, E, k, N, K):
+    ops = _ops()
+    x = _rand(T, K, dtype=torch.bfloat16, seed=1)
+    w = _rand(E, N, K, dtype=torch.bfloat16, scale=0.1, seed=2)
+    g = torch.Generator().manual_seed(T)
+    ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32).to(DEV)
+    if E == 4:
+        ids[:] = 2                                     # one expert takes everything, the others nothing
+    wts = torch.rand(T, k, generator=g).to(DEV)
+    rt = ops.moe_permute(ids, wts, E)
+    got = ops.gemm_grouped(x, w, rt, True, torch.float32).cpu()
+    st = rt.sorted_token.cpu().long()
+    off = rt.offsets.cpu().tolist()
+    xf, wf = x.float().cpu(), w.float().cpu()
+    for e in range(E):
+        rows = slice(off[e], off[e + 1])
+        ref = xf[st[rows]] @ wf[e].T
+        if ref.numel():
+            assert float((got[rows] - ref).abs().max()) <= 1e-3 * float(ref.abs().max() + 1e-6), e
+    # second product: rows already sorted, bfloat16 out
+    y = ops.gemm_grouped(x[st.to(DEV)].contiguous(), w, rt, False, torch.bfloat16).float().cpu()
+    assert float((y - got).abs().max()) <= 2e-2 * float(got.abs().max())
+
+
+@pytest.mark.parametrize("nh,nkv,hd", [(8, 2, 64), (5, 5, 32), (40, 8, 128), (3, 1, 96)])
+@pytest.mark.parametrize("kind,window", [(0, 0), (1, 24), (1, 100), (2, 50)])
+@pytest.mark.parametrize("ps", [16, 32])
+def test_attention_prefill_kernel(nh, nkv, hd, kind, window, ps):
+    """Portions of several requests at different starting positions, against dense softmax."""
+    ops = _ops()
+    ctx_lens = [70, 300, 33, 129]          # context after the portion
+    portion = [70, 45, 2, 100]             # the last `portion` tokens are this step's queries
+    bt, kc, vc, ks, vs = _paged_case(ctx_lens, nh, nkv, hd, ps, torch.bfloat16, seed=nh + hd + ps, strong_key=5)
+    g = torch.Generator().manual_seed(9)
+    T = sum(portion)
+    q = torch.randn(T, nh, hd, generator=g).to(torch.bfloat16)
+    positions, tiles, ref = [], [], []
+    scale = 1.0 / math.sqrt(hd)
+    tok = 0
+    for e, (L, n) in enumerate(zip(ctx_lens, portion)):
+        for o in range(0, n, ops.PREFILL_TILE_TOKENS):
+            tiles.append((e, tok + o, min(ops.PREFILL_TILE_TOKENS, n - o)))
+        for i in range(n):
+            p = L - n + i
+            positions.append(p)
+            ref.append(_ref_attention(q[tok + i].float(), ks[e], vs[e], p, _start(p, kind, window), scale))
+        tok += n
+    ref = torch.stack(ref)
+    got = ops.attention_prefill(q.reshape(T, nh * hd).to(DEV), kc.to(DEV), vc.to(DEV), bt.to(DEV),
+                                torch.tensor(positions, dtype=torch.int32, device=DEV),
+                                torch.tensor(tiles, dtype=torch.int32, device=DEV), kind, window, scale, nh, nkv, hd)
+    got = got.float().cpu().view(T, nh, hd)
+    err = (got - ref).abs().max(dim=-1).values.max(dim=-1).values
+    assert float(err.max()) <= 2e-2, (float(err.max()), int(err.argmax()))
