@@ -292,7 +292,7 @@ class CacheManager:
         ps = self.page_size
         out = []
         for pos in range(start, start + n):
-            page = tbl[pos // ps]
+            page = tbl[pos // ps] if pos // ps < len(tbl) else -1
             if page < 0:
                 raise CacheError(f"request {req_id!r}: position {pos} has no page in group {group}")
             out.append(page * ps + pos % ps)

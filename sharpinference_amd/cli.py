@@ -1,0 +1,115 @@
+"""Command line in the manner of the reference's ``sharpi-cli`` (reference:
+src/SharpInference.Cli/RunCommand.cs:23-300 for the options, 1907-1911 for the closing line
+``Prefill: N tokens, X t/s | Decode: M tokens, Y t/s``).
+
+Options keep the reference's names and meanings where it has them: -m/--model, -p/--prompt,
+-f/--file, -n/--n-predict (512), --temp (0.7; 0 = greedy), --top-k (40), --top-p (0.95),
+--min-p (0.05), -s/--seed (-1 = from the clock), -c/--ctx-size (0 = the model's), --kv-type,
+--repeat-penalty (1.1), --repeat-last-n, --frequency-penalty, --presence-penalty,
+--verbose-prompt.  There is no tokenizer in this engine: a prompt is a list of token ids
+(``--prompt-ids 1,2,3``; -p/-f take the same comma- or space-separated ids) or ``--prompt-len N``
+random ids.  ``-m`` names a model folder (config.json + model.safetensors); with
+``--random-weights`` the folder needs only config.json.
+"""
+from __future__ import annotations
+
+import argparse
+import random
+import re
+import sys
+import time
+from typing import List, Optional
+
+
+def _ids(text: str) -> List[int]:
+    parts = [p for p in re.split(r"[,\s]+", text.strip()) if p]
+    try:
+        return [int(p) for p in parts]
+    except ValueError:
+        raise SystemExit("this engine has no tokenizer: give the prompt as token ids, e.g. -p '1,2,3'") from None
+
+
+def build_parser() -> argparse.ArgumentParser:
+    ap = argparse.ArgumentParser(prog="sharpi-cli", description="Generate with a Llama 4 model folder on one MI355X.")
+    ap.add_argument("-m", "--model", required=True, help="model folder (config.json, model.safetensors)")
+    ap.add_argument("-p", "--prompt", help="prompt as token ids (comma or space separated)")
+    ap.add_argument("-f", "--file", help="read the prompt's token ids from a file")
+    ap.add_argument("--prompt-ids", help="prompt as token ids (same as -p)")
+    ap.add_argument("--prompt-len", type=int, help="a prompt of N random token ids")
+    ap.add_argument("-n", "--n-predict", type=int, default=512, help="tokens to generate")
+    ap.add_argument("--temp", type=float, default=0.7, help="temperature; 0 = greedy")
+    ap.add_argument("--top-k", type=int, default=40)
+    ap.add_argument("--top-p", type=float, default=0.95)
+    ap.add_argument("--min-p", type=float, default=0.05)
+    ap.add_argument("-s", "--seed", type=int, default=-1, help="sampling seed; -1 = from the clock")
+    ap.add_argument("-c", "--ctx-size", type=int, default=0, help="longest sequence; 0 = the model's")
+    ap.add_argument("--kv-type", default=None, choices=["fp32", "bf16"], help="cache dtype (follows --dtype)")
+    ap.add_argument("--repeat-penalty", type=float, default=1.1)
+    ap.add_argument("--repeat-last-n", type=int, default=256)
+    ap.add_argument("--frequency-penalty", type=float, default=0.0)
+    ap.add_argument("--presence-penalty", type=float, default=0.0)
+    ap.add_argument("--verbose-prompt", action="store_true", help="print the prompt's token ids")
+    ap.add_argument("--no-display-prompt", action="store_true")
+    ap.add_argument("--stop-ids", default="", help="token ids that end generation")
+    # this engine's own
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32", "bfloat16", "float32"])
+    ap.add_argument("--random-weights", action="store_true", help="seeded random weights (folder needs config.json only)")
+    ap.add_argument("--weight-seed", type=int, default=0)
+    ap.add_argument("--parallel", type=int, default=1, help="generate this many copies of the prompt at once")
+    ap.add_argument("--max-num-seqs", type=int, default=8)
+    ap.add_argument("--max-tokens-per-step", type=int, default=2048)
+    ap.add_argument("--kv-tokens", type=int, default=None, help="size of each page pool in tokens")
+    ap.add_argument("--page-size", type=int, default=16)
+    return ap
+
+
+def main(argv: Optional[List[str]] = None) -> int:
+    args = build_parser().parse_args(argv)
+    from .config.base import load_config
+    from .engine import Engine
+    from .sampling.params import SamplingParams
+
+    dtype = {"bf16": "bfloat16", "fp32": "float32"}.get(args.dtype, args.dtype)
+    if args.kv_type and {"bf16": "bfloat16", "fp32": "float32"}[args.kv_type] != dtype:
+        raise SystemExit("--kv-type must equal --dtype: the cache is stored in the compute dtype")
+    cfg = load_config(args.model)
+    if args.file:
+        with open(args.file) as f:
+            prompt = _ids(f.read())
+    elif args.prompt_ids or args.prompt:
+        prompt = _ids(args.prompt_ids or args.prompt)
+    elif args.prompt_len:
+        rng = random.Random(args.weight_seed)
+        prompt = [rng.randrange(cfg.vocab_size) for _ in range(args.prompt_len)]
+    else:
+        raise SystemExit("no prompt: give -p / --prompt-ids / -f / --prompt-len (there is no interactive mode)")
+    ctx = args.ctx_size or None
+    common = dict(dtype=dtype, device="cuda:0", max_model_len=ctx, max_num_seqs=max(args.max_num_seqs, args.parallel),
+                  max_tokens_per_step=args.max_tokens_per_step, kv_tokens=args.kv_tokens, page_size=args.page_size)
+    if args.random_weights:
+        eng = Engine(config=cfg, weight_seed=args.weight_seed, **common)
+    else:
+        eng = Engine(args.model, **common)
+    seed = args.seed if args.seed >= 0 else int(time.time() * 1000) & 0x7FFFFFFF
+    params = [SamplingParams(temperature=args.temp, top_k=args.top_k, top_p=args.top_p, min_p=args.min_p,
+                             repetition_penalty=args.repeat_penalty, penalty_last_n=args.repeat_last_n,
+                             frequency_penalty=args.frequency_penalty, presence_penalty=args.presence_penalty,
+                             max_new_tokens=args.n_predict, stop_token_ids=tuple(_ids(args.stop_ids)) if args.stop_ids else (),
+                             seed=seed + i) for i in range(args.parallel)]
+    if args.verbose_prompt:
+        print(f"prompt tokens ({len(prompt)}): {prompt}")
+    elif not args.no_display_prompt:
+        print(" ".join(str(t) for t in prompt))
+    results = eng.generate([prompt] * args.parallel, params)
+    for i, r in enumerate(results):
+        head = f"[{i}] " if args.parallel > 1 else ""
+        print(f"{head}{' '.join(str(t) for t in r.token_ids)}  ({r.finish_reason})")
+    st = eng.last_stats
+    pre = st.prefill_tokens / st.prefill_seconds if st.prefill_seconds > 0 else 0.0
+    dec = st.decode_tokens / st.decode_seconds if st.decode_seconds > 0 else 0.0
+    print(f"Prefill: {st.prefill_tokens} tokens, {pre:.1f} t/s | Decode: {st.decode_tokens} tokens, {dec:.1f} t/s")
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -169,7 +169,7 @@ def store_bf16(t: torch.Tensor) -> torch.Tensor:
 
 
 def attention_layer(c: dict, W: Dict[str, torch.Tensor], layer: int, n: torch.Tensor,
-                    positions: torch.Tensor, store=_same) -> torch.Tensor:
+                    positions: torch.Tensor, store=_same, kv_out: Optional[list] = None, kv_in=None) -> torch.Tensor:
     """ForwardPass.cs:1576-1690 for one layer on normed input n [T, H]: projections
     without bias, rotary then weightless norm on rotary layers (1635-1648), temperature
     on the others, attention, output projection.  `store` marks where the engine stores a
@@ -195,6 +195,10 @@ def attention_layer(c: dict, W: Dict[str, torch.Tensor], layer: int, n: torch.Te
             q = q * t.to(q.dtype)[:, None, None]
         mask = attention_mask(positions, None)
     q, k = store(q), store(k)
+    if kv_out is not None:       # hand the keys and values out (a later layer may read this layer's cache)
+        kv_out.append((k, v))
+    if kv_in is not None:        # read another layer's keys and values instead of this layer's own
+        k, v = kv_in
     o = store(attention(q, k, v, mask)).reshape(T, nh * hd)
     return store(o @ W[p + "o_proj.weight"].T)
 

@@ -1,0 +1,141 @@
+"""Configuration, registry and weight loading (no GPU)."""
+import json
+import os
+
+import pytest
+import torch
+
+from sharpinference_amd import ConfigError, build_model, load_config, registered_architectures
+from sharpinference_amd.config.llama4 import Llama4TextConfig
+from sharpinference_amd.weights import safetensors_io as st
+from sharpinference_amd.weights.loader import (RandomSource, SafetensorsSource, WeightError, check_specs,
+                                               load_model_weights, storage_dtype, write_random_model)
+from tiny_configs import CONFIGS, TINY_A, TINY_B, make_model_dir
+
+
+def test_every_key_is_read_and_round_trips():
+    for d in CONFIGS.values():
+        cfg = load_config(d)
+        again = load_config(cfg.to_dict())
+        assert again == cfg
+    b = load_config(TINY_B)
+    assert (b.hidden_size, b.num_hidden_layers, b.num_attention_heads, b.num_key_value_heads, b.head_dim) == (96, 5, 6, 3, 32)
+    assert b.rope_scaling.factor == 8.0 and b.rope_scaling.original_max_position_embeddings == 32
+    assert [b.is_moe_layer(l) for l in range(5)] == [False, True, False, True, False]
+    assert [b.uses_rope(l) for l in range(5)] == [True, True, True, False, True]
+    assert not b.use_qk_norm and b.floor_scale == 32 and b.attn_scale == 0.2 and b.rms_norm_eps == 1e-6
+
+
+def test_defaults_follow_the_reference_rule():
+    d = {k: v for k, v in TINY_A.items() if k not in ("no_rope_layers", "head_dim", "num_key_value_heads")}
+    d["num_hidden_layers"] = 8
+    cfg = load_config(d)
+    assert cfg.no_rope_layers == [1, 1, 1, 0, 1, 1, 1, 0]          # every 4th layer has no rotary
+    assert cfg.head_dim == 16 and cfg.num_key_value_heads == 4
+
+
+def test_nested_text_config():
+    d = {"architectures": ["Llama4ForCausalLM"], "text_config": {k: v for k, v in TINY_A.items() if k != "architectures"}}
+    assert load_config(d).hidden_size == 64
+
+
+@pytest.mark.parametrize("change,word", [
+    ({"num_key_value_heads": 3}, "multiple"), ({"head_dim": 15}, "even"), ({"num_experts_per_tok": 9}, "num_experts_per_tok"),
+    ({"no_rope_layers": [1]}, "no_rope_layers"), ({"attention_chunk_size": 0}, "attention_chunk_size"),
+    ({"rope_scaling": {"rope_type": "yarn", "factor": 2}}, "rope_type"), ({"rms_norm_eps": 0}, "rms_norm_eps"),
+    ({"interleave_moe_layer_step": 2, "intermediate_size_mlp": 0}, "intermediate_size_mlp"),
+])
+def test_contradictions_are_refused(change, word):
+    with pytest.raises(ConfigError, match=word):
+        load_config({**TINY_A, **change})
+
+
+def test_missing_keys_and_unknown_architecture():
+    with pytest.raises(ConfigError, match="hidden_size"):
+        load_config({"architectures": ["Llama4ForCausalLM"], "vocab_size": 10})
+    with pytest.raises(ConfigError, match="not registered.*Llama4ForCausalLM"):
+        load_config({**TINY_A, "architectures": ["NoSuchModel"]})
+    assert "Llama4ForCausalLM" in registered_architectures()
+
+
+def test_model_is_assembled_layer_by_layer():
+    m = build_model(load_config(TINY_B))
+    kinds = [(type(b.mixer).__name__, b.mixer.rotary is not None, b.mixer.window_kind, type(b.ffn).__name__) for b in m.blocks]
+    assert kinds[3] == ("Attention", False, 0, "MoESwiGLU") and kinds[0] == ("Attention", True, 1, "DenseSwiGLU")
+    assert m.blocks[0].mixer.window == 24 and m.blocks[3].mixer.q_temperature == (32.0, 0.2)
+    assert m.blocks[1].ffn.k == 2 and m.blocks[1].ffn.E == 8 and m.blocks[0].ffn.inter == 160
+    specs = m.param_specs()
+    assert specs["model.layers.1.feed_forward.experts.down_proj"].shape == (8, 96, 64)
+    assert specs["model.layers.0.self_attn.q_proj.weight"].shape == (192, 96)
+
+
+def test_safetensors_round_trip(tmp_path):
+    t = {"a": torch.randn(3, 5).to(torch.bfloat16), "b": torch.arange(7, dtype=torch.int64), "c": torch.randn(2, 2)}
+    path = str(tmp_path / "x.safetensors")
+    st.write_file(path, t.items(), {"k": "v"})
+    from safetensors.torch import load_file
+
+    other = load_file(path)                      # the library reads what we write
+    for k in t:
+        assert torch.equal(other[k], t[k])
+    hdr = st.read_header(path)
+    for k in t:
+        assert torch.equal(st.read_tensor(hdr[k]), t[k]) and hdr[k].shape == tuple(t[k].shape)
+    with open(path, "r+b") as f:                 # a truncated file is noticed
+        f.truncate(os.path.getsize(path) - 4)
+    with pytest.raises(st.SafetensorsError, match="beyond the end"):
+        st.read_header(path)
+
+
+def test_random_model_folder_and_dtype_policy(tmp_path):
+    d = make_model_dir(tmp_path, "B")
+    assert sorted(os.listdir(d)) == ["config.json", "model.safetensors"]
+    assert json.load(open(os.path.join(d, "config.json")))["hidden_size"] == 96
+    src = SafetensorsSource(d, torch.bfloat16, "cpu")
+    assert src.get("model.layers.0.self_attn.q_proj.weight").dtype == torch.bfloat16
+    assert src.get("model.norm.weight").dtype == torch.float32          # stored in 32-bit: stays so
+    assert src.get("model.layers.1.feed_forward.router.weight").dtype == torch.float32
+    assert SafetensorsSource(d, torch.float32, "cpu").get("model.layers.0.self_attn.q_proj.weight").dtype == torch.float32
+    assert storage_dtype(torch.float16, torch.bfloat16) == torch.bfloat16
+    assert storage_dtype(torch.int64, torch.bfloat16) == torch.int32
+    again = make_model_dir(tmp_path / "again", "B")                       # same seed, same bytes
+    assert open(os.path.join(d, "model.safetensors"), "rb").read() == open(os.path.join(again, "model.safetensors"), "rb").read()
+    w = SafetensorsSource(d, torch.float32, "cpu").get("model.layers.0.input_layernorm.weight")
+    assert 0.9 <= float(w.min()) and float(w.max()) <= 1.1
+
+
+def test_one_error_lists_everything(tmp_path):
+    d = make_model_dir(tmp_path, "A")
+    path = os.path.join(d, "model.safetensors")
+    hdr = st.read_header(path)
+    tensors = {n: st.read_tensor(e) for n, e in hdr.items()}
+    del tensors["model.norm.weight"]
+    del tensors["model.layers.1.self_attn.o_proj.weight"]
+    tensors["model.layers.0.self_attn.k_proj.weight"] = torch.zeros(7, 64, dtype=torch.bfloat16)
+    tensors["extra.tensor"] = torch.zeros(2)
+    tensors["model.layers.0.feed_forward.router.weight"] = torch.zeros(4, 64, dtype=torch.int32)
+    st.write_file(path, tensors.items())
+    model = build_model(load_config(d))
+    with pytest.raises(WeightError) as ei:
+        load_model_weights(model, SafetensorsSource(d, torch.float32, "cpu"))
+    e = ei.value
+    assert e.missing == ["model.layers.1.self_attn.o_proj.weight", "model.norm.weight"]
+    assert e.unexpected == ["extra.tensor"]
+    assert len(e.wrong_shape) == 1 and "expected [32, 64], found [7, 64]" in e.wrong_shape[0]
+    assert len(e.wrong_kind) == 1 and "router" in e.wrong_kind[0]
+    msg = str(e)
+    for word in ("missing (2)", "unexpected (1)", "wrong shape (1)", "wrong kind (1)"):
+        assert word in msg
+
+
+def test_random_source_is_order_independent():
+    m = build_model(load_config(TINY_A))
+    specs = m.param_specs()
+    a = RandomSource(specs, 3, torch.float32, "cpu")
+    b = RandomSource(specs, 3, torch.float32, "cpu")
+    names = sorted(specs)
+    for n in names:
+        a.get(n)
+    assert torch.equal(a.get(names[-1]), b.get(names[-1]))
+    assert not torch.equal(RandomSource(specs, 4, torch.float32, "cpu").get(names[0]), b.get(names[0]))
+    check_specs(specs, a.available())

@@ -1,0 +1,145 @@
+"""Generation through the entry points, sampling kernels, long decoding."""
+import math
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+import helpers as H
+import plain_llama4 as P
+from tiny_configs import CONFIGS, make_model_dir
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+DEV = "cuda:0"
+
+
+def test_greedy_generation_matches_plain(tmp_path):
+    """Tiny A, 32-bit: prompts of 5 / 23 / 40 tokens, 16 greedy steps each, under continuous
+    batching with prompts cut into portions."""
+    d = make_model_dir(tmp_path, "A", std=0.1)
+    c, W = P.read_config(d), P.load_weights(d)
+    prompts = [H.random_tokens(n, 256, 40 + n) for n in (5, 23, 40)]
+    want = [P.generate(c, W, p, 16) for p in prompts]
+    eng = H.make_engine(d, "float32", kv_tokens=256, max_num_seqs=3, max_tokens_per_step=16)
+    got = eng.generate(prompts, max_new_tokens=16, temperature=0.0)
+    assert [r.token_ids for r in got] == want
+    assert all(r.finish_reason == "length" and r.prompt_tokens == len(p) for r, p in zip(got, prompts))
+    assert eng.last_stats.prefill_tokens == 68 and eng.last_stats.decode_tokens == 3 * 15
+    eng.cache.check_invariants()
+    assert all(g.pool.num_free == g.pool.num_pages for g in eng.cache.groups)
+    # one request at a time gives the same tokens
+    solo = H.make_engine(d, "float32", kv_tokens=128, max_num_seqs=1)
+    assert [solo.generate([p], max_new_tokens=16)[0].token_ids for p in prompts] == want
+
+
+def test_temperature_generation_matches_plain(tmp_path):
+    """Tiny B, 32-bit: prompts of 1 / 17 / 50 / 77 tokens, 24 steps at temperature 0.8 with
+    fixed seeds: the same uniforms give the same tokens."""
+    d = make_model_dir(tmp_path, "B", std=0.1)
+    c, W = P.read_config(d), P.load_weights(d)
+    prompts = [H.random_tokens(n, 384, 70 + n) for n in (1, 17, 50, 77)]
+    seeds = [11, 12, 13, 14]
+    want = [P.generate(c, W, p, 24, temperature=0.8, seed=s) for p, s in zip(prompts, seeds)]
+    eng = H.make_engine(d, "float32", kv_tokens=512, max_num_seqs=4, max_tokens_per_step=40)
+    got = eng.generate(prompts, max_new_tokens=24, temperature=0.8, seeds=seeds)
+    assert [r.token_ids for r in got] == want
+    assert len({tuple(w) for w in want}) == 4
+
+
+def test_stop_tokens_and_tiny_pool(tmp_path):
+    d = make_model_dir(tmp_path, "A", std=0.1)
+    c, W = P.read_config(d), P.load_weights(d)
+    prompts = [H.random_tokens(n, 256, 5 + n) for n in (9, 30, 12, 25, 18)]
+    free = [P.generate(c, W, p, 12) for p in prompts]
+    stop = free[1][4]
+    want = [P.generate(c, W, p, 12, stop=(stop,)) for p in prompts]
+    assert len(want[1]) < 12
+    # pool of 64 tokens: at most one or two requests fit; the rest wait for pages
+    eng = H.make_engine(d, "float32", kv_tokens=64, max_num_seqs=4, max_tokens_per_step=24)
+    got = eng.generate(prompts, max_new_tokens=12, temperature=0.0, stop_token_ids=(stop,))
+    assert [r.token_ids for r in got] == want
+    assert [r.finish_reason for r in got] == ["stop" if len(w) < 12 else "length" for w in want]
+    assert all(g.pool.total_allocs > g.pool.num_pages for g in eng.cache.groups)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(tmp_path, dtype):
+    """Hundreds of single-token steps: windows slide over many pages that are released and reused."""
+    d = make_model_dir(tmp_path, "A", std=0.1)
+    toks = H.random_tokens(330, 256, 8)
+    eng = H.make_engine(d, dtype, kv_tokens=352, max_num_seqs=1)
+    H.check_against_plain(eng, d, dtype, "long", toks, [10] + [1] * 320, f"A {dtype} long decoding")
+    assert eng.cache.groups[0].pool.total_allocs >= 20
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_first_tokens(tmp_path, dtype):
+    d = make_model_dir(tmp_path, "B", std=0.1)
+    eng = H.make_engine(d, dtype)
+    for toks in ([7], [7, 300], [1, 2, 3]):
+        H.check_against_plain(eng, d, dtype, "f", toks, [1] * len(toks), f"B {dtype} first tokens")
+
+
+def test_sampling_kernels_against_plain():
+    from sharpinference_amd import ops
+
+    g = torch.Generator().manual_seed(0)
+    V = 1003
+    logits = (torch.randn(6, V, generator=g) * 3).to(DEV)
+    logits[2, 17] = logits[2, 900] = logits[2].max() + 1.0             # a tie: the lower index wins
+    logits[3] = -5.0                                                   # all equal
+    am = ops.argmax_rows(logits).cpu().tolist()
+    assert am == [P.greedy(logits[i].cpu()) for i in range(6)] and am[2] == 17 and am[3] == 0
+    cases = [dict(temperature=0.8), dict(temperature=1.0, top_k=5), dict(temperature=1.3, top_p=0.7),
+             dict(temperature=0.9, min_p=0.1), dict(temperature=0.7, top_k=40, top_p=0.95, min_p=0.05),
+             dict(temperature=2.0, top_k=1)]
+    for case in cases:
+        us = P.uniform_stream(3, 6)
+        temp = torch.full((6,), case["temperature"], device=DEV)
+        tk = torch.full((6,), case.get("top_k", 0), dtype=torch.int32, device=DEV)
+        tp = torch.full((6,), case.get("top_p", 1.0), device=DEV)
+        mp = torch.full((6,), case.get("min_p", 0.0), device=DEV)
+        got = ops.sample_rows(logits, temp, torch.tensor(us, device=DEV), tk, tp, mp).cpu().tolist()
+        want = [P.sample(logits[i].cpu(), us[i], **case) for i in range(6)]
+        if "top_p" in case:
+            # row 3 is all ties: which of equal values the nucleus keeps is left open by the
+            # reference (an unstable sort, Sampler.cs:543); the kernel keeps them all
+            got[3] = want[3] = -1
+        assert got == want, case
+
+
+def test_penalties_and_bias_follow_the_reference_order():
+    """reference: src/SharpInference.Engine/Sampler.cs:52-69, 414-433: bias, then the repetition
+    penalty once per distinct token (divide if positive, multiply if negative), then
+    count * frequency + presence subtracted."""
+    from sharpinference_amd.sampling.params import SamplingParams
+    from sharpinference_amd.sampling.sampler import Sampler
+
+    logits = torch.tensor([[2.0, -1.0, 0.5, 3.0, 1.0]], device=DEV)
+    p = SamplingParams(temperature=1e-4, repetition_penalty=2.0, frequency_penalty=0.5, presence_penalty=0.25,
+                       logit_bias={4: 1.5}, penalty_last_n=0)
+    # history 3, 3, 0: token 3 -> 3/2 - (2*0.5 + 0.25) = 0.25; token 0 -> 2/2 - 0.75 = 0.25; token 4 -> 2.5
+    assert Sampler(DEV).sample(logits, [p], [0], [[3, 3, 0]]) == [4]
+    q = SamplingParams(temperature=1e-4, repetition_penalty=2.0, penalty_last_n=0)
+    assert Sampler(DEV).sample(logits, [q], [0], [[3]]) == [0]          # 3 -> 1.5 < 2
+    assert Sampler(DEV).sample(torch.tensor([[-1.0, -1.5]], device=DEV), [q], [0], [[0]]) == [1]   # -1 * 2 = -2 < -1.5
+    greedy = SamplingParams(temperature=0.0, repetition_penalty=5.0)    # greedy rows skip the penalties
+    assert Sampler(DEV).sample(logits, [greedy], [0], [[3]]) == [3]
+
+
+def test_command_line(tmp_path):
+    d = make_model_dir(tmp_path, "A", std=0.1)
+    c, W = P.read_config(d), P.load_weights(d)
+    prompt = H.random_tokens(12, 256, 1)
+    want = P.generate(c, W, prompt, 8)
+    out = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "sharpi-cli"), "-m", d, "-p", ",".join(map(str, prompt)),
+                          "-n", "8", "--temp", "0", "--dtype", "fp32", "--kv-tokens", "128"],
+                         capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stderr
+    lines = out.stdout.strip().splitlines()
+    assert lines[0] == " ".join(map(str, prompt))
+    assert lines[1].startswith(" ".join(map(str, want))) and lines[1].endswith("(length)")
+    assert lines[-1].startswith("Prefill: 12 tokens, ") and "| Decode: 7 tokens, " in lines[-1] and lines[-1].endswith("t/s")

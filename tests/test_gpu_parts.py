@@ -1,0 +1,288 @@
+"""Each part alone, the arrangement of layers as data, and a toy mixer with state of its own."""
+import math
+from dataclasses import dataclass
+
+import pytest
+import torch
+
+import helpers as H
+import plain_llama4 as P
+from tiny_configs import make_model_dir
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _ctx(entries, page_size=16, dtype=torch.float32, totals=None):
+    """A StepContext for requests given as (start position, tokens in this step), each with its
+    own pages in one group (`totals`: final lengths, so that pages stay put from step to step)."""
+    from sharpinference_amd.parts.base import GroupView, StepContext
+
+    T = sum(n for _, n in entries)
+    pos, ent, slots, tables, cu = [], [], [], [], [0]
+    page = 0
+    for i, (start, n) in enumerate(entries):
+        nb = ((totals[i] if totals else start + n) + page_size - 1) // page_size
+        tbl = list(range(page, page + nb))
+        page += nb
+        tables.append(tbl)
+        for p in range(start, start + n):
+            pos.append(p)
+            ent.append(i)
+            slots.append(tbl[p // page_size] * page_size + p % page_size)
+        cu.append(cu[-1] + n)
+    maxb = max(len(t) for t in tables)
+    bt = torch.full((len(entries), maxb), -1, dtype=torch.int32)
+    for i, t in enumerate(tables):
+        bt[i, :len(t)] = torch.tensor(t, dtype=torch.int32)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)  # noqa: E731
+    g = GroupView(bt.to(DEV), i32(slots), page_size, max_context=max(pos) + 1)
+    lens = [n for _, n in entries]
+    dec = [cu[i] for i, n in enumerate(lens) if n == 1]
+    tiles = [(i, cu[i] + o, min(32, n - o)) for i, n in enumerate(lens) if n > 1 for o in range(0, n, 32)]
+    ctx = StepContext(n_tokens=T, n_entries=len(entries), token_ids=i32([0] * T), positions=i32(pos), entry_of_token=i32(ent),
+                      cu_tokens=i32(cu), state_slots=i32(list(range(len(entries)))), groups=[g], act_dtype=dtype,
+                      no_store_slots=i32([-1] * T), entry_lens=lens, entry_starts=[s for s, _ in entries],
+                      max_entry_len=max(lens), n_decode=len(dec), decode_tokens=None if len(dec) == T else i32(dec),
+                      n_prefill_tiles=len(tiles), prefill_tiles=i32(tiles).view(-1, 3) if tiles else None)
+    return ctx, page
+
+
+class _Dict:
+    where = "test"
+
+    def __init__(self, tensors, dtype):
+        self.t, self.dtype = tensors, dtype
+
+    def get(self, name):
+        return self.t[name].to(self.dtype).to(DEV)
+
+
+def test_norm_part():
+    from sharpinference_amd.parts.base import ResidualStream
+    from sharpinference_amd.parts.norm import RMSNorm
+
+    h = torch.randn(9, 80)
+    delta = torch.randn(9, 80)
+    w = torch.rand(80) + 0.5
+    part = RMSNorm(80, 1e-4)
+    part.load("n.", _Dict({"n.weight": w}, torch.float32))
+    stream = ResidualStream(h.clone().to(DEV))
+    stream.pending = delta.to(DEV)
+    out = part.forward(stream, torch.float32).cpu()
+    assert torch.allclose(out, P.rms_norm(h + delta, w, 1e-4), atol=1e-5)
+    assert stream.pending is None and torch.allclose(stream.h.cpu(), h + delta)
+    rows = torch.tensor([7, 2], dtype=torch.int32, device=DEV)
+    stream.pending = delta.to(DEV)
+    some = part.forward(stream, torch.float32, rows=rows).cpu()
+    assert torch.allclose(some, P.rms_norm(h + 2 * delta, w, 1e-4)[[7, 2]], atol=1e-5)
+    assert stream.pending is not None and torch.allclose(stream.h.cpu(), h + delta)   # gathered rows leave the stream alone
+    bare = RMSNorm(80, 1e-4, has_weight=False)
+    stream.pending = None
+    assert torch.allclose(bare.forward(stream, torch.float32).cpu(), P.l2_head_norm(h + delta, 1e-4), atol=1e-5)
+
+
+def test_rotary_table_matches_plain():
+    from sharpinference_amd.config.llama4 import RopeScaling
+    from sharpinference_amd.parts.position import RotaryInterleaved
+
+    sc = {"factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0, "original_max_position_embeddings": 32}
+    for hd, theta, s in ((16, 10000.0, None), (32, 500000.0, sc), (128, 500000.0, dict(sc, factor=16.0, original_max_position_embeddings=8192))):
+        part = RotaryInterleaved(hd, theta, RopeScaling(**{"rope_type": "llama3", **s}) if s else None)
+        assert torch.equal(part.frequencies(), P.rope_inv_freq(hd, theta, s))
+
+
+@pytest.mark.parametrize("layer,dtype", [(0, torch.float32), (1, torch.float32), (0, torch.bfloat16), (1, torch.bfloat16)])
+def test_attention_part_alone(tmp_path, layer, dtype):
+    """The mixer with a cache of its own: a prompt in two portions for one request beside single
+    tokens for two others, against the plain layer on the whole sequences.  Layer 0 of tiny B has
+    rotary and a chunk of 24, layer 3 (here: index 1) has neither but the temperature."""
+    from sharpinference_amd import build_model, load_config
+    from sharpinference_amd.parts.base import LayerCache
+    from sharpinference_amd.weights.loader import SafetensorsSource
+
+    d = make_model_dir(tmp_path, "B", std=0.1)
+    lay = [0, 3][layer]
+    c, W = P.read_config(d), {k: v.float() for k, v in P.load_weights(d).items()}
+    model = build_model(load_config(d))
+    mixer = model.blocks[lay].mixer
+    mixer.load(f"model.layers.{lay}.self_attn.", SafetensorsSource(d, dtype, DEV))
+    lens = [61, 30, 47]
+    xs = [torch.randn(L, 96).to(torch.bfloat16).float() for L in lens]
+    store = P.store_bf16 if dtype == torch.bfloat16 else P._same
+    want = [P.attention_layer(c, W, lay, x, torch.arange(L), store) for x, L in zip(xs, lens)]
+    spec = mixer.cache_spec()
+    k = torch.zeros(16, spec.num_kv_heads, 16, spec.head_dim, dtype=dtype, device=DEV)
+    v = torch.zeros(16, spec.num_kv_heads, spec.head_dim, 16, dtype=dtype, device=DEV)
+    # step 1: the three requests' first parts; step 2: request 0 goes on with 21 tokens, the others decode one token
+    first = [40, 29, 46]
+    done = [0, 0, 0]
+    outs = [[], [], []]
+    for sizes in (first, [21, 1, 1]):
+        ctx, pages = _ctx([(done[i], sizes[i]) for i in range(3)], dtype=dtype, totals=lens)
+        assert pages <= 16
+        x = torch.cat([xs[i][done[i]:done[i] + sizes[i]] for i in range(3)]).to(dtype).to(DEV)
+        out = mixer.forward(x, ctx, LayerCache(ctx.groups[0], k, v)).float().cpu()
+        o = 0
+        for i in range(3):
+            outs[i].append(out[o:o + sizes[i]])
+            o += sizes[i]
+            done[i] += sizes[i]
+    for i in range(3):
+        got = torch.cat(outs[i])
+        tol = 1e-4 if dtype == torch.float32 else 3e-2
+        assert float((got - want[i]).abs().max()) <= tol * max(1.0, float(want[i].abs().max())), (i, lay)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_feed_forward_parts_alone(tmp_path, dtype):
+    from sharpinference_amd import build_model, load_config
+    from sharpinference_amd.weights.loader import SafetensorsSource
+
+    d = make_model_dir(tmp_path, "B", std=0.1)
+    c, W = P.read_config(d), {k: v.float() for k, v in P.load_weights(d).items()}
+    model = build_model(load_config(d))
+    src = SafetensorsSource(d, dtype, DEV)
+    x = torch.randn(70, 96).to(torch.bfloat16).float()
+    ctx, _ = _ctx([(0, 70)], dtype=dtype)
+    store = P.store_bf16 if dtype == torch.bfloat16 else P._same
+    tol = 1e-4 if dtype == torch.float32 else 3e-2
+    dense = model.blocks[0].ffn
+    dense.load("model.layers.0.feed_forward.", src)
+    got = dense.forward(x.to(dtype).to(DEV), ctx).float().cpu()
+    want = P.dense_layer(c, W, 0, x, store)
+    assert float((got - want).abs().max()) <= tol * float(want.abs().max())
+    moe = model.blocks[1].ffn
+    moe.load("model.layers.1.feed_forward.", src)
+    trace = []
+    ctx.extras["router_trace"] = trace
+    got = moe.forward(x.to(dtype).to(DEV), ctx).float().cpu()
+    want = P.moe_layer(c, W, 1, x, None, store, routes={1: trace[0][0].cpu()} if dtype == torch.bfloat16 else None)
+    assert float((got - want).abs().max()) <= tol * float(want.abs().max())
+
+
+def test_schedule_runs_a_layer_twice_and_shares_a_cache(tmp_path):
+    """The order of execution is data: layer 0 runs twice (two cache slots), and the second run of
+    layer 1 reads the keys and values that its first run stored."""
+    from sharpinference_amd import load_config
+    from sharpinference_amd.engine import Engine
+    from sharpinference_amd.parts.model import Run
+    from sharpinference_amd.registry import register_architecture, unregister_architecture
+    from sharpinference_amd.config.llama4 import Llama4TextConfig
+    from sharpinference_amd.models.llama4 import build_llama4
+
+    def build(cfg):
+        m = build_llama4(cfg)
+        m.schedule = [Run(0, 0), Run(1, 1), Run(0, 2), Run(1, 1, write=False)]
+        m._check_schedule()
+        return m
+
+    register_architecture("LoopedLlama4ForTest", Llama4TextConfig, build, replace=True)
+    try:
+        d = make_model_dir(tmp_path, "A", std=0.1)
+        cfg = load_config(d)
+        cfg.architecture = "LoopedLlama4ForTest"
+        import json, os
+        json.dump(cfg.to_dict(), open(os.path.join(d, "config.json"), "w"))
+        eng = Engine(d, dtype="float32", kv_tokens=256, max_num_seqs=2)
+        assert len(eng.cache.slot_specs) == 3
+        toks = H.random_tokens(45, 256, 3)
+        got = H.run_cut(eng, "x", toks, [20, 1, 1, 13, 10])
+        c, W = P.read_config(d), {k: v.float() for k, v in P.load_weights(d).items()}
+        eps, pos = c["rms_norm_eps"], torch.arange(45)
+        h = W["model.embed_tokens.weight"][torch.tensor(toks)]
+        kv1 = []
+        for lay, kv_out, kv_in in ((0, None, None), (1, kv1, None), (0, None, None), (1, None, "shared")):
+            p = f"model.layers.{lay}."
+            n = P.rms_norm(h, W[p + "input_layernorm.weight"], eps)
+            h = h + P.attention_layer(c, W, lay, n, pos, kv_out=kv_out, kv_in=kv1[0] if kv_in else None)
+            n = P.rms_norm(h, W[p + "post_attention_layernorm.weight"], eps)
+            h = h + P.moe_layer(c, W, lay, n)
+        want = P.rms_norm(h, W["model.norm.weight"], eps) @ W["lm_head.weight"].T
+        H.assert_close_fp32(got, want, "looped schedule")
+    finally:
+        unregister_architecture("LoopedLlama4ForTest")
+
+
+def test_toy_mixer_with_state_needs_no_change_to_the_framework():
+    """A mixer defined here, with per-request state of fixed size (a running sum and a count),
+    is registered, built and stepped through the ordinary engine."""
+    from sharpinference_amd.cache.spec import StateSpec
+    from sharpinference_amd.config.base import ModelConfig
+    from sharpinference_amd.engine import Engine
+    from sharpinference_amd.parts.base import Part
+    from sharpinference_amd.parts.block import PreNormBlock
+    from sharpinference_amd.parts.feedforward import DenseSwiGLU
+    from sharpinference_amd.parts.model import DecoderModel
+    from sharpinference_amd.parts.norm import RMSNorm
+    from sharpinference_amd.registry import register_architecture, unregister_architecture
+
+    @dataclass
+    class ToyConfig(ModelConfig):
+        architecture: str = "ToyRunningMean"
+        hidden_size: int = 32
+        layers: int = 2
+        vocab_size: int = 50
+        max_position_embeddings: int = 256
+
+        @classmethod
+        def from_dict(cls, d):
+            return cls(hidden_size=d["hidden_size"], layers=d["layers"], vocab_size=d["vocab_size"])
+
+        def to_dict(self):
+            return {"architectures": [self.architecture], "hidden_size": self.hidden_size, "layers": self.layers,
+                    "vocab_size": self.vocab_size}
+
+    class RunningMean(Part):
+        """out[t] = mean of the inputs of positions 0..t; state per request: [sum (H), count]."""
+
+        def __init__(self, hidden):
+            self.hidden = hidden
+
+        def cache_spec(self):
+            return StateSpec((self.hidden + 1,), torch.float32)
+
+        def forward(self, x, ctx, cache):
+            out = torch.empty_like(x)
+            o = 0
+            slots = ctx.state_slots.cpu().tolist()
+            for e, n in enumerate(ctx.entry_lens):
+                st = cache.state[slots[e]]
+                cs = torch.cumsum(x[o:o + n].float(), 0) + st[:-1]
+                cnt = st[-1] + torch.arange(1, n + 1, device=x.device)
+                out[o:o + n] = (cs / cnt[:, None]).to(x.dtype)
+                st[:-1] = cs[-1]
+                st[-1] = cnt[-1]
+                o += n
+            return out
+
+    def build(cfg):
+        blocks = [PreNormBlock(RMSNorm(cfg.hidden_size, 1e-5), RunningMean(cfg.hidden_size), RMSNorm(cfg.hidden_size, 1e-5),
+                               DenseSwiGLU(cfg.hidden_size, 48), names={"norm1": "n1.", "mixer": "mix.", "norm2": "n2.", "ffn": "ff."})
+                  for _ in range(cfg.layers)]
+        return DecoderModel(cfg.vocab_size, cfg.hidden_size, blocks, RMSNorm(cfg.hidden_size, 1e-5), config=cfg)
+
+    register_architecture("ToyRunningMean", ToyConfig, build, replace=True)
+    try:
+        eng = Engine(config=ToyConfig(), weight_seed=7, dtype="float32", kv_tokens=64, max_num_seqs=3, weight_std=0.3)
+        assert eng.cache.groups == [] and eng.cache.state[0].shape == (3, 33)
+        a, b = H.random_tokens(40, 50, 1), H.random_tokens(25, 50, 2)
+        whole_a = H.run_cut(eng, "a", a, [40])
+        whole_b = H.run_cut(eng, "b", b, [25])
+        # the same two requests interleaved, in portions and single tokens; a third takes and frees a slot between
+        steps = H.mixed_trace({"a": a, "b": b, "c": H.random_tokens(9, 50, 3)}, seed=2, max_live=3, tail=6)
+        got = H.replay(eng, steps)
+        assert float((got["a"] - whole_a).abs().max()) <= 1e-4 and float((got["b"] - whole_b).abs().max()) <= 1e-4
+        # and against the formula itself
+        m = eng.model
+        h = m.embed[torch.tensor(a, device=DEV)].float()
+        for blk in m.blocks:
+            n = P.rms_norm(h, blk.norm1.weight, 1e-5)
+            h = h + torch.cumsum(n, 0) / torch.arange(1, 41, device=DEV)[:, None]
+            n = P.rms_norm(h, blk.norm2.weight, 1e-5)
+            gu = n @ blk.ffn.w_gate_up.T
+            h = h + (P.silu(gu[:, :48]) * gu[:, 48:]) @ blk.ffn.w_down.T
+        want = P.rms_norm(h, m.final_norm.weight, 1e-5) @ m.head.T
+        assert float((whole_a - want.cpu()).abs().max()) <= 1e-4
+    finally:
+        unregister_architecture("ToyRunningMean")

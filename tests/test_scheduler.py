@@ -1,0 +1,132 @@
+"""The scheduler's decisions, driven by a scripted step function (no GPU), in the way the
+reference tests its engines with a scripted forward pass
+(reference: tests/SharpInference.Tests.ForwardPass/InferenceEngineChunkTests.cs:417-456)."""
+from sharpinference_amd.cache.manager import CacheManager
+from sharpinference_amd.cache.spec import KVSpec, WINDOW_CHUNK, WINDOW_NONE
+from sharpinference_amd.engine.scheduler import Request, Scheduler
+from sharpinference_amd.sampling.params import SamplingParams
+
+
+def _cache(num_pages, max_requests=8):
+    return CacheManager([KVSpec(1, 16, WINDOW_CHUNK, 32), KVSpec(1, 16, WINDOW_NONE, 0)], 16, num_pages, max_requests,
+                        allocate=False)
+
+
+def _run(sched, script, max_iters=10000):
+    """script(request) -> next token.  Plays steps until nothing is left; returns the batches."""
+    batches = []
+    for _ in range(max_iters):
+        if not sched.has_work():
+            break
+        batch = sched.schedule()
+        if not batch:
+            break
+        for s in batch:                                   # what the step function does to the cache
+            assert sched.cache.append(s.request.req_id, len(s.tokens)), "a running request ran out of pages"
+        for s in batch:
+            sched.cache.commit(s.request.req_id)
+        sched.cache.check_invariants()
+        batches.append([(s.request.req_id, list(s.tokens), s.samples) for s in batch])
+        sched.update(batch, [script(s.request) if s.samples else None for s in batch])
+    return batches
+
+
+def _req(i, n_prompt, max_new, stop=()):
+    return Request(i, list(range(1, n_prompt + 1)), SamplingParams(temperature=0.0, max_new_tokens=max_new, stop_token_ids=stop))
+
+
+def test_portions_respect_the_budget_and_decodes_come_first():
+    sched = Scheduler(_cache(64), max_num_seqs=4, max_tokens_per_step=16, max_model_len=256)
+    reqs = [_req(0, 5, 3), _req(1, 40, 2), _req(2, 7, 2)]
+    for r in reqs:
+        sched.add(r)
+    batches = _run(sched, lambda r: 100 + len(r.output))
+    assert all(sum(len(t) for _, t, _ in b) <= 16 for b in batches)
+    # step 0: request 0 whole (5), request 1 gets the rest of the budget (11)
+    assert batches[0] == [(0, [1, 2, 3, 4, 5], True), (1, list(range(1, 12)), False)]
+    # step 1: request 0 decodes first, then prompts in arrival order
+    assert batches[1][0] == (0, [100], True) and batches[1][1][0] == 1 and len(batches[1][1][1]) == 15
+    # each request's prompt went through exactly once, in order
+    for r in reqs:
+        seen = [t for b in batches for rid, toks, _ in b if rid == r.req_id for t in toks]
+        assert seen[:len(r.prompt)] == r.prompt
+        assert seen[len(r.prompt):] == r.output[:-1]      # the last token drawn is never fed back
+    assert [r.finish_reason for r in reqs] == ["length"] * 3
+    assert [len(r.output) for r in reqs] == [3, 2, 2]
+    assert all(g.pool.num_free == g.pool.num_pages for g in sched.cache.groups)
+
+
+def test_stop_token_ends_without_being_emitted_even_as_first_token():
+    sched = Scheduler(_cache(64), 4, 64, 256)
+    a, b = _req("a", 4, 10, stop=(7,)), _req("b", 4, 10, stop=(7,))
+    sched.add(a)
+    sched.add(b)
+    _run(sched, lambda r: 7 if r.req_id == "a" or len(r.output) == 2 else 50)
+    assert a.output == [] and a.finish_reason == "stop"
+    assert b.output == [50, 50] and b.finish_reason == "stop"
+
+
+def test_fifo_admission_waits_for_pages_and_everything_completes():
+    """A pool too small for all requests at once: later ones wait for the earlier ones' pages
+    (reference: tests/SharpInference.Tests.ForwardPass/ContinuousBatchingTests.cs:504-539)."""
+    sched = Scheduler(_cache(num_pages=6), max_num_seqs=8, max_tokens_per_step=32, max_model_len=256)
+    reqs = [_req(i, 30 + i, 10) for i in range(5)]        # each needs 3 pages of the all-keys group
+    for r in reqs:
+        sched.add(r)
+    first_step = {}
+    batches = _run(sched, lambda r: 9)
+    for n, b in enumerate(batches):
+        for rid, _, _ in b:
+            first_step.setdefault(rid, n)
+    assert [first_step[i] for i in range(5)] == sorted(first_step[i] for i in range(5))   # nobody overtakes
+    assert first_step[2] > first_step[1]                   # the third had to wait for pages
+    assert all(len(set(rid for rid, _, _ in b)) <= 2 for b in batches)
+    assert all(r.finish_reason == "length" and len(r.output) == 10 for r in reqs)
+    assert all(g.pool.total_allocs > g.pool.num_pages for g in sched.cache.groups[1:])
+
+
+def test_a_request_that_can_never_fit_is_refused_not_admitted():
+    sched = Scheduler(_cache(num_pages=4), 4, 32, max_model_len=1000)
+    big, ok = _req("big", 100, 10), _req("ok", 20, 5)
+    sched.add(big)
+    sched.add(ok)
+    _run(sched, lambda r: 3)
+    assert big.finish_reason == "too_long" and big.output == []
+    assert ok.finish_reason == "length" and len(ok.output) == 5
+    too_long = _req("ctx", 300, 5)
+    sched2 = Scheduler(_cache(64), 4, 32, max_model_len=256)
+    sched2.add(too_long)
+    _run(sched2, lambda r: 3)
+    assert too_long.finish_reason == "too_long"
+
+
+def test_context_limit_and_zero_tokens_and_cancel():
+    sched = Scheduler(_cache(64), 4, 32, max_model_len=24)
+    r = _req("r", 20, 100)
+    z = _req("z", 5, 0)
+    c = _req("c", 5, 50)
+    for x in (r, z, c):
+        sched.add(x)
+    steps = {"n": 0}
+
+    def script(req):
+        steps["n"] += 1
+        if steps["n"] == 3:
+            c.cancelled = True
+        return 4
+
+    _run(sched, script)
+    assert r.finish_reason == "length" and len(r.prompt) + len(r.output) == 24
+    assert z.finish_reason == "length" and z.output == []
+    assert c.finish_reason == "abort" and 0 < len(c.output) < 50
+    assert all(g.pool.num_free == g.pool.num_pages for g in sched.cache.groups)
+
+
+def test_max_num_seqs_bounds_the_batch():
+    sched = Scheduler(_cache(256), max_num_seqs=2, max_tokens_per_step=64, max_model_len=128)
+    reqs = [_req(i, 3, 4) for i in range(5)]
+    for r in reqs:
+        sched.add(r)
+    batches = _run(sched, lambda r: 1)
+    assert max(len(b) for b in batches) == 2
+    assert all(r.finish_reason == "length" for r in reqs)
