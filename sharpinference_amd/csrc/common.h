@@ -48,6 +48,32 @@ template <typename T> __device__ __forceinline__ T from_f32(float v);
 template <> __device__ __forceinline__ float from_f32<float>(float v) { return v; }
 template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float v) { return f32_to_bf16(v); }
 
+// eight consecutive elements as floats (p must be 16-byte aligned for bfloat16, 32 for float)
+__device__ __forceinline__ void load8(const float* p, float* v) {
+  const float4 a = *reinterpret_cast<const float4*>(p);
+  const float4 b = *reinterpret_cast<const float4*>(p + 4);
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+__device__ __forceinline__ void load8(const bf16_t* p, float* v) {
+  const uint4 a = *reinterpret_cast<const uint4*>(p);
+  v[0] = bf16_bits_to_f32(a.x & 0xffffu); v[1] = bf16_bits_to_f32(a.x >> 16);
+  v[2] = bf16_bits_to_f32(a.y & 0xffffu); v[3] = bf16_bits_to_f32(a.y >> 16);
+  v[4] = bf16_bits_to_f32(a.z & 0xffffu); v[5] = bf16_bits_to_f32(a.z >> 16);
+  v[6] = bf16_bits_to_f32(a.w & 0xffffu); v[7] = bf16_bits_to_f32(a.w >> 16);
+}
+__device__ __forceinline__ void store8(float* p, const float* v) {
+  *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  *reinterpret_cast<float4*>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+}
+__device__ __forceinline__ void store8(bf16_t* p, const float* v) {
+  uint4 o;
+  o.x = (uint32_t)f32_to_bf16(v[0]).bits | ((uint32_t)f32_to_bf16(v[1]).bits << 16);
+  o.y = (uint32_t)f32_to_bf16(v[2]).bits | ((uint32_t)f32_to_bf16(v[3]).bits << 16);
+  o.z = (uint32_t)f32_to_bf16(v[4]).bits | ((uint32_t)f32_to_bf16(v[5]).bits << 16);
+  o.w = (uint32_t)f32_to_bf16(v[6]).bits | ((uint32_t)f32_to_bf16(v[7]).bits << 16);
+  *reinterpret_cast<uint4*>(p) = o;
+}
+
 // dtype codes shared with the Python side
 enum : int { DT_F32 = 0, DT_BF16 = 1 };
 

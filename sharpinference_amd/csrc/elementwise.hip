@@ -67,19 +67,91 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__
   }
 }
 
+// The same with rows a multiple of 8 wide: 16-byte accesses, the row kept in registers between
+// the two passes (up to kNormKeep runs of 8 per thread; wider rows are read again).
+constexpr int kNormKeep = 4;
+
+template <typename TD, typename TW, typename TO>
+__global__ void add_rmsnorm_vec_kernel(float* __restrict__ h, const TD* __restrict__ delta,
+                                       const TW* __restrict__ w, TO* __restrict__ out,
+                                       const int* __restrict__ rows, int hidden, float eps, int write_back) {
+  __shared__ float red[16];
+  const int i = blockIdx.x;
+  const int r = rows ? rows[i] : i;
+  float* hr = h + (size_t)r * hidden;
+  const TD* dr = delta ? delta + (size_t)r * hidden : nullptr;
+  float keep[kNormKeep][8];
+  float ss = 0.f;
+  int n = 0;
+  for (int c = threadIdx.x * 8; c < hidden; c += blockDim.x * 8, ++n) {
+    float x[8];
+    load8(hr + c, x);
+    if (dr) {
+      float d[8];
+      load8(dr + c, d);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) x[j] += d[j];
+      if (write_back) store8(hr + c, x);
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ss += x[j] * x[j];
+    if (n < kNormKeep) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) keep[n][j] = x[j];
+    }
+  }
+  const float total = block_sum(ss, red);
+  const float s = 1.0f / sqrtf(total / (float)hidden + eps);
+  TO* o = out + (size_t)i * hidden;
+  n = 0;
+  for (int c = threadIdx.x * 8; c < hidden; c += blockDim.x * 8, ++n) {
+    float x[8];
+    if (n < kNormKeep) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) x[j] = keep[n][j];
+    } else {
+      load8(hr + c, x);
+      if (dr && !write_back) {
+        float d[8];
+        load8(dr + c, d);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) x[j] += d[j];
+      }
+    }
+    float y[8];
+    if (w) {
+      float wv[8];
+      load8(w + c, wv);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) y[j] = (x[j] * s) * wv[j];
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) y[j] = x[j] * s;
+    }
+    store8(o + c, y);
+  }
+}
+
 template <typename TD, typename TW>
 static int launch_add_rmsnorm_o(float* h, const void* delta, const void* w, void* out, int out_dtype,
                                 const int* rows, int n_out, int hidden, float eps, int write_back,
                                 hipStream_t stream) {
   dim3 grid(n_out), block(hidden >= 2048 ? 512 : 256);
-  if (out_dtype == DT_F32)
+  if (out_dtype != DT_F32 && out_dtype != DT_BF16) return SHARPI_ERR_ARG;
+  if ((hidden & 7) == 0) {
+    dim3 vblock(hidden >= 4096 ? 256 : hidden >= 1024 ? 128 : 64);
+    if (out_dtype == DT_F32)
+      add_rmsnorm_vec_kernel<TD, TW, float><<<grid, vblock, 0, stream>>>(h, (const TD*)delta, (const TW*)w,
+                                                                        (float*)out, rows, hidden, eps, write_back);
+    else
+      add_rmsnorm_vec_kernel<TD, TW, bf16_t><<<grid, vblock, 0, stream>>>(h, (const TD*)delta, (const TW*)w,
+                                                                         (bf16_t*)out, rows, hidden, eps, write_back);
+  } else if (out_dtype == DT_F32)
     add_rmsnorm_kernel<TD, TW, float><<<grid, block, 0, stream>>>(h, (const TD*)delta, (const TW*)w,
                                                                  (float*)out, rows, hidden, eps, write_back);
-  else if (out_dtype == DT_BF16)
+  else
     add_rmsnorm_kernel<TD, TW, bf16_t><<<grid, block, 0, stream>>>(h, (const TD*)delta, (const TW*)w,
                                                                   (bf16_t*)out, rows, hidden, eps, write_back);
-  else
-    return SHARPI_ERR_ARG;
   SHARPI_CHECK_LAUNCH();
   return SHARPI_OK;
 }
@@ -130,17 +202,45 @@ __global__ void silu_mul_kernel(const T* __restrict__ gu, const float* __restric
   out[(size_t)m * inter + i] = from_f32<T>(a * u);
 }
 
+template <typename T>
+__global__ void silu_mul_vec_kernel(const T* __restrict__ gu, const float* __restrict__ scale,
+                                    T* __restrict__ out, int inter) {
+  const int m = blockIdx.x;
+  const int i = (blockIdx.y * blockDim.x + threadIdx.x) * 8;
+  if (i >= inter) return;
+  const T* row = gu + (size_t)m * 2 * inter;
+  float g[8], u[8], o[8];
+  load8(row + i, g);
+  load8(row + inter + i, u);
+  const float s = scale ? scale[m] : 1.0f;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    float gj = g[j], uj = u[j];
+    if (scale) {
+      gj *= s;
+      uj *= s;
+    }
+    o[j] = (gj / (1.0f + expf(-gj))) * uj;
+  }
+  store8(out + (size_t)m * inter + i, o);
+}
+
 SHARPI_EXPORT int sharpi_silu_mul(const void* gu, const float* scale, void* out, int dtype, int rows, int inter,
                                   hipStream_t stream) {
   if (rows <= 0) return SHARPI_OK;
   if (inter <= 0 || ceil_div(inter, 256) > 65535) return SHARPI_ERR_ARG;
   dim3 block(256), grid(rows, ceil_div(inter, 256));
-  if (dtype == DT_F32)
+  if (dtype != DT_F32 && dtype != DT_BF16) return SHARPI_ERR_ARG;
+  if ((inter & 7) == 0) {
+    dim3 vgrid(rows, ceil_div(inter, 256 * 8));
+    if (dtype == DT_F32)
+      silu_mul_vec_kernel<float><<<vgrid, block, 0, stream>>>((const float*)gu, scale, (float*)out, inter);
+    else
+      silu_mul_vec_kernel<bf16_t><<<vgrid, block, 0, stream>>>((const bf16_t*)gu, scale, (bf16_t*)out, inter);
+  } else if (dtype == DT_F32)
     silu_mul_kernel<float><<<grid, block, 0, stream>>>((const float*)gu, scale, (float*)out, inter);
-  else if (dtype == DT_BF16)
-    silu_mul_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)gu, scale, (bf16_t*)out, inter);
   else
-    return SHARPI_ERR_ARG;
+    silu_mul_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)gu, scale, (bf16_t*)out, inter);
   SHARPI_CHECK_LAUNCH();
   return SHARPI_OK;
 }
@@ -160,19 +260,48 @@ __global__ void moe_combine_kernel(const T* __restrict__ y, const int* __restric
   out[(size_t)t * hidden + c] = from_f32<T>(acc);
 }
 
+template <typename T>
+__global__ void moe_combine_vec_kernel(const T* __restrict__ y, const int* __restrict__ inv_pos,
+                                       const T* __restrict__ shared, T* __restrict__ out, int hidden, int k) {
+  const int t = blockIdx.x;
+  const int c = (blockIdx.y * blockDim.x + threadIdx.x) * 8;
+  if (c >= hidden) return;
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  for (int j = 0; j < k; ++j) {
+    float v[8];
+    load8(y + (size_t)inv_pos[t * k + j] * hidden + c, v);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] += v[i];
+  }
+  if (shared) {
+    float v[8];
+    load8(shared + (size_t)t * hidden + c, v);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] += v[i];
+  }
+  store8(out + (size_t)t * hidden + c, acc);
+}
+
 SHARPI_EXPORT int sharpi_moe_combine(const void* y, const int* inv_pos, const void* shared, void* out, int dtype,
                                      int n_tokens, int hidden, int k, hipStream_t stream) {
   if (n_tokens <= 0) return SHARPI_OK;
   if (hidden <= 0 || k <= 0 || ceil_div(hidden, 256) > 65535) return SHARPI_ERR_ARG;
   dim3 block(256), grid(n_tokens, ceil_div(hidden, 256));
-  if (dtype == DT_F32)
+  if (dtype != DT_F32 && dtype != DT_BF16) return SHARPI_ERR_ARG;
+  if ((hidden & 7) == 0) {
+    dim3 vblock(128), vgrid(n_tokens, ceil_div(hidden, 128 * 8));
+    if (dtype == DT_F32)
+      moe_combine_vec_kernel<float><<<vgrid, vblock, 0, stream>>>((const float*)y, inv_pos, (const float*)shared,
+                                                                 (float*)out, hidden, k);
+    else
+      moe_combine_vec_kernel<bf16_t><<<vgrid, vblock, 0, stream>>>((const bf16_t*)y, inv_pos, (const bf16_t*)shared,
+                                                                  (bf16_t*)out, hidden, k);
+  } else if (dtype == DT_F32)
     moe_combine_kernel<float><<<grid, block, 0, stream>>>((const float*)y, inv_pos, (const float*)shared,
                                                          (float*)out, hidden, k);
-  else if (dtype == DT_BF16)
+  else
     moe_combine_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)y, inv_pos, (const bf16_t*)shared,
                                                           (bf16_t*)out, hidden, k);
-  else
-    return SHARPI_ERR_ARG;
   SHARPI_CHECK_LAUNCH();
   return SHARPI_OK;
 }

@@ -2,32 +2,36 @@
 //   out[row, :] = x[a_rows[row], :] * W[e]^T   for the rows of expert e in the expert-sorted list,
 // bfloat16 inputs, float accumulation on the matrix cores.
 //
-// A block computes a 64-row x 256-column tile of one expert.  The tiles are listed on the
-// device by the routing kernel (tile_expert, tile_row0, n_tiles), so no block is launched for
-// an (expert, row range) that does not exist and the host never learns the routing.  Tiles of
-// the same expert and column range are neighbours in launch order, so a second row tile finds
-// the expert's weights in the memory-side cache.
-//  * Each of the 4 waves owns 64 weight rows (4 MFMA tiles) and reads them straight from global
-//    memory into registers: a weight element is used by one wave only.
-//  * The 64 x rows (gathered through a_rows) are shared by the waves and staged through LDS,
-//    128 columns of K at a time, double-buffered; rows are padded to 136 elements so that the
-//    16 lanes of a quarter-wave read 16 different banks.
+// The product is bound by reading the experts' weights, so a block takes ALL rows of its expert
+// that fit one tile (192, about one and a half times the mean load of 2,048 tokens over 16
+// experts) against 128 weight rows: a typical expert's weights are then read once.  Tiles are
+// listed on the device by the routing kernel (tile_expert, tile_row0, n_tiles); the host never
+// learns the routing, and 16-row groups beyond an expert's last row are skipped, not multiplied.
+//  * Each of the 4 waves owns 32 weight rows (2 MFMA tiles) and reads them straight from global
+//    memory into registers, one 64-wide K stage ahead: a weight element is used by one wave only.
+//  * The x rows (gathered through a_rows) are shared by the waves and staged through LDS, 64
+//    columns of K at a time, double-buffered; rows are padded to 72 elements so that the 16
+//    lanes of a quarter-wave read 16 different banks.
 //  * W is the A operand (rows = n), x the B operand: a lane ends up with 4 consecutive n of one
 //    row, stored as one 8-byte write.  Each output is one chain over k in ascending order, so a
 //    row's result does not depend on which other rows share its tile.
-// Limits: K % 128 == 0, N % 4 == 0.
+// Limits: K % 64 == 0, N % 4 == 0.
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
-constexpr int GM = 64;        // rows per tile (the routing kernel lists tiles of this height)
-constexpr int GN = 256;       // columns per tile
-constexpr int GK = 128;       // K per LDS stage
+constexpr int GM = 192;       // rows per tile (the routing kernel lists tiles of this height)
+constexpr int GMT = GM / 16;  // 16-row groups per tile
+constexpr int GW = 4;         // waves per block, 32 weight rows each
+constexpr int GN = 32 * GW;   // columns per tile
+constexpr int GK = 64;        // K per LDS stage
 constexpr int GPAD = GK + 8;  // padded LDS row
+constexpr int GROWS = GW * 8;     // rows staged per pass: 8 threads per 64-wide row
+constexpr int GPASS = GM / GROWS;  // staging passes
 
 template <typename TO>
-__global__ __launch_bounds__(256) void grouped_gemm_kernel(
+__global__ __launch_bounds__(GW* kWave) void grouped_gemm_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ W, TO* __restrict__ out, int N, int K,
     const int* __restrict__ a_rows, const int* __restrict__ group_offsets, const int* __restrict__ tile_expert,
     const int* __restrict__ tile_row0, const int* __restrict__ n_tiles) {
@@ -37,79 +41,93 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(
   const int e = tile_expert[tile];
   const int row0 = tile_row0[tile];
   const int row_end = group_offsets[e + 1];
+  const int n_rows = min(GM, row_end - row0);
+  const int n_mt = (n_rows + 15) >> 4;           // 16-row groups that hold rows
   const int lane = threadIdx.x & (kWave - 1);
   const int w = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
-  const int n_base = blockIdx.y * GN + w * 64;
+  const int n_base = blockIdx.y * GN + w * 32;
   const bf16_t* We = W + (size_t)e * N * K;
 
-  // weight rows of this lane: 4 tiles of 16
-  const bf16_t* wrow[4];
+  const bf16_t* wrow[2];
 #pragma unroll
-  for (int t = 0; t < 4; ++t) {
+  for (int t = 0; t < 2; ++t) {
     int n = n_base + t * 16 + r;
     if (n >= N) n = N - 1;  // loaded, never stored
     wrow[t] = We + (size_t)n * K + g * 8;
   }
-  // staging role: thread loads 16 bytes of row (tid / 16 + 16 * pass), columns (tid % 16) * 8
-  const int srow = threadIdx.x >> 4, scol = (threadIdx.x & 15) * 8;
-  const bf16_t* xsrc[4];
+  // staging role: thread loads 16 bytes of row (tid / 8 + GROWS * pass), columns (tid % 8) * 8
+  const int srow = threadIdx.x >> 3, scol = (threadIdx.x & 7) * 8;
+  const bf16_t* xsrc[GPASS];
 #pragma unroll
-  for (int ps = 0; ps < 4; ++ps) {
-    const int row = row0 + srow + 16 * ps;
+  for (int ps = 0; ps < GPASS; ++ps) {
+    const int row = row0 + srow + GROWS * ps;
     xsrc[ps] = row < row_end ? x + (size_t)(a_rows ? a_rows[row] : row) * K + scol : nullptr;
   }
 
-  f32x4 acc[4][4];
+  f32x4 acc[2][GMT];
 #pragma unroll
-  for (int t = 0; t < 4; ++t)
+  for (int t = 0; t < 2; ++t)
 #pragma unroll
-    for (int mb = 0; mb < 4; ++mb) acc[t][mb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int mb = 0; mb < GMT; ++mb) acc[t][mb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   const int chunks = K / GK;
-  uint4 stage[4];
+  uint4 stage[GPASS];
+  bf16x8 wf[2][2], wnext[2][2];
 #pragma unroll
-  for (int ps = 0; ps < 4; ++ps)
+  for (int ps = 0; ps < GPASS; ++ps)
     stage[ps] = xsrc[ps] ? *reinterpret_cast<const uint4*>(xsrc[ps]) : uint4{0u, 0u, 0u, 0u};
 #pragma unroll
-  for (int ps = 0; ps < 4; ++ps) *reinterpret_cast<uint4*>(&xs[0][srow + 16 * ps][scol]) = stage[ps];
+  for (int j = 0; j < 2; ++j)
+#pragma unroll
+    for (int t = 0; t < 2; ++t) wf[j][t] = *reinterpret_cast<const bf16x8*>(wrow[t] + j * 32);
+#pragma unroll
+  for (int ps = 0; ps < GPASS; ++ps)
+    if (srow + GROWS * ps < n_mt * 16) *reinterpret_cast<uint4*>(&xs[0][srow + GROWS * ps][scol]) = stage[ps];
   __syncthreads();
 
   for (int c = 0; c < chunks; ++c) {
     const int buf = c & 1;
-    const int k0 = c * GK;
-    if (c + 1 < chunks) {
+    const int k1 = (c + 1) * GK;
+    if (c + 1 < chunks) {   // the next stage's x rows and weight rows are on their way while this one is multiplied
 #pragma unroll
-      for (int ps = 0; ps < 4; ++ps)
-        stage[ps] = xsrc[ps] ? *reinterpret_cast<const uint4*>(xsrc[ps] + k0 + GK) : uint4{0u, 0u, 0u, 0u};
+      for (int ps = 0; ps < GPASS; ++ps)
+        stage[ps] = xsrc[ps] ? *reinterpret_cast<const uint4*>(xsrc[ps] + k1) : uint4{0u, 0u, 0u, 0u};
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) wnext[j][t] = *reinterpret_cast<const bf16x8*>(wrow[t] + k1 + j * 32);
     }
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      bf16x8 wf[4], xf[4];
+    for (int j = 0; j < 2; ++j) {
 #pragma unroll
-      for (int t = 0; t < 4; ++t) wf[t] = *reinterpret_cast<const bf16x8*>(wrow[t] + k0 + j * 32);
-#pragma unroll
-      for (int mb = 0; mb < 4; ++mb) xf[mb] = *reinterpret_cast<const bf16x8*>(&xs[buf][mb * 16 + r][j * 32 + g * 8]);
-#pragma unroll
-      for (int t = 0; t < 4; ++t)
-#pragma unroll
-        for (int mb = 0; mb < 4; ++mb)
-          acc[t][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[t], xf[mb], acc[t][mb], 0, 0, 0);
+      for (int mb = 0; mb < GMT; ++mb) {
+        if (mb < n_mt) {   // uniform over the block
+          const bf16x8 xf = *reinterpret_cast<const bf16x8*>(&xs[buf][mb * 16 + r][j * 32 + g * 8]);
+          acc[0][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j][0], xf, acc[0][mb], 0, 0, 0);
+          acc[1][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j][1], xf, acc[1][mb], 0, 0, 0);
+        }
+      }
     }
     if (c + 1 < chunks) {
 #pragma unroll
-      for (int ps = 0; ps < 4; ++ps) *reinterpret_cast<uint4*>(&xs[buf ^ 1][srow + 16 * ps][scol]) = stage[ps];
+      for (int ps = 0; ps < GPASS; ++ps)
+        if (srow + GROWS * ps < n_mt * 16) *reinterpret_cast<uint4*>(&xs[buf ^ 1][srow + GROWS * ps][scol]) = stage[ps];
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) wf[j][t] = wnext[j][t];
     }
     __syncthreads();
   }
 
   // lane holds out[row0 + mb*16 + r][n_base + t*16 + 4g + 0..3]
 #pragma unroll
-  for (int mb = 0; mb < 4; ++mb) {
+  for (int mb = 0; mb < GMT; ++mb) {
     const int row = row0 + mb * 16 + r;
-    if (row >= row_end) continue;
+    if (mb >= n_mt || row >= row_end) continue;
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
+    for (int t = 0; t < 2; ++t) {
       const int n = n_base + t * 16 + 4 * g;
       if (n >= N) continue;
       TO* dst = out + (size_t)row * N + n;
@@ -127,7 +145,7 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(
 
 // x [*, K] bf16 (rows gathered through a_rows if given), W [E, N, K] bf16, out [n_rows, N];
 // group_offsets [E + 1]; tile_expert / tile_row0 [max_tiles], n_tiles [1] from the routing kernel
-// (tiles of 64 rows).  max_tiles >= ceil(n_rows / 64) + E bounds the grid.
+// (tiles of sharpi_gemm_grouped_tile_rows() rows).  max_tiles bounds the grid.
 SHARPI_EXPORT int sharpi_gemm_grouped(const void* x, const void* W, void* out, int out_dtype, int n_rows, int N,
                                       int K, const int* a_rows, const int* group_offsets, const int* tile_expert,
                                       const int* tile_row0, const int* n_tiles, int max_tiles,
@@ -136,7 +154,7 @@ SHARPI_EXPORT int sharpi_gemm_grouped(const void* x, const void* W, void* out, i
   if (N <= 0 || (N & 3) || K <= 0 || K % GK != 0 || max_tiles <= 0) return SHARPI_ERR_ARG;
   if (!group_offsets || !tile_expert || !tile_row0 || !n_tiles) return SHARPI_ERR_ARG;
   if (ceil_div(N, GN) > 65535) return SHARPI_ERR_ARG;
-  dim3 grid(max_tiles, ceil_div(N, GN)), block(256);
+  dim3 grid(max_tiles, ceil_div(N, GN)), block(GW * kWave);
   if (out_dtype == DT_BF16)
     grouped_gemm_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)x, (const bf16_t*)W, (bf16_t*)out, N, K,
                                                            a_rows, group_offsets, tile_expert, tile_row0, n_tiles);

@@ -96,6 +96,76 @@ __global__ void rope_kv_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
   }
 }
 
+// The same for head sizes 32, 64, 128, 256: one block per token, a thread per run of 8 elements
+// (4 rotary pairs), 16-byte accesses; the hd/8 lanes of a head are neighbours in a wave and sum
+// their squares with shuffles.
+template <typename T>
+__global__ __launch_bounds__(256) void rope_kv_vec_kernel(
+    const T* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
+    const int* __restrict__ slot_mapping, const int* __restrict__ positions, const float* __restrict__ inv_freq,
+    int qk_norm, float eps, int temp_tuning, float floor_scale, float attn_scale, int nh, int nkv, int hd,
+    int page_size) {
+  const int t = blockIdx.x;
+  const int per_head = hd >> 3;                    // lanes per head: 4, 8, 16 or 32
+  const int chunks = (nh + 2 * nkv) * per_head;
+  const int pos = positions[t];
+  const int slot = slot_mapping[t];
+  const T* src = qkv + (size_t)t * (nh + 2 * nkv) * hd;
+  float post = 1.0f;
+  if (temp_tuning) post = 1.0f + attn_scale * logf(floorf(((float)pos + 1.0f) / floor_scale) + 1.0f);
+  for (int base = 0; base < chunks; base += blockDim.x) {
+    const int ci = base + threadIdx.x;
+    const bool valid = ci < chunks;
+    const int head = valid ? ci / per_head : 0;
+    const int run = valid ? ci % per_head : 0;
+    const bool is_q = head < nh;
+    const bool is_k = !is_q && head < nh + nkv;
+    float x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (valid) load8(src + (size_t)head * hd + run * 8, x);
+    float ss = 0.f;
+    if (valid && (is_q || is_k)) {
+      if (inv_freq) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float ang = (float)pos * inv_freq[run * 4 + j];
+          const float c = cosf(ang), sn = sinf(ang);
+          const float a = x[2 * j], b = x[2 * j + 1];
+          x[2 * j] = a * c - b * sn;
+          x[2 * j + 1] = a * sn + b * c;
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ss += x[j] * x[j];
+    }
+    if (qk_norm) {   // every lane takes part in the shuffles
+      for (int off = per_head >> 1; off > 0; off >>= 1) ss += __shfl_xor(ss, off, kWave);
+      const float mul = 1.0f / sqrtf(ss / (float)hd + eps);
+      if (is_q || is_k) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) x[j] *= mul;
+      }
+    }
+    if (!valid) continue;
+    if (is_q) {
+      if (temp_tuning) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) x[j] *= post;
+      }
+      store8(q_out + ((size_t)t * nh + head) * hd + run * 8, x);
+    } else if (slot >= 0) {
+      const size_t page = (size_t)(slot / page_size);
+      const int off = slot % page_size;
+      if (is_k) {
+        store8(k_cache + ((page * nkv + (head - nh)) * page_size + off) * hd + run * 8, x);
+      } else {
+        T* dst = v_cache + (page * nkv + (head - nh - nkv)) * hd * page_size + off;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) dst[(size_t)(run * 8 + j) * page_size] = from_f32<T>(x[j]);
+      }
+    }
+  }
+}
+
 SHARPI_EXPORT int sharpi_rope_kv(const void* qkv, void* q_out, void* k_cache, void* v_cache, int dtype,
                                  const int* slot_mapping, const int* positions, const float* inv_freq,
                                  int qk_norm, float eps, int temp_tuning, float floor_scale, float attn_scale,
@@ -105,6 +175,21 @@ SHARPI_EXPORT int sharpi_rope_kv(const void* qkv, void* q_out, void* k_cache, vo
   if (nh + 2 * nkv > 65535) return SHARPI_ERR_ARG;
   if (temp_tuning && !(floor_scale > 0.f)) return SHARPI_ERR_ARG;
   dim3 grid(n_tokens, nh + 2 * nkv), block(kWave);
+  if (dtype != DT_F32 && dtype != DT_BF16) return SHARPI_ERR_ARG;
+  if (hd == 32 || hd == 64 || hd == 128 || hd == 256) {
+    if (dtype == DT_F32)
+      rope_kv_vec_kernel<float><<<n_tokens, 256, 0, stream>>>((const float*)qkv, (float*)q_out, (float*)k_cache,
+                                                             (float*)v_cache, slot_mapping, positions, inv_freq,
+                                                             qk_norm, eps, temp_tuning, floor_scale, attn_scale,
+                                                             nh, nkv, hd, page_size);
+    else
+      rope_kv_vec_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>((const bf16_t*)qkv, (bf16_t*)q_out,
+                                                              (bf16_t*)k_cache, (bf16_t*)v_cache, slot_mapping,
+                                                              positions, inv_freq, qk_norm, eps, temp_tuning,
+                                                              floor_scale, attn_scale, nh, nkv, hd, page_size);
+    SHARPI_CHECK_LAUNCH();
+    return SHARPI_OK;
+  }
   if (dtype == DT_F32)
     rope_kv_kernel<float><<<grid, block, 0, stream>>>((const float*)qkv, (float*)q_out, (float*)k_cache,
                                                      (float*)v_cache, slot_mapping, positions, inv_freq, qk_norm,

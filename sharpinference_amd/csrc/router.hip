@@ -14,20 +14,6 @@
 
 constexpr int kMaxExperts = 1024;
 
-// eight consecutive elements as floats
-__device__ __forceinline__ void load8(const float* p, float* v) {
-  const float4 a = *reinterpret_cast<const float4*>(p);
-  const float4 b = *reinterpret_cast<const float4*>(p + 4);
-  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
-}
-__device__ __forceinline__ void load8(const bf16_t* p, float* v) {
-  const uint4 a = *reinterpret_cast<const uint4*>(p);
-  v[0] = bf16_bits_to_f32(a.x & 0xffffu); v[1] = bf16_bits_to_f32(a.x >> 16);
-  v[2] = bf16_bits_to_f32(a.y & 0xffffu); v[3] = bf16_bits_to_f32(a.y >> 16);
-  v[4] = bf16_bits_to_f32(a.z & 0xffffu); v[5] = bf16_bits_to_f32(a.z >> 16);
-  v[6] = bf16_bits_to_f32(a.w & 0xffffu); v[7] = bf16_bits_to_f32(a.w >> 16);
-}
-
 template <typename T, typename TW>
 __global__ __launch_bounds__(1024) void router_topk_kernel(const T* __restrict__ x, const TW* __restrict__ wr,
                                                            int* __restrict__ topk_ids,

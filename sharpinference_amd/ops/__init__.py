@@ -372,7 +372,7 @@ def router_topk(x: torch.Tensor, wr: torch.Tensor, k: int, gate: int = GATE_SIGM
     return (ids, wts, gates) if want_gates else (ids, wts)
 
 
-GROUPED_TILE_ROWS = 64
+GROUPED_TILE_ROWS = 192   # rows per tile of the grouped product (csrc/gemm_grouped.hip GM)
 
 
 class Routing:
@@ -388,7 +388,7 @@ class Routing:
 
 def moe_permute(ids: torch.Tensor, wts: torch.Tensor, n_experts: int) -> Routing:
     """(token, pick) pairs sorted by expert: offsets [E+1], sorted_token, sorted_w, inv_pos, and
-    the list of 64-row tiles of the experts that have rows."""
+    the list of row tiles (GROUPED_TILE_ROWS high) of the experts that have rows."""
     _dev(ids, wts)
     _i32(ids, "ids")
     _need(ids.shape == wts.shape and wts.dtype == torch.float32 and ids.dim() == 2, "moe_permute: ids/wts [T, k]")
@@ -420,7 +420,7 @@ def gemm_grouped(x: torch.Tensor, w: torch.Tensor, rt: Routing, gather: bool, ou
     _need(w.dim() == 3 and w.shape[0] == rt.n_experts and x.dim() == 2 and x.shape[1] == w.shape[2],
           f"gemm_grouped: x {tuple(x.shape)} vs w {tuple(w.shape)}")
     E, N, K = w.shape
-    _need(K % 128 == 0 and N % 4 == 0, "gemm_grouped: K % 128 == 0 and N % 4 == 0 wanted")
+    _need(K % 64 == 0 and N % 4 == 0, "gemm_grouped: K % 64 == 0 and N % 4 == 0 wanted")
     _need(x.shape[0] == (rt.n_tokens if gather else rt.n_rows), "gemm_grouped: x has the wrong number of rows")
     out = torch.empty(rt.n_rows, N, dtype=out_dtype, device=x.device)
     _run("sharpi_gemm_grouped", _ptr(x), _ptr(w), _ptr(out), _code(out_dtype), rt.n_rows, N, K,
