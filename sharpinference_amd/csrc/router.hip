@@ -9,7 +9,9 @@
 // moe_permute: one block. Counts rows per expert, prefix-sums them into offsets[E + 1] and
 // writes, in expert order, the token and weight of every (token, pick) pair plus the inverse
 // map inv_pos[t * k + j] = row in that order, and the list of (expert, first row) tiles of
-// tile_rows rows that the grouped product of many rows walks.
+// tile_rows rows that the grouped product of many rows walks.  With shared_group the list gets one
+// more group after the experts: every token once, weight 1 (an always-on expert that shares the
+// experts' weight tensor); offsets then has n_experts + 2 entries and the row arrays n_tokens more.
 #include "common.h"
 
 constexpr int kMaxExperts = 1024;
@@ -112,7 +114,8 @@ __global__ __launch_bounds__(1024) void moe_permute_kernel(const int* __restrict
                                                            int* __restrict__ tile_expert,
                                                            int* __restrict__ tile_row0,
                                                            int* __restrict__ n_tiles, int n_pairs, int k,
-                                                           int n_experts, int tile_rows, int max_tiles) {
+                                                           int n_experts, int tile_rows, int max_tiles,
+                                                           int shared_group) {
   __shared__ int count[kMaxExperts];
   __shared__ int cursor[kMaxExperts];
   for (int e = threadIdx.x; e < n_experts; e += blockDim.x) count[e] = 0;
@@ -138,6 +141,14 @@ __global__ __launch_bounds__(1024) void moe_permute_kernel(const int* __restrict
         }
       }
     n_tiles[0] = nt;
+    // an always-on expert as one more group: every token once, in token order, with weight 1
+    if (shared_group) offsets[n_experts + 1] = run + n_pairs / k;
+  }
+  if (shared_group) {
+    for (int t = threadIdx.x; t < n_pairs / k; t += blockDim.x) {
+      sorted_token[n_pairs + t] = t;
+      sorted_w[n_pairs + t] = 1.0f;
+    }
   }
   __syncthreads();
   for (int i = threadIdx.x; i < n_pairs; i += blockDim.x) {
@@ -152,13 +163,13 @@ __global__ __launch_bounds__(1024) void moe_permute_kernel(const int* __restrict
 SHARPI_EXPORT int sharpi_moe_permute(const int* topk_ids, const float* topk_w, int* offsets, int* sorted_token,
                                      float* sorted_w, int* inv_pos, int* tile_expert, int* tile_row0,
                                      int* n_tiles, int n_tokens, int k, int n_experts, int tile_rows,
-                                     int max_tiles, hipStream_t stream) {
+                                     int max_tiles, int shared_group, hipStream_t stream) {
   if (n_experts <= 0 || n_experts > kMaxExperts || k <= 0) return SHARPI_ERR_ARG;
   if (n_tokens < 0 || tile_rows <= 0) return SHARPI_ERR_ARG;
   if (max_tiles < (n_tokens * k + tile_rows - 1) / tile_rows + n_experts) return SHARPI_ERR_ARG;
   moe_permute_kernel<<<1, 1024, 0, stream>>>(topk_ids, topk_w, offsets, sorted_token, sorted_w, inv_pos,
                                              tile_expert, tile_row0, n_tiles, n_tokens * k, k, n_experts,
-                                             tile_rows, max_tiles);
+                                             tile_rows, max_tiles, shared_group);
   SHARPI_CHECK_LAUNCH();
   return SHARPI_OK;
 }

@@ -292,8 +292,9 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, a_rows
     _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_skinny: bfloat16 operands only")
     grouped = offsets is not None
     if grouped:
-        _need(w.dim() == 3 and offsets.shape == (w.shape[0] + 1,), "gemm_skinny: grouped needs w [E, N, K], offsets [E+1]")
-        E, N, K = w.shape
+        _need(w.dim() == 3 and 2 <= offsets.shape[0] <= w.shape[0] + 1,
+              "gemm_skinny: grouped needs w [E, N, K] and offsets of at most E + 1 entries")
+        E, N, K = offsets.shape[0] - 1, w.shape[1], w.shape[2]
         M = int(n_rows)
         if a_rows is not None:
             _need(a_rows.shape == (M,), "gemm_skinny: a_rows must be [n_rows]")
@@ -340,8 +341,9 @@ def grouped_gemm(x: torch.Tensor, w: torch.Tensor, offsets: torch.Tensor, a_rows
     _i32(a_rows, "a_rows")
     _need(w.dim() == 3 and x.dim() == 2 and x.shape[1] == w.shape[2] and x.dtype == w.dtype,
           f"grouped_gemm: x {tuple(x.shape)} vs w {tuple(w.shape)}")
-    E, N, K = w.shape
-    _need(offsets.shape == (E + 1,), "grouped_gemm: offsets must be [E + 1]")
+    N, K = w.shape[1], w.shape[2]
+    E = offsets.shape[0] - 1          # the weight may hold more experts than the routing has groups
+    _need(1 <= E <= w.shape[0], "grouped_gemm: offsets must have at most E + 1 entries")
     if a_rows is not None:
         _need(a_rows.shape == (n_rows,), "grouped_gemm: a_rows must be [n_rows]")
     else:
@@ -378,17 +380,19 @@ GROUPED_TILE_ROWS = 192   # rows per tile of the grouped product (csrc/gemm_grou
 class Routing:
     """The expert-sorted view of a step's (token, pick) pairs, all on the device."""
 
-    __slots__ = ("n_tokens", "k", "n_experts", "offsets", "sorted_token", "sorted_w", "inv_pos", "tile_expert",
-                 "tile_row0", "n_tiles", "max_tiles")
+    __slots__ = ("n_tokens", "k", "n_experts", "n_groups", "offsets", "sorted_token", "sorted_w", "inv_pos",
+                 "tile_expert", "tile_row0", "n_tiles", "max_tiles")
 
     @property
     def n_rows(self) -> int:
-        return self.n_tokens * self.k
+        """Rows of the sorted list: one per (token, pick), plus one per token for a shared group."""
+        return self.n_tokens * self.k + (self.n_tokens if self.n_groups > self.n_experts else 0)
 
 
-def moe_permute(ids: torch.Tensor, wts: torch.Tensor, n_experts: int) -> Routing:
+def moe_permute(ids: torch.Tensor, wts: torch.Tensor, n_experts: int, shared_group: bool = False) -> Routing:
     """(token, pick) pairs sorted by expert: offsets [E+1], sorted_token, sorted_w, inv_pos, and
-    the list of row tiles (GROUPED_TILE_ROWS high) of the experts that have rows."""
+    the list of row tiles (GROUPED_TILE_ROWS high) of the experts that have rows.  With
+    shared_group one more group follows the experts: every token once with weight 1."""
     _dev(ids, wts)
     _i32(ids, "ids")
     _need(ids.shape == wts.shape and wts.dtype == torch.float32 and ids.dim() == 2, "moe_permute: ids/wts [T, k]")
@@ -396,19 +400,21 @@ def moe_permute(ids: torch.Tensor, wts: torch.Tensor, n_experts: int) -> Routing
     dev = ids.device
     rt = Routing()
     rt.n_tokens, rt.k, rt.n_experts = T, k, n_experts
+    rt.n_groups = n_experts + (1 if shared_group else 0)
+    rows = T * k + (T if shared_group else 0)
     rt.max_tiles = (T * k + GROUPED_TILE_ROWS - 1) // GROUPED_TILE_ROWS + n_experts
-    ints = torch.empty(n_experts + 1 + 2 * T * k + 2 * rt.max_tiles + 1, dtype=torch.int32, device=dev)
+    ints = torch.empty(rt.n_groups + 1 + rows + T * k + 2 * rt.max_tiles + 1, dtype=torch.int32, device=dev)
     o = 0
-    rt.offsets = ints[o:o + n_experts + 1]; o += n_experts + 1
-    rt.sorted_token = ints[o:o + T * k]; o += T * k
+    rt.offsets = ints[o:o + rt.n_groups + 1]; o += rt.n_groups + 1
+    rt.sorted_token = ints[o:o + rows]; o += rows
     rt.inv_pos = ints[o:o + T * k]; o += T * k
     rt.tile_expert = ints[o:o + rt.max_tiles]; o += rt.max_tiles
     rt.tile_row0 = ints[o:o + rt.max_tiles]; o += rt.max_tiles
     rt.n_tiles = ints[o:o + 1]
-    rt.sorted_w = torch.empty(T * k, dtype=torch.float32, device=dev)
+    rt.sorted_w = torch.empty(rows, dtype=torch.float32, device=dev)
     _run("sharpi_moe_permute", _ptr(ids), _ptr(wts), _ptr(rt.offsets), _ptr(rt.sorted_token), _ptr(rt.sorted_w),
          _ptr(rt.inv_pos), _ptr(rt.tile_expert), _ptr(rt.tile_row0), _ptr(rt.n_tiles), T, k, n_experts,
-         GROUPED_TILE_ROWS, rt.max_tiles, _stream())
+         GROUPED_TILE_ROWS, rt.max_tiles, 1 if shared_group else 0, _stream())
     return rt
 
 
@@ -417,8 +423,8 @@ def gemm_grouped(x: torch.Tensor, w: torch.Tensor, rt: Routing, gather: bool, ou
     through the routing's token list; otherwise x is already in expert-sorted order."""
     _dev(x, w)
     _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_grouped: bfloat16 operands only")
-    _need(w.dim() == 3 and w.shape[0] == rt.n_experts and x.dim() == 2 and x.shape[1] == w.shape[2],
-          f"gemm_grouped: x {tuple(x.shape)} vs w {tuple(w.shape)}")
+    _need(w.dim() == 3 and w.shape[0] >= rt.n_experts and rt.n_groups == rt.n_experts and x.dim() == 2
+          and x.shape[1] == w.shape[2], f"gemm_grouped: x {tuple(x.shape)} vs w {tuple(w.shape)}")
     E, N, K = w.shape
     _need(K % 64 == 0 and N % 4 == 0, "gemm_grouped: K % 64 == 0 and N % 4 == 0 wanted")
     _need(x.shape[0] == (rt.n_tokens if gather else rt.n_rows), "gemm_grouped: x has the wrong number of rows")

@@ -59,6 +59,8 @@ class MoESwiGLU(Part):
     (2060-2066); the outputs are summed (2096-2097).  ``gate`` is "sigmoid" or "softmax"
     (2031-2034); ``renormalise`` divides the k scores by their sum (2156-2162)."""
 
+    MERGE_MAX_TOKENS = 16   # one row block of the few-rows kernel for the shared group
+
     def __init__(self, hidden: int, num_experts: int, top_k: int, expert_intermediate: int,
                  shared_intermediate: Optional[int] = None, gate: str = "sigmoid", renormalise: bool = False,
                  score_on_input: bool = True):
@@ -95,8 +97,23 @@ class MoESwiGLU(Part):
         self.w_gate_up = _fuse_rows(g, u)
         del g, u
         self.w_down = source.get(prefix + "experts.down_proj")
+        self.merged = False
         if self.shared is not None:
             self.shared.load(prefix + "shared_expert.", source)
+            sh = self.shared
+            if (sh.inter == self.inter and sh.w_gate_up.dtype == self.w_gate_up.dtype == torch.bfloat16
+                    and sh.w_down.dtype == self.w_down.dtype == torch.bfloat16):
+                # The shared expert becomes expert E of the experts' tensors (its own tensors turn
+                # into views of them): few-row steps then run it in the same launches as the routed ones.
+                gu = torch.empty(self.E + 1, 2 * self.inter, self.hidden, dtype=torch.bfloat16, device=self.w_gate_up.device)
+                gu[:self.E].copy_(self.w_gate_up)
+                gu[self.E].copy_(sh.w_gate_up)
+                self.w_gate_up, sh.w_gate_up = gu, gu[self.E]
+                dn = torch.empty(self.E + 1, self.hidden, self.inter, dtype=torch.bfloat16, device=self.w_down.device)
+                dn[:self.E].copy_(self.w_down)
+                dn[self.E].copy_(sh.w_down)
+                self.w_down, sh.w_down = dn, dn[self.E]
+                self.merged = True
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         T = x.shape[0]
@@ -104,6 +121,13 @@ class MoESwiGLU(Part):
         trace = ctx.extras.get("router_trace")
         if trace is not None:      # the picks of this step, layer by layer (reference: ForwardPass.cs:2042-2056)
             trace.append((ids, wts))
+        if self.merged and T <= self.MERGE_MAX_TOKENS and ctx.act_dtype == torch.bfloat16:
+            # few rows: the shared expert rides along as one more group of the same two launches
+            rt = ops.moe_permute(ids, wts, self.E, shared_group=True)
+            gu = ops.grouped_linear(x, self.w_gate_up, rt, True, ctx.act_dtype)
+            act = ops.silu_mul(gu, rt.sorted_w)
+            y = ops.grouped_linear(act, self.w_down, rt, False, ctx.act_dtype)
+            return ops.moe_combine(y[:T * self.k], rt.inv_pos, y[T * self.k:], T, self.k)
         rt = ops.moe_permute(ids, wts, self.E)
         shared = self.shared.forward(x, ctx) if self.shared is not None else None
         gu = ops.grouped_linear(x, self.w_gate_up, rt, True, ctx.act_dtype)
