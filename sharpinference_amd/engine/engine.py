@@ -55,7 +55,8 @@ class Engine:
                  weight_seed: Optional[int] = None, dtype="bfloat16", device="cuda:0",
                  max_model_len: Optional[int] = None, max_num_seqs: int = 8, max_tokens_per_step: int = 2048,
                  kv_tokens: Optional[int] = None, page_size: int = 16, weight_std: float = 0.02,
-                 weight_std_by_suffix: Optional[Dict[str, float]] = None, verbose: bool = False):
+                 weight_std_by_suffix: Optional[Dict[str, float]] = None, verbose: bool = False,
+                 decode_graphs: bool = True):
         self.dtype = parse_dtype(dtype)
         self.device = torch.device(device)
         if self.device.type != "cuda":
@@ -100,7 +101,8 @@ class Engine:
         num_pages = max(1, (int(kv_tokens) + page_size - 1) // page_size)
         self.cache = CacheManager(self.model.cache_specs(), page_size, num_pages, self.max_num_seqs, self.dtype,
                                   self.device)
-        self.runner = ModelRunner(self.model, self.cache, self.dtype, self.device)
+        self.runner = ModelRunner(self.model, self.cache, self.dtype, self.device, decode_graphs=decode_graphs,
+                                  max_context=self.max_model_len)
         self.sampler = Sampler(self.device)
         self.last_stats = GenerationStats()
 

@@ -20,6 +20,7 @@ from ..cache.manager import CacheError, CacheManager
 from ..parts.base import GroupView, LayerCache, StepContext
 
 
+MAX_GRAPH_BATCH = 64   # decode steps of up to this many requests are replayed from a HIP graph
 TILE = 32   # tokens per attention tile of multi-token entries (ops.PREFILL_TILE_TOKENS)
 
 
@@ -35,12 +36,20 @@ class StepEntry:
 
 
 class ModelRunner:
-    def __init__(self, model, cache: CacheManager, act_dtype: torch.dtype, device):
+    def __init__(self, model, cache: CacheManager, act_dtype: torch.dtype, device, decode_graphs: bool = False,
+                 max_context: int = 0):
         self.model = model
         self.cache = cache
         self.act_dtype = act_dtype
         self.device = torch.device(device)
         self.steps_run = 0
+        # Steps made of single decoded tokens only are launch-bound: they are captured once per
+        # batch size into a HIP graph over fixed index buffers and replayed.
+        # (not for mixers with state of their own: the capture's trial run would advance it)
+        self.decode_graphs = bool(decode_graphs) and max_context > 0 and all(t is None for t in cache.state)
+        self.max_context = int(max_context)
+        self._graphs: dict = {}
+        self.graph_replays = 0
 
     # ------------------------------------------------------------------
     def _validate(self, entries: Sequence[StepEntry]) -> None:
@@ -61,8 +70,9 @@ class ModelRunner:
                 if not 0 <= int(w) < len(e.tokens):
                     raise ValueError(f"request {e.req_id!r}: wanted place {w} outside its {len(e.tokens)} tokens")
 
-    def build_context(self, entries: Sequence[StepEntry]):
-        """Host side of a step: lay the batch out flat and pack all index arrays into one upload."""
+    def _host_arrays(self, entries: Sequence[StepEntry], static_blocks: Optional[int] = None):
+        """Host side of a step: lay the batch out flat.  Returns the index arrays in upload order
+        and what the context needs to know about them."""
         cache = self.cache
         ps = cache.page_size
         n = len(entries)
@@ -87,8 +97,11 @@ class ModelRunner:
         group_tables, group_slots = [], []
         for g in range(len(cache.groups)):
             tables = [cache.block_table(e.req_id, g) for e in entries]
-            maxb = max(1, max(len(t) for t in tables))
-            maxb = (maxb + 3) // 4 * 4
+            if static_blocks is not None:
+                maxb = static_blocks
+            else:
+                maxb = max(1, max(len(t) for t in tables))
+                maxb = (maxb + 3) // 4 * 4
             bt = np.full((n, maxb), -1, dtype=np.int32)
             for i, t in enumerate(tables):
                 bt[i, :len(t)] = t
@@ -112,24 +125,37 @@ class ModelRunner:
                   dec_np, tiles_np]
         for bt, sm in zip(group_tables, group_slots):
             pieces += [bt.reshape(-1), sm]
-        flat = np.concatenate(pieces) if pieces else np.zeros(0, dtype=np.int32)
-        dev = torch.from_numpy(flat).to(self.device)
+        info = dict(n=n, T=T, lens=lens, starts=starts, n_rows=len(rows), n_dec=len(dec), n_tiles=len(tiles),
+                    max_blocks=[bt.shape[1] for bt in group_tables],
+                    max_context=int(positions.max()) + 1 if T else 0)
+        return pieces, info
+
+    def _context_from(self, dev: torch.Tensor, sizes: Sequence[int], info: dict):
+        """The step's context over one device tensor that holds the index arrays back to back."""
         views, off = [], 0
-        for p in pieces:
-            views.append(dev[off:off + p.size])
-            off += p.size
+        for size in sizes:
+            views.append(dev[off:off + size])
+            off += size
         d_tok, d_pos, d_ent, d_cu, d_state, d_nostore, d_rows, d_dec, d_tiles = views[:9]
+        n, T = info["n"], info["T"]
         groups = []
-        for g in range(len(cache.groups)):
-            bt = views[9 + 2 * g].view(n, group_tables[g].shape[1])
-            groups.append(GroupView(bt, views[10 + 2 * g], ps, max_context=int(positions.max()) + 1 if T else 0))
+        for g in range(len(self.cache.groups)):
+            bt = views[9 + 2 * g].view(n, info["max_blocks"][g])
+            groups.append(GroupView(bt, views[10 + 2 * g], self.cache.page_size, max_context=info["max_context"]))
         ctx = StepContext(n_tokens=T, n_entries=n, token_ids=d_tok, positions=d_pos, entry_of_token=d_ent,
                           cu_tokens=d_cu, state_slots=d_state, groups=groups, act_dtype=self.act_dtype,
-                          no_store_slots=d_nostore, entry_lens=lens, entry_starts=starts,
-                          max_entry_len=max(lens) if lens else 1, n_decode=len(dec),
-                          decode_tokens=None if len(dec) == T else d_dec, n_prefill_tiles=len(tiles),
-                          prefill_tiles=d_tiles.view(-1, 3) if tiles else None)
-        return ctx, (d_rows if rows else None)
+                          no_store_slots=d_nostore, entry_lens=info["lens"], entry_starts=info["starts"],
+                          max_entry_len=max(info["lens"]) if info["lens"] else 1, n_decode=info["n_dec"],
+                          decode_tokens=None if info["n_dec"] == T else d_dec, n_prefill_tiles=info["n_tiles"],
+                          prefill_tiles=d_tiles.view(-1, 3) if info["n_tiles"] else None)
+        return ctx, (d_rows if info["n_rows"] else None)
+
+    def build_context(self, entries: Sequence[StepEntry]):
+        """Index arrays of a step packed into ONE upload, and the context over them."""
+        pieces, info = self._host_arrays(entries)
+        flat = np.concatenate(pieces) if pieces else np.zeros(0, dtype=np.int32)
+        dev = torch.from_numpy(flat).to(self.device)
+        return self._context_from(dev, [p.size for p in pieces], info)
 
     def layer_caches(self, ctx: StepContext) -> List[LayerCache]:
         cache = self.cache
@@ -141,6 +167,34 @@ class ModelRunner:
         return out
 
     # ------------------------------------------------------------------
+    def _decode_graph_step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        """Replay the captured graph of this batch size if the step qualifies: every entry one
+        token whose logits are wanted, all contexts within the captured bound.  None otherwise."""
+        n = len(entries)
+        if not self.decode_graphs or n > MAX_GRAPH_BATCH:
+            return None
+        for e in entries:
+            if len(e.tokens) != 1 or len(e.want) != 1 or int(e.want[0]) != 0:
+                return None
+            if self.cache.length(e.req_id) + 1 > self.max_context:
+                return None
+        graph = self._graphs.get(n)
+        if graph is False:
+            return None
+        static_blocks = (self.max_context + self.cache.page_size - 1) // self.cache.page_size
+        pieces, info = self._host_arrays(entries, static_blocks=static_blocks)
+        if graph is None:
+            try:
+                graph = _DecodeGraph(self, pieces, info)
+            except Exception as e:  # noqa: BLE001 - capture is an optimisation: report once, go on eagerly
+                print(f"[sharpi] decode graph for batch {n} not captured ({type(e).__name__}: {e}); running eagerly",
+                      flush=True)
+                self._graphs[n] = False
+                return None
+            self._graphs[n] = graph
+        self.graph_replays += 1
+        return graph.replay(pieces)
+
     def step(self, entries: Sequence[StepEntry], router_trace: Optional[list] = None) -> Optional[torch.Tensor]:
         """Run one batch.  Returns float32 logits [wanted, vocab] in the order of the entries and
         of their ``want`` lists, or None when nothing is wanted.  A list given as ``router_trace``
@@ -155,10 +209,12 @@ class ModelRunner:
                 if not self.cache.append(e.req_id, len(e.tokens)):
                     raise CacheExhausted(f"no pages left for request {e.req_id!r} ({len(e.tokens)} more tokens)")
                 appended.append(e.req_id)
-            ctx, rows = self.build_context(entries)
-            if router_trace is not None:
-                ctx.extras["router_trace"] = router_trace
-            logits = self.model.forward(ctx, self.layer_caches(ctx), rows)
+            logits = self._decode_graph_step(entries) if router_trace is None else None
+            if logits is None:
+                ctx, rows = self.build_context(entries)
+                if router_trace is not None:
+                    ctx.extras["router_trace"] = router_trace
+                logits = self.model.forward(ctx, self.layer_caches(ctx), rows)
         except BaseException:
             for r in appended:
                 self.cache.rollback(r)
@@ -167,3 +223,60 @@ class ModelRunner:
             self.cache.commit(e.req_id)
         self.steps_run += 1
         return logits
+
+
+class _DecodeGraph:
+    """One captured decode step of a fixed batch size over fixed index buffers.
+
+    The index arrays of a step are written into a pinned host buffer, copied into the device
+    buffer the graph was captured over, and the graph is replayed; shapes that vary from step to
+    step (block table width, context bound of the decode kernel) are fixed at their maxima.
+    The logits tensor belongs to the graph: the caller gets a copy."""
+
+    def __init__(self, runner: ModelRunner, pieces, info: dict):
+        self.runner = runner
+        self.sizes = [p.size for p in pieces]
+        total = sum(self.sizes)
+        self.host = torch.empty(total, dtype=torch.int32).pin_memory()
+        self.host_np = self.host.numpy()
+        self.dev = torch.empty(total, dtype=torch.int32, device=runner.device)
+        self.copied = torch.cuda.Event()
+        info = dict(info, max_context=runner.max_context)
+        # capture over harmless contents: nothing is stored (slots -1) and no key is visible (tables -1)
+        null = [np.zeros_like(p) for p in pieces]
+        n = info["n"]
+        null[2] = np.arange(n, dtype=np.int32)            # entry of token
+        null[3] = np.arange(n + 1, dtype=np.int32)        # cu_tokens
+        null[4] = pieces[4]                               # state slots (any valid slot)
+        null[5] = np.full(n, -1, dtype=np.int32)
+        null[6] = np.arange(n, dtype=np.int32)            # logit rows
+        null[7] = np.arange(n, dtype=np.int32)
+        for i in range(9, len(null)):
+            null[i] = np.full_like(pieces[i], -1)
+        self._upload(null)
+        ctx, rows = runner._context_from(self.dev, self.sizes, info)
+        caches = runner.layer_caches(ctx)
+        side = torch.cuda.Stream(device=runner.device)
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):                     # once eagerly: libraries initialise outside the capture
+            runner.model.forward(ctx, caches, rows)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self.logits = runner.model.forward(ctx, caches, rows)
+
+    def _upload(self, pieces) -> None:
+        self.copied.synchronize()                         # the previous copy has left the pinned buffer
+        off = 0
+        for p, size in zip(pieces, self.sizes):
+            assert p.size == size
+            self.host_np[off:off + size] = p.reshape(-1)
+            off += size
+        self.dev.copy_(self.host, non_blocking=True)
+        self.copied.record()
+
+    def replay(self, pieces) -> torch.Tensor:
+        self._upload(pieces)
+        self.graph.replay()
+        return self.logits.clone()
