@@ -238,3 +238,112 @@ def test_attention_prefill_kernel(nh, nkv, hd, kind, window, ps):
     got = got.float().cpu().view(T, nh, hd)
     err = (got - ref).abs().max(dim=-1).values.max(dim=-1).values
     assert float(err.max()) <= 2e-2, (float(err.max()), int(err.argmax()))
+
+
+# ---------------------------------------------------------------------------
+# row kernels, at widths with and without 16-byte runs
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("H", [80, 203, 1000, 5120, 9000])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_add_rmsnorm_kernel(H, dtype):
+    ops = _ops()
+    T = 7
+    h = _rand(T, H, seed=1)
+    delta = _rand(T, H, dtype=dtype, seed=2)
+    w = (torch.rand(H) + 0.5).to(DEV)
+    want_sum = h + delta.float()
+    want = want_sum * torch.rsqrt(want_sum.pow(2).mean(-1, keepdim=True) + 1e-5) * w
+    tol = 1e-5 if dtype == torch.float32 else 1e-2
+    for wt in (w, w.to(torch.bfloat16)):
+        hh = h.clone()
+        out = ops.add_rmsnorm(hh, delta, wt, 1e-5, dtype)
+        ref = want if wt.dtype == torch.float32 else want / w * wt.float()
+        assert float((out.float() - ref).abs().max()) <= tol * float(ref.abs().max())
+        assert torch.allclose(hh, want_sum, atol=1e-6)               # the sum went back into the stream
+    hh = h.clone()
+    rows = torch.tensor([5, 0, 5], dtype=torch.int32, device=DEV)
+    out = ops.add_rmsnorm(hh, delta, None, 1e-5, dtype, rows=rows)
+    assert torch.equal(hh, h)                                        # gathered rows leave the stream alone
+    assert float((out.float() - (want / w)[[5, 0, 5]]).abs().max()) <= tol * float(want.abs().max())
+    plain = ops.add_rmsnorm(h.clone(), None, w, 1e-5, torch.float32)
+    assert torch.allclose(plain, h * torch.rsqrt(h.pow(2).mean(-1, keepdim=True) + 1e-5) * w, atol=1e-5)
+
+
+@pytest.mark.parametrize("I", [48, 77, 8192])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_silu_mul_and_combine_and_embed(I, dtype):
+    ops = _ops()
+    M = 9
+    gu = _rand(M, 2 * I, dtype=dtype, seed=3)
+    scale = torch.rand(M).to(DEV) + 0.2
+    g, u = gu.float()[:, :I], gu.float()[:, I:]
+    tol = 1e-5 if dtype == torch.float32 else 1e-2
+    got = ops.silu_mul(gu).float()
+    assert float((got - torch.nn.functional.silu(g) * u).abs().max()) <= tol * 4
+    got = ops.silu_mul(gu, scale).float()
+    gs, us = g * scale[:, None], u * scale[:, None]
+    assert float((got - torch.nn.functional.silu(gs) * us).abs().max()) <= tol * 4
+    # combine: 3 tokens, 2 picks each, plus a shared row
+    y = _rand(6, I, dtype=dtype, seed=4)
+    sh = _rand(3, I, dtype=dtype, seed=5)
+    inv = torch.tensor([4, 1, 0, 5, 2, 3], dtype=torch.int32, device=DEV)
+    got = ops.moe_combine(y, inv, sh, 3, 2).float()
+    want = y.float()[inv.long()].view(3, 2, I).sum(1) + sh.float()
+    assert float((got - want).abs().max()) <= tol * 4
+    assert float((ops.moe_combine(y, inv, None, 3, 2).float() - (want - sh.float())).abs().max()) <= tol * 4
+    table = _rand(50, I, dtype=dtype, seed=6)
+    ids = torch.tensor([3, 49, 0, 3], dtype=torch.int32, device=DEV)
+    assert torch.equal(ops.embed_gather(ids, table), table.float()[ids.long()])
+
+
+@pytest.mark.parametrize("nh,nkv,hd", [(4, 2, 16), (6, 3, 32), (5, 5, 48), (40, 8, 128)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("mode", ["rope+norm", "rope", "temperature", "bare"])
+def test_rope_kv_kernel(nh, nkv, hd, dtype, mode):
+    ops = _ops()
+    import plain_llama4 as P
+
+    T, ps, pages = 11, 16, 6
+    qkv = _rand(T, (nh + 2 * nkv) * hd, dtype=dtype, seed=hd)
+    positions = torch.tensor([0, 1, 2, 17, 31, 32, 100, 1000, 4095, 70000, 5], dtype=torch.int32)
+    slots = torch.tensor([0, 1, 2, 33, 47, 64, 20, 21, 95, 50, -1], dtype=torch.int32)   # the last one stores nothing
+    inv = P.rope_inv_freq(hd, 500000.0, None) if mode.startswith("rope") else None
+    kc = torch.zeros(pages, nkv, ps, hd, dtype=dtype, device=DEV)
+    vc = torch.zeros(pages, nkv, hd, ps, dtype=dtype, device=DEV)
+    q = ops.rope_kv(qkv, kc, vc, slots.to(DEV), positions.to(DEV), inv.to(DEV) if inv is not None else None,
+                    mode == "rope+norm", 1e-5, (32.0, 0.2) if mode == "temperature" else None, nh, nkv, hd)
+    x = qkv.float().cpu().view(T, nh + 2 * nkv, hd)
+    qr, kr, vr = x[:, :nh], x[:, nh:nh + nkv], x[:, nh + nkv:]
+    if inv is not None:
+        qr, kr = P.apply_rope_interleaved(qr, positions, inv), P.apply_rope_interleaved(kr, positions, inv)
+    if mode == "rope+norm":
+        qr, kr = P.l2_head_norm(qr, 1e-5), P.l2_head_norm(kr, 1e-5)
+    if mode == "temperature":
+        qr = qr * P.query_temperature(positions, 32.0, 0.2)[:, None, None]
+    tol = 2e-5 if dtype == torch.float32 else 1e-2
+    scale = max(1.0, float(qr.abs().max()))
+    assert float((q.float().cpu().view(T, nh, hd) - qr).abs().max()) <= tol * scale
+    kcc, vcc = kc.float().cpu(), vc.float().cpu()
+    for t in range(T - 1):
+        page, off = int(slots[t]) // ps, int(slots[t]) % ps
+        assert float((kcc[page, :, off, :] - kr[t]).abs().max()) <= tol * scale, t
+        assert float((vcc[page, :, :, off] - vr[t]).abs().max()) <= tol * scale, t
+    written = torch.zeros(pages * ps, dtype=torch.bool)
+    written[slots[:-1].long()] = True
+    assert float(kcc.permute(0, 2, 1, 3).reshape(pages * ps, -1)[~written].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 5, 3), (70, 130, 50), (64, 64, 16), (129, 203, 96)])
+def test_gemm_tiled_is_a_true_float_product_and_batch_invariant(M, N, K):
+    ops = _ops()
+    x, w = _rand(M, K, seed=1), _rand(N, K, seed=2)
+    got = ops.gemm_tiled(x, w)
+    want = (x.double() @ w.double().T).float()
+    assert float((got - want).abs().max()) <= 2e-6 * K * float(want.abs().max() + 1)
+    # values that bfloat16 or tf32 products would lose
+    a = torch.tensor([[1.0, 2.0 ** -20]], device=DEV)
+    b = torch.tensor([[1.0, 1.0]], device=DEV)
+    assert float(ops.gemm_tiled(a, b)[0, 0]) == 1.0 + 2.0 ** -20
+    if M > 1:
+        assert torch.equal(ops.gemm_tiled(x[:1].contiguous(), w), got[:1])
+        assert torch.equal(ops.gemm_tiled(x[M // 2:].contiguous(), w), got[M // 2:])
