@@ -1,53 +1,64 @@
 // Attention for entries of several tokens (prompt portions): flash attention on the matrix cores
 // over the paged cache, causal and window masks applied per element.
 //
-// A wave owns a tile of up to 32 consecutive tokens of one entry and one query head, and walks
-// the keys its rows can see in 32-key chunks (two 16-key blocks aligned to absolute positions,
-// so a block never straddles a page).  As in the decode kernel everything is transposed:
+// A block owns a tile of up to 128 consecutive tokens of one entry and one query head; each of its
+// four waves takes 32 of the tokens.  The block walks the keys its rows can see in 32-key chunks
+// (two 16-key blocks aligned to absolute positions, so a block never straddles a page); a chunk's
+// keys and values are fetched from the cache once, staged in LDS (double-buffered, one chunk
+// ahead) and read from there by all four waves.  As in the decode kernel everything is transposed:
 //   S^T[key, q]  = K[key, :] . Q[q, :]          A = K block, B = Q^T
 //   O^T[d, q]   += V^T[d, key] * P^T[key, q]    A = V^T block (values are stored transposed
 //                                               inside a page), B = P^T
 // and the S^T accumulator of a lane is the B operand of the second product once exponentiated
-// and split into a bfloat16 pair hi + lo.  Softmax state (running max and sum per query) is
-// float.  The keys of a query are always visited in the same blocks, whatever the portion it
-// arrived in, so its sums do not depend on how the prompt was cut.  Waves do not share data:
-// there is no LDS and no barrier.
+// and split into a bfloat16 pair hi + lo.  In LDS the value columns are permuted so that the
+// eight keys a lane needs (4 of each 16-key block) sit side by side; rows are padded so that the
+// 16 lanes of a quarter-wave hit 16 different bank groups.  Softmax state (running max and sum
+// per query) is float, kept in base-2 units (scores times log2 e, the hardware's exp2).  The keys of a query are always visited in the same blocks, whatever the
+// portion it arrived in, so its sums do not depend on how the prompt was cut.
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 constexpr int kPreWaves = 4;
-constexpr int kQT = 2;            // 16-token column tiles per wave
-constexpr int kTileTokens = 16 * kQT;
+constexpr int kQT = 2;                               // 16-token column tiles per wave
+constexpr int kWaveTokens = 16 * kQT;
+constexpr int kTileTokens = kWaveTokens * kPreWaves; // 128 tokens per block
+constexpr int kVPad = 40;                            // LDS row of the value tile: 32 keys + 8
 
 template <int HD>
 __global__ __launch_bounds__(kPreWaves* kWave) void attn_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ block_table, const int* __restrict__ positions, const int* __restrict__ tiles,
-    bf16_t* __restrict__ out, int n_tiles, int window_kind, int window, float scale, int nh, int nkv,
-    int page_size, int max_blocks, int num_pages) {
+    bf16_t* __restrict__ out, int window_kind, int window, float scale, int nh, int nkv, int page_size,
+    int max_blocks, int num_pages) {
   constexpr int NJ = HD / 32;
   constexpr int ND = HD / 16;
-  const int lane = threadIdx.x & (kWave - 1);
-  const int w = threadIdx.x >> 6;
+  constexpr int KPAD = HD + 8;
+  constexpr int PIECES = 4 * HD;                                   // 16-byte pieces of a K (or V) chunk
+  constexpr int NST = (PIECES + kPreWaves * kWave - 1) / (kPreWaves * kWave);
+  __shared__ __attribute__((aligned(16))) bf16_t Ks[2][32][KPAD];
+  __shared__ __attribute__((aligned(16))) bf16_t Vs[2][HD][kVPad];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int w = tid >> 6;
   const int r = lane & 15, g = lane >> 4;
-  const int ti = blockIdx.x * kPreWaves + w;
-  if (ti >= n_tiles) return;
+  const int ti = blockIdx.x;
   const int h = blockIdx.y;
   const int kvh = h / (nh / nkv);
   const int entry = tiles[ti * 3], tok0 = tiles[ti * 3 + 1], rows = tiles[ti * 3 + 2];
   const int pos0 = positions[tok0];
   const int* bt = block_table + (size_t)entry * max_blocks;
 
-  // per column tile: this lane's query row, its position and the first key it may see
+  // this wave's 32 tokens: per column tile, the lane's query row, its position, its first key
+  const int wrow0 = w * kWaveTokens;
   int qpos[kQT], qstart[kQT];
   bool qok[kQT];
   bf16x8 qf[kQT][NJ];
 #pragma unroll
   for (int c = 0; c < kQT; ++c) {
-    const int row = c * 16 + r;
+    const int row = wrow0 + c * 16 + r;
     qok[c] = row < rows;
     qpos[c] = pos0 + row;
     int st = 0;
@@ -60,10 +71,22 @@ __global__ __launch_bounds__(kPreWaves* kWave) void attn_prefill_kernel(
       else qf[c][j] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
     }
   }
-  int first = pos0;   // the first key of the tile's first row
+  const int wave_last = pos0 + min(rows, wrow0 + kWaveTokens) - 1;   // last position of this wave's rows
+  const bool wave_has_rows = wrow0 < rows;
+  const bool wave_full = wrow0 + kWaveTokens <= rows;                 // all 32 rows exist
+  const int wave_first_pos = pos0 + wrow0;
+  int wave_last_start = 0;                                            // first key the wave's last row may see
+  if (window_kind == 1) wave_last_start = (wave_last / window) * window;
+  else if (window_kind == 2) wave_last_start = wave_last - window + 1 > 0 ? wave_last - window + 1 : 0;
+  const float scale_log2 = scale * 1.4426950408889634f;               // softmax in base 2: exp(x) = 2^(x log2 e)
+  int wave_first = pos0 + wrow0;                                      // first key the wave's first row may see
+  if (window_kind == 1) wave_first = (wave_first / window) * window;
+  else if (window_kind == 2) wave_first = wave_first - window + 1 > 0 ? wave_first - window + 1 : 0;
+  else wave_first = 0;
+
+  int first = 0;   // the first key of the tile's first row
   if (window_kind == 1) first = (pos0 / window) * window;
   else if (window_kind == 2) first = pos0 - window + 1 > 0 ? pos0 - window + 1 : 0;
-  else first = 0;
   const int b_first = first >> 4;
   const int b_last = (pos0 + rows - 1) >> 4;
 
@@ -77,10 +100,11 @@ __global__ __launch_bounds__(kPreWaves* kWave) void attn_prefill_kernel(
     for (int d = 0; d < ND; ++d) acc[c][d] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
-  for (int b = b_first; b <= b_last; b += 2) {
+  // staging: fetch the chunk that starts at 16-key block b into registers
+  uint4 kst[NST], vst[NST];
+  auto fetch = [&](int b) {
     long long kbase[2], vbase[2];
     bool have[2];
-    f32x4 s[kQT][2];
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const int bb = b + u;
@@ -94,69 +118,126 @@ __global__ __launch_bounds__(kPreWaves* kWave) void attn_prefill_kernel(
       const int off = (bb << 4) % page_size;
       kbase[u] = have[u] ? (((long long)page * nkv + kvh) * page_size + off) * HD : 0;
       vbase[u] = have[u] ? ((long long)page * nkv + kvh) * HD * page_size + off : 0;
+    }
 #pragma unroll
-      for (int c = 0; c < kQT; ++c) s[c][u] = f32x4{0.f, 0.f, 0.f, 0.f};
-      if (have[u]) {
-#pragma unroll
-        for (int j = 0; j < NJ; ++j) {
-          const bf16x8 kf = *reinterpret_cast<const bf16x8*>(k_cache + kbase[u] + (size_t)r * HD + j * 32 + g * 8);
-#pragma unroll
-          for (int c = 0; c < kQT; ++c) s[c][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[c][j], s[c][u], 0, 0, 0);
-        }
+    for (int i = 0; i < NST; ++i) {
+      const int piece = tid + i * kPreWaves * kWave;
+      kst[i] = uint4{0u, 0u, 0u, 0u};
+      vst[i] = uint4{0u, 0u, 0u, 0u};
+      if (piece < PIECES) {
+        const int key = piece / (HD / 8), dcol = (piece % (HD / 8)) * 8;     // K: 32 keys x HD
+        if (have[key >> 4])
+          kst[i] = *reinterpret_cast<const uint4*>(k_cache + kbase[key >> 4] + (size_t)(key & 15) * HD + dcol);
+        const int d = piece >> 2, blk = (piece >> 1) & 1, half = piece & 1;  // V^T: HD rows x 2 blocks x 2 halves
+        if (have[blk])
+          vst[i] = *reinterpret_cast<const uint4*>(v_cache + vbase[blk] + (size_t)d * page_size + half * 8);
       }
     }
-    bf16x8 pf[kQT], pf_lo[kQT];
-    float corr[kQT];
+  };
+  auto stash = [&](int buf) {
 #pragma unroll
-    for (int c = 0; c < kQT; ++c) {
-      // lane holds S^T[key = 16*(b+u) + 4g + i][query row c*16 + r]
-      float cm = -INFINITY;
+    for (int i = 0; i < NST; ++i) {
+      const int piece = tid + i * kPreWaves * kWave;
+      if (piece < PIECES) {
+        const int key = piece / (HD / 8), dcol = (piece % (HD / 8)) * 8;
+        *reinterpret_cast<uint4*>(&Ks[buf][key][dcol]) = kst[i];
+        // keys 8*half .. 8*half+7 of block blk: groups g = 2*half and 2*half + 1, four keys each;
+        // column of (g, blk) = g*8 + blk*4
+        const int d = piece >> 2, blk = (piece >> 1) & 1, half = piece & 1;
+        *reinterpret_cast<uint2*>(&Vs[buf][d][(2 * half) * 8 + blk * 4]) = uint2{vst[i].x, vst[i].y};
+        *reinterpret_cast<uint2*>(&Vs[buf][d][(2 * half + 1) * 8 + blk * 4]) = uint2{vst[i].z, vst[i].w};
+      }
+    }
+  };
+
+  fetch(b_first);
+  stash(0);
+  __syncthreads();
+  int buf = 0;
+  for (int b = b_first; b <= b_last; b += 2, buf ^= 1) {
+    const bool more = b + 2 <= b_last;
+    if (more) fetch(b + 2);
+    // does any row of this wave see a key of this chunk?
+    const bool active = wave_has_rows && (b << 4) <= wave_last && ((b + 2) << 4) > wave_first;
+    if (active) {
+      bool have[2];
+      f32x4 s[kQT][2];
 #pragma unroll
-      for (int u = 0; u < 2; ++u)
+      for (int u = 0; u < 2; ++u) {
+        have[u] = b + u <= b_last;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int key = ((b + u) << 4) + 4 * g + i;
-          const bool ok = have[u] && qok[c] && key >= qstart[c] && key <= qpos[c];
-          s[c][u][i] = ok ? s[c][u][i] * scale : -INFINITY;
-          cm = fmaxf(cm, s[c][u][i]);
+        for (int c = 0; c < kQT; ++c) s[c][u] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (have[u]) {
+#pragma unroll
+          for (int j = 0; j < NJ; ++j) {
+            const bf16x8 kf = *reinterpret_cast<const bf16x8*>(&Ks[buf][u * 16 + r][j * 32 + g * 8]);
+#pragma unroll
+            for (int c = 0; c < kQT; ++c) s[c][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[c][j], s[c][u], 0, 0, 0);
+          }
         }
-      cm = fmaxf(cm, __shfl_xor(cm, 16, kWave));
-      cm = fmaxf(cm, __shfl_xor(cm, 32, kWave));
-      const float m_new = fmaxf(m[c], cm);
-      corr[c] = 1.0f;
-      if (m_new == -INFINITY) {
-        pf[c] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
-        pf_lo[c] = pf[c];
-      } else {
-        corr[c] = expf(m[c] - m_new);
-        float ls = 0.f;
+      }
+      bf16x8 pf[kQT], pf_lo[kQT];
+      float corr[kQT];
+      // a chunk that every row of the wave sees whole needs no mask
+      const bool whole = wave_full && have[1] && ((b + 2) << 4) - 1 <= wave_first_pos && (b << 4) >= wave_last_start;
+#pragma unroll
+      for (int c = 0; c < kQT; ++c) {
+        // lane holds S^T[key = 16*(b+u) + 4g + i][query row c*16 + r]; scores go to base-2 units
+        float cm = -INFINITY;
 #pragma unroll
         for (int u = 0; u < 2; ++u)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const float e = expf(s[c][u][i] - m_new);
-            ls += e;
-            const bf16_t hi = f32_to_bf16(e);
-            pf[c][u * 4 + i] = __builtin_bit_cast(__bf16, hi.bits);
-            pf_lo[c][u * 4 + i] = __builtin_bit_cast(__bf16, f32_to_bf16(e - bf16_to_f32(hi)).bits);
+            float t = s[c][u][i] * scale_log2;
+            if (!whole) {
+              const int key = ((b + u) << 4) + 4 * g + i;
+              const bool ok = have[u] && qok[c] && key >= qstart[c] && key <= qpos[c];
+              t = ok ? t : -INFINITY;
+            }
+            s[c][u][i] = t;
+            cm = fmaxf(cm, t);
           }
-        l[c] = l[c] * corr[c] + ls;
-        m[c] = m_new;
+        cm = fmaxf(cm, __shfl_xor(cm, 16, kWave));
+        cm = fmaxf(cm, __shfl_xor(cm, 32, kWave));
+        const float m_new = fmaxf(m[c], cm);
+        corr[c] = 1.0f;
+        if (m_new == -INFINITY) {
+          pf[c] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+          pf_lo[c] = pf[c];
+        } else {
+          corr[c] = __builtin_amdgcn_exp2f(m[c] - m_new);
+          float ls = 0.f;
+#pragma unroll
+          for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const float e = __builtin_amdgcn_exp2f(s[c][u][i] - m_new);   // masked: 2^-inf = 0
+              ls += e;
+              const __bf16 hi = (__bf16)e;                                   // round to nearest even
+              pf[c][u * 4 + i] = hi;
+              pf_lo[c][u * 4 + i] = (__bf16)(e - (float)hi);
+            }
+          l[c] = l[c] * corr[c] + ls;
+          m[c] = m_new;
+        }
+      }
+      bool rescale[kQT];
+#pragma unroll
+      for (int c = 0; c < kQT; ++c) rescale[c] = __builtin_amdgcn_ballot_w64(corr[c] != 1.0f) != 0;   // wave-uniform
+#pragma unroll
+      for (int d = 0; d < ND; ++d) {
+        // lane (d row r, group g): keys 4g..4g+3 of block b, then of block b + 1, side by side in LDS
+        const bf16x8 vf = *reinterpret_cast<const bf16x8*>(&Vs[buf][d * 16 + r][g * 8]);
+#pragma unroll
+        for (int c = 0; c < kQT; ++c) {
+          if (rescale[c]) acc[c][d] *= corr[c];
+          acc[c][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[c], acc[c][d], 0, 0, 0);
+          acc[c][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf_lo[c], acc[c][d], 0, 0, 0);
+        }
       }
     }
-#pragma unroll
-    for (int d = 0; d < ND; ++d) {
-      bf16x4 va = bf16x4{0, 0, 0, 0}, vb = bf16x4{0, 0, 0, 0};
-      if (have[0]) va = *reinterpret_cast<const bf16x4*>(v_cache + vbase[0] + (size_t)(d * 16 + r) * page_size + 4 * g);
-      if (have[1]) vb = *reinterpret_cast<const bf16x4*>(v_cache + vbase[1] + (size_t)(d * 16 + r) * page_size + 4 * g);
-      const bf16x8 vf = __builtin_shufflevector(va, vb, 0, 1, 2, 3, 4, 5, 6, 7);
-#pragma unroll
-      for (int c = 0; c < kQT; ++c) {
-        acc[c][d] *= corr[c];
-        acc[c][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[c], acc[c][d], 0, 0, 0);
-        acc[c][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf_lo[c], acc[c][d], 0, 0, 0);
-      }
-    }
+    if (more) stash(buf ^ 1);
+    __syncthreads();
   }
 
 #pragma unroll
@@ -166,7 +247,7 @@ __global__ __launch_bounds__(kPreWaves* kWave) void attn_prefill_kernel(
     L += __shfl_xor(L, 32, kWave);
     if (!qok[c]) continue;
     const float inv = L > 0.f ? 1.0f / L : 0.f;
-    bf16_t* orow = out + ((size_t)(tok0 + c * 16 + r) * nh + h) * HD;
+    bf16_t* orow = out + ((size_t)(tok0 + wrow0 + c * 16 + r) * nh + h) * HD;
 #pragma unroll
     for (int d = 0; d < ND; ++d) {
       // lane holds O^T[d*16 + 4g + i][query row]
@@ -180,7 +261,7 @@ __global__ __launch_bounds__(kPreWaves* kWave) void attn_prefill_kernel(
 }
 
 // q [T, nh, hd] bf16; caches K [pages, nkv, page_size, hd], V [pages, nkv, hd, page_size] bf16;
-// tiles int32 [n_tiles, 3] = (entry, first token, rows <= 32), tokens of a tile consecutive in
+// tiles int32 [n_tiles, 3] = (entry, first token, rows <= 128), tokens of a tile consecutive in
 // one entry; out [T, nh, hd] bf16 (rows of the listed tiles).
 SHARPI_EXPORT int sharpi_attention_prefill(const void* q, const void* k_cache, const void* v_cache,
                                            const int* block_table, const int* positions, const int* tiles,
@@ -191,19 +272,19 @@ SHARPI_EXPORT int sharpi_attention_prefill(const void* q, const void* k_cache, c
   if (nh <= 0 || nkv <= 0 || nh % nkv != 0 || nh > 65535) return SHARPI_ERR_ARG;
   if (page_size <= 0 || page_size % 16 != 0 || max_blocks <= 0 || num_pages <= 0) return SHARPI_ERR_ARG;
   if (window_kind < 0 || window_kind > 2 || (window_kind != 0 && window <= 0)) return SHARPI_ERR_ARG;
-  dim3 grid(ceil_div(n_tiles, kPreWaves), nh), block(kPreWaves * kWave);
+  dim3 grid(n_tiles, nh), block(kPreWaves * kWave);
 #define PRE(HDV)                                                                                              \
   if (hd == HDV) {                                                                                            \
     attn_prefill_kernel<HDV><<<grid, block, 0, stream>>>((const bf16_t*)q, (const bf16_t*)k_cache,            \
                                                         (const bf16_t*)v_cache, block_table, positions, tiles, \
-                                                        (bf16_t*)out, n_tiles, window_kind, window, scale, nh, \
-                                                        nkv, page_size, max_blocks, num_pages);               \
+                                                        (bf16_t*)out, window_kind, window, scale, nh, nkv,     \
+                                                        page_size, max_blocks, num_pages);                    \
     SHARPI_CHECK_LAUNCH();                                                                                    \
     return SHARPI_OK;                                                                                         \
   }
-  PRE(32) PRE(64) PRE(96) PRE(128) PRE(192) PRE(256)
+  PRE(32) PRE(64) PRE(96) PRE(128) PRE(192)
 #undef PRE
-  return SHARPI_ERR_ARG;  // head sizes that are no multiple of 32 go to the generic kernel
+  return SHARPI_ERR_ARG;  // other head sizes go to the generic kernel
 }
 
 SHARPI_EXPORT int sharpi_attention_prefill_tile_tokens() { return kTileTokens; }

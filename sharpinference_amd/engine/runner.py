@@ -21,7 +21,7 @@ from ..parts.base import GroupView, LayerCache, StepContext
 
 
 MAX_GRAPH_BATCH = 64   # decode steps of up to this many requests are replayed from a HIP graph
-TILE = 32   # tokens per attention tile of multi-token entries (ops.PREFILL_TILE_TOKENS)
+TILE = 128   # tokens per attention tile of multi-token entries (ops.PREFILL_TILE_TOKENS)
 
 
 class CacheExhausted(CacheError):

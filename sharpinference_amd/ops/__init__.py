@@ -222,20 +222,25 @@ def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     return out
 
 
-PREFILL_TILE_TOKENS = 32   # tokens per wave of the prefill kernel
+PREFILL_TILE_TOKENS = 128   # tokens per block of the prefill kernel (32 per wave)
+
+
+def prefill_attention_ok(dtype: torch.dtype, hd: int) -> bool:
+    return dtype == torch.bfloat16 and hd % 32 == 0 and 32 <= hd <= 192
 
 
 def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                       positions: torch.Tensor, tiles: torch.Tensor, window_kind: int, window: int, scale: float,
                       nh: int, nkv: int, hd: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Flash attention for the listed tiles: tiles int32 [n, 3] = (entry, first token, rows <= 32),
+    """Flash attention for the listed tiles: tiles int32 [n, 3] = (entry, first token, rows <= 128),
     the tokens of a tile consecutive in one entry."""
     _dev(q, k_cache, v_cache, block_table, positions, tiles, out)
     _i32(block_table, "block_table")
     _i32(positions, "positions")
     _i32(tiles, "tiles")
     T = q.shape[0]
-    _need(q.shape == (T, nh * hd) and decode_attention_ok(q.dtype, hd), "attention_prefill: q must be bfloat16 [T, nh*hd], hd a multiple of 32")
+    _need(q.shape == (T, nh * hd) and prefill_attention_ok(q.dtype, hd),
+          "attention_prefill: q must be bfloat16 [T, nh*hd], hd a multiple of 32 up to 192")
     _need(_cache_shapes_ok(k_cache, v_cache, nkv, hd) and k_cache.dtype == q.dtype and v_cache.dtype == q.dtype,
           "attention_prefill: caches must be K [pages, nkv, page_size, hd], V [pages, nkv, hd, page_size] bfloat16")
     _need(block_table.dim() == 2 and positions.shape == (T,) and tiles.dim() == 2 and tiles.shape[1] == 3,
@@ -483,8 +488,8 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, gro
               window: int, scale: float, nh: int, nkv: int, hd: int) -> torch.Tensor:
     """Attention of the step's tokens over their requests' pages (`group`: the cache group's
     block tables, `ctx`: the step)."""
-    if decode_attention_ok(q.dtype, hd):
-        # entries of one token: split-K decode kernel; longer entries: flash kernel, 32 tokens a wave
+    if decode_attention_ok(q.dtype, hd) and (prefill_attention_ok(q.dtype, hd) or not ctx.n_prefill_tiles):
+        # entries of one token: split-K decode kernel; longer entries: flash kernel, 128 tokens a block
         out = torch.empty_like(q)
         if ctx.n_prefill_tiles:
             attention_prefill(q, k_cache, v_cache, group.block_table, ctx.positions, ctx.prefill_tiles, window_kind,

@@ -50,7 +50,7 @@ class StepContext:
     groups: List[GroupView]
     act_dtype: torch.dtype
     no_store_slots: Optional[torch.Tensor] = None   # int32 [tokens] of -1: "store nothing" for cache readers
-    # how attention kernels split the batch: entries of one token, and 32-token tiles of the others
+    # how attention kernels split the batch: entries of one token, and 128-token tiles of the others
     n_decode: int = 0
     decode_tokens: Optional[torch.Tensor] = None    # int32 [n_decode] token indices; None = every token
     n_prefill_tiles: int = 0

@@ -10,7 +10,7 @@ pytestmark = pytest.mark.gpu
 PROMPTS = {"A": [5, 23, 40 + 16], "B": [1, 17, 50, 77 + 24], "C": [3, 64, 95]}
 
 
-@pytest.fixture(scope="module", params=[("A", 0.02), ("B", 0.02), ("C", 0.02), ("A", 0.15), ("B", 0.12), ("C", 0.1)],
+@pytest.fixture(scope="module", params=[("A", 0.02), ("B", 0.02), ("C", 0.02), ("A", 0.1), ("B", 0.08), ("C", 0.1)],
                 ids=lambda p: f"{p[0]}-std{p[1]}")
 def model_dir(request, tmp_path_factory):
     which, std = request.param

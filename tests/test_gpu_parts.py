@@ -16,6 +16,7 @@ DEV = "cuda:0"
 def _ctx(entries, page_size=16, dtype=torch.float32, totals=None):
     """A StepContext for requests given as (start position, tokens in this step), each with its
     own pages in one group (`totals`: final lengths, so that pages stay put from step to step)."""
+    from sharpinference_amd.ops import PREFILL_TILE_TOKENS as TILE
     from sharpinference_amd.parts.base import GroupView, StepContext
 
     T = sum(n for _, n in entries)
@@ -39,7 +40,7 @@ def _ctx(entries, page_size=16, dtype=torch.float32, totals=None):
     g = GroupView(bt.to(DEV), i32(slots), page_size, max_context=max(pos) + 1)
     lens = [n for _, n in entries]
     dec = [cu[i] for i, n in enumerate(lens) if n == 1]
-    tiles = [(i, cu[i] + o, min(32, n - o)) for i, n in enumerate(lens) if n > 1 for o in range(0, n, 32)]
+    tiles = [(i, cu[i] + o, min(TILE, n - o)) for i, n in enumerate(lens) if n > 1 for o in range(0, n, TILE)]
     ctx = StepContext(n_tokens=T, n_entries=len(entries), token_ids=i32([0] * T), positions=i32(pos), entry_of_token=i32(ent),
                       cu_tokens=i32(cu), state_slots=i32(list(range(len(entries)))), groups=[g], act_dtype=dtype,
                       no_store_slots=i32([-1] * T), entry_lens=lens, entry_starts=[s for s, _ in entries],
