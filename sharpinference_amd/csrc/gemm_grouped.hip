@@ -8,7 +8,7 @@
 // listed on the device by the routing kernel (tile_expert, tile_row0, n_tiles); the host never
 // learns the routing, and 16-row groups beyond an expert's last row are skipped, not multiplied.
 //  * Each of the 4 waves owns 32 weight rows (2 MFMA tiles) and reads them straight from global
-//    memory into registers, one 64-wide K stage ahead: a weight element is used by one wave only.
+//    memory into registers, four 64-wide K stages ahead: a weight element is used by one wave only.
 //  * The x rows (gathered through a_rows) are shared by the waves and staged through LDS, 64
 //    columns of K at a time, double-buffered; rows are padded to 72 elements so that the 16
 //    lanes of a quarter-wave read 16 different banks.
@@ -16,6 +16,8 @@
 //    row, stored as one 8-byte write.  Each output is one chain over k in ascending order, so a
 //    row's result does not depend on which other rows share its tile.
 // Limits: K % 64 == 0, N % 4 == 0.
+#include <type_traits>
+
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -23,21 +25,32 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 constexpr int GM = 192;       // rows per tile (the routing kernel lists tiles of this height)
 constexpr int GMT = GM / 16;  // 16-row groups per tile
-constexpr int GW = 4;         // waves per block, 32 weight rows each
-constexpr int GN = 32 * GW;   // columns per tile
+constexpr int GW = 4;         // waves per block
+constexpr int NT = 2;         // 16-row weight tiles per wave
+constexpr int GN = 16 * NT * GW;   // columns per tile
 constexpr int GK = 64;        // K per LDS stage
 constexpr int GPAD = GK + 8;  // padded LDS row
 constexpr int GROWS = GW * 8;     // rows staged per pass: 8 threads per 64-wide row
 constexpr int GPASS = GM / GROWS;  // staging passes
+constexpr int kXcds = 8;           // accelerator dies, each with its own L2
+constexpr int kAhead = 4;           // K stages of weights in flight per wave
+constexpr int kHalves = 2;         // a tile's column blocks are split over this many XCDs
 
 template <typename TO>
 __global__ __launch_bounds__(GW* kWave) void grouped_gemm_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ W, TO* __restrict__ out, int N, int K,
     const int* __restrict__ a_rows, const int* __restrict__ group_offsets, const int* __restrict__ tile_expert,
-    const int* __restrict__ tile_row0, const int* __restrict__ n_tiles) {
+    const int* __restrict__ tile_row0, const int* __restrict__ n_tiles, int nb_per_unit) {
   __shared__ __attribute__((aligned(16))) bf16_t xs[2][GM][GPAD];
-  const int tile = blockIdx.x;
-  if (tile >= n_tiles[0]) return;
+  // Workgroups go to the 8 XCDs round-robin by their linear id, and each XCD has an L2 of its
+  // own.  All column blocks of one (tile, half of the columns) unit are therefore given ids that
+  // are equal modulo 8: the unit's x rows are fetched into one L2 and stay there.
+  const int xcd = blockIdx.x % kXcds;
+  const int slot = blockIdx.x / kXcds;
+  const int unit = (slot / nb_per_unit) * kXcds + xcd;
+  const int tile = unit / kHalves;
+  const int nblock = (unit % kHalves) * nb_per_unit + slot % nb_per_unit;
+  if (tile >= n_tiles[0] || nblock * GN >= N) return;
   const int e = tile_expert[tile];
   const int row0 = tile_row0[tile];
   const int row_end = group_offsets[e + 1];
@@ -46,12 +59,12 @@ __global__ __launch_bounds__(GW* kWave) void grouped_gemm_kernel(
   const int lane = threadIdx.x & (kWave - 1);
   const int w = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
-  const int n_base = blockIdx.y * GN + w * 32;
+  const int n_base = nblock * GN + w * 16 * NT;
   const bf16_t* We = W + (size_t)e * N * K;
 
-  const bf16_t* wrow[2];
+  const bf16_t* wrow[NT];
 #pragma unroll
-  for (int t = 0; t < 2; ++t) {
+  for (int t = 0; t < NT; ++t) {
     int n = n_base + t * 16 + r;
     if (n >= N) n = N - 1;  // loaded, never stored
     wrow[t] = We + (size_t)n * K + g * 8;
@@ -65,38 +78,39 @@ __global__ __launch_bounds__(GW* kWave) void grouped_gemm_kernel(
     xsrc[ps] = row < row_end ? x + (size_t)(a_rows ? a_rows[row] : row) * K + scol : nullptr;
   }
 
-  f32x4 acc[2][GMT];
+  f32x4 acc[NT][GMT];
 #pragma unroll
-  for (int t = 0; t < 2; ++t)
+  for (int t = 0; t < NT; ++t)
 #pragma unroll
     for (int mb = 0; mb < GMT; ++mb) acc[t][mb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   const int chunks = K / GK;
   uint4 stage[GPASS];
-  bf16x8 wf[2][2], wnext[2][2];
+  bf16x8 wf[kAhead][2][NT];   // weight fragments of the next kAhead stages, a ring indexed by stage % kAhead
 #pragma unroll
   for (int ps = 0; ps < GPASS; ++ps)
     stage[ps] = xsrc[ps] ? *reinterpret_cast<const uint4*>(xsrc[ps]) : uint4{0u, 0u, 0u, 0u};
 #pragma unroll
-  for (int j = 0; j < 2; ++j)
+  for (int a = 0; a < kAhead; ++a)
+    if (a < chunks) {
 #pragma unroll
-    for (int t = 0; t < 2; ++t) wf[j][t] = *reinterpret_cast<const bf16x8*>(wrow[t] + j * 32);
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) wf[a][j][t] = *reinterpret_cast<const bf16x8*>(wrow[t] + a * GK + j * 32);
+    }
 #pragma unroll
   for (int ps = 0; ps < GPASS; ++ps)
     if (srow + GROWS * ps < n_mt * 16) *reinterpret_cast<uint4*>(&xs[0][srow + GROWS * ps][scol]) = stage[ps];
   __syncthreads();
 
-  for (int c = 0; c < chunks; ++c) {
+  // one K stage; `slot` is the stage's place in the ring and a compile-time constant
+  auto stage_step = [&](int c, auto slot_tag) {
+    constexpr int slot = decltype(slot_tag)::value;
     const int buf = c & 1;
-    const int k1 = (c + 1) * GK;
-    if (c + 1 < chunks) {   // the next stage's x rows and weight rows are on their way while this one is multiplied
+    if (c + 1 < chunks) {   // the next stage's x rows are on their way while this one is multiplied
 #pragma unroll
       for (int ps = 0; ps < GPASS; ++ps)
-        stage[ps] = xsrc[ps] ? *reinterpret_cast<const uint4*>(xsrc[ps] + k1) : uint4{0u, 0u, 0u, 0u};
-#pragma unroll
-      for (int j = 0; j < 2; ++j)
-#pragma unroll
-        for (int t = 0; t < 2; ++t) wnext[j][t] = *reinterpret_cast<const bf16x8*>(wrow[t] + k1 + j * 32);
+        stage[ps] = xsrc[ps] ? *reinterpret_cast<const uint4*>(xsrc[ps] + (c + 1) * GK) : uint4{0u, 0u, 0u, 0u};
     }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
@@ -104,21 +118,32 @@ __global__ __launch_bounds__(GW* kWave) void grouped_gemm_kernel(
       for (int mb = 0; mb < GMT; ++mb) {
         if (mb < n_mt) {   // uniform over the block
           const bf16x8 xf = *reinterpret_cast<const bf16x8*>(&xs[buf][mb * 16 + r][j * 32 + g * 8]);
-          acc[0][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j][0], xf, acc[0][mb], 0, 0, 0);
-          acc[1][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j][1], xf, acc[1][mb], 0, 0, 0);
+#pragma unroll
+          for (int t = 0; t < NT; ++t)
+            acc[t][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[slot][j][t], xf, acc[t][mb], 0, 0, 0);
         }
       }
+    }
+    if (c + kAhead < chunks) {   // this slot's weights are used up: fetch those of kAhead stages on
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+          wf[slot][j][t] = *reinterpret_cast<const bf16x8*>(wrow[t] + (c + kAhead) * GK + j * 32);
     }
     if (c + 1 < chunks) {
 #pragma unroll
       for (int ps = 0; ps < GPASS; ++ps)
         if (srow + GROWS * ps < n_mt * 16) *reinterpret_cast<uint4*>(&xs[buf ^ 1][srow + GROWS * ps][scol]) = stage[ps];
-#pragma unroll
-      for (int j = 0; j < 2; ++j)
-#pragma unroll
-        for (int t = 0; t < 2; ++t) wf[j][t] = wnext[j][t];
     }
     __syncthreads();
+  };
+  static_assert(kAhead == 4, "the loop below is unrolled for a ring of four");
+  for (int c = 0; c < chunks; c += kAhead) {
+    stage_step(c, std::integral_constant<int, 0>{});
+    if (c + 1 < chunks) stage_step(c + 1, std::integral_constant<int, 1>{});
+    if (c + 2 < chunks) stage_step(c + 2, std::integral_constant<int, 2>{});
+    if (c + 3 < chunks) stage_step(c + 3, std::integral_constant<int, 3>{});
   }
 
   // lane holds out[row0 + mb*16 + r][n_base + t*16 + 4g + 0..3]
@@ -127,7 +152,7 @@ __global__ __launch_bounds__(GW* kWave) void grouped_gemm_kernel(
     const int row = row0 + mb * 16 + r;
     if (mb >= n_mt || row >= row_end) continue;
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
+    for (int t = 0; t < NT; ++t) {
       const int n = n_base + t * 16 + 4 * g;
       if (n >= N) continue;
       TO* dst = out + (size_t)row * N + n;
@@ -153,14 +178,17 @@ SHARPI_EXPORT int sharpi_gemm_grouped(const void* x, const void* W, void* out, i
   if (n_rows <= 0) return SHARPI_OK;
   if (N <= 0 || (N & 3) || K <= 0 || K % GK != 0 || max_tiles <= 0) return SHARPI_ERR_ARG;
   if (!group_offsets || !tile_expert || !tile_row0 || !n_tiles) return SHARPI_ERR_ARG;
-  if (ceil_div(N, GN) > 65535) return SHARPI_ERR_ARG;
-  dim3 grid(max_tiles, ceil_div(N, GN)), block(GW * kWave);
+  const int nb_per_unit = ceil_div(ceil_div(N, GN), kHalves);
+  const int units = ceil_div(max_tiles * kHalves, kXcds) * kXcds;
+  dim3 grid(units * nb_per_unit), block(GW * kWave);
   if (out_dtype == DT_BF16)
     grouped_gemm_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)x, (const bf16_t*)W, (bf16_t*)out, N, K,
-                                                           a_rows, group_offsets, tile_expert, tile_row0, n_tiles);
+                                                           a_rows, group_offsets, tile_expert, tile_row0, n_tiles,
+                                                           nb_per_unit);
   else if (out_dtype == DT_F32)
     grouped_gemm_kernel<float><<<grid, block, 0, stream>>>((const bf16_t*)x, (const bf16_t*)W, (float*)out, N, K,
-                                                          a_rows, group_offsets, tile_expert, tile_row0, n_tiles);
+                                                          a_rows, group_offsets, tile_expert, tile_row0, n_tiles,
+                                                          nb_per_unit);
   else
     return SHARPI_ERR_ARG;
   SHARPI_CHECK_LAUNCH();
