@@ -7,10 +7,10 @@ from tiny_configs import CONFIGS, make_model_dir
 
 pytestmark = pytest.mark.gpu
 
-PROMPTS = {"A": [5, 23, 40 + 16], "B": [1, 17, 50, 77 + 24], "C": [3, 64, 95]}
+PROMPTS = {"A": [5, 23, 40 + 16], "B": [1, 17, 50, 77 + 24], "C": [3, 64, 95], "D": [2, 70, 150, 260]}
 
 
-@pytest.fixture(scope="module", params=[("A", 0.02), ("B", 0.02), ("C", 0.02), ("A", 0.1), ("B", 0.08), ("C", 0.1)],
+@pytest.fixture(scope="module", params=[("A", 0.02), ("B", 0.02), ("C", 0.02), ("A", 0.1), ("B", 0.08), ("C", 0.1), ("D", 0.02), ("D", 0.06)],
                 ids=lambda p: f"{p[0]}-std{p[1]}")
 def model_dir(request, tmp_path_factory):
     which, std = request.param

@@ -39,10 +39,26 @@ TINY_C = {
     "tie_word_embeddings": True, "max_position_embeddings": 512, "torch_dtype": "bfloat16",
 }
 
-SEEDS = {"A": 0, "B": 1, "C": 5}
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+# a fourth one whose widths are multiples of 128 and whose head size is 64: the sizes at which the
+# matrix-core kernels (few-row and grouped products, flash attention) take over from the generic ones
+TINY_D = {
+    "architectures": ["Llama4ForCausalLM"],
+    "hidden_size": 256, "num_hidden_layers": 3, "num_attention_heads": 6, "num_key_value_heads": 2,
+    "head_dim": 64, "vocab_size": 500,
+    "intermediate_size": 128, "intermediate_size_mlp": 384,
+    "num_local_experts": 6, "num_experts_per_tok": 1, "interleave_moe_layer_step": 1,
+    "no_rope_layers": [1, 0, 1], "attention_chunk_size": 48,
+    "use_qk_norm": True, "attn_temperature_tuning": True, "floor_scale": 16, "attn_scale": 0.15,
+    "rms_norm_eps": 1e-5, "rope_theta": 500000.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 4.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 64},
+    "tie_word_embeddings": False, "max_position_embeddings": 1024, "torch_dtype": "bfloat16",
+}
+
+SEEDS = {"A": 0, "B": 1, "C": 5, "D": 9}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
 # tensors kept in float32 in B's file: shows that 32-bit tensors stay 32-bit in a bfloat16 run
-FLOAT32_NAMES = {"A": (), "B": ("layernorm.weight", "model.norm.weight", "router.weight"), "C": ()}
+FLOAT32_NAMES = {"A": (), "B": ("layernorm.weight", "model.norm.weight", "router.weight"), "C": (), "D": ()}
 
 
 def make_model_dir(tmp_path, which: str, std: float = 0.02, **overrides) -> str:
