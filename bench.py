@@ -44,7 +44,7 @@ def log(msg: str) -> None:
     print(f"[bench] {msg}", file=sys.stderr, flush=True)
 
 
-def build_engine(layers: int, max_batch: int, page_size: int):
+def build_engine(layers: int, max_batch: int, page_size: int, graphs: bool = True):
     from sharpinference_amd.engine import Engine
 
     cfg = dict(SCOUT)
@@ -54,7 +54,7 @@ def build_engine(layers: int, max_batch: int, page_size: int):
     t0 = time.time()
     eng = Engine(config=cfg, weight_seed=2, dtype="bfloat16", device="cuda:0", max_model_len=CONTEXT,
                  max_num_seqs=max_batch, max_tokens_per_step=8192, kv_tokens=max_batch * per_req,
-                 page_size=page_size)
+                 page_size=page_size, decode_graphs=graphs)
     log(f"engine with {layers} layers ready in {time.time() - t0:.1f}s")
     return eng
 
@@ -144,6 +144,7 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 points")
+    ap.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel instead of replaying a HIP graph")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this engine has no multi-GPU path (N=1 only)")
@@ -153,7 +154,7 @@ def main() -> int:
 
     rng = random.Random(2)
     max_batch = args.batch if args.no_points else max(args.batch, 64)
-    eng = build_engine(args.layers, max_batch, args.page_size)
+    eng = build_engine(args.layers, max_batch, args.page_size, graphs=not args.no_graphs)
     cfg = eng.config
 
     # prefill: one 2,048-token prompt alone, once to warm up, once timed

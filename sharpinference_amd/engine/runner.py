@@ -20,7 +20,7 @@ from ..cache.manager import CacheError, CacheManager
 from ..parts.base import GroupView, LayerCache, StepContext
 
 
-MAX_GRAPH_BATCH = 64   # decode steps of up to this many requests are replayed from a HIP graph
+MAX_GRAPH_BATCH = 16   # decode steps of up to this many requests are replayed from a HIP graph (beyond, launches no longer bound the step and the fixed maxima cost more than they save)
 TILE = 128   # tokens per attention tile of multi-token entries (ops.PREFILL_TILE_TOKENS)
 
 
