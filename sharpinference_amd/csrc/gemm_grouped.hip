@@ -23,14 +23,20 @@
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
-constexpr int GM = 192;       // rows per tile (the routing kernel lists tiles of this height)
+#ifndef SHARPI_GM
+#define SHARPI_GM 192
+#endif
+#ifndef SHARPI_GK
+#define SHARPI_GK 64
+#endif
+constexpr int GM = SHARPI_GM;  // rows per tile (the routing kernel lists tiles of this height)
 constexpr int GMT = GM / 16;  // 16-row groups per tile
 constexpr int GW = 4;         // waves per block
 constexpr int NT = 2;         // 16-row weight tiles per wave
 constexpr int GN = 16 * NT * GW;   // columns per tile
-constexpr int GK = 64;        // K per LDS stage
+constexpr int GK = SHARPI_GK;  // K per LDS stage
 constexpr int GPAD = GK + 8;  // padded LDS row
-constexpr int GROWS = GW * 8;     // rows staged per pass: 8 threads per 64-wide row
+constexpr int GROWS = GW * 64 / (GK / 8);   // rows staged per pass: GK / 8 threads per row
 constexpr int GPASS = GM / GROWS;  // staging passes
 constexpr int kXcds = 8;           // accelerator dies, each with its own L2
 constexpr int kAhead = 4;           // K stages of weights in flight per wave
@@ -70,7 +76,7 @@ __global__ __launch_bounds__(GW* kWave) void grouped_gemm_kernel(
     wrow[t] = We + (size_t)n * K + g * 8;
   }
   // staging role: thread loads 16 bytes of row (tid / 8 + GROWS * pass), columns (tid % 8) * 8
-  const int srow = threadIdx.x >> 3, scol = (threadIdx.x & 7) * 8;
+  const int srow = threadIdx.x / (GK / 8), scol = (threadIdx.x % (GK / 8)) * 8;
   const bf16_t* xsrc[GPASS];
 #pragma unroll
   for (int ps = 0; ps < GPASS; ++ps) {
@@ -86,7 +92,7 @@ __global__ __launch_bounds__(GW* kWave) void grouped_gemm_kernel(
 
   const int chunks = K / GK;
   uint4 stage[GPASS];
-  bf16x8 wf[kAhead][2][NT];   // weight fragments of the next kAhead stages, a ring indexed by stage % kAhead
+  bf16x8 wf[kAhead][GK / 32][NT];   // weight fragments of the next kAhead stages, a ring indexed by stage % kAhead
 #pragma unroll
   for (int ps = 0; ps < GPASS; ++ps)
     stage[ps] = xsrc[ps] ? *reinterpret_cast<const uint4*>(xsrc[ps]) : uint4{0u, 0u, 0u, 0u};
@@ -94,7 +100,7 @@ __global__ __launch_bounds__(GW* kWave) void grouped_gemm_kernel(
   for (int a = 0; a < kAhead; ++a)
     if (a < chunks) {
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+      for (int j = 0; j < GK / 32; ++j)
 #pragma unroll
         for (int t = 0; t < NT; ++t) wf[a][j][t] = *reinterpret_cast<const bf16x8*>(wrow[t] + a * GK + j * 32);
     }
@@ -113,7 +119,7 @@ __global__ __launch_bounds__(GW* kWave) void grouped_gemm_kernel(
         stage[ps] = xsrc[ps] ? *reinterpret_cast<const uint4*>(xsrc[ps] + (c + 1) * GK) : uint4{0u, 0u, 0u, 0u};
     }
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < GK / 32; ++j) {
 #pragma unroll
       for (int mb = 0; mb < GMT; ++mb) {
         if (mb < n_mt) {   // uniform over the block
@@ -126,7 +132,7 @@ __global__ __launch_bounds__(GW* kWave) void grouped_gemm_kernel(
     }
     if (c + kAhead < chunks) {   // this slot's weights are used up: fetch those of kAhead stages on
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+      for (int j = 0; j < GK / 32; ++j)
 #pragma unroll
         for (int t = 0; t < NT; ++t)
           wf[slot][j][t] = *reinterpret_cast<const bf16x8*>(wrow[t] + (c + kAhead) * GK + j * 32);
