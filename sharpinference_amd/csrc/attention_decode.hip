@@ -75,10 +75,12 @@ __global__ __launch_bounds__(kDecWaves* kWave) void attn_decode_kernel(
   for (int d = 0; d < ND; ++d) acc[d] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   for (int b = b_first + 2 * w; b <= b_last; b += 2 * kDecWaves) {
-    // two 16-key blocks: b and b + 1 (the second may lie beyond the range)
+    // two 16-key blocks: b and b + 1 (the second may lie beyond the range).  Keys AND values of
+    // the chunk are requested before anything is computed: the values do not wait for the scores.
     f32x4 s[2];
-    long long kbase[2], vbase[2];
     bool have[2];
+    bf16x8 kf[2][NJ];
+    bf16x4 vq[2][ND];
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const int bb = b + u;
@@ -90,16 +92,25 @@ __global__ __launch_bounds__(kDecWaves* kWave) void attn_decode_kernel(
         if (page < 0 || page >= num_pages) have[u] = false;
       }
       const int off = (bb << 4) % page_size;
-      kbase[u] = have[u] ? (((long long)page * nkv + kvh) * page_size + off) * HD : 0;
-      vbase[u] = have[u] ? ((long long)page * nkv + kvh) * HD * page_size + off : 0;
-      s[u] = f32x4{0.f, 0.f, 0.f, 0.f};
-      if (have[u]) {
+      const long long kbase = have[u] ? (((long long)page * nkv + kvh) * page_size + off) * HD : 0;
+      const long long vbase = have[u] ? ((long long)page * nkv + kvh) * HD * page_size + off : 0;
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) {
-          const bf16x8 kf = *reinterpret_cast<const bf16x8*>(k_cache + kbase[u] + (size_t)r * HD + j * 32 + g * 8);
-          s[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[j], s[u], 0, 0, 0);
-        }
+      for (int j = 0; j < NJ; ++j) {
+        if (have[u]) kf[u][j] = *reinterpret_cast<const bf16x8*>(k_cache + kbase + (size_t)r * HD + j * 32 + g * 8);
+        else kf[u][j] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
       }
+#pragma unroll
+      for (int d = 0; d < ND; ++d) {
+        // V^T fragment: lane (d row r, group g) holds keys 4g..4g+3 of the block
+        if (have[u]) vq[u][d] = *reinterpret_cast<const bf16x4*>(v_cache + vbase + (size_t)(d * 16 + r) * page_size + 4 * g);
+        else vq[u][d] = bf16x4{0, 0, 0, 0};
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      s[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) s[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[u][j], qf[j], s[u], 0, 0, 0);
     }
     // lane holds S^T[key = 16*(b+u) + 4g + i][head r]
     float cm = -INFINITY;
@@ -138,11 +149,8 @@ __global__ __launch_bounds__(kDecWaves* kWave) void attn_decode_kernel(
     }
 #pragma unroll
     for (int d = 0; d < ND; ++d) {
-      // V^T fragment: lane (d row r, group g) holds keys 4g..4g+3 of block b, then of block b + 1
-      bf16x4 va = bf16x4{0, 0, 0, 0}, vb = bf16x4{0, 0, 0, 0};
-      if (have[0]) va = *reinterpret_cast<const bf16x4*>(v_cache + vbase[0] + (size_t)(d * 16 + r) * page_size + 4 * g);
-      if (have[1]) vb = *reinterpret_cast<const bf16x4*>(v_cache + vbase[1] + (size_t)(d * 16 + r) * page_size + 4 * g);
-      const bf16x8 vf = __builtin_shufflevector(va, vb, 0, 1, 2, 3, 4, 5, 6, 7);
+      // keys 4g..4g+3 of block b, then of block b + 1
+      const bf16x8 vf = __builtin_shufflevector(vq[0][d], vq[1][d], 0, 1, 2, 3, 4, 5, 6, 7);
       acc[d] *= corr;   // corr belongs to head r = the accumulator's column
       acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, acc[d], 0, 0, 0);
       acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf_lo, acc[d], 0, 0, 0);
