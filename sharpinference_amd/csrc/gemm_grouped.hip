@@ -6,7 +6,7 @@
 // that fit one tile (192, about one and a half times the mean load of 2,048 tokens over 16
 // experts) against 128 weight rows: a typical expert's weights are then read once.  Tiles are
 // listed on the device by the routing kernel (tile_expert, tile_row0, n_tiles); the host never
-// learns the routing, and 16-row groups beyond an expert's last row are skipped, not multiplied.
+// learns the routing, and quartets of 16-row groups beyond an expert's last row are skipped, not multiplied.
 //  * Each of the 4 waves owns 32 weight rows (2 MFMA tiles) and reads them straight from global
 //    memory into registers, four 64-wide K stages ahead: a weight element is used by one wave only.
 //  * The x rows (gathered through a_rows) are shared by the waves and staged through LDS, 64
@@ -22,6 +22,7 @@
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
 #ifndef SHARPI_GM
 #define SHARPI_GM 192
@@ -80,8 +81,10 @@ __global__ __launch_bounds__(GW* kWave) void grouped_gemm_kernel(
   const bf16_t* xsrc[GPASS];
 #pragma unroll
   for (int ps = 0; ps < GPASS; ++ps) {
-    const int row = row0 + srow + GROWS * ps;
-    xsrc[ps] = row < row_end ? x + (size_t)(a_rows ? a_rows[row] : row) * K + scol : nullptr;
+    // rows beyond the expert's last read its last row again: every load is unconditional, and what
+    // such rows produce is never stored
+    const int row = min(row0 + srow + GROWS * ps, row_end - 1);
+    xsrc[ps] = x + (size_t)(a_rows ? a_rows[row] : row) * K + scol;
   }
 
   f32x4 acc[NT][GMT];
@@ -91,65 +94,88 @@ __global__ __launch_bounds__(GW* kWave) void grouped_gemm_kernel(
     for (int mb = 0; mb < GMT; ++mb) acc[t][mb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   const int chunks = K / GK;
-  uint4 stage[GPASS];
+  u32x4 stage[GPASS];
   bf16x8 wf[kAhead][GK / 32][NT];   // weight fragments of the next kAhead stages, a ring indexed by stage % kAhead
 #pragma unroll
   for (int ps = 0; ps < GPASS; ++ps)
-    stage[ps] = xsrc[ps] ? *reinterpret_cast<const uint4*>(xsrc[ps]) : uint4{0u, 0u, 0u, 0u};
+    stage[ps] = *reinterpret_cast<const u32x4*>(xsrc[ps]);
+  auto fill_ring = [&](auto all_tag) {
 #pragma unroll
-  for (int a = 0; a < kAhead; ++a)
-    if (a < chunks) {
+    for (int a = 0; a < kAhead; ++a)
+      if (decltype(all_tag)::value || a < chunks) {
 #pragma unroll
-      for (int j = 0; j < GK / 32; ++j)
+        for (int j = 0; j < GK / 32; ++j)
 #pragma unroll
-        for (int t = 0; t < NT; ++t) wf[a][j][t] = *reinterpret_cast<const bf16x8*>(wrow[t] + a * GK + j * 32);
-    }
+          for (int t = 0; t < NT; ++t) wf[a][j][t] = *reinterpret_cast<const bf16x8*>(wrow[t] + a * GK + j * 32);
+      }
+  };
+  if (chunks >= kAhead) fill_ring(std::true_type{}); else fill_ring(std::false_type{});
 #pragma unroll
   for (int ps = 0; ps < GPASS; ++ps)
-    if (srow + GROWS * ps < n_mt * 16) *reinterpret_cast<uint4*>(&xs[0][srow + GROWS * ps][scol]) = stage[ps];
+    *reinterpret_cast<u32x4*>(&xs[0][srow + GROWS * ps][scol]) = stage[ps];
   __syncthreads();
 
   // one K stage; `slot` is the stage's place in the ring and a compile-time constant
-  auto stage_step = [&](int c, auto slot_tag) {
+  // `steady`: every load of the stage is known to be in range, so none sits behind a branch.  The
+  // compiler counts outstanding loads statically; a load that may or may not have been issued makes
+  // it wait for all of them, and the ring would hide nothing.
+  auto stage_step = [&](int c, auto slot_tag, auto steady_tag) {
     constexpr int slot = decltype(slot_tag)::value;
+    constexpr bool steady = decltype(steady_tag)::value;
     const int buf = c & 1;
-    if (c + 1 < chunks) {   // the next stage's x rows are on their way while this one is multiplied
+    if (steady || c + 1 < chunks) {   // the next stage's x rows are on their way while this one is multiplied
 #pragma unroll
-      for (int ps = 0; ps < GPASS; ++ps)
-        stage[ps] = xsrc[ps] ? *reinterpret_cast<const uint4*>(xsrc[ps] + (c + 1) * GK) : uint4{0u, 0u, 0u, 0u};
+      for (int ps = 0; ps < GPASS; ++ps) stage[ps] = *reinterpret_cast<const u32x4*>(xsrc[ps] + (c + 1) * GK);
     }
+    // the loads above are issued here and waited for after the products: without the fence the
+    // compiler moves each load down to the LDS store that uses it and waits for it at once
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int j = 0; j < GK / 32; ++j) {
+      // 16-row groups four at a time: four LDS reads go out together, then their eight MFMAs;
+      // a quartet with no rows at all is skipped (uniform over the block), a partly filled one is
+      // multiplied whole (rows beyond the expert's last are never stored)
 #pragma unroll
-      for (int mb = 0; mb < GMT; ++mb) {
-        if (mb < n_mt) {   // uniform over the block
-          const bf16x8 xf = *reinterpret_cast<const bf16x8*>(&xs[buf][mb * 16 + r][j * 32 + g * 8]);
+      for (int mq = 0; mq < GMT; mq += 4) {
+        if (mq < n_mt) {
+          bf16x8 xf[4];
 #pragma unroll
-          for (int t = 0; t < NT; ++t)
-            acc[t][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[slot][j][t], xf, acc[t][mb], 0, 0, 0);
+          for (int i = 0; i < 4; ++i) xf[i] = *reinterpret_cast<const bf16x8*>(&xs[buf][(mq + i) * 16 + r][j * 32 + g * 8]);
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+              acc[t][mq + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[slot][j][t], xf[i], acc[t][mq + i], 0, 0, 0);
         }
       }
     }
-    if (c + kAhead < chunks) {   // this slot's weights are used up: fetch those of kAhead stages on
+    __builtin_amdgcn_sched_barrier(0);
+    if (steady || c + kAhead < chunks) {   // this slot's weights are used up: fetch those of kAhead stages on
 #pragma unroll
       for (int j = 0; j < GK / 32; ++j)
 #pragma unroll
         for (int t = 0; t < NT; ++t)
           wf[slot][j][t] = *reinterpret_cast<const bf16x8*>(wrow[t] + (c + kAhead) * GK + j * 32);
     }
-    if (c + 1 < chunks) {
+    if (steady || c + 1 < chunks) {
 #pragma unroll
-      for (int ps = 0; ps < GPASS; ++ps)
-        if (srow + GROWS * ps < n_mt * 16) *reinterpret_cast<uint4*>(&xs[buf ^ 1][srow + GROWS * ps][scol]) = stage[ps];
+      for (int ps = 0; ps < GPASS; ++ps) *reinterpret_cast<u32x4*>(&xs[buf ^ 1][srow + GROWS * ps][scol]) = stage[ps];
     }
     __syncthreads();
   };
   static_assert(kAhead == 4, "the loop below is unrolled for a ring of four");
-  for (int c = 0; c < chunks; c += kAhead) {
-    stage_step(c, std::integral_constant<int, 0>{});
-    if (c + 1 < chunks) stage_step(c + 1, std::integral_constant<int, 1>{});
-    if (c + 2 < chunks) stage_step(c + 2, std::integral_constant<int, 2>{});
-    if (c + 3 < chunks) stage_step(c + 3, std::integral_constant<int, 3>{});
+  int c = 0;
+  for (; c + 2 * kAhead <= chunks; c += kAhead) {   // all four stages fetch weights of stages that exist
+    stage_step(c, std::integral_constant<int, 0>{}, std::true_type{});
+    stage_step(c + 1, std::integral_constant<int, 1>{}, std::true_type{});
+    stage_step(c + 2, std::integral_constant<int, 2>{}, std::true_type{});
+    stage_step(c + 3, std::integral_constant<int, 3>{}, std::true_type{});
+  }
+  for (; c < chunks; c += kAhead) {   // the last stages: what they fetch is checked one by one
+    stage_step(c, std::integral_constant<int, 0>{}, std::false_type{});
+    if (c + 1 < chunks) stage_step(c + 1, std::integral_constant<int, 1>{}, std::false_type{});
+    if (c + 2 < chunks) stage_step(c + 2, std::integral_constant<int, 2>{}, std::false_type{});
+    if (c + 3 < chunks) stage_step(c + 3, std::integral_constant<int, 3>{}, std::false_type{});
   }
 
   // lane holds out[row0 + mb*16 + r][n_base + t*16 + 4g + 0..3]
