@@ -12,19 +12,22 @@
 // and the S^T accumulator of a lane is the B operand of the second product once exponentiated
 // and split into a bfloat16 pair hi + lo.  In LDS the value columns are permuted so that the
 // eight keys a lane needs (4 of each 16-key block) sit side by side; rows are padded so that the
-// 16 lanes of a quarter-wave hit 16 different bank groups.  Softmax state (running max and sum
-// per query) is float, kept in base-2 units (scores times log2 e, the hardware's exp2).  The keys of a query are always visited in the same blocks, whatever the
-// portion it arrived in, so its sums do not depend on how the prompt was cut.
+// 16 lanes of a quarter-wave hit 16 different bank groups.  Softmax state (a reference maximum and
+// the sum per query) is float, kept in base-2 units (scores times log2 e, the hardware's exp2).
+// The keys of a query are always visited in the same blocks, whatever the portion it arrived in,
+// so its sums do not depend on how the prompt was cut.
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
 constexpr int kPreWaves = 4;
 constexpr int kQT = 2;                               // 16-token column tiles per wave
 constexpr int kWaveTokens = 16 * kQT;
 constexpr int kTileTokens = kWaveTokens * kPreWaves; // 128 tokens per block
 constexpr int kVPad = 40;                            // LDS row of the value tile: 32 keys + 8
+constexpr float kLazyMax = 8.0f;                     // how far the row maximum may outgrow its reference
 
 template <int HD>
 __global__ __launch_bounds__(kPreWaves* kWave) void attn_prefill_kernel(
@@ -44,8 +47,10 @@ __global__ __launch_bounds__(kPreWaves* kWave) void attn_prefill_kernel(
   const int lane = tid & (kWave - 1);
   const int w = tid >> 6;
   const int r = lane & 15, g = lane >> 4;
-  const int ti = blockIdx.x;
-  const int h = blockIdx.y;
+  // heads run fastest and tiles from the last backwards: later tiles of a prompt see more keys, and
+  // the longest blocks should start first
+  const int ti = gridDim.y - 1 - blockIdx.y;
+  const int h = blockIdx.x;
   const int kvh = h / (nh / nkv);
   const int entry = tiles[ti * 3], tok0 = tiles[ti * 3 + 1], rows = tiles[ti * 3 + 2];
   const int pos0 = positions[tok0];
@@ -65,11 +70,12 @@ __global__ __launch_bounds__(kPreWaves* kWave) void attn_prefill_kernel(
     if (window_kind == 1) st = (qpos[c] / window) * window;
     else if (window_kind == 2) st = qpos[c] - window + 1 > 0 ? qpos[c] - window + 1 : 0;
     qstart[c] = st;
+    // rows beyond the tile's last read its last row (every load unconditional, see the note on the
+    // chunk loop); their scores are masked and their output is never stored
+    const int qrow = min(row, rows - 1);
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-      if (qok[c]) qf[c][j] = *reinterpret_cast<const bf16x8*>(q + ((size_t)(tok0 + row) * nh + h) * HD + j * 32 + g * 8);
-      else qf[c][j] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
-    }
+    for (int j = 0; j < NJ; ++j)
+      qf[c][j] = *reinterpret_cast<const bf16x8*>(q + ((size_t)(tok0 + qrow) * nh + h) * HD + j * 32 + g * 8);
   }
   const int wave_last = pos0 + min(rows, wrow0 + kWaveTokens) - 1;   // last position of this wave's rows
   const bool wave_has_rows = wrow0 < rows;
@@ -100,38 +106,41 @@ __global__ __launch_bounds__(kPreWaves* kWave) void attn_prefill_kernel(
     for (int d = 0; d < ND; ++d) acc[c][d] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
-  // staging: fetch the chunk that starts at 16-key block b into registers
-  uint4 kst[NST], vst[NST];
+  // The block table of the entry, 64 pages at a time, one per lane (and the next 64 behind them):
+  // a chunk's pages come out of a register with a uniform lane read, not out of memory, so the
+  // address of a chunk's keys does not wait for a load of its own.
+  int pv_base = (b_first << 4) / page_size;
+  auto load_pages = [&](int base) { return bt[min(base + lane, max_blocks - 1)]; };
+  int pv = load_pages(pv_base), pv_next = load_pages(pv_base + kWave);
+  auto page_of = [&](int bb) {                               // bb uniform, within the 128 pages held
+    const int pi = (bb << 4) / page_size - pv_base;
+    const int page = pi < kWave ? __builtin_amdgcn_readlane(pv, pi) : __builtin_amdgcn_readlane(pv_next, pi - kWave);
+    return min(max(page, 0), num_pages - 1);                 // a table that is wrong reads a wrong page, never outside
+  };
+
+  // staging: fetch the chunk that starts at 16-key block b into registers.  Every load is
+  // unconditional: a 16-key block beyond the tile's last is fetched as the last one again (its
+  // keys are masked, its values are finite and meet probabilities of zero).  The compiler counts
+  // outstanding loads statically; one load behind a branch and every wait in the loop becomes a
+  // wait for all loads, the chunk in flight included.
+  u32x4 kst[NST], vst[NST];
   auto fetch = [&](int b) {
     long long kbase[2], vbase[2];
-    bool have[2];
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
-      const int bb = b + u;
-      have[u] = bb <= b_last;
-      int page = -1;
-      if (have[u]) {
-        const int pi = (bb << 4) / page_size;
-        page = pi < max_blocks ? bt[pi] : -1;
-        if (page < 0 || page >= num_pages) have[u] = false;
-      }
+      const int bb = min(b + u, b_last);
+      const int page = page_of(bb);
       const int off = (bb << 4) % page_size;
-      kbase[u] = have[u] ? (((long long)page * nkv + kvh) * page_size + off) * HD : 0;
-      vbase[u] = have[u] ? ((long long)page * nkv + kvh) * HD * page_size + off : 0;
+      kbase[u] = (((long long)page * nkv + kvh) * page_size + off) * HD;
+      vbase[u] = ((long long)page * nkv + kvh) * HD * page_size + off;
     }
 #pragma unroll
     for (int i = 0; i < NST; ++i) {
-      const int piece = tid + i * kPreWaves * kWave;
-      kst[i] = uint4{0u, 0u, 0u, 0u};
-      vst[i] = uint4{0u, 0u, 0u, 0u};
-      if (piece < PIECES) {
-        const int key = piece / (HD / 8), dcol = (piece % (HD / 8)) * 8;     // K: 32 keys x HD
-        if (have[key >> 4])
-          kst[i] = *reinterpret_cast<const uint4*>(k_cache + kbase[key >> 4] + (size_t)(key & 15) * HD + dcol);
-        const int d = piece >> 2, blk = (piece >> 1) & 1, half = piece & 1;  // V^T: HD rows x 2 blocks x 2 halves
-        if (have[blk])
-          vst[i] = *reinterpret_cast<const uint4*>(v_cache + vbase[blk] + (size_t)d * page_size + half * 8);
-      }
+      const int piece = min(tid + i * kPreWaves * kWave, PIECES - 1);
+      const int key = piece / (HD / 8), dcol = (piece % (HD / 8)) * 8;     // K: 32 keys x HD
+      kst[i] = *reinterpret_cast<const u32x4*>(k_cache + kbase[key >> 4] + (size_t)(key & 15) * HD + dcol);
+      const int d = piece >> 2, blk = (piece >> 1) & 1, half = piece & 1;  // V^T: HD rows x 2 blocks x 2 halves
+      vst[i] = *reinterpret_cast<const u32x4*>(v_cache + vbase[blk] + (size_t)d * page_size + half * 8);
     }
   };
   auto stash = [&](int buf) {
@@ -140,7 +149,7 @@ __global__ __launch_bounds__(kPreWaves* kWave) void attn_prefill_kernel(
       const int piece = tid + i * kPreWaves * kWave;
       if (piece < PIECES) {
         const int key = piece / (HD / 8), dcol = (piece % (HD / 8)) * 8;
-        *reinterpret_cast<uint4*>(&Ks[buf][key][dcol]) = kst[i];
+        *reinterpret_cast<u32x4*>(&Ks[buf][key][dcol]) = kst[i];
         // keys 8*half .. 8*half+7 of block blk: groups g = 2*half and 2*half + 1, four keys each;
         // column of (g, blk) = g*8 + blk*4
         const int d = piece >> 2, blk = (piece >> 1) & 1, half = piece & 1;
@@ -156,7 +165,14 @@ __global__ __launch_bounds__(kPreWaves* kWave) void attn_prefill_kernel(
   int buf = 0;
   for (int b = b_first; b <= b_last; b += 2, buf ^= 1) {
     const bool more = b + 2 <= b_last;
-    if (more) fetch(b + 2);
+    const int b_next = more ? b + 2 : b;                     // after the last chunk: the same one again, unused
+    if ((((b_next + 1) << 4) / page_size) - pv_base >= 2 * kWave - 1) {   // the pages held run out: move on by 64
+      pv = pv_next;
+      pv_base += kWave;
+      pv_next = load_pages(pv_base + kWave);
+    }
+    fetch(b_next);
+    __builtin_amdgcn_sched_barrier(0);                       // the loads are issued here, not where they are used
     // does any row of this wave see a key of this chunk?
     const bool active = wave_has_rows && (b << 4) <= wave_last && ((b + 2) << 4) > wave_first;
     if (active) {
@@ -199,7 +215,13 @@ __global__ __launch_bounds__(kPreWaves* kWave) void attn_prefill_kernel(
           }
         cm = fmaxf(cm, __shfl_xor(cm, 16, kWave));
         cm = fmaxf(cm, __shfl_xor(cm, 32, kWave));
-        const float m_new = fmaxf(m[c], cm);
+        // m is a reference, not the exact running maximum: it moves only when the maximum has grown
+        // past it by more than kLazyMax (base-2 units), so probabilities reach 2^kLazyMax at most, which
+        // float sums carry easily, and the accumulators are rescaled in few chunks.  The decision
+        // is the row's own (its four lanes hold the same m and cm), so what a row ends up with does
+        // not depend on the rows it shares a wave with.
+        const float m_true = fmaxf(m[c], cm);
+        const float m_new = (m_true - m[c] > kLazyMax) ? m_true : m[c];   // from -inf: inf > kLazyMax; all masked: NaN, stays
         corr[c] = 1.0f;
         if (m_new == -INFINITY) {
           pf[c] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
@@ -236,7 +258,8 @@ __global__ __launch_bounds__(kPreWaves* kWave) void attn_prefill_kernel(
         }
       }
     }
-    if (more) stash(buf ^ 1);
+    __builtin_amdgcn_sched_barrier(0);
+    stash(buf ^ 1);
     __syncthreads();
   }
 
@@ -269,10 +292,10 @@ SHARPI_EXPORT int sharpi_attention_prefill(const void* q, const void* k_cache, c
                                            int nh, int nkv, int hd, int page_size, int max_blocks, int num_pages,
                                            hipStream_t stream) {
   if (n_tiles <= 0) return SHARPI_OK;
-  if (nh <= 0 || nkv <= 0 || nh % nkv != 0 || nh > 65535) return SHARPI_ERR_ARG;
+  if (nh <= 0 || nkv <= 0 || nh % nkv != 0 || n_tiles > 65535) return SHARPI_ERR_ARG;
   if (page_size <= 0 || page_size % 16 != 0 || max_blocks <= 0 || num_pages <= 0) return SHARPI_ERR_ARG;
   if (window_kind < 0 || window_kind > 2 || (window_kind != 0 && window <= 0)) return SHARPI_ERR_ARG;
-  dim3 grid(n_tiles, nh), block(kPreWaves * kWave);
+  dim3 grid(nh, n_tiles), block(kPreWaves * kWave);
 #define PRE(HDV)                                                                                              \
   if (hd == HDV) {                                                                                            \
     attn_prefill_kernel<HDV><<<grid, block, 0, stream>>>((const bf16_t*)q, (const bf16_t*)k_cache,            \

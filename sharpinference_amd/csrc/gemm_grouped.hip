@@ -6,12 +6,14 @@
 // that fit one tile (192, about one and a half times the mean load of 2,048 tokens over 16
 // experts) against 128 weight rows: a typical expert's weights are then read once.  Tiles are
 // listed on the device by the routing kernel (tile_expert, tile_row0, n_tiles); the host never
-// learns the routing, and quartets of 16-row groups beyond an expert's last row are skipped, not multiplied.
+// learns the routing.  The tile's work is compiled three times, for 64, 128 and 192 rows, and a
+// block takes the smallest that holds its rows: no branch inside a K stage, nothing multiplied or
+// staged for 64-row quarters that hold no row.
 //  * Each of the 4 waves owns 32 weight rows (2 MFMA tiles) and reads them straight from global
-//    memory into registers, four 64-wide K stages ahead: a weight element is used by one wave only.
+//    memory into registers, a ring of 64-wide K stages ahead: a weight element is used by one wave only.
 //  * The x rows (gathered through a_rows) are shared by the waves and staged through LDS, 64
-//    columns of K at a time, double-buffered; rows are padded to 72 elements so that the 16
-//    lanes of a quarter-wave read 16 different banks.
+//    columns of K at a time, double-buffered and fetched two stages ahead; rows are padded to 72
+//    elements so that the 16 lanes of a quarter-wave read 16 different banks.
 //  * W is the A operand (rows = n), x the B operand: a lane ends up with 4 consecutive n of one
 //    row, stored as one 8-byte write.  Each output is one chain over k in ascending order, so a
 //    row's result does not depend on which other rows share its tile.
@@ -27,6 +29,12 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 #ifndef SHARPI_GM
 #define SHARPI_GM 192
 #endif
+#ifndef SHARPI_GAHEAD
+#define SHARPI_GAHEAD 2
+#endif
+#ifndef SHARPI_GQ
+#define SHARPI_GQ 4
+#endif
 #ifndef SHARPI_GK
 #define SHARPI_GK 64
 #endif
@@ -36,69 +44,65 @@ constexpr int GW = 4;         // waves per block
 constexpr int NT = 2;         // 16-row weight tiles per wave
 constexpr int GN = 16 * NT * GW;   // columns per tile
 constexpr int GK = SHARPI_GK;  // K per LDS stage
-constexpr int GPAD = GK + 8;  // padded LDS row
+#ifndef SHARPI_GPADX
+#define SHARPI_GPADX 8
+#endif
+constexpr int GPAD = GK + SHARPI_GPADX;  // padded LDS row
 constexpr int GROWS = GW * 64 / (GK / 8);   // rows staged per pass: GK / 8 threads per row
 constexpr int GPASS = GM / GROWS;  // staging passes
 constexpr int kXcds = 8;           // accelerator dies, each with its own L2
-constexpr int kAhead = 4;           // K stages of weights in flight per wave
+constexpr int kAhead = SHARPI_GAHEAD;  // K stages of weights in flight per wave (2, 3 or 4)
+constexpr int GQ = SHARPI_GQ;       // 16-row groups whose LDS reads go out together (divides 4)
 constexpr int kHalves = 2;         // a tile's column blocks are split over this many XCDs
 
-template <typename TO>
-__global__ __launch_bounds__(GW* kWave) void grouped_gemm_kernel(
-    const bf16_t* __restrict__ x, const bf16_t* __restrict__ W, TO* __restrict__ out, int N, int K,
-    const int* __restrict__ a_rows, const int* __restrict__ group_offsets, const int* __restrict__ tile_expert,
-    const int* __restrict__ tile_row0, const int* __restrict__ n_tiles, int nb_per_unit) {
-  __shared__ __attribute__((aligned(16))) bf16_t xs[2][GM][GPAD];
-  // Workgroups go to the 8 XCDs round-robin by their linear id, and each XCD has an L2 of its
-  // own.  All column blocks of one (tile, half of the columns) unit are therefore given ids that
-  // are equal modulo 8: the unit's x rows are fetched into one L2 and stay there.
-  const int xcd = blockIdx.x % kXcds;
-  const int slot = blockIdx.x / kXcds;
-  const int unit = (slot / nb_per_unit) * kXcds + xcd;
-  const int tile = unit / kHalves;
-  const int nblock = (unit % kHalves) * nb_per_unit + slot % nb_per_unit;
-  if (tile >= n_tiles[0] || nblock * GN >= N) return;
-  const int e = tile_expert[tile];
-  const int row0 = tile_row0[tile];
-  const int row_end = group_offsets[e + 1];
-  const int n_rows = min(GM, row_end - row0);
-  const int n_mt = (n_rows + 15) >> 4;           // 16-row groups that hold rows
+// The work of one tile of NQ * 64 rows (the block's rows, rounded up) against GN weight rows.
+template <typename TO, int NQ>
+__device__ __forceinline__ void grouped_tile(const bf16_t* __restrict__ x, const bf16_t* __restrict__ We,
+                                             TO* __restrict__ out, int N, int K, const int* __restrict__ a_rows,
+                                             int row0, int row_end, int n_base, bf16_t (*xs)[GM][GPAD]) {
+  constexpr int MT = NQ * 4;                    // 16-row groups
+  constexpr int PASS = NQ * 64 / GROWS;         // staging passes
   const int lane = threadIdx.x & (kWave - 1);
-  const int w = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
-  const int n_base = nblock * GN + w * 16 * NT;
-  const bf16_t* We = W + (size_t)e * N * K;
 
-  const bf16_t* wrow[NT];
+  // 32-bit element offsets from uniform bases (the host checks that they fit): half the address registers
+  uint32_t woff[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
     int n = n_base + t * 16 + r;
     if (n >= N) n = N - 1;  // loaded, never stored
-    wrow[t] = We + (size_t)n * K + g * 8;
+    woff[t] = (uint32_t)n * (uint32_t)K + g * 8;
   }
   // staging role: thread loads 16 bytes of row (tid / 8 + GROWS * pass), columns (tid % 8) * 8
   const int srow = threadIdx.x / (GK / 8), scol = (threadIdx.x % (GK / 8)) * 8;
-  const bf16_t* xsrc[GPASS];
+  uint32_t xoff[PASS];
 #pragma unroll
-  for (int ps = 0; ps < GPASS; ++ps) {
+  for (int ps = 0; ps < PASS; ++ps) {
     // rows beyond the expert's last read its last row again: every load is unconditional, and what
     // such rows produce is never stored
     const int row = min(row0 + srow + GROWS * ps, row_end - 1);
-    xsrc[ps] = x + (size_t)(a_rows ? a_rows[row] : row) * K + scol;
+    xoff[ps] = (uint32_t)(a_rows ? a_rows[row] : row) * (uint32_t)K + scol;
   }
 
-  f32x4 acc[NT][GMT];
+  f32x4 acc[NT][MT];
 #pragma unroll
   for (int t = 0; t < NT; ++t)
 #pragma unroll
-    for (int mb = 0; mb < GMT; ++mb) acc[t][mb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int mb = 0; mb < MT; ++mb) acc[t][mb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   const int chunks = K / GK;
-  u32x4 stage[GPASS];
+  // The memory counter retires loads in order, so waiting for one load waits for every load issued
+  // before it.  Both streams therefore run the same distance ahead: x rows of stage c + 2 go into
+  // one of two register sets while stage c is multiplied (and into LDS one stage later), weights
+  // of stage c + kAhead into the ring slot that stage c has just used up.
+  u32x4 stage[2][PASS];
   bf16x8 wf[kAhead][GK / 32][NT];   // weight fragments of the next kAhead stages, a ring indexed by stage % kAhead
 #pragma unroll
-  for (int ps = 0; ps < GPASS; ++ps)
-    stage[ps] = *reinterpret_cast<const u32x4*>(xsrc[ps]);
+  for (int ps = 0; ps < PASS; ++ps) stage[0][ps] = *reinterpret_cast<const u32x4*>(x + xoff[ps]);
+  if (chunks > 1) {
+#pragma unroll
+    for (int ps = 0; ps < PASS; ++ps) stage[1][ps] = *reinterpret_cast<const u32x4*>(x + xoff[ps] + GK);
+  }
   auto fill_ring = [&](auto all_tag) {
 #pragma unroll
     for (int a = 0; a < kAhead; ++a)
@@ -106,47 +110,42 @@ __global__ __launch_bounds__(GW* kWave) void grouped_gemm_kernel(
 #pragma unroll
         for (int j = 0; j < GK / 32; ++j)
 #pragma unroll
-          for (int t = 0; t < NT; ++t) wf[a][j][t] = *reinterpret_cast<const bf16x8*>(wrow[t] + a * GK + j * 32);
+          for (int t = 0; t < NT; ++t) wf[a][j][t] = *reinterpret_cast<const bf16x8*>(We + woff[t] + a * GK + j * 32);
       }
   };
   if (chunks >= kAhead) fill_ring(std::true_type{}); else fill_ring(std::false_type{});
 #pragma unroll
-  for (int ps = 0; ps < GPASS; ++ps)
-    *reinterpret_cast<u32x4*>(&xs[0][srow + GROWS * ps][scol]) = stage[ps];
+  for (int ps = 0; ps < PASS; ++ps) *reinterpret_cast<u32x4*>(&xs[0][srow + GROWS * ps][scol]) = stage[0][ps];
   __syncthreads();
 
-  // one K stage; `slot` is the stage's place in the ring and a compile-time constant
-  // `steady`: every load of the stage is known to be in range, so none sits behind a branch.  The
-  // compiler counts outstanding loads statically; a load that may or may not have been issued makes
-  // it wait for all of them, and the ring would hide nothing.
-  auto stage_step = [&](int c, auto slot_tag, auto steady_tag) {
+  // One K stage; `slot` (the stage's place in the ring) and `par` (its parity) are compile-time
+  // constants.  `steady`: every load of the stage is known to be in range, so none sits behind a
+  // branch.  The compiler counts outstanding loads statically; a load that may or may not have been
+  // issued makes it wait for all of them, and nothing would be hidden.
+  auto stage_step = [&](int c, auto slot_tag, auto par_tag, auto steady_tag) {
     constexpr int slot = decltype(slot_tag)::value;
+    constexpr int par = decltype(par_tag)::value;
     constexpr bool steady = decltype(steady_tag)::value;
-    const int buf = c & 1;
-    if (steady || c + 1 < chunks) {   // the next stage's x rows are on their way while this one is multiplied
+    if (steady || c + 2 < chunks) {   // this stage's register set went to LDS a stage ago
 #pragma unroll
-      for (int ps = 0; ps < GPASS; ++ps) stage[ps] = *reinterpret_cast<const u32x4*>(xsrc[ps] + (c + 1) * GK);
+      for (int ps = 0; ps < PASS; ++ps) stage[par][ps] = *reinterpret_cast<const u32x4*>(x + xoff[ps] + (c + 2) * GK);
     }
-    // the loads above are issued here and waited for after the products: without the fence the
-    // compiler moves each load down to the LDS store that uses it and waits for it at once
+    // the loads above are issued here and waited for a stage later: without the fence the compiler
+    // moves each load down to the LDS store that uses it and waits for it at once
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int j = 0; j < GK / 32; ++j) {
-      // 16-row groups four at a time: four LDS reads go out together, then their eight MFMAs;
-      // a quartet with no rows at all is skipped (uniform over the block), a partly filled one is
-      // multiplied whole (rows beyond the expert's last are never stored)
+      // 16-row groups GQ at a time: their LDS reads go out together, then their MFMAs
 #pragma unroll
-      for (int mq = 0; mq < GMT; mq += 4) {
-        if (mq < n_mt) {
-          bf16x8 xf[4];
+      for (int mq = 0; mq < MT; mq += GQ) {
+        bf16x8 xf[GQ];
 #pragma unroll
-          for (int i = 0; i < 4; ++i) xf[i] = *reinterpret_cast<const bf16x8*>(&xs[buf][(mq + i) * 16 + r][j * 32 + g * 8]);
+        for (int i = 0; i < GQ; ++i) xf[i] = *reinterpret_cast<const bf16x8*>(&xs[par][(mq + i) * 16 + r][j * 32 + g * 8]);
 #pragma unroll
-          for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < GQ; ++i)
 #pragma unroll
-            for (int t = 0; t < NT; ++t)
-              acc[t][mq + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[slot][j][t], xf[i], acc[t][mq + i], 0, 0, 0);
-        }
+          for (int t = 0; t < NT; ++t)
+            acc[t][mq + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[slot][j][t], xf[i], acc[t][mq + i], 0, 0, 0);
       }
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -155,34 +154,37 @@ __global__ __launch_bounds__(GW* kWave) void grouped_gemm_kernel(
       for (int j = 0; j < GK / 32; ++j)
 #pragma unroll
         for (int t = 0; t < NT; ++t)
-          wf[slot][j][t] = *reinterpret_cast<const bf16x8*>(wrow[t] + (c + kAhead) * GK + j * 32);
+          wf[slot][j][t] = *reinterpret_cast<const bf16x8*>(We + woff[t] + (c + kAhead) * GK + j * 32);
     }
-    if (steady || c + 1 < chunks) {
+    if (steady || c + 1 < chunks) {   // the next stage's x rows, fetched a stage ago
 #pragma unroll
-      for (int ps = 0; ps < GPASS; ++ps) *reinterpret_cast<u32x4*>(&xs[buf ^ 1][srow + GROWS * ps][scol]) = stage[ps];
+      for (int ps = 0; ps < PASS; ++ps) *reinterpret_cast<u32x4*>(&xs[par ^ 1][srow + GROWS * ps][scol]) = stage[par ^ 1][ps];
     }
     __syncthreads();
   };
-  static_assert(kAhead == 4, "the loop below is unrolled for a ring of four");
+  // stages are unrolled over ring slot x parity, so that both are constants
+  constexpr int kUnroll = (kAhead % 2 == 0) ? kAhead : 2 * kAhead;
+  auto stage_group = [&](int c, auto steady_tag) {
+    auto one = [&](auto i_tag) {
+      constexpr int i = decltype(i_tag)::value;
+      if (decltype(steady_tag)::value || c + i < chunks)
+        stage_step(c + i, std::integral_constant<int, i % kAhead>{}, std::integral_constant<int, i % 2>{}, steady_tag);
+    };
+    // exactly kUnroll stages: the loops below advance by that many
+    one(std::integral_constant<int, 0>{}); one(std::integral_constant<int, 1>{});
+    if constexpr (kUnroll > 2) { one(std::integral_constant<int, 2>{}); one(std::integral_constant<int, 3>{}); }
+    if constexpr (kUnroll > 4) { one(std::integral_constant<int, 4>{}); one(std::integral_constant<int, 5>{}); }
+    static_assert(kUnroll == 2 || kUnroll == 4 || kUnroll == 6, "stage_group lists two, four or six stages");
+  };
   int c = 0;
-  for (; c + 2 * kAhead <= chunks; c += kAhead) {   // all four stages fetch weights of stages that exist
-    stage_step(c, std::integral_constant<int, 0>{}, std::true_type{});
-    stage_step(c + 1, std::integral_constant<int, 1>{}, std::true_type{});
-    stage_step(c + 2, std::integral_constant<int, 2>{}, std::true_type{});
-    stage_step(c + 3, std::integral_constant<int, 3>{}, std::true_type{});
-  }
-  for (; c < chunks; c += kAhead) {   // the last stages: what they fetch is checked one by one
-    stage_step(c, std::integral_constant<int, 0>{}, std::false_type{});
-    if (c + 1 < chunks) stage_step(c + 1, std::integral_constant<int, 1>{}, std::false_type{});
-    if (c + 2 < chunks) stage_step(c + 2, std::integral_constant<int, 2>{}, std::false_type{});
-    if (c + 3 < chunks) stage_step(c + 3, std::integral_constant<int, 3>{}, std::false_type{});
-  }
+  for (; c + kUnroll + kAhead <= chunks; c += kUnroll) stage_group(c, std::true_type{});   // every fetch is of a stage that exists
+  for (; c < chunks; c += kUnroll) stage_group(c, std::false_type{});                      // the last stages check each fetch
 
   // lane holds out[row0 + mb*16 + r][n_base + t*16 + 4g + 0..3]
 #pragma unroll
-  for (int mb = 0; mb < GMT; ++mb) {
+  for (int mb = 0; mb < MT; ++mb) {
     const int row = row0 + mb * 16 + r;
-    if (mb >= n_mt || row >= row_end) continue;
+    if (row >= row_end) continue;
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       const int n = n_base + t * 16 + 4 * g;
@@ -200,16 +202,49 @@ __global__ __launch_bounds__(GW* kWave) void grouped_gemm_kernel(
   }
 }
 
-// x [*, K] bf16 (rows gathered through a_rows if given), W [E, N, K] bf16, out [n_rows, N];
+template <typename TO>
+__global__ __launch_bounds__(GW* kWave, 2) void grouped_gemm_kernel(
+    const bf16_t* __restrict__ x, const bf16_t* __restrict__ W, TO* __restrict__ out, int N, int K,
+    const int* __restrict__ a_rows, const int* __restrict__ group_offsets, const int* __restrict__ tile_expert,
+    const int* __restrict__ tile_row0, const int* __restrict__ n_tiles, int nb_per_unit) {
+  __shared__ __attribute__((aligned(16))) bf16_t xs[2][GM][GPAD];
+  // Workgroups go to the 8 XCDs round-robin by their linear id, and each XCD has an L2 of its
+  // own.  All column blocks of one (tile, half of the columns) unit are therefore given ids that
+  // are equal modulo 8: the unit's x rows are fetched into one L2 and stay there.
+  const int xcd = blockIdx.x % kXcds;
+  const int slot = blockIdx.x / kXcds;
+  const int unit = (slot / nb_per_unit) * kXcds + xcd;
+  const int tile = unit / kHalves;
+  const int nblock = (unit % kHalves) * nb_per_unit + slot % nb_per_unit;
+  if (tile >= n_tiles[0] || nblock * GN >= N) return;
+  const int e = tile_expert[tile];
+  const int row0 = tile_row0[tile];
+  const int row_end = min(group_offsets[e + 1], row0 + GM);   // the tile's rows end here; later ones are another tile's
+  const int n_rows = row_end - row0;
+  if (n_rows <= 0) return;
+  const int n_base = nblock * GN + (threadIdx.x >> 6) * 16 * NT;
+  const bf16_t* We = W + (size_t)e * N * K;
+  static_assert(GM == 192, "three tile heights are compiled: 64, 128 and 192 rows");
+  if (n_rows <= 64)
+    grouped_tile<TO, 1>(x, We, out, N, K, a_rows, row0, row_end, n_base, xs);
+  else if (n_rows <= 128)
+    grouped_tile<TO, 2>(x, We, out, N, K, a_rows, row0, row_end, n_base, xs);
+  else
+    grouped_tile<TO, 3>(x, We, out, N, K, a_rows, row0, row_end, n_base, xs);
+}
+
+// x [x_rows, K] bf16 (rows gathered through a_rows if given), W [E, N, K] bf16, out [n_rows, N];
 // group_offsets [E + 1]; tile_expert / tile_row0 [max_tiles], n_tiles [1] from the routing kernel
 // (tiles of sharpi_gemm_grouped_tile_rows() rows).  max_tiles bounds the grid.
-SHARPI_EXPORT int sharpi_gemm_grouped(const void* x, const void* W, void* out, int out_dtype, int n_rows, int N,
-                                      int K, const int* a_rows, const int* group_offsets, const int* tile_expert,
+SHARPI_EXPORT int sharpi_gemm_grouped(const void* x, int x_rows, const void* W, void* out, int out_dtype, int n_rows,
+                                      int N, int K, const int* a_rows, const int* group_offsets, const int* tile_expert,
                                       const int* tile_row0, const int* n_tiles, int max_tiles,
                                       hipStream_t stream) {
   if (n_rows <= 0) return SHARPI_OK;
   if (N <= 0 || (N & 3) || K <= 0 || K % GK != 0 || max_tiles <= 0) return SHARPI_ERR_ARG;
   if (!group_offsets || !tile_expert || !tile_row0 || !n_tiles) return SHARPI_ERR_ARG;
+  // the kernel addresses x and one expert's weights with 32-bit element offsets
+  if ((long long)N * K > 0x7fffffffLL || x_rows <= 0 || (long long)x_rows * K > 0x7fffffffLL) return SHARPI_ERR_ARG;
   const int nb_per_unit = ceil_div(ceil_div(N, GN), kHalves);
   const int units = ceil_div(max_tiles * kHalves, kXcds) * kXcds;
   dim3 grid(units * nb_per_unit), block(GW * kWave);

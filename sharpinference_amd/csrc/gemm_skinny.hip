@@ -154,7 +154,8 @@ static int dispatch_mb(int MB, const void* x, const void* W, void* out, int out_
 // x [M, K] bf16 (rows gathered through a_rows if given), W [N, K] or [groups, N, K] bf16,
 // out [M, N] (out_dtype float or bf16).  groups == 0: plain.  groups > 0: rows are the
 // expert-sorted list, group_offsets [groups + 1].  R in {1, 2, 4}: 16-row weight tiles per block;
-// NW in {4, 8, 16}: waves per block splitting K.
+// NW in {4, 8, 16}: waves per block splitting K (16 only with R = 1: a block of 1,024 threads has
+// 128 registers a lane, which wider tiles do not fit).
 SHARPI_EXPORT int sharpi_gemm_skinny(const void* x, const void* W, void* out, int out_dtype, int M, int N, int K,
                                      const int* a_rows, const int* group_offsets, int groups, int R, int NW,
                                      hipStream_t stream) {
@@ -167,8 +168,8 @@ SHARPI_EXPORT int sharpi_gemm_skinny(const void* x, const void* W, void* out, in
 #define SK(RR, WW) \
   if (R == RR && NW == WW) return dispatch_mb<RR, WW>(MB, x, W, out, out_dtype, M, N, K, a_rows, group_offsets, groups, stream)
   SK(1, 4); SK(1, 8); SK(1, 16);
-  SK(2, 4); SK(2, 8); SK(2, 16);
-  SK(4, 4); SK(4, 8); SK(4, 16);
+  SK(2, 4); SK(2, 8);
+  SK(4, 4); SK(4, 8);
 #undef SK
   return SHARPI_ERR_ARG;
 }

@@ -434,7 +434,7 @@ def gemm_grouped(x: torch.Tensor, w: torch.Tensor, rt: Routing, gather: bool, ou
     _need(K % 64 == 0 and N % 4 == 0, "gemm_grouped: K % 64 == 0 and N % 4 == 0 wanted")
     _need(x.shape[0] == (rt.n_tokens if gather else rt.n_rows), "gemm_grouped: x has the wrong number of rows")
     out = torch.empty(rt.n_rows, N, dtype=out_dtype, device=x.device)
-    _run("sharpi_gemm_grouped", _ptr(x), _ptr(w), _ptr(out), _code(out_dtype), rt.n_rows, N, K,
+    _run("sharpi_gemm_grouped", _ptr(x), x.shape[0], _ptr(w), _ptr(out), _code(out_dtype), rt.n_rows, N, K,
          _ptr(rt.sorted_token) if gather else None, _ptr(rt.offsets), _ptr(rt.tile_expert), _ptr(rt.tile_row0),
          _ptr(rt.n_tiles), rt.max_tiles, _stream())
     return out

@@ -30,6 +30,8 @@ def test_gemm_skinny(M, N, K, out_dtype):
     ref = x.float() @ w.float().T
     for R in (1, 2, 4):
         for NW in (4, 8, 16):
+            if NW == 16 and R > 1:
+                continue   # refused: 1,024-thread blocks only take one weight tile
             got = ops.gemm_skinny(x, w, out_dtype, R=R, NW=NW).float()
             tol = 2e-2 if out_dtype == torch.bfloat16 else 1e-3
             assert float((got - ref).abs().max()) <= tol * float(ref.abs().max()), (M, N, K, R, NW)
@@ -183,7 +185,9 @@ def test_router_ties_pick_the_lowest_index():
     assert ids.cpu().tolist() == [[0, 1]] * 4 and float((wts - 0.5).abs().max()) == 0.0
 
 
-@pytest.mark.parametrize("T,E,k,N,K", [(300, 4, 1, 264, 256), (700, 16, 2, 512, 128), (65, 3, 1, 20, 384)])
+# the last two are deep enough in K for the kernel's steady loop (and its tail of 4 and of 1 stages)
+@pytest.mark.parametrize("T,E,k,N,K", [(300, 4, 1, 264, 256), (700, 16, 2, 512, 128), (65, 3, 1, 20, 384),
+                                       (500, 5, 1, 200, 640), (260, 2, 2, 136, 1216)])
 def test_gemm_grouped(T, E, k, N, K):
     ops = _ops()
     x = _rand(T, K, dtype=torch.bfloat16, seed=1)
