@@ -96,9 +96,10 @@ __global__ void rope_kv_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
   }
 }
 
-// The same for head sizes 32, 64, 128, 256: one block per token, a thread per run of 8 elements
-// (4 rotary pairs), 16-byte accesses; the hd/8 lanes of a head are neighbours in a wave and sum
-// their squares with shuffles.
+// The same for head sizes 32, 64, 128, 256: a thread per run of 8 elements (4 rotary pairs),
+// 16-byte accesses; the hd/8 lanes of a head are neighbours in a wave and sum their squares with
+// shuffles.  Blocks (token, y) share a token's heads between them, 256 runs each, so that a
+// handful of decode tokens still spreads over many compute units.
 template <typename T>
 __global__ __launch_bounds__(256) void rope_kv_vec_kernel(
     const T* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
@@ -113,7 +114,7 @@ __global__ __launch_bounds__(256) void rope_kv_vec_kernel(
   const T* src = qkv + (size_t)t * (nh + 2 * nkv) * hd;
   float post = 1.0f;
   if (temp_tuning) post = 1.0f + attn_scale * logf(floorf(((float)pos + 1.0f) / floor_scale) + 1.0f);
-  for (int base = 0; base < chunks; base += blockDim.x) {
+  for (int base = blockIdx.y * blockDim.x; base < chunks; base += gridDim.y * blockDim.x) {
     const int ci = base + threadIdx.x;
     const bool valid = ci < chunks;
     const int head = valid ? ci / per_head : 0;
@@ -177,13 +178,14 @@ SHARPI_EXPORT int sharpi_rope_kv(const void* qkv, void* q_out, void* k_cache, vo
   dim3 grid(n_tokens, nh + 2 * nkv), block(kWave);
   if (dtype != DT_F32 && dtype != DT_BF16) return SHARPI_ERR_ARG;
   if (hd == 32 || hd == 64 || hd == 128 || hd == 256) {
+    const dim3 vgrid(n_tokens, ceil_div((nh + 2 * nkv) * (hd >> 3), 256));
     if (dtype == DT_F32)
-      rope_kv_vec_kernel<float><<<n_tokens, 256, 0, stream>>>((const float*)qkv, (float*)q_out, (float*)k_cache,
+      rope_kv_vec_kernel<float><<<vgrid, 256, 0, stream>>>((const float*)qkv, (float*)q_out, (float*)k_cache,
                                                              (float*)v_cache, slot_mapping, positions, inv_freq,
                                                              qk_norm, eps, temp_tuning, floor_scale, attn_scale,
                                                              nh, nkv, hd, page_size);
     else
-      rope_kv_vec_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>((const bf16_t*)qkv, (bf16_t*)q_out,
+      rope_kv_vec_kernel<bf16_t><<<vgrid, 256, 0, stream>>>((const bf16_t*)qkv, (bf16_t*)q_out,
                                                               (bf16_t*)k_cache, (bf16_t*)v_cache, slot_mapping,
                                                               positions, inv_freq, qk_norm, eps, temp_tuning,
                                                               floor_scale, attn_scale, nh, nkv, hd, page_size);

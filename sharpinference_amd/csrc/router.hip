@@ -16,6 +16,45 @@
 
 constexpr int kMaxExperts = 1024;
 
+// One thread: gate the logits g[0 .. n_experts) in place, pick k of them (ascending scan with a
+// strict >, so the lowest index wins a tie) into ids / w.
+__device__ void gate_and_pick(float* g, int n_experts, int k, int gate, int renorm, int* ids, float* w,
+                              float* gate_out) {
+  if (gate == 0) {
+    for (int e = 0; e < n_experts; ++e) g[e] = 1.0f / (1.0f + expf(-g[e]));
+  } else {
+    float mx = g[0];
+    for (int e = 1; e < n_experts; ++e) mx = fmaxf(mx, g[e]);
+    float sum = 0.f;
+    for (int e = 0; e < n_experts; ++e) {
+      g[e] = expf(g[e] - mx);
+      sum += g[e];
+    }
+    const float inv = 1.0f / sum;
+    for (int e = 0; e < n_experts; ++e) g[e] *= inv;
+  }
+  if (gate_out)
+    for (int e = 0; e < n_experts; ++e) gate_out[e] = g[e];
+  float wsum = 0.f;
+  for (int j = 0; j < k; ++j) {
+    int best = -1;
+    float bv = -INFINITY;
+    for (int e = 0; e < n_experts; ++e) {
+      bool taken = false;
+      for (int i = 0; i < j; ++i) taken |= (ids[i] == e);
+      if (!taken && (best < 0 || g[e] > bv)) {
+        bv = g[e];
+        best = e;
+      }
+    }
+    ids[j] = best;
+    w[j] = bv;
+    wsum += bv;
+  }
+  if (renorm && k > 1 && wsum > 0.f)
+    for (int j = 0; j < k; ++j) w[j] /= wsum;
+}
+
 template <typename T, typename TW>
 __global__ __launch_bounds__(1024) void router_topk_kernel(const T* __restrict__ x, const TW* __restrict__ wr,
                                                            int* __restrict__ topk_ids,
@@ -33,7 +72,22 @@ __global__ __launch_bounds__(1024) void router_topk_kernel(const T* __restrict__
     const TW* wrow = wr + (size_t)e * hidden;
     float s = 0.f;
     if (vec) {  // lane-strided runs of 8: the order of the additions depends on the width only
-      for (int c = lane * 8; c < hidden; c += kWave * 8) {
+      // four runs are fetched before the first is added: a row is a dozen dependent round trips
+      // to the cache otherwise, and the kernel is nothing but their latency
+      int c = lane * 8;
+      for (; c + 3 * kWave * 8 < hidden; c += 4 * kWave * 8) {
+        float a[4][8], b[4][8];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          load8(xr + c + q * kWave * 8, a[q]);
+          load8(wrow + c + q * kWave * 8, b[q]);
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int i = 0; i < 8; ++i) s = fmaf(a[q][i], b[q][i], s);
+      }
+      for (; c < hidden; c += kWave * 8) {
         float a[8], b[8];
         load8(xr + c, a);
         load8(wrow + c, b);
@@ -47,41 +101,9 @@ __global__ __launch_bounds__(1024) void router_topk_kernel(const T* __restrict__
     if (lane == 0) g[e] = s;
   }
   __syncthreads();
-  if (threadIdx.x == 0) {
-    if (gate == 0) {
-      for (int e = 0; e < n_experts; ++e) g[e] = 1.0f / (1.0f + expf(-g[e]));
-    } else {
-      float mx = g[0];
-      for (int e = 1; e < n_experts; ++e) mx = fmaxf(mx, g[e]);
-      float sum = 0.f;
-      for (int e = 0; e < n_experts; ++e) {
-        g[e] = expf(g[e] - mx);
-        sum += g[e];
-      }
-      const float inv = 1.0f / sum;
-      for (int e = 0; e < n_experts; ++e) g[e] *= inv;
-    }
-    if (gate_out)
-      for (int e = 0; e < n_experts; ++e) gate_out[(size_t)t * n_experts + e] = g[e];
-    float wsum = 0.f;
-    for (int j = 0; j < k; ++j) {
-      int best = -1;
-      float bv = -INFINITY;
-      for (int e = 0; e < n_experts; ++e) {
-        bool taken = false;
-        for (int i = 0; i < j; ++i) taken |= (topk_ids[t * k + i] == e);
-        if (!taken && (best < 0 || g[e] > bv)) {
-          bv = g[e];
-          best = e;
-        }
-      }
-      topk_ids[t * k + j] = best;
-      topk_w[t * k + j] = bv;
-      wsum += bv;
-    }
-    if (renorm && k > 1 && wsum > 0.f)
-      for (int j = 0; j < k; ++j) topk_w[t * k + j] /= wsum;
-  }
+  if (threadIdx.x == 0)
+    gate_and_pick(g, n_experts, k, gate, renorm, topk_ids + (size_t)t * k, topk_w + (size_t)t * k,
+                  gate_out ? gate_out + (size_t)t * n_experts : nullptr);
 }
 
 SHARPI_EXPORT int sharpi_router_topk(const void* x, int x_dtype, const void* wr, int w_dtype, int* topk_ids,
@@ -105,19 +127,14 @@ SHARPI_EXPORT int sharpi_router_topk(const void* x, int x_dtype, const void* wr,
   return SHARPI_OK;
 }
 
-__global__ __launch_bounds__(1024) void moe_permute_kernel(const int* __restrict__ topk_ids,
-                                                           const float* __restrict__ topk_w,
-                                                           int* __restrict__ offsets,
-                                                           int* __restrict__ sorted_token,
-                                                           float* __restrict__ sorted_w,
-                                                           int* __restrict__ inv_pos,
-                                                           int* __restrict__ tile_expert,
-                                                           int* __restrict__ tile_row0,
-                                                           int* __restrict__ n_tiles, int n_pairs, int k,
-                                                           int n_experts, int tile_rows, int max_tiles,
-                                                           int shared_group) {
-  __shared__ int count[kMaxExperts];
-  __shared__ int cursor[kMaxExperts];
+// One block: the expert-sorted list of the (token, pick) pairs; count and cursor are LDS of
+// n_experts ints.  Every thread of the block calls it; the pairs must be visible to the block.
+__device__ void permute_block(const int* __restrict__ topk_ids, const float* __restrict__ topk_w,
+                              int* __restrict__ offsets, int* __restrict__ sorted_token,
+                              float* __restrict__ sorted_w, int* __restrict__ inv_pos,
+                              int* __restrict__ tile_expert, int* __restrict__ tile_row0, int* __restrict__ n_tiles,
+                              int n_pairs, int k, int n_experts, int tile_rows, int max_tiles, int shared_group,
+                              int* count, int* cursor) {
   for (int e = threadIdx.x; e < n_experts; e += blockDim.x) count[e] = 0;
   __syncthreads();
   for (int i = threadIdx.x; i < n_pairs; i += blockDim.x) atomicAdd(&count[topk_ids[i]], 1);
@@ -132,14 +149,17 @@ __global__ __launch_bounds__(1024) void moe_permute_kernel(const int* __restrict
     offsets[n_experts] = run;
     // row tiles of the experts that have rows, for the grouped product of many rows
     int nt = 0;
-    for (int e = 0; e < n_experts; ++e)
-      for (int r0 = offsets[e]; r0 < offsets[e] + count[e]; r0 += tile_rows) {
+    run = 0;
+    for (int e = 0; e < n_experts; ++e) {
+      for (int r0 = run; r0 < run + count[e]; r0 += tile_rows) {
         if (nt < max_tiles) {
           tile_expert[nt] = e;
           tile_row0[nt] = r0;
           ++nt;
         }
       }
+      run += count[e];
+    }
     n_tiles[0] = nt;
     // an always-on expert as one more group: every token once, in token order, with weight 1
     if (shared_group) offsets[n_experts + 1] = run + n_pairs / k;
@@ -158,6 +178,23 @@ __global__ __launch_bounds__(1024) void moe_permute_kernel(const int* __restrict
     sorted_w[r] = topk_w[i];
     inv_pos[i] = r;
   }
+}
+
+__global__ __launch_bounds__(1024) void moe_permute_kernel(const int* __restrict__ topk_ids,
+                                                           const float* __restrict__ topk_w,
+                                                           int* __restrict__ offsets,
+                                                           int* __restrict__ sorted_token,
+                                                           float* __restrict__ sorted_w,
+                                                           int* __restrict__ inv_pos,
+                                                           int* __restrict__ tile_expert,
+                                                           int* __restrict__ tile_row0,
+                                                           int* __restrict__ n_tiles, int n_pairs, int k,
+                                                           int n_experts, int tile_rows, int max_tiles,
+                                                           int shared_group) {
+  __shared__ int count[kMaxExperts];
+  __shared__ int cursor[kMaxExperts];
+  permute_block(topk_ids, topk_w, offsets, sorted_token, sorted_w, inv_pos, tile_expert, tile_row0, n_tiles,
+                n_pairs, k, n_experts, tile_rows, max_tiles, shared_group, count, cursor);
 }
 
 SHARPI_EXPORT int sharpi_moe_permute(const int* topk_ids, const float* topk_w, int* offsets, int* sorted_token,

@@ -394,15 +394,7 @@ class Routing:
         return self.n_tokens * self.k + (self.n_tokens if self.n_groups > self.n_experts else 0)
 
 
-def moe_permute(ids: torch.Tensor, wts: torch.Tensor, n_experts: int, shared_group: bool = False) -> Routing:
-    """(token, pick) pairs sorted by expert: offsets [E+1], sorted_token, sorted_w, inv_pos, and
-    the list of row tiles (GROUPED_TILE_ROWS high) of the experts that have rows.  With
-    shared_group one more group follows the experts: every token once with weight 1."""
-    _dev(ids, wts)
-    _i32(ids, "ids")
-    _need(ids.shape == wts.shape and wts.dtype == torch.float32 and ids.dim() == 2, "moe_permute: ids/wts [T, k]")
-    T, k = ids.shape
-    dev = ids.device
+def _new_routing(T: int, k: int, n_experts: int, shared_group: bool, dev) -> Routing:
     rt = Routing()
     rt.n_tokens, rt.k, rt.n_experts = T, k, n_experts
     rt.n_groups = n_experts + (1 if shared_group else 0)
@@ -417,10 +409,29 @@ def moe_permute(ids: torch.Tensor, wts: torch.Tensor, n_experts: int, shared_gro
     rt.tile_row0 = ints[o:o + rt.max_tiles]; o += rt.max_tiles
     rt.n_tiles = ints[o:o + 1]
     rt.sorted_w = torch.empty(rows, dtype=torch.float32, device=dev)
+    return rt
+
+
+def moe_permute(ids: torch.Tensor, wts: torch.Tensor, n_experts: int, shared_group: bool = False) -> Routing:
+    """(token, pick) pairs sorted by expert: offsets [E+1], sorted_token, sorted_w, inv_pos, and
+    the list of row tiles (GROUPED_TILE_ROWS high) of the experts that have rows.  With
+    shared_group one more group follows the experts: every token once with weight 1."""
+    _dev(ids, wts)
+    _i32(ids, "ids")
+    _need(ids.shape == wts.shape and wts.dtype == torch.float32 and ids.dim() == 2, "moe_permute: ids/wts [T, k]")
+    T, k = ids.shape
+    rt = _new_routing(T, k, n_experts, shared_group, ids.device)
     _run("sharpi_moe_permute", _ptr(ids), _ptr(wts), _ptr(rt.offsets), _ptr(rt.sorted_token), _ptr(rt.sorted_w),
          _ptr(rt.inv_pos), _ptr(rt.tile_expert), _ptr(rt.tile_row0), _ptr(rt.n_tiles), T, k, n_experts,
          GROUPED_TILE_ROWS, rt.max_tiles, 1 if shared_group else 0, _stream())
     return rt
+
+
+def route(x: torch.Tensor, wr: torch.Tensor, k: int, gate: int = GATE_SIGMOID, renorm: bool = False,
+          shared_group: bool = False):
+    """router_topk then moe_permute: (ids, weights, Routing)."""
+    ids, wts = router_topk(x, wr, k, gate, renorm)
+    return ids, wts, moe_permute(ids, wts, wr.shape[0], shared_group)
 
 
 def gemm_grouped(x: torch.Tensor, w: torch.Tensor, rt: Routing, gather: bool, out_dtype: torch.dtype) -> torch.Tensor:

@@ -117,18 +117,17 @@ class MoESwiGLU(Part):
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         T = x.shape[0]
-        ids, wts = ops.router_topk(x, self.w_router, self.k, self.gate, self.renormalise)
+        merge = self.merged and T <= self.MERGE_MAX_TOKENS and ctx.act_dtype == torch.bfloat16
+        ids, wts, rt = ops.route(x, self.w_router, self.k, self.gate, self.renormalise, shared_group=merge)
         trace = ctx.extras.get("router_trace")
         if trace is not None:      # the picks of this step, layer by layer (reference: ForwardPass.cs:2042-2056)
             trace.append((ids, wts))
-        if self.merged and T <= self.MERGE_MAX_TOKENS and ctx.act_dtype == torch.bfloat16:
+        if merge:
             # few rows: the shared expert rides along as one more group of the same two launches
-            rt = ops.moe_permute(ids, wts, self.E, shared_group=True)
             gu = ops.grouped_linear(x, self.w_gate_up, rt, True, ctx.act_dtype)
             act = ops.silu_mul(gu, rt.sorted_w)
             y = ops.grouped_linear(act, self.w_down, rt, False, ctx.act_dtype)
             return ops.moe_combine(y[:T * self.k], rt.inv_pos, y[T * self.k:], T, self.k)
-        rt = ops.moe_permute(ids, wts, self.E)
         shared = self.shared.forward(x, ctx) if self.shared is not None else None
         gu = ops.grouped_linear(x, self.w_gate_up, rt, True, ctx.act_dtype)
         act = ops.silu_mul(gu, rt.sorted_w)
