@@ -65,8 +65,8 @@ __global__ __launch_bounds__(kDecWaves* kWave) void attn_decode_kernel(
   bf16x8 qf[NJ];
 #pragma unroll
   for (int j = 0; j < NJ; ++j) {
-    if (r < hcount) qf[j] = *reinterpret_cast<const bf16x8*>(q + ((size_t)t * nh + h0 + r) * HD + j * 32 + g * 8);
-    else qf[j] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    // columns beyond the group's heads repeat its last head; they are never stored
+    qf[j] = *reinterpret_cast<const bf16x8*>(q + ((size_t)t * nh + h0 + min(r, hcount - 1)) * HD + j * 32 + g * 8);
   }
 
   float m = -INFINITY, l = 0.f;   // for head r: m identical in the 4 lanes of a column, l a partial sum
@@ -74,43 +74,46 @@ __global__ __launch_bounds__(kDecWaves* kWave) void attn_decode_kernel(
 #pragma unroll
   for (int d = 0; d < ND; ++d) acc[d] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  for (int b = b_first + 2 * w; b <= b_last; b += 2 * kDecWaves) {
-    // two 16-key blocks: b and b + 1 (the second may lie beyond the range).  Keys AND values of
-    // the chunk are requested before anything is computed: the values do not wait for the scores.
-    f32x4 s[2];
-    bool have[2];
-    bf16x8 kf[2][NJ];
-    bf16x4 vq[2][ND];
+  // A wave's chunks of the run are 2 * kDecWaves blocks apart; PRE of them are requested before
+  // anything is computed (all of a 256-key run where the registers allow it: the run is then one
+  // round trip to memory, not one per chunk).  Every load is unconditional: a block beyond the
+  // run's last is fetched as the last one again and masked, so that the compiler's count of
+  // outstanding loads stays exact and the first chunk does not wait for the second.
+  constexpr int PRE = HD <= 128 ? 2 : 1;
+  for (int b0 = b_first + 2 * w; b0 <= b_last; b0 += 2 * kDecWaves * PRE) {
+    bf16x8 kf[PRE][2][NJ];
+    bf16x4 vq[PRE][2][ND];
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const int bb = b + u;
-      have[u] = bb <= b_last;
-      int page = -1;
-      if (have[u]) {
-        const int pi = (bb << 4) / page_size;
-        page = pi < max_blocks ? bt[pi] : -1;
-        if (page < 0 || page >= num_pages) have[u] = false;
-      }
-      const int off = (bb << 4) % page_size;
-      const long long kbase = have[u] ? (((long long)page * nkv + kvh) * page_size + off) * HD : 0;
-      const long long vbase = have[u] ? ((long long)page * nkv + kvh) * HD * page_size + off : 0;
+    for (int it = 0; it < PRE; ++it) {
 #pragma unroll
-      for (int j = 0; j < NJ; ++j) {
-        if (have[u]) kf[u][j] = *reinterpret_cast<const bf16x8*>(k_cache + kbase + (size_t)r * HD + j * 32 + g * 8);
-        else kf[u][j] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
-      }
+      for (int u = 0; u < 2; ++u) {
+        const int bb = min(b0 + it * 2 * kDecWaves + u, b_last);
+        const int pi = min((bb << 4) / page_size, max_blocks - 1);
+        const int page = min(max(bt[pi], 0), num_pages - 1);   // a table that is wrong reads a wrong page, never outside
+        const int off = (bb << 4) % page_size;
+        const long long kbase = (((long long)page * nkv + kvh) * page_size + off) * HD;
+        const long long vbase = ((long long)page * nkv + kvh) * HD * page_size + off;
 #pragma unroll
-      for (int d = 0; d < ND; ++d) {
-        // V^T fragment: lane (d row r, group g) holds keys 4g..4g+3 of the block
-        if (have[u]) vq[u][d] = *reinterpret_cast<const bf16x4*>(v_cache + vbase + (size_t)(d * 16 + r) * page_size + 4 * g);
-        else vq[u][d] = bf16x4{0, 0, 0, 0};
+        for (int j = 0; j < NJ; ++j)
+          kf[it][u][j] = *reinterpret_cast<const bf16x8*>(k_cache + kbase + (size_t)r * HD + j * 32 + g * 8);
+#pragma unroll
+        for (int d = 0; d < ND; ++d)   // V^T fragment: lane (d row r, group g) holds keys 4g..4g+3 of the block
+          vq[it][u][d] = *reinterpret_cast<const bf16x4*>(v_cache + vbase + (size_t)(d * 16 + r) * page_size + 4 * g);
       }
     }
+#pragma unroll
+    for (int it = 0; it < PRE; ++it) {
+    const int b = b0 + it * 2 * kDecWaves;
+    if (b > b_last) break;   // wave-uniform
+    f32x4 s[2];
+    bool have[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) have[u] = b + u <= b_last;
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       s[u] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int j = 0; j < NJ; ++j) s[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[u][j], qf[j], s[u], 0, 0, 0);
+      for (int j = 0; j < NJ; ++j) s[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[it][u][j], qf[j], s[u], 0, 0, 0);
     }
     // lane holds S^T[key = 16*(b+u) + 4g + i][head r]
     float cm = -INFINITY;
@@ -150,10 +153,11 @@ __global__ __launch_bounds__(kDecWaves* kWave) void attn_decode_kernel(
 #pragma unroll
     for (int d = 0; d < ND; ++d) {
       // keys 4g..4g+3 of block b, then of block b + 1
-      const bf16x8 vf = __builtin_shufflevector(vq[0][d], vq[1][d], 0, 1, 2, 3, 4, 5, 6, 7);
+      const bf16x8 vf = __builtin_shufflevector(vq[it][0][d], vq[it][1][d], 0, 1, 2, 3, 4, 5, 6, 7);
       acc[d] *= corr;   // corr belongs to head r = the accumulator's column
       acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, acc[d], 0, 0, 0);
       acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf_lo, acc[d], 0, 0, 0);
+    }
     }
   }
 

@@ -74,6 +74,16 @@ __device__ __forceinline__ void store8(bf16_t* p, const float* v) {
   *reinterpret_cast<uint4*>(p) = o;
 }
 
+// SwiGLU of one element: silu(s g) * (s u), silu(x) = x / (1 + exp(-x)); one definition for the
+// activation kernel and for the product that applies it in its epilogue, so both give the same bits
+__device__ __forceinline__ float swiglu_f32(float g, float u, float s, bool scaled) {
+  if (scaled) {
+    g *= s;
+    u *= s;
+  }
+  return (g / (1.0f + expf(-g))) * u;
+}
+
 // dtype codes shared with the Python side
 enum : int { DT_F32 = 0, DT_BF16 = 1 };
 

@@ -71,15 +71,47 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__
 // the two passes (up to kNormKeep runs of 8 per thread; wider rows are read again).
 constexpr int kNormKeep = 4;
 
+// delta of row r, columns c .. c + 7, as floats.  Plain: delta[r].  As an expert sum (sum_pos
+// given): the rows sum_pos[r*k .. r*k + k) of delta plus sum_shared[r], added in that order in
+// float and rounded to the storage type, which is what the separate combine kernel would have
+// stored for the norm to read.
+template <typename TD>
+__device__ __forceinline__ void load_delta8(const TD* __restrict__ delta, const int* __restrict__ sum_pos,
+                                            const TD* __restrict__ sum_shared, int sum_k, int r, int hidden,
+                                            int c, float* d) {
+  if (!sum_pos) {
+    load8(delta + (size_t)r * hidden + c, d);
+    return;
+  }
+#pragma unroll
+  for (int j = 0; j < 8; ++j) d[j] = 0.f;
+  for (int q = 0; q < sum_k; ++q) {
+    float v[8];
+    load8(delta + (size_t)sum_pos[r * sum_k + q] * hidden + c, v);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) d[j] += v[j];
+  }
+  if (sum_shared) {
+    float v[8];
+    load8(sum_shared + (size_t)r * hidden + c, v);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) d[j] += v[j];
+  }
+#pragma unroll
+  for (int j = 0; j < 8; ++j) d[j] = to_f32<TD>(from_f32<TD>(d[j]));
+}
+
 template <typename TD, typename TW, typename TO>
 __global__ void add_rmsnorm_vec_kernel(float* __restrict__ h, const TD* __restrict__ delta,
                                        const TW* __restrict__ w, TO* __restrict__ out,
-                                       const int* __restrict__ rows, int hidden, float eps, int write_back) {
+                                       const int* __restrict__ rows, int hidden, float eps, int write_back,
+                                       const int* __restrict__ sum_pos, const TD* __restrict__ sum_shared,
+                                       int sum_k) {
   __shared__ float red[16];
   const int i = blockIdx.x;
   const int r = rows ? rows[i] : i;
   float* hr = h + (size_t)r * hidden;
-  const TD* dr = delta ? delta + (size_t)r * hidden : nullptr;
+  const bool dr = delta != nullptr;
   float keep[kNormKeep][8];
   float ss = 0.f;
   int n = 0;
@@ -88,7 +120,7 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ h, const TD* __restri
     load8(hr + c, x);
     if (dr) {
       float d[8];
-      load8(dr + c, d);
+      load_delta8<TD>(delta, sum_pos, sum_shared, sum_k, r, hidden, c, d);
 #pragma unroll
       for (int j = 0; j < 8; ++j) x[j] += d[j];
       if (write_back) store8(hr + c, x);
@@ -113,7 +145,7 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ h, const TD* __restri
       load8(hr + c, x);
       if (dr && !write_back) {
         float d[8];
-        load8(dr + c, d);
+        load_delta8<TD>(delta, sum_pos, sum_shared, sum_k, r, hidden, c, d);
 #pragma unroll
         for (int j = 0; j < 8; ++j) x[j] += d[j];
       }
@@ -135,18 +167,22 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ h, const TD* __restri
 template <typename TD, typename TW>
 static int launch_add_rmsnorm_o(float* h, const void* delta, const void* w, void* out, int out_dtype,
                                 const int* rows, int n_out, int hidden, float eps, int write_back,
-                                hipStream_t stream) {
+                                const int* sum_pos, const void* sum_shared, int sum_k, hipStream_t stream) {
   dim3 grid(n_out), block(hidden >= 2048 ? 512 : 256);
   if (out_dtype != DT_F32 && out_dtype != DT_BF16) return SHARPI_ERR_ARG;
   if ((hidden & 7) == 0) {
     dim3 vblock(hidden >= 4096 ? 256 : hidden >= 1024 ? 128 : 64);
     if (out_dtype == DT_F32)
       add_rmsnorm_vec_kernel<TD, TW, float><<<grid, vblock, 0, stream>>>(h, (const TD*)delta, (const TW*)w,
-                                                                        (float*)out, rows, hidden, eps, write_back);
+                                                                        (float*)out, rows, hidden, eps, write_back,
+                                                                        sum_pos, (const TD*)sum_shared, sum_k);
     else
       add_rmsnorm_vec_kernel<TD, TW, bf16_t><<<grid, vblock, 0, stream>>>(h, (const TD*)delta, (const TW*)w,
-                                                                         (bf16_t*)out, rows, hidden, eps, write_back);
-  } else if (out_dtype == DT_F32)
+                                                                         (bf16_t*)out, rows, hidden, eps, write_back,
+                                                                         sum_pos, (const TD*)sum_shared, sum_k);
+  } else if (sum_pos)
+    return SHARPI_ERR_ARG;   // an expert sum is folded in by the vector kernel only (width % 8 == 0)
+  else if (out_dtype == DT_F32)
     add_rmsnorm_kernel<TD, TW, float><<<grid, block, 0, stream>>>(h, (const TD*)delta, (const TW*)w,
                                                                  (float*)out, rows, hidden, eps, write_back);
   else
@@ -159,24 +195,34 @@ static int launch_add_rmsnorm_o(float* h, const void* delta, const void* w, void
 template <typename TD>
 static int launch_add_rmsnorm_w(float* h, const void* delta, const void* w, int w_dtype, void* out,
                                 int out_dtype, const int* rows, int n_out, int hidden, float eps,
-                                int write_back, hipStream_t stream) {
+                                int write_back, const int* sum_pos, const void* sum_shared, int sum_k,
+                                hipStream_t stream) {
   if (w_dtype == DT_F32 || w == nullptr)
-    return launch_add_rmsnorm_o<TD, float>(h, delta, w, out, out_dtype, rows, n_out, hidden, eps, write_back, stream);
+    return launch_add_rmsnorm_o<TD, float>(h, delta, w, out, out_dtype, rows, n_out, hidden, eps, write_back,
+                                           sum_pos, sum_shared, sum_k, stream);
   if (w_dtype == DT_BF16)
-    return launch_add_rmsnorm_o<TD, bf16_t>(h, delta, w, out, out_dtype, rows, n_out, hidden, eps, write_back, stream);
+    return launch_add_rmsnorm_o<TD, bf16_t>(h, delta, w, out, out_dtype, rows, n_out, hidden, eps, write_back,
+                                            sum_pos, sum_shared, sum_k, stream);
   return SHARPI_ERR_ARG;
 }
 
+// h [*, hidden] float; delta the branch output to add first (null: none).  With sum_pos the
+// delta is an expert sum: row r = delta[sum_pos[r*sum_k ..]] summed (+ sum_shared[r]), see
+// load_delta8; hidden % 8 == 0 then.
 SHARPI_EXPORT int sharpi_add_rmsnorm(float* h, const void* delta, int delta_dtype, const void* w, int w_dtype,
                                      void* out, int out_dtype, const int* rows, int n_out, int hidden,
-                                     float eps, int write_back, hipStream_t stream) {
+                                     float eps, int write_back, const int* sum_pos, const void* sum_shared,
+                                     int sum_k, hipStream_t stream) {
   if (n_out <= 0) return SHARPI_OK;
   if (hidden <= 0 || !(eps > 0.f)) return SHARPI_ERR_ARG;
   if (rows && write_back) return SHARPI_ERR_ARG;  // gathered rows never write the stream back
+  if (sum_pos && (delta == nullptr || sum_k <= 0)) return SHARPI_ERR_ARG;
   if (delta == nullptr || delta_dtype == DT_F32)
-    return launch_add_rmsnorm_w<float>(h, delta, w, w_dtype, out, out_dtype, rows, n_out, hidden, eps, write_back, stream);
+    return launch_add_rmsnorm_w<float>(h, delta, w, w_dtype, out, out_dtype, rows, n_out, hidden, eps, write_back,
+                                       sum_pos, sum_shared, sum_k, stream);
   if (delta_dtype == DT_BF16)
-    return launch_add_rmsnorm_w<bf16_t>(h, delta, w, w_dtype, out, out_dtype, rows, n_out, hidden, eps, write_back, stream);
+    return launch_add_rmsnorm_w<bf16_t>(h, delta, w, w_dtype, out, out_dtype, rows, n_out, hidden, eps, write_back,
+                                        sum_pos, sum_shared, sum_k, stream);
   return SHARPI_ERR_ARG;
 }
 
@@ -191,15 +237,9 @@ __global__ void silu_mul_kernel(const T* __restrict__ gu, const float* __restric
   const int i = blockIdx.y * blockDim.x + threadIdx.x;
   if (i >= inter) return;
   const T* row = gu + (size_t)m * 2 * inter;
-  float g = to_f32<T>(row[i]);
-  float u = to_f32<T>(row[inter + i]);
-  if (scale) {
-    const float s = scale[m];
-    g *= s;
-    u *= s;
-  }
-  const float a = g / (1.0f + expf(-g));
-  out[(size_t)m * inter + i] = from_f32<T>(a * u);
+  const float g = to_f32<T>(row[i]);
+  const float u = to_f32<T>(row[inter + i]);
+  out[(size_t)m * inter + i] = from_f32<T>(swiglu_f32(g, u, scale ? scale[m] : 1.0f, scale != nullptr));
 }
 
 template <typename T>
@@ -214,14 +254,7 @@ __global__ void silu_mul_vec_kernel(const T* __restrict__ gu, const float* __res
   load8(row + inter + i, u);
   const float s = scale ? scale[m] : 1.0f;
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    float gj = g[j], uj = u[j];
-    if (scale) {
-      gj *= s;
-      uj *= s;
-    }
-    o[j] = (gj / (1.0f + expf(-gj))) * uj;
-  }
+  for (int j = 0; j < 8; ++j) o[j] = swiglu_f32(g[j], u[j], s, scale != nullptr);
   store8(out + (size_t)m * inter + i, o);
 }
 

@@ -14,6 +14,11 @@
 //    [offsets[e], offsets[e + 1]) of the expert-sorted row list with W[e], sixteen at a time;
 //    x rows are gathered through a_rows.  Experts without rows return at once.
 //
+//  * SwiGLU form (ACT): W holds gate rows [0, N/2) and up rows [N/2, N); a block takes R/2 tiles
+//    of each at the same columns, and the wave that adds up a gate tile adds up its up tile too,
+//    rounds both to bfloat16 (what a separate activation kernel would have read) and stores
+//    silu(s g) * (s u), s the row's score: out is [M, N/2] and the gate|up rows never go to memory.
+//
 // Limits (the caller falls back to other kernels otherwise): K % 128 == 0, N % 4 == 0, M <= 64.
 #include "common.h"
 
@@ -33,11 +38,14 @@ template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, f32x4 v) {
 
 constexpr int kRedTiles = 2;  // (tile, row block) pairs summed per LDS round
 
-template <int R, int MB, int NW, typename TO>
+template <int R, int MB, int NW, typename TO, bool ACT>
 __global__ __launch_bounds__(NW* kWave) void skinny_gemm_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ W, TO* __restrict__ out, int M, int N, int K,
-    const int* __restrict__ a_rows, const int* __restrict__ group_offsets) {
-  __shared__ f32x4 red[NW][kRedTiles][kWave];
+    const int* __restrict__ a_rows, const int* __restrict__ group_offsets, const float* __restrict__ act_scale) {
+  static_assert(!ACT || (R % 2 == 0 && MB == 1), "the SwiGLU form pairs gate and up tiles of one row block");
+  constexpr int RT = ACT ? R : kRedTiles;   // tiles that meet in LDS per round
+  constexpr int TG = ACT ? R / 2 : R;       // tiles of distinct output columns per block
+  __shared__ f32x4 red[NW][RT][kWave];
   const int lane = threadIdx.x & (kWave - 1);
   const int w = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
@@ -51,7 +59,8 @@ __global__ __launch_bounds__(NW* kWave) void skinny_gemm_kernel(
   }
   const int n_rows = row_end - row_begin;
   if (n_rows <= 0) return;
-  const int n_base = nb * 16 * R;
+  const int n_base = nb * 16 * TG;
+  const int n_out = ACT ? N / 2 : N;        // output columns
 
   // this wave's K units
   const int U = K >> 7;
@@ -61,8 +70,9 @@ __global__ __launch_bounds__(NW* kWave) void skinny_gemm_kernel(
   const bf16_t* wrow[R];
 #pragma unroll
   for (int t = 0; t < R; ++t) {
-    int n = n_base + t * 16 + r;
-    if (n >= N) n = N - 1;  // loaded, never stored
+    int n = n_base + (t % TG) * 16 + r;
+    if (n >= n_out) n = n_out - 1;  // loaded, never stored
+    if (ACT && t >= TG) n += n_out;  // the up row of the same column
     wrow[t] = W + (size_t)n * K + g * 32;
   }
 
@@ -105,6 +115,32 @@ __global__ __launch_bounds__(NW* kWave) void skinny_gemm_kernel(
             acc[t][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[t][j], xf[mb][j], acc[t][mb], 0, 0, 0);
     }
 
+    if constexpr (ACT) {
+      // all tiles meet at once; wave t < TG adds up gate tile t and up tile t + TG in wave order
+      __syncthreads();
+#pragma unroll
+      for (int t = 0; t < R; ++t) red[w][t][lane] = acc[t][0];
+      __syncthreads();
+      if (w < TG) {
+        f32x4 gv = red[0][w][lane], uv = red[0][w + TG][lane];
+#pragma unroll
+        for (int ww = 1; ww < NW; ++ww) {
+          gv += red[ww][w][lane];
+          uv += red[ww][w + TG][lane];
+        }
+        const int row = row_begin + rb0 * 16 + r;
+        const int n = n_base + w * 16 + g * 4;
+        if (row < row_end && n < n_out) {
+          const float sc = act_scale ? act_scale[row] : 1.0f;
+          f32x4 o;
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            o[i] = swiglu_f32(bf16_to_f32(f32_to_bf16(gv[i])), bf16_to_f32(f32_to_bf16(uv[i])), sc, act_scale != nullptr);
+          store4<TO>(out + (size_t)row * n_out + n, o);
+        }
+      }
+      continue;
+    }
     // add the waves' K slices in wave order, kRedTiles (tile, row block) pairs per round;
     // pair p of a round is summed and stored by wave p
 #pragma unroll
@@ -128,17 +164,18 @@ __global__ __launch_bounds__(NW* kWave) void skinny_gemm_kernel(
   }
 }
 
-template <int R, int MB, int NW>
+template <int R, int MB, int NW, bool ACT>
 static int launch_skinny(const void* x, const void* W, void* out, int out_dtype, int M, int N, int K,
-                         const int* a_rows, const int* group_offsets, int groups, hipStream_t stream) {
-  dim3 grid(ceil_div(N, 16 * R), groups > 0 ? groups : 1), block(NW * kWave);
+                         const int* a_rows, const int* group_offsets, int groups, const float* act_scale,
+                         hipStream_t stream) {
+  dim3 grid(ceil_div(ACT ? N / 2 : N, 16 * (ACT ? R / 2 : R)), groups > 0 ? groups : 1), block(NW * kWave);
   const int* go = groups > 0 ? group_offsets : nullptr;
   if (out_dtype == DT_F32)
-    skinny_gemm_kernel<R, MB, NW, float><<<grid, block, 0, stream>>>((const bf16_t*)x, (const bf16_t*)W,
-                                                                    (float*)out, M, N, K, a_rows, go);
+    skinny_gemm_kernel<R, MB, NW, float, ACT><<<grid, block, 0, stream>>>(
+        (const bf16_t*)x, (const bf16_t*)W, (float*)out, M, N, K, a_rows, go, act_scale);
   else
-    skinny_gemm_kernel<R, MB, NW, bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)x, (const bf16_t*)W,
-                                                                     (bf16_t*)out, M, N, K, a_rows, go);
+    skinny_gemm_kernel<R, MB, NW, bf16_t, ACT><<<grid, block, 0, stream>>>(
+        (const bf16_t*)x, (const bf16_t*)W, (bf16_t*)out, M, N, K, a_rows, go, act_scale);
   SHARPI_CHECK_LAUNCH();
   return SHARPI_OK;
 }
@@ -146,9 +183,9 @@ static int launch_skinny(const void* x, const void* W, void* out, int out_dtype,
 template <int R, int NW>
 static int dispatch_mb(int MB, const void* x, const void* W, void* out, int out_dtype, int M, int N, int K,
                        const int* a_rows, const int* group_offsets, int groups, hipStream_t stream) {
-  if (MB == 1) return launch_skinny<R, 1, NW>(x, W, out, out_dtype, M, N, K, a_rows, group_offsets, groups, stream);
-  if (MB == 2) return launch_skinny<R, 2, NW>(x, W, out, out_dtype, M, N, K, a_rows, group_offsets, groups, stream);
-  return launch_skinny<R, 4, NW>(x, W, out, out_dtype, M, N, K, a_rows, group_offsets, groups, stream);
+  if (MB == 1) return launch_skinny<R, 1, NW, false>(x, W, out, out_dtype, M, N, K, a_rows, group_offsets, groups, nullptr, stream);
+  if (MB == 2) return launch_skinny<R, 2, NW, false>(x, W, out, out_dtype, M, N, K, a_rows, group_offsets, groups, nullptr, stream);
+  return launch_skinny<R, 4, NW, false>(x, W, out, out_dtype, M, N, K, a_rows, group_offsets, groups, nullptr, stream);
 }
 
 // x [M, K] bf16 (rows gathered through a_rows if given), W [N, K] or [groups, N, K] bf16,
@@ -171,5 +208,24 @@ SHARPI_EXPORT int sharpi_gemm_skinny(const void* x, const void* W, void* out, in
   SK(2, 4); SK(2, 8);
   SK(4, 4); SK(4, 8);
 #undef SK
+  return SHARPI_ERR_ARG;
+}
+
+// The grouped product with SwiGLU applied in its epilogue: W [groups, N, K] holds gate rows
+// [0, N/2) and up rows [N/2, N) of every expert; out [M, N/2] bf16 =
+// silu(s g) * (s u) with g, u the two products rounded to bfloat16 and s = act_scale[row] (null: 1).
+// Rows are the expert-sorted list (sixteen of an expert at a time).  R in {2, 4}, NW in {4, 8}.
+SHARPI_EXPORT int sharpi_gemm_skinny_swiglu(const void* x, const void* W, void* out, int M, int N, int K,
+                                            const int* a_rows, const int* group_offsets, int groups,
+                                            const float* act_scale, int R, int NW, hipStream_t stream) {
+  if (M <= 0) return SHARPI_OK;
+  if (M > 64 || N <= 0 || (N & 7) || K <= 0 || (K & 127) || groups <= 0 || groups > 65535) return SHARPI_ERR_ARG;
+  if (group_offsets == nullptr) return SHARPI_ERR_ARG;
+#define SKA(RR, WW)           \
+  if (R == RR && NW == WW)    \
+  return launch_skinny<RR, 1, WW, true>(x, W, out, DT_BF16, M, N, K, a_rows, group_offsets, groups, act_scale, stream)
+  SKA(2, 4); SKA(2, 8);
+  SKA(4, 4); SKA(4, 8);
+#undef SKA
   return SHARPI_ERR_ARG;
 }

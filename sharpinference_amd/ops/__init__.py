@@ -74,16 +74,47 @@ def embed_gather(ids: torch.Tensor, table: torch.Tensor, out: Optional[torch.Ten
     return out
 
 
-def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: Optional[torch.Tensor], eps: float,
+class ExpertSum:
+    """A branch output that is still a sum to be formed: row t = sum_j y[inv_pos[t*k + j]]
+    (+ shared[t]).  ``add_rmsnorm`` forms it on the fly; ``tensor()`` forms it with a kernel of
+    its own.  Either way the sum is rounded once to y's storage type."""
+
+    __slots__ = ("y", "inv_pos", "shared", "n_tokens", "k")
+
+    def __init__(self, y: torch.Tensor, inv_pos: torch.Tensor, shared: Optional[torch.Tensor], n_tokens: int, k: int):
+        _need(y.dim() == 2 and inv_pos.numel() == n_tokens * k, "ExpertSum: y [rows, H], inv_pos [T*k]")
+        if shared is not None:
+            _need(shared.shape == (n_tokens, y.shape[1]) and shared.dtype == y.dtype and shared.is_contiguous(),
+                  "ExpertSum: shared must be contiguous [T, H] of y's dtype")
+        self.y, self.inv_pos, self.shared, self.n_tokens, self.k = y, inv_pos, shared, n_tokens, k
+
+    @property
+    def shape(self):
+        return (self.n_tokens, self.y.shape[1])
+
+    @property
+    def dtype(self):
+        return self.y.dtype
+
+    def tensor(self) -> torch.Tensor:
+        return moe_combine(self.y[: self.n_tokens * self.k], self.inv_pos, self.shared, self.n_tokens, self.k)
+
+
+def add_rmsnorm(h: torch.Tensor, delta, weight: Optional[torch.Tensor], eps: float,
                 out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None, write_back: bool = True,
                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """(h + delta) -> RMSNorm -> out; the sum goes back into h unless rows are gathered."""
-    _dev(h, delta, weight, rows, out)
+    """(h + delta) -> RMSNorm -> out; the sum goes back into h unless rows are gathered.
+    delta: a tensor, an ExpertSum, or None."""
+    lazy = delta if isinstance(delta, ExpertSum) else None
+    if lazy is not None and h.shape[1] % 8 != 0:
+        delta, lazy = lazy.tensor(), None          # the kernel folds a sum in only at widths that are multiples of 8
+    base = lazy.y if lazy is not None else delta
+    _dev(h, base, weight, rows, out)
     _i32(rows, "rows")
     _need(h.dim() == 2 and h.dtype == torch.float32, "add_rmsnorm: h must be float32 [T, H]")
     T, H = h.shape
     if delta is not None:
-        _need(delta.shape == h.shape, f"add_rmsnorm: delta {tuple(delta.shape)} vs h {tuple(h.shape)}")
+        _need(tuple(delta.shape) == tuple(h.shape), f"add_rmsnorm: delta {tuple(delta.shape)} vs h {tuple(h.shape)}")
     if weight is not None:
         _need(weight.shape == (H,), f"add_rmsnorm: weight {tuple(weight.shape)} vs width {H}")
     n_out = T if rows is None else rows.shape[0]
@@ -92,9 +123,11 @@ def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: Optional
     if out is None:
         out = torch.empty(n_out, H, dtype=out_dtype, device=h.device)
     _need(out.shape == (n_out, H) and out.dtype == out_dtype, "add_rmsnorm: out has the wrong shape or dtype")
-    _run("sharpi_add_rmsnorm", _ptr(h), _ptr(delta), _code(delta.dtype) if delta is not None else 0,
+    _run("sharpi_add_rmsnorm", _ptr(h), _ptr(base), _code(base.dtype) if base is not None else 0,
          _ptr(weight), _code(weight.dtype) if weight is not None else 0, _ptr(out), _code(out_dtype), _ptr(rows),
-         n_out, H, float(eps), 1 if write_back else 0, _stream())
+         n_out, H, float(eps), 1 if write_back else 0,
+         _ptr(lazy.inv_pos) if lazy is not None else None, _ptr(lazy.shared) if lazy is not None else None,
+         lazy.k if lazy is not None else 0, _stream())
     return out
 
 
@@ -319,6 +352,36 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, a_rows
     return out
 
 
+def gemm_skinny_swiglu(x: torch.Tensor, w: torch.Tensor, offsets: torch.Tensor, a_rows: Optional[torch.Tensor],
+                       n_rows: int, scale: Optional[torch.Tensor], R: Optional[int] = None,
+                       NW: Optional[int] = None) -> torch.Tensor:
+    """Per expert, silu(s g) * (s u) with (g | u) = x @ w[e]^T rounded to bfloat16, w [E, 2I, K]
+    holding gate rows then up rows: the product and the activation in one kernel, for at most
+    64 rows.  Returns [n_rows, I] bfloat16."""
+    _dev(x, w, a_rows, offsets, scale)
+    _i32(a_rows, "a_rows")
+    _i32(offsets, "offsets")
+    _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_skinny_swiglu: bfloat16 operands only")
+    _need(w.dim() == 3 and 2 <= offsets.shape[0] <= w.shape[0] + 1,
+          "gemm_skinny_swiglu: w [E, 2I, K] and offsets of at most E + 1 entries")
+    E, N, K = offsets.shape[0] - 1, w.shape[1], w.shape[2]
+    M = int(n_rows)
+    if a_rows is not None:
+        _need(a_rows.shape == (M,), "gemm_skinny_swiglu: a_rows must be [n_rows]")
+    else:
+        _need(x.shape[0] == M, "gemm_skinny_swiglu: x must have n_rows rows when not gathered")
+    _need(x.dim() == 2 and x.shape[1] == K, f"gemm_skinny_swiglu: x {tuple(x.shape)} vs w {tuple(w.shape)}")
+    _need(0 < M <= SKINNY_MAX_ROWS and K % 128 == 0 and N % 8 == 0,
+          f"gemm_skinny_swiglu: shape M={M} N={N} K={K} is not taken (M <= 64, K % 128 == 0, N % 8 == 0)")
+    if scale is not None:
+        _need(scale.dtype == torch.float32 and scale.shape == (M,), "gemm_skinny_swiglu: scale must be float32 [n_rows]")
+    pr, pw = skinny_plan(N, K)
+    out = torch.empty(M, N // 2, dtype=torch.bfloat16, device=x.device)
+    _run("sharpi_gemm_skinny_swiglu", _ptr(x), _ptr(w), _ptr(out), M, N, K, _ptr(a_rows), _ptr(offsets), E,
+         _ptr(scale), R or pr, NW or pw, _stream())
+    return out
+
+
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """y = x W^T.  float32 weights: the float FMA kernel (true 32-bit, whatever x was stored
     as).  bfloat16 weights: the library's matrix product with float accumulation."""
@@ -511,6 +574,17 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, gro
         return out
     return attention_generic(q, k_cache, v_cache, group.block_table, ctx.entry_of_token, ctx.positions, window_kind,
                              window, scale, nh, nkv, hd)
+
+
+def grouped_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, rt: Routing, out_dtype: torch.dtype) -> torch.Tensor:
+    """The experts' gate|up products of the routed tokens and their activation,
+    silu(s g) * (s u) with s the pick's weight: [n_rows, I] in expert-sorted order.  A few rows
+    take one kernel; otherwise the product and the activation are two."""
+    N, K = w_gate_up.shape[1], w_gate_up.shape[2]
+    if (x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16 and out_dtype == torch.bfloat16
+            and rt.n_rows <= SKINNY_MAX_ROWS and K % 128 == 0 and N % 8 == 0):
+        return gemm_skinny_swiglu(x, w_gate_up, rt.offsets, rt.sorted_token, rt.n_rows, rt.sorted_w)
+    return silu_mul(grouped_linear(x, w_gate_up, rt, True, out_dtype), rt.sorted_w)
 
 
 def grouped_linear(x: torch.Tensor, w: torch.Tensor, rt: Routing, gather: bool, out_dtype: torch.dtype) -> torch.Tensor:

@@ -77,8 +77,14 @@ class ResidualStream:
     """The float32 residual sum ``h`` and the branch output still to be added to it.
 
     A branch (mixer, feed-forward) leaves its output in ``pending``; the next norm adds it into
-    ``h`` in the same kernel that normalises, so the sum is formed once, in float."""
+    ``h`` in the same kernel that normalises, so the sum is formed once, in float.  ``pending``
+    is a tensor [T, H] or an object with ``shape``, ``dtype`` and ``tensor()`` that stands for one
+    (``ops.ExpertSum``); a norm that cannot fold such an object in calls ``pending_tensor()``."""
 
     def __init__(self, h: torch.Tensor):
         self.h = h
-        self.pending: Optional[torch.Tensor] = None
+        self.pending = None
+
+    def pending_tensor(self) -> Optional[torch.Tensor]:
+        p = self.pending
+        return p if p is None or isinstance(p, torch.Tensor) else p.tensor()

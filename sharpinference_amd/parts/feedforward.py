@@ -124,12 +124,11 @@ class MoESwiGLU(Part):
             trace.append((ids, wts))
         if merge:
             # few rows: the shared expert rides along as one more group of the same two launches
-            gu = ops.grouped_linear(x, self.w_gate_up, rt, True, ctx.act_dtype)
-            act = ops.silu_mul(gu, rt.sorted_w)
+            act = ops.grouped_swiglu(x, self.w_gate_up, rt, ctx.act_dtype)
             y = ops.grouped_linear(act, self.w_down, rt, False, ctx.act_dtype)
-            return ops.moe_combine(y[:T * self.k], rt.inv_pos, y[T * self.k:], T, self.k)
+            # left as a sum: the next norm forms it while it reads the residual stream
+            return ops.ExpertSum(y, rt.inv_pos, y[T * self.k:], T, self.k)
         shared = self.shared.forward(x, ctx) if self.shared is not None else None
-        gu = ops.grouped_linear(x, self.w_gate_up, rt, True, ctx.act_dtype)
-        act = ops.silu_mul(gu, rt.sorted_w)
+        act = ops.grouped_swiglu(x, self.w_gate_up, rt, ctx.act_dtype)
         y = ops.grouped_linear(act, self.w_down, rt, False, ctx.act_dtype)
         return ops.moe_combine(y, rt.inv_pos, shared, T, self.k)

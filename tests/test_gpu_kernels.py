@@ -185,6 +185,37 @@ def test_router_ties_pick_the_lowest_index():
     assert ids.cpu().tolist() == [[0, 1]] * 4 and float((wts - 0.5).abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("M,E,I,K", [(8, 4, 40, 128), (64, 16, 264, 256), (33, 5, 8192, 384), (1, 3, 20, 640)])
+def test_gemm_skinny_swiglu_equals_product_then_activation(M, E, I, K):
+    """The product with the activation in its epilogue gives the bits of the two kernels in a row."""
+    ops = _ops()
+    x = _rand(M, K, dtype=torch.bfloat16, seed=M)
+    w = _rand(E, 2 * I, K, dtype=torch.bfloat16, scale=0.1, seed=I)
+    g = torch.Generator().manual_seed(M + E)
+    ex = torch.sort(torch.randint(0, E, (M,), generator=g)).values
+    offsets = torch.zeros(E + 1, dtype=torch.int32)
+    for e in range(E):
+        offsets[e + 1] = offsets[e] + int((ex == e).sum())
+    a_rows = torch.randperm(M, generator=g).to(torch.int32).to(DEV)
+    scale = (torch.rand(M, generator=g) + 0.25).to(DEV)
+    for sc in (scale, None):
+        for R, NW in ((2, 4), (2, 8), (4, 4), (4, 8)):
+            gu = ops.gemm_skinny(x, w, torch.bfloat16, a_rows=a_rows, offsets=offsets.to(DEV), n_rows=M, R=R, NW=NW)
+            want = ops.silu_mul(gu, sc)
+            got = ops.gemm_skinny_swiglu(x, w, offsets.to(DEV), a_rows, M, sc, R=R, NW=NW)
+            assert torch.equal(got, want), (R, NW, sc is None)
+    # and against the formula
+    xs = x[a_rows.long()].float().cpu()
+    ref = torch.zeros(M, I)
+    off = offsets.tolist()
+    for e in range(E):
+        rows = slice(off[e], off[e + 1])
+        gu = (xs[rows] @ w[e].float().cpu().T).to(torch.bfloat16).float() * scale.cpu()[rows, None]
+        ref[rows] = torch.nn.functional.silu(gu[:, :I]) * gu[:, I:]
+    got = ops.gemm_skinny_swiglu(x, w, offsets.to(DEV), a_rows, M, scale).float().cpu()
+    assert float((got - ref).abs().max()) <= 2e-2 * float(ref.abs().max())
+
+
 # the last two are deep enough in K for the kernel's steady loop (and its tail of 4 and of 1 stages)
 @pytest.mark.parametrize("T,E,k,N,K", [(300, 4, 1, 264, 256), (700, 16, 2, 512, 128), (65, 3, 1, 20, 384),
                                        (500, 5, 1, 200, 640), (260, 2, 2, 136, 1216)])
