@@ -31,7 +31,38 @@ __global__ __launch_bounds__(kSampThreads) void argmax_rows_kernel(const float* 
   const float* x = logits + (size_t)blockIdx.x * vocab;
   float best = -INFINITY;
   int idx = 0x7fffffff;
-  for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
+  int i0 = 0;
+  if ((vocab & 3) == 0) {
+    // 16-byte loads, two in flight per thread: one block reads a row at a compute unit's full rate.
+    // A thread's indices still ascend, so a strict > keeps the lowest index of equal values.
+    const int v4 = vocab >> 2;
+    const float4* x4 = reinterpret_cast<const float4*>(x);
+    int q = threadIdx.x;
+    for (; q + (int)blockDim.x < v4; q += 2 * blockDim.x) {
+      const float4 a = x4[q], b = x4[q + blockDim.x];
+      const float va[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int i = (j < 4 ? q : q + (int)blockDim.x) * 4 + (j & 3);
+        if (va[j] > best || idx == 0x7fffffff) {
+          best = va[j];
+          idx = i;
+        }
+      }
+    }
+    for (; q < v4; q += blockDim.x) {
+      const float4 a = x4[q];
+      const float va[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (va[j] > best || idx == 0x7fffffff) {
+          best = va[j];
+          idx = q * 4 + j;
+        }
+    }
+    i0 = vocab;
+  }
+  for (int i = i0 + threadIdx.x; i < vocab; i += blockDim.x) {
     const float v = x[i];
     if (v > best || idx == 0x7fffffff) {  // ascending i per thread: strict > keeps the lowest index
       best = v;
