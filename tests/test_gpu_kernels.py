@@ -99,6 +99,27 @@ def _paged_case(lens, nh, nkv, hd, ps, dtype, seed, strong_key=None):
     return bt, kc.to(dtype), vc.to(dtype), ks, vs
 
 
+def _pages_from(ks, vs, ps, dtype, seed):
+    """Given dense per-request k, v [L, nkv, hd]: the same scattered over shuffled pages."""
+    g = torch.Generator().manual_seed(seed)
+    nkv, hd = ks[0].shape[1], ks[0].shape[2]
+    blocks = [(k.shape[0] + ps - 1) // ps for k in ks]
+    n_pages = sum(blocks) + 3
+    it = iter(torch.randperm(n_pages, generator=g).tolist())
+    bt = torch.full((len(ks), max(blocks)), -1, dtype=torch.int32)
+    kc = torch.zeros(n_pages, nkv, ps, hd)
+    vc = torch.zeros(n_pages, nkv, hd, ps)
+    for i, (k, v) in enumerate(zip(ks, vs)):
+        for b in range(blocks[i]):
+            page = next(it)
+            bt[i, b] = page
+            seg = slice(b * ps, min(k.shape[0], (b + 1) * ps))
+            m = seg.stop - seg.start
+            kc[page, :, :m, :] = k[seg].permute(1, 0, 2)
+            vc[page, :, :, :m] = v[seg].permute(1, 2, 0)
+    return bt, kc.to(dtype), vc.to(dtype)
+
+
 def _ref_attention(q, k, v, p, start, scale):
     """q [nh, hd]; k, v [L, nkv, hd]: softmax over keys start..p."""
     nh, hd = q.shape
@@ -141,6 +162,59 @@ def test_attention_decode_kernel(nh, nkv, hd, kind, window, ps):
     ops.attention_decode(*args, sel, max(lens), kind, window, scale, nh, nkv, hd, out=out)
     out = out.float().cpu().view(n, nh, hd)
     assert torch.equal(out[[4, 1, 3]], got[[4, 1, 3]]) and float(out[[0, 2, 5]].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("kind,window", [(0, 0), (1, 256), (2, 89)])
+@pytest.mark.parametrize("ps", [16, 32])
+def test_attention_sees_one_key_at_every_edge(kind, window, ps):
+    """Random keys would average a missed key away.  Here one key at a time is made to carry all
+    the weight (it points along the query), at the first and last position, at both sides of a
+    page's edge, of the decode kernel's 256-key runs and of the window's first key: the output
+    must be that key's value when the key is visible and must not be when it is not."""
+    ops = _ops()
+    nh, nkv, hd, L = 4, 2, 64, 600
+    scale = 1.0 / math.sqrt(hd)
+    g = torch.Generator().manual_seed(3)
+    u = torch.randn(hd, generator=g)
+    u = (u / u.norm() * math.sqrt(hd)).to(torch.bfloat16).float()
+    q1 = (2.0 * u).expand(nh, hd)                                   # every head asks the same question
+    portion = 100                                                   # prefill: the last 100 positions are queries
+    p_last = L - 1
+    start = _start(p_last, kind, window)
+    edges = {0, 1, ps - 1, ps, ps + 1, 255, 256, 257, 511, 512, 513, L - portion - 1, L - portion, L - 2, L - 1,
+             max(start - 1, 0), start, start + 1}
+    for j in sorted(edges):
+        k = (0.05 * torch.randn(L, nkv, hd, generator=g)).to(torch.bfloat16).float()
+        v = torch.randn(L, nkv, hd, generator=g).to(torch.bfloat16).float()
+        k[j] = 2.0 * u                                              # score 4 * hd * scale = 32 above the rest
+        bt, kc, vc = _pages_from([k], [v], ps, torch.bfloat16, seed=j)
+        dev = [t.to(DEV) for t in (kc, vc, bt)]
+        # decode: one query at the last position
+        qd = q1.reshape(1, nh * hd).to(torch.bfloat16).to(DEV)
+        one = torch.zeros(1, dtype=torch.int32, device=DEV)
+        pos = torch.tensor([p_last], dtype=torch.int32, device=DEV)
+        ref = _ref_attention(q1, k, v, p_last, start, scale)
+        for name, got in (("decode", ops.attention_decode(qd, *dev, one, pos, None, L, kind, window, scale, nh, nkv, hd)),
+                          ("generic", ops.attention_generic(qd, *dev, one, pos, kind, window, scale, nh, nkv, hd))):
+            got = got.float().cpu().view(nh, hd)
+            assert float((got - ref).abs().max()) <= 2e-2, (name, j)
+            near = float((got - v[j].repeat_interleave(nh // nkv, 0)).abs().max())
+            assert (near <= 2e-2) == (j >= start), (name, j, near)
+        # prefill: the last `portion` positions in one step, every query the same question
+        T = portion
+        qp = q1.reshape(1, nh * hd).expand(T, nh * hd).to(torch.bfloat16).contiguous().to(DEV)
+        positions = torch.arange(L - T, L, dtype=torch.int32)
+        tiles = torch.tensor([(0, o, min(ops.PREFILL_TILE_TOKENS, T - o)) for o in range(0, T, ops.PREFILL_TILE_TOKENS)],
+                             dtype=torch.int32, device=DEV)
+        got = ops.attention_prefill(qp, *dev, positions.to(DEV), tiles, kind, window, scale, nh, nkv, hd)
+        got = got.float().cpu().view(T, nh, hd)
+        for i in (0, 1, T // 2, T - 2, T - 1):
+            p = int(positions[i])
+            st = _start(p, kind, window)
+            ref = _ref_attention(q1, k, v, p, st, scale)
+            assert float((got[i] - ref).abs().max()) <= 2e-2, ("prefill", j, p)
+            near = float((got[i] - v[j].repeat_interleave(nh // nkv, 0)).abs().max())
+            assert (near <= 2e-2) == (st <= j <= p), ("prefill", j, p, near)
 
 
 # ---------------------------------------------------------------------------
