@@ -56,7 +56,7 @@ constexpr int GQ = SHARPI_GQ;       // 16-row groups whose LDS reads go out toge
 constexpr int kHalves = 2;         // a tile's column blocks are split over this many XCDs
 
 // The work of one tile of NQ * 64 rows (the block's rows, rounded up) against GN weight rows.
-template <typename TO, int NQ>
+template <typename TO, int NQ, bool PACKED>
 __device__ __forceinline__ void grouped_tile(const bf16_t* __restrict__ x, const bf16_t* __restrict__ We,
                                              TO* __restrict__ out, int N, int K, const int* __restrict__ a_rows,
                                              int row0, int row_end, int n_base, bf16_t (*xs)[GM][GPAD]) {
@@ -66,12 +66,24 @@ __device__ __forceinline__ void grouped_tile(const bf16_t* __restrict__ x, const
   const int r = lane & 15, g = lane >> 4;
 
   // 32-bit element offsets from uniform bases (the host checks that they fit): half the address registers
+  // Row layout: lane (r, g) reads 16 bytes of row n at k = c*GK + j*32 + g*8.  Packed layout (the
+  // matrix stored as [N/16][K/128][16 runs of 8 k][16 rows][8]): the same element sits at
+  // tile*16*K + c*GK*16 + j*512 + lane*8, and a wave's load is one contiguous 1 KB.
+  constexpr uint32_t kStageStep = PACKED ? GK * 16 : GK;
+  constexpr uint32_t kSubStep = PACKED ? 512 : 32;
+  static_assert(128 % GK == 0, "a K stage must not straddle a packed 128-wide unit");
   uint32_t woff[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
-    int n = n_base + t * 16 + r;
-    if (n >= N) n = N - 1;  // loaded, never stored
-    woff[t] = (uint32_t)n * (uint32_t)K + g * 8;
+    if constexpr (PACKED) {
+      int n = n_base + t * 16;
+      if (n >= N) n = N - 16;  // loaded, never stored
+      woff[t] = (uint32_t)n * (uint32_t)K + lane * 8;
+    } else {
+      int n = n_base + t * 16 + r;
+      if (n >= N) n = N - 1;  // loaded, never stored
+      woff[t] = (uint32_t)n * (uint32_t)K + g * 8;
+    }
   }
   // staging role: thread loads 16 bytes of row (tid / 8 + GROWS * pass), columns (tid % 8) * 8
   const int srow = threadIdx.x / (GK / 8), scol = (threadIdx.x % (GK / 8)) * 8;
@@ -110,7 +122,7 @@ __device__ __forceinline__ void grouped_tile(const bf16_t* __restrict__ x, const
 #pragma unroll
         for (int j = 0; j < GK / 32; ++j)
 #pragma unroll
-          for (int t = 0; t < NT; ++t) wf[a][j][t] = *reinterpret_cast<const bf16x8*>(We + woff[t] + a * GK + j * 32);
+          for (int t = 0; t < NT; ++t) wf[a][j][t] = *reinterpret_cast<const bf16x8*>(We + woff[t] + a * kStageStep + j * kSubStep);
       }
   };
   if (chunks >= kAhead) fill_ring(std::true_type{}); else fill_ring(std::false_type{});
@@ -154,7 +166,7 @@ __device__ __forceinline__ void grouped_tile(const bf16_t* __restrict__ x, const
       for (int j = 0; j < GK / 32; ++j)
 #pragma unroll
         for (int t = 0; t < NT; ++t)
-          wf[slot][j][t] = *reinterpret_cast<const bf16x8*>(We + woff[t] + (c + kAhead) * GK + j * 32);
+          wf[slot][j][t] = *reinterpret_cast<const bf16x8*>(We + woff[t] + (c + kAhead) * kStageStep + j * kSubStep);
     }
     if (steady || c + 1 < chunks) {   // the next stage's x rows, fetched a stage ago
 #pragma unroll
@@ -202,7 +214,7 @@ __device__ __forceinline__ void grouped_tile(const bf16_t* __restrict__ x, const
   }
 }
 
-template <typename TO>
+template <typename TO, bool PACKED>
 __global__ __launch_bounds__(GW* kWave, 2) void grouped_gemm_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ W, TO* __restrict__ out, int N, int K,
     const int* __restrict__ a_rows, const int* __restrict__ group_offsets, const int* __restrict__ tile_expert,
@@ -226,38 +238,42 @@ __global__ __launch_bounds__(GW* kWave, 2) void grouped_gemm_kernel(
   const bf16_t* We = W + (size_t)e * N * K;
   static_assert(GM == 192, "three tile heights are compiled: 64, 128 and 192 rows");
   if (n_rows <= 64)
-    grouped_tile<TO, 1>(x, We, out, N, K, a_rows, row0, row_end, n_base, xs);
+    grouped_tile<TO, 1, PACKED>(x, We, out, N, K, a_rows, row0, row_end, n_base, xs);
   else if (n_rows <= 128)
-    grouped_tile<TO, 2>(x, We, out, N, K, a_rows, row0, row_end, n_base, xs);
+    grouped_tile<TO, 2, PACKED>(x, We, out, N, K, a_rows, row0, row_end, n_base, xs);
   else
-    grouped_tile<TO, 3>(x, We, out, N, K, a_rows, row0, row_end, n_base, xs);
+    grouped_tile<TO, 3, PACKED>(x, We, out, N, K, a_rows, row0, row_end, n_base, xs);
 }
 
 // x [x_rows, K] bf16 (rows gathered through a_rows if given), W [E, N, K] bf16, out [n_rows, N];
 // group_offsets [E + 1]; tile_expert / tile_row0 [max_tiles], n_tiles [1] from the routing kernel
-// (tiles of sharpi_gemm_grouped_tile_rows() rows).  max_tiles bounds the grid.
+// (tiles of sharpi_gemm_grouped_tile_rows() rows).  max_tiles bounds the grid.  packed: W is stored
+// tile by tile, [E][N/16][K/128][16 runs of 8 k][16 rows][8] (N % 16 == 0, K % 128 == 0).
 SHARPI_EXPORT int sharpi_gemm_grouped(const void* x, int x_rows, const void* W, void* out, int out_dtype, int n_rows,
                                       int N, int K, const int* a_rows, const int* group_offsets, const int* tile_expert,
-                                      const int* tile_row0, const int* n_tiles, int max_tiles,
+                                      const int* tile_row0, const int* n_tiles, int max_tiles, int packed,
                                       hipStream_t stream) {
   if (n_rows <= 0) return SHARPI_OK;
   if (N <= 0 || (N & 3) || K <= 0 || K % GK != 0 || max_tiles <= 0) return SHARPI_ERR_ARG;
+  if (packed && ((N & 15) || (K & 127))) return SHARPI_ERR_ARG;
   if (!group_offsets || !tile_expert || !tile_row0 || !n_tiles) return SHARPI_ERR_ARG;
   // the kernel addresses x and one expert's weights with 32-bit element offsets
   if ((long long)N * K > 0x7fffffffLL || x_rows <= 0 || (long long)x_rows * K > 0x7fffffffLL) return SHARPI_ERR_ARG;
   const int nb_per_unit = ceil_div(ceil_div(N, GN), kHalves);
   const int units = ceil_div(max_tiles * kHalves, kXcds) * kXcds;
   dim3 grid(units * nb_per_unit), block(GW * kWave);
-  if (out_dtype == DT_BF16)
-    grouped_gemm_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)x, (const bf16_t*)W, (bf16_t*)out, N, K,
-                                                           a_rows, group_offsets, tile_expert, tile_row0, n_tiles,
-                                                           nb_per_unit);
-  else if (out_dtype == DT_F32)
-    grouped_gemm_kernel<float><<<grid, block, 0, stream>>>((const bf16_t*)x, (const bf16_t*)W, (float*)out, N, K,
-                                                          a_rows, group_offsets, tile_expert, tile_row0, n_tiles,
-                                                          nb_per_unit);
-  else
+#define GG_LAUNCH(TOV, PK)                                                                                        \
+  grouped_gemm_kernel<TOV, PK><<<grid, block, 0, stream>>>((const bf16_t*)x, (const bf16_t*)W, (TOV*)out, N, K,    \
+                                                          a_rows, group_offsets, tile_expert, tile_row0, n_tiles,  \
+                                                          nb_per_unit)
+  if (out_dtype == DT_BF16) {
+    if (packed) GG_LAUNCH(bf16_t, true); else GG_LAUNCH(bf16_t, false);
+  } else if (out_dtype == DT_F32) {
+    if (packed) GG_LAUNCH(float, true); else GG_LAUNCH(float, false);
+  } else {
     return SHARPI_ERR_ARG;
+  }
+#undef GG_LAUNCH
   SHARPI_CHECK_LAUNCH();
   return SHARPI_OK;
 }

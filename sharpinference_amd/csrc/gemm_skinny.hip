@@ -14,6 +14,10 @@
 //    [offsets[e], offsets[e + 1]) of the expert-sorted row list with W[e], sixteen at a time;
 //    x rows are gathered through a_rows.  Experts without rows return at once.
 //
+//  * Packed weights (PACKED): the matrix is stored tile by tile instead of row by row, the 4 KB
+//    of a (16-row tile, 128-wide K unit) contiguous and in the order the lanes want them, and
+//    the K units are dealt to the waves in turn: a block's reads are contiguous runs of NW * 4 KB
+//    rather than 256-byte pieces a row apart, worth about a tenth of the bandwidth.
 //  * SwiGLU form (ACT): W holds gate rows [0, N/2) and up rows [N/2, N); a block takes R/2 tiles
 //    of each at the same columns, and the wave that adds up a gate tile adds up its up tile too,
 //    rounds both to bfloat16 (what a separate activation kernel would have read) and stores
@@ -38,7 +42,7 @@ template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, f32x4 v) {
 
 constexpr int kRedTiles = 2;  // (tile, row block) pairs summed per LDS round
 
-template <int R, int MB, int NW, typename TO, bool ACT>
+template <int R, int MB, int NW, typename TO, bool ACT, bool PACKED>
 __global__ __launch_bounds__(NW* kWave) void skinny_gemm_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ W, TO* __restrict__ out, int M, int N, int K,
     const int* __restrict__ a_rows, const int* __restrict__ group_offsets, const float* __restrict__ act_scale) {
@@ -67,14 +71,27 @@ __global__ __launch_bounds__(NW* kWave) void skinny_gemm_kernel(
   const int u_begin = (U * w) / NW;
   const int u_end = (U * (w + 1)) / NW;
 
+  // Row layout: lane (row r, group g) reads the 64-byte run k0 + g*32 .. + 32 of its row, 16 bytes
+  // per MFMA step j.  Packed layout: the 4 KB of a (16-row tile, 128-wide unit) are contiguous
+  // in the order [j][g][r][8 elements], so step j of a wave is one contiguous 1 KB read and the
+  // lane's 8 elements are k0 + (4j + g)*8 .. + 8 of row r; x is read at the same k.
   const bf16_t* wrow[R];
 #pragma unroll
   for (int t = 0; t < R; ++t) {
-    int n = n_base + (t % TG) * 16 + r;
-    if (n >= n_out) n = n_out - 1;  // loaded, never stored
-    if (ACT && t >= TG) n += n_out;  // the up row of the same column
-    wrow[t] = W + (size_t)n * K + g * 32;
+    if constexpr (PACKED) {
+      int tile = (n_base >> 4) + (t % TG);
+      if (tile * 16 >= n_out) tile = (n_out >> 4) - 1;   // loaded, never stored
+      if (ACT && t >= TG) tile += n_out >> 4;            // the up tile of the same columns
+      wrow[t] = W + (size_t)tile * 16 * K + lane * 8;
+    } else {
+      int n = n_base + (t % TG) * 16 + r;
+      if (n >= n_out) n = n_out - 1;  // loaded, never stored
+      if (ACT && t >= TG) n += n_out;  // the up row of the same column
+      wrow[t] = W + (size_t)n * K + g * 32;
+    }
   }
+  constexpr int XG = PACKED ? 8 : 32;    // x: a lane's first k within a unit is g * XG, step j adds XJ
+  constexpr int XJ = PACKED ? 32 : 8;
 
   for (int rb0 = 0; rb0 * 16 < n_rows; rb0 += MB) {
     const bf16_t* xrow[MB];
@@ -84,7 +101,7 @@ __global__ __launch_bounds__(NW* kWave) void skinny_gemm_kernel(
       const int m = row_begin + (rb0 + mb) * 16 + r;
       xvalid[mb] = m < row_end;
       const int src = xvalid[mb] ? (a_rows ? a_rows[m] : m) : 0;
-      xrow[mb] = x + (size_t)src * K + g * 32;
+      xrow[mb] = x + (size_t)src * K + g * XG;
     }
     f32x4 acc[R][MB];
 #pragma unroll
@@ -92,18 +109,21 @@ __global__ __launch_bounds__(NW* kWave) void skinny_gemm_kernel(
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) acc[t][mb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    for (int u = u_begin; u < u_end; ++u) {
+    // Row layout: a wave takes a contiguous slice of K.  Packed layout: units are dealt to the
+    // waves in turn, so that the block reads NW * 4 KB of a tile side by side at every step.
+    for (int u = PACKED ? w : u_begin; u < (PACKED ? U : u_end); u += PACKED ? NW : 1) {
       const int k0 = u << 7;
       bf16x8 wf[R][4], xf[MB][4];
 #pragma unroll
       for (int t = 0; t < R; ++t)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) wf[t][j] = *reinterpret_cast<const bf16x8*>(wrow[t] + k0 + j * 8);
+        for (int j = 0; j < 4; ++j)
+          wf[t][j] = *reinterpret_cast<const bf16x8*>(wrow[t] + (PACKED ? (size_t)u * 2048 + j * 512 : (size_t)k0 + j * 8));
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          if (xvalid[mb]) xf[mb][j] = *reinterpret_cast<const bf16x8*>(xrow[mb] + k0 + j * 8);
+          if (xvalid[mb]) xf[mb][j] = *reinterpret_cast<const bf16x8*>(xrow[mb] + k0 + j * XJ);
           else xf[mb][j] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
         }
 #pragma unroll
@@ -164,46 +184,50 @@ __global__ __launch_bounds__(NW* kWave) void skinny_gemm_kernel(
   }
 }
 
-template <int R, int MB, int NW, bool ACT>
+template <int R, int MB, int NW, bool ACT, bool PACKED>
 static int launch_skinny(const void* x, const void* W, void* out, int out_dtype, int M, int N, int K,
                          const int* a_rows, const int* group_offsets, int groups, const float* act_scale,
                          hipStream_t stream) {
   dim3 grid(ceil_div(ACT ? N / 2 : N, 16 * (ACT ? R / 2 : R)), groups > 0 ? groups : 1), block(NW * kWave);
   const int* go = groups > 0 ? group_offsets : nullptr;
   if (out_dtype == DT_F32)
-    skinny_gemm_kernel<R, MB, NW, float, ACT><<<grid, block, 0, stream>>>(
+    skinny_gemm_kernel<R, MB, NW, float, ACT, PACKED><<<grid, block, 0, stream>>>(
         (const bf16_t*)x, (const bf16_t*)W, (float*)out, M, N, K, a_rows, go, act_scale);
   else
-    skinny_gemm_kernel<R, MB, NW, bf16_t, ACT><<<grid, block, 0, stream>>>(
+    skinny_gemm_kernel<R, MB, NW, bf16_t, ACT, PACKED><<<grid, block, 0, stream>>>(
         (const bf16_t*)x, (const bf16_t*)W, (bf16_t*)out, M, N, K, a_rows, go, act_scale);
   SHARPI_CHECK_LAUNCH();
   return SHARPI_OK;
 }
 
-template <int R, int NW>
+template <int R, int NW, bool PACKED>
 static int dispatch_mb(int MB, const void* x, const void* W, void* out, int out_dtype, int M, int N, int K,
                        const int* a_rows, const int* group_offsets, int groups, hipStream_t stream) {
-  if (MB == 1) return launch_skinny<R, 1, NW, false>(x, W, out, out_dtype, M, N, K, a_rows, group_offsets, groups, nullptr, stream);
-  if (MB == 2) return launch_skinny<R, 2, NW, false>(x, W, out, out_dtype, M, N, K, a_rows, group_offsets, groups, nullptr, stream);
-  return launch_skinny<R, 4, NW, false>(x, W, out, out_dtype, M, N, K, a_rows, group_offsets, groups, nullptr, stream);
+  if (MB == 1) return launch_skinny<R, 1, NW, false, PACKED>(x, W, out, out_dtype, M, N, K, a_rows, group_offsets, groups, nullptr, stream);
+  if (MB == 2) return launch_skinny<R, 2, NW, false, PACKED>(x, W, out, out_dtype, M, N, K, a_rows, group_offsets, groups, nullptr, stream);
+  return launch_skinny<R, 4, NW, false, PACKED>(x, W, out, out_dtype, M, N, K, a_rows, group_offsets, groups, nullptr, stream);
 }
 
 // x [M, K] bf16 (rows gathered through a_rows if given), W [N, K] or [groups, N, K] bf16,
 // out [M, N] (out_dtype float or bf16).  groups == 0: plain.  groups > 0: rows are the
 // expert-sorted list, group_offsets [groups + 1].  R in {1, 2, 4}: 16-row weight tiles per block;
 // NW in {4, 8, 16}: waves per block splitting K (16 only with R = 1: a block of 1,024 threads has
-// 128 registers a lane, which wider tiles do not fit).
+// 128 registers a lane, which wider tiles do not fit).  packed: W is stored tile by tile,
+// [N/16][K/128][16 runs of 8 k][16 rows][8] (N % 16 == 0), instead of row by row.
 SHARPI_EXPORT int sharpi_gemm_skinny(const void* x, const void* W, void* out, int out_dtype, int M, int N, int K,
                                      const int* a_rows, const int* group_offsets, int groups, int R, int NW,
-                                     hipStream_t stream) {
+                                     int packed, hipStream_t stream) {
   if (M <= 0) return SHARPI_OK;
   if (M > 64 || N <= 0 || (N & 3) || K <= 0 || (K & 127) || groups < 0 || groups > 65535) return SHARPI_ERR_ARG;
   if (groups > 0 && group_offsets == nullptr) return SHARPI_ERR_ARG;
   if (out_dtype != DT_F32 && out_dtype != DT_BF16) return SHARPI_ERR_ARG;
+  if (packed && (N & 15)) return SHARPI_ERR_ARG;
   // grouped rows are spread over experts: one row block at a time; plain: all row blocks at once
   const int MB = groups > 0 ? 1 : ceil_div(M, 16);
-#define SK(RR, WW) \
-  if (R == RR && NW == WW) return dispatch_mb<RR, WW>(MB, x, W, out, out_dtype, M, N, K, a_rows, group_offsets, groups, stream)
+#define SK(RR, WW)                                                                                                        \
+  if (R == RR && NW == WW)                                                                                                \
+  return packed ? dispatch_mb<RR, WW, true>(MB, x, W, out, out_dtype, M, N, K, a_rows, group_offsets, groups, stream)     \
+                : dispatch_mb<RR, WW, false>(MB, x, W, out, out_dtype, M, N, K, a_rows, group_offsets, groups, stream)
   SK(1, 4); SK(1, 8); SK(1, 16);
   SK(2, 4); SK(2, 8);
   SK(4, 4); SK(4, 8);
@@ -214,16 +238,19 @@ SHARPI_EXPORT int sharpi_gemm_skinny(const void* x, const void* W, void* out, in
 // The grouped product with SwiGLU applied in its epilogue: W [groups, N, K] holds gate rows
 // [0, N/2) and up rows [N/2, N) of every expert; out [M, N/2] bf16 =
 // silu(s g) * (s u) with g, u the two products rounded to bfloat16 and s = act_scale[row] (null: 1).
-// Rows are the expert-sorted list (sixteen of an expert at a time).  R in {2, 4}, NW in {4, 8}.
+// Rows are the expert-sorted list (sixteen of an expert at a time).  R in {2, 4}, NW in {4, 8};
+// packed as above (N % 32 == 0 then).
 SHARPI_EXPORT int sharpi_gemm_skinny_swiglu(const void* x, const void* W, void* out, int M, int N, int K,
                                             const int* a_rows, const int* group_offsets, int groups,
-                                            const float* act_scale, int R, int NW, hipStream_t stream) {
+                                            const float* act_scale, int R, int NW, int packed, hipStream_t stream) {
   if (M <= 0) return SHARPI_OK;
   if (M > 64 || N <= 0 || (N & 7) || K <= 0 || (K & 127) || groups <= 0 || groups > 65535) return SHARPI_ERR_ARG;
   if (group_offsets == nullptr) return SHARPI_ERR_ARG;
-#define SKA(RR, WW)           \
-  if (R == RR && NW == WW)    \
-  return launch_skinny<RR, 1, WW, true>(x, W, out, DT_BF16, M, N, K, a_rows, group_offsets, groups, act_scale, stream)
+  if (packed && (N & 31)) return SHARPI_ERR_ARG;
+#define SKA(RR, WW)                                                                                                              \
+  if (R == RR && NW == WW)                                                                                                       \
+  return packed ? launch_skinny<RR, 1, WW, true, true>(x, W, out, DT_BF16, M, N, K, a_rows, group_offsets, groups, act_scale, stream)  \
+                : launch_skinny<RR, 1, WW, true, false>(x, W, out, DT_BF16, M, N, K, a_rows, group_offsets, groups, act_scale, stream)
   SKA(2, 4); SKA(2, 8);
   SKA(4, 4); SKA(4, 8);
 #undef SKA

@@ -303,6 +303,69 @@ def gemm_tiled(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype
 
 
 # ---------------------------------------------------------------------------
+# weights stored for streaming
+# ---------------------------------------------------------------------------
+class PackedWeight:
+    """A bfloat16 matrix [N, K] (or a stack [E, N, K]) stored tile by tile for the decode kernels:
+    [N/16][K/128][16 runs of 8 k][16 rows][8], the 4 KB of a (16-row tile, 128-wide unit) in the
+    order a wave's lanes read them, so that a wave's load is one contiguous kilobyte.  ``packed``
+    has the logical shape but that element order; ``rows`` is the ordinary row-major matrix, kept
+    where the library's product (which wants rows) also multiplies by it, else None."""
+
+    __slots__ = ("packed", "rows", "shape", "dtype")
+
+    def __init__(self, packed: torch.Tensor, rows: Optional[torch.Tensor]):
+        self.packed, self.rows = packed, rows
+        self.shape, self.dtype = packed.shape, packed.dtype
+
+    def dim(self) -> int:
+        return len(self.shape)
+
+    def select(self, e: int) -> "PackedWeight":
+        """Matrix e of a stack (a view)."""
+        return PackedWeight(self.packed[e], self.rows[e] if self.rows is not None else None)
+
+
+def can_pack(w: torch.Tensor) -> bool:
+    return w.dtype == torch.bfloat16 and w.dim() in (2, 3) and w.shape[-2] % 16 == 0 and w.shape[-1] % 128 == 0
+
+
+def pack_into(dst: torch.Tensor, w: torch.Tensor) -> None:
+    """Write w [.., N, K] into dst (same shape, contiguous) in packed order."""
+    _need(dst.shape == w.shape and dst.is_contiguous() and can_pack(w), "pack_into: shapes must match and be packable")
+    N, K = w.shape[-2], w.shape[-1]
+    lead = w.shape[:-2]
+    src = w.reshape(*lead, N // 16, 16, K // 128, 16, 8)
+    n = len(lead)
+    dst.view(*lead, N // 16, K // 128, 16, 16, 8).copy_(src.permute(*range(n), n, n + 2, n + 3, n + 1, n + 4))
+
+
+def pack_weight(w: torch.Tensor, keep_rows: bool = True):
+    """w as a PackedWeight if its shape and type allow it, else w itself."""
+    if not can_pack(w):
+        return w
+    packed = torch.empty_like(w, memory_format=torch.contiguous_format)
+    pack_into(packed, w)
+    return PackedWeight(packed, w if keep_rows else None)
+
+
+def unpack_weight(w: "PackedWeight") -> torch.Tensor:
+    """The row-major matrix of a PackedWeight (a copy unless it is kept)."""
+    if w.rows is not None:
+        return w.rows
+    N, K = w.shape[-2], w.shape[-1]
+    lead = tuple(w.shape[:-2])
+    n = len(lead)
+    src = w.packed.view(*lead, N // 16, K // 128, 16, 16, 8)
+    return src.permute(*range(n), n, n + 3, n + 1, n + 2, n + 4).reshape(*lead, N, K).contiguous()
+
+
+def _unwrap(w):
+    """(tensor in the kernel's order, packed?) of a weight given as a tensor or a PackedWeight."""
+    return (w.packed, True) if isinstance(w, PackedWeight) else (w, False)
+
+
+# ---------------------------------------------------------------------------
 # the weight-streaming product for few rows (decode)
 # ---------------------------------------------------------------------------
 SKINNY_MAX_ROWS = 64          # grouped form: rows of all experts together
@@ -320,10 +383,12 @@ def skinny_plan(N: int, K: int):
     return (4 if N >= 12288 else 2), 8
 
 
-def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, a_rows: Optional[torch.Tensor] = None,
+def gemm_skinny(x: torch.Tensor, w, out_dtype: torch.dtype, a_rows: Optional[torch.Tensor] = None,
                 offsets: Optional[torch.Tensor] = None, n_rows: Optional[int] = None, R: Optional[int] = None,
                 NW: Optional[int] = None) -> torch.Tensor:
-    """x [M, K] @ w[N, K]^T (or per expert with w [E, N, K]) for M <= 64 on the matrix cores."""
+    """x [M, K] @ w[N, K]^T (or per expert with w [E, N, K]) for M <= 64 on the matrix cores;
+    w a tensor (row-major) or a PackedWeight."""
+    w, packed = _unwrap(w)
     _dev(x, w, a_rows, offsets)
     _i32(a_rows, "a_rows")
     _i32(offsets, "offsets")
@@ -348,16 +413,17 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, a_rows
     pr, pw = skinny_plan(N, K)
     out = torch.empty(M, N, dtype=out_dtype, device=x.device)
     _run("sharpi_gemm_skinny", _ptr(x), _ptr(w), _ptr(out), _code(out_dtype), M, N, K, _ptr(a_rows), _ptr(offsets), E,
-         R or pr, NW or pw, _stream())
+         R or pr, NW or pw, 1 if packed else 0, _stream())
     return out
 
 
-def gemm_skinny_swiglu(x: torch.Tensor, w: torch.Tensor, offsets: torch.Tensor, a_rows: Optional[torch.Tensor],
+def gemm_skinny_swiglu(x: torch.Tensor, w, offsets: torch.Tensor, a_rows: Optional[torch.Tensor],
                        n_rows: int, scale: Optional[torch.Tensor], R: Optional[int] = None,
                        NW: Optional[int] = None) -> torch.Tensor:
     """Per expert, silu(s g) * (s u) with (g | u) = x @ w[e]^T rounded to bfloat16, w [E, 2I, K]
     holding gate rows then up rows: the product and the activation in one kernel, for at most
     64 rows.  Returns [n_rows, I] bfloat16."""
+    w, packed = _unwrap(w)
     _dev(x, w, a_rows, offsets, scale)
     _i32(a_rows, "a_rows")
     _i32(offsets, "offsets")
@@ -373,19 +439,27 @@ def gemm_skinny_swiglu(x: torch.Tensor, w: torch.Tensor, offsets: torch.Tensor, 
     _need(x.dim() == 2 and x.shape[1] == K, f"gemm_skinny_swiglu: x {tuple(x.shape)} vs w {tuple(w.shape)}")
     _need(0 < M <= SKINNY_MAX_ROWS and K % 128 == 0 and N % 8 == 0,
           f"gemm_skinny_swiglu: shape M={M} N={N} K={K} is not taken (M <= 64, K % 128 == 0, N % 8 == 0)")
+    _need(not packed or N % 32 == 0, "gemm_skinny_swiglu: packed weights need gate and up rows in whole 16-row tiles")
     if scale is not None:
         _need(scale.dtype == torch.float32 and scale.shape == (M,), "gemm_skinny_swiglu: scale must be float32 [n_rows]")
     pr, pw = skinny_plan(N, K)
     out = torch.empty(M, N // 2, dtype=torch.bfloat16, device=x.device)
     _run("sharpi_gemm_skinny_swiglu", _ptr(x), _ptr(w), _ptr(out), M, N, K, _ptr(a_rows), _ptr(offsets), E,
-         _ptr(scale), R or pr, NW or pw, _stream())
+         _ptr(scale), R or pr, NW or pw, 1 if packed else 0, _stream())
     return out
 
 
-def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+def linear(x: torch.Tensor, w, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """y = x W^T.  float32 weights: the float FMA kernel (true 32-bit, whatever x was stored
-    as).  bfloat16 weights: the library's matrix product with float accumulation."""
+    as).  bfloat16 weights: the weight-streaming kernel for a few rows (over the packed form if w
+    is a PackedWeight), the library's matrix product with float accumulation otherwise."""
     out_dtype = out_dtype or x.dtype
+    if isinstance(w, PackedWeight):
+        xb = x if x.dtype == torch.bfloat16 else cast(x, torch.bfloat16)
+        _need(xb.dim() == 2 and xb.shape[1] == w.shape[1], f"linear: x {tuple(x.shape)} vs w {tuple(w.shape)}")
+        if skinny_ok(xb.shape[0], w.shape[0], w.shape[1]):
+            return gemm_skinny(xb, w, out_dtype)
+        w = unpack_weight(w)
     if w.dtype == torch.float32:
         xf = x if x.dtype == torch.float32 else cast(x, torch.float32)
         y = gemm_tiled(xf, w, torch.float32)
@@ -497,9 +571,10 @@ def route(x: torch.Tensor, wr: torch.Tensor, k: int, gate: int = GATE_SIGMOID, r
     return ids, wts, moe_permute(ids, wts, wr.shape[0], shared_group)
 
 
-def gemm_grouped(x: torch.Tensor, w: torch.Tensor, rt: Routing, gather: bool, out_dtype: torch.dtype) -> torch.Tensor:
+def gemm_grouped(x: torch.Tensor, w, rt: Routing, gather: bool, out_dtype: torch.dtype) -> torch.Tensor:
     """Per-expert products for many rows on the matrix cores (bfloat16).  gather: x rows are read
     through the routing's token list; otherwise x is already in expert-sorted order."""
+    w, packed = _unwrap(w)
     _dev(x, w)
     _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_grouped: bfloat16 operands only")
     _need(w.dim() == 3 and w.shape[0] >= rt.n_experts and rt.n_groups == rt.n_experts and x.dim() == 2
@@ -510,7 +585,7 @@ def gemm_grouped(x: torch.Tensor, w: torch.Tensor, rt: Routing, gather: bool, ou
     out = torch.empty(rt.n_rows, N, dtype=out_dtype, device=x.device)
     _run("sharpi_gemm_grouped", _ptr(x), x.shape[0], _ptr(w), _ptr(out), _code(out_dtype), rt.n_rows, N, K,
          _ptr(rt.sorted_token) if gather else None, _ptr(rt.offsets), _ptr(rt.tile_expert), _ptr(rt.tile_row0),
-         _ptr(rt.n_tiles), rt.max_tiles, _stream())
+         _ptr(rt.n_tiles), rt.max_tiles, 1 if packed else 0, _stream())
     return out
 
 
@@ -576,20 +651,21 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, gro
                              window, scale, nh, nkv, hd)
 
 
-def grouped_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, rt: Routing, out_dtype: torch.dtype) -> torch.Tensor:
+def grouped_swiglu(x: torch.Tensor, w_gate_up, rt: Routing, out_dtype: torch.dtype) -> torch.Tensor:
     """The experts' gate|up products of the routed tokens and their activation,
     silu(s g) * (s u) with s the pick's weight: [n_rows, I] in expert-sorted order.  A few rows
     take one kernel; otherwise the product and the activation are two."""
     N, K = w_gate_up.shape[1], w_gate_up.shape[2]
     if (x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16 and out_dtype == torch.bfloat16
-            and rt.n_rows <= SKINNY_MAX_ROWS and K % 128 == 0 and N % 8 == 0):
+            and rt.n_rows <= SKINNY_MAX_ROWS and K % 128 == 0 and N % (32 if isinstance(w_gate_up, PackedWeight) else 8) == 0):
         return gemm_skinny_swiglu(x, w_gate_up, rt.offsets, rt.sorted_token, rt.n_rows, rt.sorted_w)
     return silu_mul(grouped_linear(x, w_gate_up, rt, True, out_dtype), rt.sorted_w)
 
 
-def grouped_linear(x: torch.Tensor, w: torch.Tensor, rt: Routing, gather: bool, out_dtype: torch.dtype) -> torch.Tensor:
-    """Per-expert products over the routing's expert-sorted row list: w [E, N, K]; x rows are read
-    through the token list (gather) or are already in sorted order.  Returns [n_rows, N]."""
+def grouped_linear(x: torch.Tensor, w, rt: Routing, gather: bool, out_dtype: torch.dtype) -> torch.Tensor:
+    """Per-expert products over the routing's expert-sorted row list: w [E, N, K] (a tensor or a
+    PackedWeight); x rows are read through the token list (gather) or are already in sorted order.
+    Returns [n_rows, N]."""
     if x.dtype != w.dtype:
         x = cast(x, w.dtype)
     N, K = w.shape[1], w.shape[2]

@@ -63,8 +63,9 @@ class Attention(Part):
         for p in parts:
             fused[o:o + p.shape[0]].copy_(p)
             o += p.shape[0]
-        self.w_qkv = fused
-        self.w_o = source.get(prefix + "o_proj.weight")
+        # both also in the order the few-rows kernel streams them; the rows stay for prompt-sized steps
+        self.w_qkv = ops.pack_weight(fused)
+        self.w_o = ops.pack_weight(source.get(prefix + "o_proj.weight"))
 
     # -- compute --------------------------------------------------------------
     def forward(self, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> torch.Tensor:

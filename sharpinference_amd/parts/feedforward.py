@@ -20,6 +20,10 @@ def _fuse_rows(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def _rows(w) -> torch.Tensor:
+    return ops.unpack_weight(w) if isinstance(w, ops.PackedWeight) else w
+
+
 class DenseSwiGLU(Part):
     """down( silu(gate x) * (up x) ) (reference: src/SharpInference.Engine/ForwardPass.cs:2006-2015;
     silu(g) = g / (1 + exp(-g)), src/SharpInference.Cpu/SimdKernels.cs:4377-4408)."""
@@ -39,9 +43,10 @@ class DenseSwiGLU(Part):
     def load(self, prefix: str, source: TensorSource) -> None:
         g = source.get(prefix + "gate_proj.weight")
         u = source.get(prefix + "up_proj.weight")
-        self.w_gate_up = _fuse_rows(g, u)
+        # both also in the order the few-rows kernel streams them; the rows stay for prompt-sized steps
+        self.w_gate_up = ops.pack_weight(_fuse_rows(g, u))
         del g, u
-        self.w_down = source.get(prefix + "down_proj.weight")
+        self.w_down = ops.pack_weight(source.get(prefix + "down_proj.weight"))
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         gu = ops.linear(x, self.w_gate_up, ctx.act_dtype)
@@ -94,26 +99,43 @@ class MoESwiGLU(Part):
         self.w_router = source.get(prefix + "router.weight")
         g = source.get(prefix + "experts.gate_proj")
         u = source.get(prefix + "experts.up_proj")
-        self.w_gate_up = _fuse_rows(g, u)
-        del g, u
-        self.w_down = source.get(prefix + "experts.down_proj")
+        d = source.get(prefix + "experts.down_proj")
         self.merged = False
-        if self.shared is not None:
-            self.shared.load(prefix + "shared_expert.", source)
-            sh = self.shared
-            if (sh.inter == self.inter and sh.w_gate_up.dtype == self.w_gate_up.dtype == torch.bfloat16
-                    and sh.w_down.dtype == self.w_down.dtype == torch.bfloat16):
-                # The shared expert becomes expert E of the experts' tensors (its own tensors turn
-                # into views of them): few-row steps then run it in the same launches as the routed ones.
-                gu = torch.empty(self.E + 1, 2 * self.inter, self.hidden, dtype=torch.bfloat16, device=self.w_gate_up.device)
-                gu[:self.E].copy_(self.w_gate_up)
-                gu[self.E].copy_(sh.w_gate_up)
-                self.w_gate_up, sh.w_gate_up = gu, gu[self.E]
-                dn = torch.empty(self.E + 1, self.hidden, self.inter, dtype=torch.bfloat16, device=self.w_down.device)
-                dn[:self.E].copy_(self.w_down)
-                dn[self.E].copy_(sh.w_down)
-                self.w_down, sh.w_down = dn, dn[self.E]
-                self.merged = True
+        sh = self.shared
+        if sh is not None:
+            sh.load(prefix + "shared_expert.", source)
+        bf16 = g.dtype == u.dtype == d.dtype == torch.bfloat16
+        # The experts' matrices are kept only in the order the kernels stream them (no rows: both
+        # the few-rows and the many-rows product of the experts read that order), if the sizes allow.
+        pack = bf16 and self.inter % 128 == 0 and self.hidden % 128 == 0
+        merge = (bf16 and sh is not None and sh.inter == self.inter and sh.w_gate_up.dtype == torch.bfloat16
+                 and sh.w_down.dtype == torch.bfloat16)   # (dtype: of a tensor or of a packed weight)
+        if not bf16:
+            self.w_gate_up, self.w_down = _fuse_rows(g, u), d
+            return
+        # With a shared expert of the experts' width, it becomes expert E of their tensors: few-row
+        # steps then run it in the same launches as the routed ones.
+        n = self.E + (1 if merge else 0)
+        gu = torch.empty(n, 2 * self.inter, self.hidden, dtype=torch.bfloat16, device=g.device)
+        dn = torch.empty(n, self.hidden, self.inter, dtype=torch.bfloat16, device=d.device)
+        put = ops.pack_into if pack else (lambda dst, src: dst.copy_(src))
+        for e in range(self.E):
+            put(gu[e, :self.inter], g[e])
+            put(gu[e, self.inter:], u[e])
+            put(dn[e], d[e])
+        del g, u, d
+        if merge:
+            sgu, sdn = _rows(sh.w_gate_up), _rows(sh.w_down)
+            put(gu[self.E, :self.inter], sgu[:self.inter])
+            put(gu[self.E, self.inter:], sgu[self.inter:])
+            put(dn[self.E], sdn)
+            if pack:   # the shared expert's own packed copies give way to these
+                sh.w_gate_up, sh.w_down = ops.PackedWeight(gu[self.E], sgu), ops.PackedWeight(dn[self.E], sdn)
+            else:      # its own tensors turn into views
+                sh.w_gate_up, sh.w_down = gu[self.E], dn[self.E]
+            self.merged = True
+        self.w_gate_up = ops.PackedWeight(gu, None) if pack else gu
+        self.w_down = ops.PackedWeight(dn, None) if pack else dn
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         T = x.shape[0]

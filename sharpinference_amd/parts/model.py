@@ -90,7 +90,9 @@ class DecoderModel(Part):
         for i, b in enumerate(self.blocks):
             b.load(f"{self.layer_prefix}{i}.", source)
         self.final_norm.load(self.norm_prefix, source)
-        self.head = self.embed if self.tie_embeddings else source.get(self.head_name)
+        # the head also in the order the few-rows kernel streams it (the rows stay for many-row steps
+        # and, when tied, for the embedding gather)
+        self.head = ops.pack_weight(self.embed if self.tie_embeddings else source.get(self.head_name))
 
     # -- compute ------------------------------------------------------------------
     def forward(self, ctx: StepContext, caches: Sequence[LayerCache], logit_rows: Optional[torch.Tensor]) -> Optional[torch.Tensor]:

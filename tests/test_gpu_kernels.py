@@ -21,36 +21,43 @@ def _rand(*shape, dtype=torch.float32, scale=1.0, seed=0):
 
 
 @pytest.mark.parametrize("M", [1, 5, 16, 17, 40, 64])
-@pytest.mark.parametrize("N,K", [(132, 128), (1000, 256), (5120, 1024), (20, 384)])
+@pytest.mark.parametrize("N,K", [(132, 128), (1000, 256), (5120, 1024), (20, 384), (48, 640), (208, 1152)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 def test_gemm_skinny(M, N, K, out_dtype):
     ops = _ops()
     x = _rand(M, K, dtype=torch.bfloat16, seed=M)
     w = _rand(N, K, dtype=torch.bfloat16, scale=0.1, seed=N)
     ref = x.float() @ w.float().T
-    for R in (1, 2, 4):
-        for NW in (4, 8, 16):
-            if NW == 16 and R > 1:
-                continue   # refused: 1,024-thread blocks only take one weight tile
-            got = ops.gemm_skinny(x, w, out_dtype, R=R, NW=NW).float()
-            tol = 2e-2 if out_dtype == torch.bfloat16 else 1e-3
-            assert float((got - ref).abs().max()) <= tol * float(ref.abs().max()), (M, N, K, R, NW)
+    forms = [w]
+    if ops.can_pack(w):                       # the same matrix stored tile by tile
+        forms.append(ops.pack_weight(w, keep_rows=False))
+        assert torch.equal(ops.unpack_weight(forms[1]), w)
+    for form in forms:
+        for R in (1, 2, 4):
+            for NW in (4, 8, 16):
+                if NW == 16 and R > 1:
+                    continue   # refused: 1,024-thread blocks only take one weight tile
+                got = ops.gemm_skinny(x, form, out_dtype, R=R, NW=NW).float()
+                tol = 2e-2 if out_dtype == torch.bfloat16 else 1e-3
+                assert float((got - ref).abs().max()) <= tol * float(ref.abs().max()), (M, N, K, R, NW, form is w)
 
 
 def test_gemm_skinny_rows_do_not_depend_on_the_batch():
     ops = _ops()
     x = _rand(64, 512, dtype=torch.bfloat16, seed=3)
-    w = _rand(516, 512, dtype=torch.bfloat16, scale=0.1, seed=4)
-    full = ops.gemm_skinny(x, w, torch.float32)
-    for m in (1, 7, 16, 33):
-        part = ops.gemm_skinny(x[:m].contiguous(), w, torch.float32)
-        assert torch.equal(part, full[:m]), m
+    for w in (_rand(516, 512, dtype=torch.bfloat16, scale=0.1, seed=4),
+              ops.pack_weight(_rand(528, 512, dtype=torch.bfloat16, scale=0.1, seed=5), keep_rows=False)):
+        full = ops.gemm_skinny(x, w, torch.float32)
+        for m in (1, 7, 16, 33):
+            part = ops.gemm_skinny(x[:m].contiguous(), w, torch.float32)
+            assert torch.equal(part, full[:m]), m
 
 
 @pytest.mark.parametrize("rows,E", [(8, 4), (64, 16), (33, 5), (1, 3)])
-def test_gemm_skinny_grouped(rows, E):
+@pytest.mark.parametrize("N", [264, 272])
+def test_gemm_skinny_grouped(rows, E, N):
     ops = _ops()
-    N, K, T = 264, 256, 40
+    K, T = 256, 40
     g = torch.Generator().manual_seed(rows)
     x = _rand(T, K, dtype=torch.bfloat16, seed=1)
     w = _rand(E, N, K, dtype=torch.bfloat16, scale=0.1, seed=2)
@@ -60,9 +67,11 @@ def test_gemm_skinny_grouped(rows, E):
         offsets[e + 1] = offsets[e] + int((expert == e).sum())
     a_rows = torch.randint(0, T, (rows,), generator=g, dtype=torch.int32)
     ref = torch.stack([x[int(a_rows[i])].float() @ w[int(expert[i])].float().T for i in range(rows)])
-    for R, NW in ((1, 16), (2, 8), (4, 4)):
-        got = ops.gemm_skinny(x, w, torch.float32, a_rows=a_rows.to(DEV), offsets=offsets.to(DEV), n_rows=rows, R=R, NW=NW)
-        assert float((got - ref).abs().max()) <= 1e-3 * float(ref.abs().max()), (R, NW)
+    for form in ([w, ops.pack_weight(w, keep_rows=False)] if ops.can_pack(w) else [w]):
+        for R, NW in ((1, 16), (2, 8), (4, 4)):
+            got = ops.gemm_skinny(x, form, torch.float32, a_rows=a_rows.to(DEV), offsets=offsets.to(DEV), n_rows=rows,
+                                  R=R, NW=NW)
+            assert float((got - ref).abs().max()) <= 1e-3 * float(ref.abs().max()), (R, NW, form is w)
 
 
 # ---------------------------------------------------------------------------
@@ -259,7 +268,8 @@ def test_router_ties_pick_the_lowest_index():
     assert ids.cpu().tolist() == [[0, 1]] * 4 and float((wts - 0.5).abs().max()) == 0.0
 
 
-@pytest.mark.parametrize("M,E,I,K", [(8, 4, 40, 128), (64, 16, 264, 256), (33, 5, 8192, 384), (1, 3, 20, 640)])
+@pytest.mark.parametrize("M,E,I,K", [(8, 4, 40, 128), (64, 16, 264, 256), (33, 5, 8192, 384), (1, 3, 20, 640),
+                                     (16, 3, 48, 256)])
 def test_gemm_skinny_swiglu_equals_product_then_activation(M, E, I, K):
     """The product with the activation in its epilogue gives the bits of the two kernels in a row."""
     ops = _ops()
@@ -288,11 +298,19 @@ def test_gemm_skinny_swiglu_equals_product_then_activation(M, E, I, K):
         ref[rows] = torch.nn.functional.silu(gu[:, :I]) * gu[:, I:]
     got = ops.gemm_skinny_swiglu(x, w, offsets.to(DEV), a_rows, M, scale).float().cpu()
     assert float((got - ref).abs().max()) <= 2e-2 * float(ref.abs().max())
+    if ops.can_pack(w) and (2 * I) % 32 == 0:      # the same from weights stored tile by tile
+        pw = ops.pack_weight(w, keep_rows=False)
+        for R, NW in ((2, 4), (2, 8), (4, 4), (4, 8)):
+            gu = ops.gemm_skinny(x, pw, torch.bfloat16, a_rows=a_rows, offsets=offsets.to(DEV), n_rows=M, R=R, NW=NW)
+            got = ops.gemm_skinny_swiglu(x, pw, offsets.to(DEV), a_rows, M, scale, R=R, NW=NW)
+            assert torch.equal(got, ops.silu_mul(gu, scale)), (R, NW)
+            assert float((got.float().cpu() - ref).abs().max()) <= 2e-2 * float(ref.abs().max())
 
 
 # the last two are deep enough in K for the kernel's steady loop (and its tail of 4 and of 1 stages)
 @pytest.mark.parametrize("T,E,k,N,K", [(300, 4, 1, 264, 256), (700, 16, 2, 512, 128), (65, 3, 1, 20, 384),
-                                       (500, 5, 1, 200, 640), (260, 2, 2, 136, 1216)])
+                                       (500, 5, 1, 200, 640), (260, 2, 2, 136, 1216), (500, 5, 1, 208, 640),
+                                       (260, 2, 2, 144, 1280), (70, 3, 1, 16, 128)])
 def test_gemm_grouped(T, E, k, N, K):
     ops = _ops()
     x = _rand(T, K, dtype=torch.bfloat16, seed=1)
@@ -315,6 +333,9 @@ def test_gemm_grouped(T, E, k, N, K):
     # second product: rows already sorted, bfloat16 out
     y = ops.gemm_grouped(x[st.to(DEV)].contiguous(), w, rt, False, torch.bfloat16).float().cpu()
     assert float((y - got).abs().max()) <= 2e-2 * float(got.abs().max())
+    if ops.can_pack(w):                       # the same from weights stored tile by tile: the same sums, the same bits
+        pw = ops.pack_weight(w, keep_rows=False)
+        assert torch.equal(ops.gemm_grouped(x, pw, rt, True, torch.float32).cpu(), got)
 
 
 @pytest.mark.parametrize("nh,nkv,hd", [(8, 2, 64), (5, 5, 32), (40, 8, 128), (3, 1, 96)])
