@@ -12,8 +12,8 @@
 //  * Each of the 4 waves owns 32 weight rows (2 MFMA tiles) and reads them straight from global
 //    memory into registers, a ring of 64-wide K stages ahead: a weight element is used by one wave only.
 //  * The x rows (gathered through a_rows) are shared by the waves and staged through LDS, 64
-//    columns of K at a time, double-buffered and fetched two stages ahead; rows are padded to 72
-//    elements so that the 16 lanes of a quarter-wave read 16 different banks.
+//    columns of K at a time, double-buffered and fetched two stages ahead; the 16-byte chunks of
+//    a row are swizzled so that reads and stores are free of bank conflicts.
 //  * W is the A operand (rows = n), x the B operand: a lane ends up with 4 consecutive n of one
 //    row, stored as one 8-byte write.  Each output is one chain over k in ascending order, so a
 //    row's result does not depend on which other rows share its tile.
@@ -44,16 +44,23 @@ constexpr int GW = 4;         // waves per block
 constexpr int NT = 2;         // 16-row weight tiles per wave
 constexpr int GN = 16 * NT * GW;   // columns per tile
 constexpr int GK = SHARPI_GK;  // K per LDS stage
-#ifndef SHARPI_GPADX
-#define SHARPI_GPADX 8
-#endif
-constexpr int GPAD = GK + SHARPI_GPADX;  // padded LDS row
+constexpr int GPAD = GK;      // LDS row: no pad, the 16-byte chunks of a row are swizzled instead (xs_col)
 constexpr int GROWS = GW * 64 / (GK / 8);   // rows staged per pass: GK / 8 threads per row
 constexpr int GPASS = GM / GROWS;  // staging passes
 constexpr int kXcds = 8;           // accelerator dies, each with its own L2
 constexpr int kAhead = SHARPI_GAHEAD;  // K stages of weights in flight per wave (2, 3 or 4)
 constexpr int GQ = SHARPI_GQ;       // 16-row groups whose LDS reads go out together (divides 4)
 constexpr int kHalves = 2;         // a tile's column blocks are split over this many XCDs
+
+// Where column `col` (a multiple of 8 elements = one 16-byte chunk) of LDS row `row` is kept: the
+// chunk index is XORed with bits 1..3 of the row.  The LDS serves a 16-byte read of a wave in four
+// turns of two octets of lanes, one octet from rows 0..7 and one from rows 8..15 of the operand
+// (measured with the bank-conflict counter: rows padded to 144 bytes conflict two ways).  With the
+// swizzle the eight chunks an octet reads fall into eight different 16-byte bank groups of its half
+// (even rows use one half of the 256-byte bank space, odd rows the other), and the two octets of a
+// turn into different ones; an octet of the staging stores fills one whole row, i.e. one half.
+static_assert(GK == 64, "the swizzle assumes rows of eight 16-byte chunks");
+__device__ __forceinline__ int xs_col(int row, int col) { return col ^ (((row >> 1) & 7) << 3); }
 
 // The work of one tile of NQ * 64 rows (the block's rows, rounded up) against GN weight rows.
 template <typename TO, int NQ, bool PACKED>
@@ -127,7 +134,7 @@ __device__ __forceinline__ void grouped_tile(const bf16_t* __restrict__ x, const
   };
   if (chunks >= kAhead) fill_ring(std::true_type{}); else fill_ring(std::false_type{});
 #pragma unroll
-  for (int ps = 0; ps < PASS; ++ps) *reinterpret_cast<u32x4*>(&xs[0][srow + GROWS * ps][scol]) = stage[0][ps];
+  for (int ps = 0; ps < PASS; ++ps) *reinterpret_cast<u32x4*>(&xs[0][srow + GROWS * ps][xs_col(srow + GROWS * ps, scol)]) = stage[0][ps];
   __syncthreads();
 
   // One K stage; `slot` (the stage's place in the ring) and `par` (its parity) are compile-time
@@ -152,7 +159,7 @@ __device__ __forceinline__ void grouped_tile(const bf16_t* __restrict__ x, const
       for (int mq = 0; mq < MT; mq += GQ) {
         bf16x8 xf[GQ];
 #pragma unroll
-        for (int i = 0; i < GQ; ++i) xf[i] = *reinterpret_cast<const bf16x8*>(&xs[par][(mq + i) * 16 + r][j * 32 + g * 8]);
+        for (int i = 0; i < GQ; ++i) xf[i] = *reinterpret_cast<const bf16x8*>(&xs[par][(mq + i) * 16 + r][xs_col(r, j * 32 + g * 8)]);
 #pragma unroll
         for (int i = 0; i < GQ; ++i)
 #pragma unroll
@@ -170,7 +177,7 @@ __device__ __forceinline__ void grouped_tile(const bf16_t* __restrict__ x, const
     }
     if (steady || c + 1 < chunks) {   // the next stage's x rows, fetched a stage ago
 #pragma unroll
-      for (int ps = 0; ps < PASS; ++ps) *reinterpret_cast<u32x4*>(&xs[par ^ 1][srow + GROWS * ps][scol]) = stage[par ^ 1][ps];
+      for (int ps = 0; ps < PASS; ++ps) *reinterpret_cast<u32x4*>(&xs[par ^ 1][srow + GROWS * ps][xs_col(srow + GROWS * ps, scol)]) = stage[par ^ 1][ps];
     }
     __syncthreads();
   };
