@@ -85,3 +85,21 @@ def test_mixed_batches_with_page_reuse(model_dir, seed):
         for g in eng.cache.groups:
             assert g.pool.total_allocs > g.pool.num_pages, "the pool was large enough to never reuse a page"
             assert g.pool.num_free == g.pool.num_pages
+
+
+@pytest.mark.parametrize("page_size", [32, 64])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_other_page_sizes(model_dir, page_size, dtype):
+    """Pages of 32 and 64 positions: the windows' edges, the decode kernel's runs and the prefill
+    kernel's chunks then fall inside pages, not on their edges."""
+    which, d = model_dir
+    if which not in ("B", "D"):
+        pytest.skip("two configurations are enough here")
+    toks = _requests(which)[-1]
+    eng = H.make_engine(d, dtype, kv_tokens=2 * ((len(toks) + page_size - 1) // page_size) * page_size,
+                        max_num_seqs=2, page_size=page_size)
+    H.check_against_plain(eng, d, dtype, "a", toks, H.changing_portions(len(toks), 5), f"{which} {dtype} pages of {page_size}")
+    H.check_against_plain(eng, d, dtype, "b", toks, H.last_decoded(len(toks)), f"{which} {dtype} pages of {page_size}, decoded")
+    for g in eng.cache.groups:
+        assert g.pool.num_free == g.pool.num_pages
+
