@@ -311,3 +311,117 @@ def test_toy_mixer_with_state_needs_no_change_to_the_framework():
         assert float((whole_a - want.cpu()).abs().max()) <= 1e-4
     finally:
         unregister_architecture("ToyRunningMean")
+
+
+def test_toy_position_encoding_and_routed_feed_forward_need_no_change_to_the_framework():
+    """Two more parts defined here: a learned absolute position encoding (added to the mixer's
+    input, around an attention without rotation) and a feed-forward that routes by position
+    (expert = position mod E, no router weights), built from the framework's routing and
+    grouped-product operations.  Registered, built, stepped whole, cut and mixed."""
+    from sharpinference_amd import ops
+    from sharpinference_amd.config.base import ModelConfig
+    from sharpinference_amd.engine import Engine
+    from sharpinference_amd.parts.attention import Attention
+    from sharpinference_amd.parts.base import ParamSpec, Part
+    from sharpinference_amd.parts.block import PreNormBlock
+    from sharpinference_amd.parts.model import DecoderModel
+    from sharpinference_amd.parts.norm import RMSNorm
+    from sharpinference_amd.registry import register_architecture, unregister_architecture
+
+    HID, NH, NKV, HD, E, INTER, MAXPOS, VOCAB = 32, 2, 1, 16, 3, 40, 128, 60
+
+    @dataclass
+    class ToyConfig(ModelConfig):
+        architecture: str = "ToyLearnedPositions"
+        vocab_size: int = VOCAB
+        max_position_embeddings: int = MAXPOS
+
+        @classmethod
+        def from_dict(cls, d):
+            return cls()
+
+        def to_dict(self):
+            return {"architectures": [self.architecture]}
+
+    class LearnedPositions(Part):
+        """mixer(x + table[position]): a position encoding as a part around any mixer."""
+
+        def __init__(self, inner, hidden, max_pos):
+            self.inner, self.hidden, self.max_pos = inner, hidden, max_pos
+
+        def param_specs(self, prefix):
+            out = {prefix + "positions.weight": ParamSpec((self.max_pos, self.hidden))}
+            out.update(self.inner.param_specs(prefix))
+            return out
+
+        def load(self, prefix, source):
+            self.table = source.get(prefix + "positions.weight")
+            self.inner.load(prefix, source)
+
+        def cache_spec(self):
+            return self.inner.cache_spec()
+
+        def forward(self, x, ctx, cache):
+            return self.inner.forward((x + self.table[ctx.positions.long()].to(x.dtype)), ctx, cache)
+
+    class RoutedByPosition(Part):
+        """Expert (position mod E) of E SwiGLU experts: routing without a router."""
+
+        def param_specs(self, prefix):
+            return {prefix + "gate_up": ParamSpec((E, 2 * INTER, HID)), prefix + "down": ParamSpec((E, HID, INTER))}
+
+        def load(self, prefix, source):
+            self.w_gate_up, self.w_down = source.get(prefix + "gate_up"), source.get(prefix + "down")
+
+        def forward(self, x, ctx):
+            T = x.shape[0]
+            ids = (ctx.positions % E).to(torch.int32).view(T, 1)
+            rt = ops.moe_permute(ids, torch.ones(T, 1, device=x.device), E)
+            act = ops.grouped_swiglu(x, self.w_gate_up, rt, ctx.act_dtype)
+            y = ops.grouped_linear(act, self.w_down, rt, False, ctx.act_dtype)
+            return ops.moe_combine(y, rt.inv_pos, None, T, 1)
+
+    def build(cfg):
+        blocks = [PreNormBlock(RMSNorm(HID, 1e-5), LearnedPositions(Attention(HID, NH, NKV, HD), HID, MAXPOS),
+                               RMSNorm(HID, 1e-5), RoutedByPosition(),
+                               names={"norm1": "n1.", "mixer": "mix.", "norm2": "n2.", "ffn": "ff."}) for _ in range(2)]
+        return DecoderModel(VOCAB, HID, blocks, RMSNorm(HID, 1e-5), config=cfg)
+
+    register_architecture("ToyLearnedPositions", ToyConfig, build, replace=True)
+    try:
+        eng = Engine(config=ToyConfig(), weight_seed=11, dtype="float32", kv_tokens=128, max_num_seqs=3, weight_std=0.3)
+        a, b = H.random_tokens(50, VOCAB, 1), H.random_tokens(33, VOCAB, 2)
+        whole_a = H.run_cut(eng, "a", a, [50])
+        whole_b = H.run_cut(eng, "b", b, [33])
+        assert float((H.run_cut(eng, "a2", a, H.changing_portions(50, 4)) - whole_a).abs().max()) <= 1e-4
+        steps = H.mixed_trace({"a": a, "b": b, "c": H.random_tokens(7, VOCAB, 3)}, seed=1, max_live=3, tail=5)
+        got = H.replay(eng, steps)
+        assert float((got["a"] - whole_a).abs().max()) <= 1e-4 and float((got["b"] - whole_b).abs().max()) <= 1e-4
+        # and against the formulas
+        m = eng.model
+        pos = torch.arange(50, device=DEV)
+        h = m.embed[torch.tensor(a, device=DEV)].float()
+        causal = torch.tril(torch.ones(50, 50, device=DEV, dtype=torch.bool))
+        for blk in m.blocks:
+            n = P.rms_norm(h, blk.norm1.weight, 1e-5) + blk.mixer.table[pos]
+            att = blk.mixer.inner
+            qkv = n @ att.w_qkv.T
+            q, k, v = qkv[:, :NH * HD].view(50, NH, HD), qkv[:, NH * HD:(NH + NKV) * HD].view(50, NKV, HD), \
+                qkv[:, (NH + NKV) * HD:].view(50, NKV, HD)
+            outs = []
+            for hh in range(NH):
+                sc = (q[:, hh] @ k[:, hh // (NH // NKV)].T) / math.sqrt(HD)
+                outs.append(torch.softmax(sc.masked_fill(~causal, float("-inf")), -1) @ v[:, hh // (NH // NKV)])
+            h = h + torch.cat(outs, -1) @ att.w_o.T
+            n = P.rms_norm(h, blk.norm2.weight, 1e-5)
+            y = torch.empty_like(n)
+            for e in range(E):
+                rows = pos % E == e
+                gu = n[rows] @ blk.ffn.w_gate_up[e].T
+                y[rows] = (P.silu(gu[:, :INTER]) * gu[:, INTER:]) @ blk.ffn.w_down[e].T
+            h = h + y
+        want = P.rms_norm(h, m.final_norm.weight, 1e-5) @ m.head.T
+        assert float((whole_a - want.cpu()).abs().max()) <= 1e-4
+    finally:
+        unregister_architecture("ToyLearnedPositions")
+
