@@ -40,8 +40,14 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 #endif
 constexpr int GM = SHARPI_GM;  // rows per tile (the routing kernel lists tiles of this height)
 constexpr int GMT = GM / 16;  // 16-row groups per tile
-constexpr int GW = 4;         // waves per block
-constexpr int NT = 2;         // 16-row weight tiles per wave
+#ifndef SHARPI_GW
+#define SHARPI_GW 4
+#endif
+#ifndef SHARPI_GNT
+#define SHARPI_GNT 2
+#endif
+constexpr int GW = SHARPI_GW;   // waves per block
+constexpr int NT = SHARPI_GNT;  // 16-row weight tiles per wave
 constexpr int GN = 16 * NT * GW;   // columns per tile
 constexpr int GK = SHARPI_GK;  // K per LDS stage
 constexpr int GPAD = GK;      // LDS row: no pad, the 16-byte chunks of a row are swizzled instead (xs_col)
@@ -243,13 +249,18 @@ __global__ __launch_bounds__(GW* kWave, 2) void grouped_gemm_kernel(
   if (n_rows <= 0) return;
   const int n_base = nblock * GN + (threadIdx.x >> 6) * 16 * NT;
   const bf16_t* We = W + (size_t)e * N * K;
-  static_assert(GM == 192, "three tile heights are compiled: 64, 128 and 192 rows");
-  if (n_rows <= 64)
+  static_assert(GM % 64 == 0 && GM >= 128 && GM <= 256, "tile heights are compiled in steps of 64 rows, up to GM");
+  if (n_rows <= 64) {
     grouped_tile<TO, 1, PACKED>(x, We, out, N, K, a_rows, row0, row_end, n_base, xs);
-  else if (n_rows <= 128)
+  } else if (n_rows <= 128) {
     grouped_tile<TO, 2, PACKED>(x, We, out, N, K, a_rows, row0, row_end, n_base, xs);
-  else
-    grouped_tile<TO, 3, PACKED>(x, We, out, N, K, a_rows, row0, row_end, n_base, xs);
+  } else if constexpr (GM >= 192) {
+    if (GM == 192 || n_rows <= 192) {
+      grouped_tile<TO, 3, PACKED>(x, We, out, N, K, a_rows, row0, row_end, n_base, xs);
+    } else if constexpr (GM >= 256) {
+      grouped_tile<TO, 4, PACKED>(x, We, out, N, K, a_rows, row0, row_end, n_base, xs);
+    }
+  }
 }
 
 // x [x_rows, K] bf16 (rows gathered through a_rows if given), W [E, N, K] bf16, out [n_rows, N];
