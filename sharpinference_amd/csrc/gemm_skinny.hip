@@ -46,7 +46,7 @@ template <int R, int MB, int NW, typename TO, bool ACT, bool PACKED>
 __global__ __launch_bounds__(NW* kWave) void skinny_gemm_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ W, TO* __restrict__ out, int M, int N, int K,
     const int* __restrict__ a_rows, const int* __restrict__ group_offsets, const float* __restrict__ act_scale) {
-  static_assert(!ACT || (R % 2 == 0 && MB == 1), "the SwiGLU form pairs gate and up tiles of one row block");
+  static_assert(!ACT || R % 2 == 0, "the SwiGLU form pairs gate and up tiles");
   constexpr int RT = ACT ? R : kRedTiles;   // tiles that meet in LDS per round
   constexpr int TG = ACT ? R / 2 : R;       // tiles of distinct output columns per block
   __shared__ f32x4 red[NW][RT][kWave];
@@ -136,27 +136,30 @@ __global__ __launch_bounds__(NW* kWave) void skinny_gemm_kernel(
     }
 
     if constexpr (ACT) {
-      // all tiles meet at once; wave t < TG adds up gate tile t and up tile t + TG in wave order
-      __syncthreads();
+      // per row block all tiles meet at once; wave t < TG adds up gate tile t and up tile t + TG in wave order
 #pragma unroll
-      for (int t = 0; t < R; ++t) red[w][t][lane] = acc[t][0];
-      __syncthreads();
-      if (w < TG) {
-        f32x4 gv = red[0][w][lane], uv = red[0][w + TG][lane];
+      for (int mb = 0; mb < MB; ++mb) {
+        __syncthreads();
 #pragma unroll
-        for (int ww = 1; ww < NW; ++ww) {
-          gv += red[ww][w][lane];
-          uv += red[ww][w + TG][lane];
-        }
-        const int row = row_begin + rb0 * 16 + r;
-        const int n = n_base + w * 16 + g * 4;
-        if (row < row_end && n < n_out) {
-          const float sc = act_scale ? act_scale[row] : 1.0f;
-          f32x4 o;
+        for (int t = 0; t < R; ++t) red[w][t][lane] = acc[t][mb];
+        __syncthreads();
+        if (w < TG) {
+          f32x4 gv = red[0][w][lane], uv = red[0][w + TG][lane];
 #pragma unroll
-          for (int i = 0; i < 4; ++i)
-            o[i] = swiglu_f32(bf16_to_f32(f32_to_bf16(gv[i])), bf16_to_f32(f32_to_bf16(uv[i])), sc, act_scale != nullptr);
-          store4<TO>(out + (size_t)row * n_out + n, o);
+          for (int ww = 1; ww < NW; ++ww) {
+            gv += red[ww][w][lane];
+            uv += red[ww][w + TG][lane];
+          }
+          const int row = row_begin + (rb0 + mb) * 16 + r;
+          const int n = n_base + w * 16 + g * 4;
+          if (row < row_end && n < n_out) {
+            const float sc = act_scale ? act_scale[row] : 1.0f;
+            f32x4 o;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              o[i] = swiglu_f32(bf16_to_f32(f32_to_bf16(gv[i])), bf16_to_f32(f32_to_bf16(uv[i])), sc, act_scale != nullptr);
+            store4<TO>(out + (size_t)row * n_out + n, o);
+          }
         }
       }
       continue;
@@ -216,14 +219,17 @@ static int dispatch_mb(int MB, const void* x, const void* W, void* out, int out_
 // [N/16][K/128][16 runs of 8 k][16 rows][8] (N % 16 == 0), instead of row by row.
 SHARPI_EXPORT int sharpi_gemm_skinny(const void* x, const void* W, void* out, int out_dtype, int M, int N, int K,
                                      const int* a_rows, const int* group_offsets, int groups, int R, int NW,
-                                     int packed, hipStream_t stream) {
+                                     int packed, int row_blocks, hipStream_t stream) {
   if (M <= 0) return SHARPI_OK;
-  if (M > 64 || N <= 0 || (N & 3) || K <= 0 || (K & 127) || groups < 0 || groups > 65535) return SHARPI_ERR_ARG;
+  if (N <= 0 || (N & 3) || K <= 0 || (K & 127) || groups < 0 || groups > 65535) return SHARPI_ERR_ARG;
+  if (groups == 0 && M > 64) return SHARPI_ERR_ARG;
   if (groups > 0 && group_offsets == nullptr) return SHARPI_ERR_ARG;
   if (out_dtype != DT_F32 && out_dtype != DT_BF16) return SHARPI_ERR_ARG;
   if (packed && (N & 15)) return SHARPI_ERR_ARG;
-  // grouped rows are spread over experts: one row block at a time; plain: all row blocks at once
-  const int MB = groups > 0 ? 1 : ceil_div(M, 16);
+  // plain: all row blocks at once.  Grouped: row_blocks (1, 2 or 4) blocks of 16 rows of an expert at
+  // a time; an expert with more rows is walked in turns, reading its weights again for each
+  const int MB = groups > 0 ? (row_blocks > 0 ? row_blocks : 1) : ceil_div(M, 16);
+  if (MB < 1 || MB > 4) return SHARPI_ERR_ARG;
 #define SK(RR, WW)                                                                                                        \
   if (R == RR && NW == WW)                                                                                                \
   return packed ? dispatch_mb<RR, WW, true>(MB, x, W, out, out_dtype, M, N, K, a_rows, group_offsets, groups, stream)     \
@@ -238,21 +244,29 @@ SHARPI_EXPORT int sharpi_gemm_skinny(const void* x, const void* W, void* out, in
 // The grouped product with SwiGLU applied in its epilogue: W [groups, N, K] holds gate rows
 // [0, N/2) and up rows [N/2, N) of every expert; out [M, N/2] bf16 =
 // silu(s g) * (s u) with g, u the two products rounded to bfloat16 and s = act_scale[row] (null: 1).
-// Rows are the expert-sorted list (sixteen of an expert at a time).  R in {2, 4}, NW in {4, 8};
+// Rows are the expert-sorted list (row_blocks * 16 of an expert at a time).  R in {2, 4}, NW in {4, 8};
 // packed as above (N % 32 == 0 then).
 SHARPI_EXPORT int sharpi_gemm_skinny_swiglu(const void* x, const void* W, void* out, int M, int N, int K,
                                             const int* a_rows, const int* group_offsets, int groups,
-                                            const float* act_scale, int R, int NW, int packed, hipStream_t stream) {
+                                            const float* act_scale, int R, int NW, int packed, int row_blocks,
+                                            hipStream_t stream) {
   if (M <= 0) return SHARPI_OK;
-  if (M > 64 || N <= 0 || (N & 7) || K <= 0 || (K & 127) || groups <= 0 || groups > 65535) return SHARPI_ERR_ARG;
+  if (N <= 0 || (N & 7) || K <= 0 || (K & 127) || groups <= 0 || groups > 65535) return SHARPI_ERR_ARG;
   if (group_offsets == nullptr) return SHARPI_ERR_ARG;
   if (packed && (N & 31)) return SHARPI_ERR_ARG;
-#define SKA(RR, WW)                                                                                                              \
-  if (R == RR && NW == WW)                                                                                                       \
-  return packed ? launch_skinny<RR, 1, WW, true, true>(x, W, out, DT_BF16, M, N, K, a_rows, group_offsets, groups, act_scale, stream)  \
-                : launch_skinny<RR, 1, WW, true, false>(x, W, out, DT_BF16, M, N, K, a_rows, group_offsets, groups, act_scale, stream)
+  const int MB = row_blocks > 0 ? row_blocks : 1;
+#define SKA1(RR, WW, MBV, PK) \
+  return launch_skinny<RR, MBV, WW, true, PK>(x, W, out, DT_BF16, M, N, K, a_rows, group_offsets, groups, act_scale, stream)
+#define SKA(RR, WW)                                    \
+  if (R == RR && NW == WW) {                           \
+    if (MB == 1) { if (packed) SKA1(RR, WW, 1, true); else SKA1(RR, WW, 1, false); }  \
+    if (MB == 2) { if (packed) SKA1(RR, WW, 2, true); else SKA1(RR, WW, 2, false); }  \
+    if (MB == 4) { if (packed) SKA1(RR, WW, 4, true); else SKA1(RR, WW, 4, false); }  \
+    return SHARPI_ERR_ARG;                             \
+  }
   SKA(2, 4); SKA(2, 8);
   SKA(4, 4); SKA(4, 8);
 #undef SKA
+#undef SKA1
   return SHARPI_ERR_ARG;
 }

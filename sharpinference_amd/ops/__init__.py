@@ -368,7 +368,7 @@ def _unwrap(w):
 # ---------------------------------------------------------------------------
 # the weight-streaming product for few rows (decode)
 # ---------------------------------------------------------------------------
-SKINNY_MAX_ROWS = 64          # grouped form: rows of all experts together
+SKINNY_MAX_ROWS = 64          # rows the kernel multiplies against one stream of a weight tile (4 blocks of 16)
 SKINNY_MAX_ROWS_PLAIN = 16    # plain form: beyond one row block the library's product is faster
 
 
@@ -383,10 +383,19 @@ def skinny_plan(N: int, K: int):
     return (4 if N >= 12288 else 2), 8
 
 
+def _row_blocks(group_rows: Optional[int]) -> int:
+    """16-row blocks of one expert that a grouped launch multiplies at a time: enough for the
+    largest group (its bound is the caller's), 1, 2 or 4; larger groups are walked in turns."""
+    if not group_rows or group_rows <= 16:
+        return 1
+    return 2 if group_rows <= 32 else 4
+
+
 def gemm_skinny(x: torch.Tensor, w, out_dtype: torch.dtype, a_rows: Optional[torch.Tensor] = None,
                 offsets: Optional[torch.Tensor] = None, n_rows: Optional[int] = None, R: Optional[int] = None,
-                NW: Optional[int] = None) -> torch.Tensor:
-    """x [M, K] @ w[N, K]^T (or per expert with w [E, N, K]) for M <= 64 on the matrix cores;
+                NW: Optional[int] = None, group_rows: Optional[int] = None) -> torch.Tensor:
+    """x [M, K] @ w[N, K]^T for M <= 64, or per expert with w [E, N, K] over an expert-sorted row
+    list (``group_rows``: a bound on the rows of one expert, if known), on the matrix cores;
     w a tensor (row-major) or a PackedWeight."""
     w, packed = _unwrap(w)
     _dev(x, w, a_rows, offsets)
@@ -408,18 +417,18 @@ def gemm_skinny(x: torch.Tensor, w, out_dtype: torch.dtype, a_rows: Optional[tor
         E, (N, K) = 0, w.shape
         M = x.shape[0]
     _need(x.dim() == 2 and x.shape[1] == K, f"gemm_skinny: x {tuple(x.shape)} vs w {tuple(w.shape)}")
-    _need(0 < M <= SKINNY_MAX_ROWS and K % 128 == 0 and N % 4 == 0,
-          f"gemm_skinny: shape M={M} N={N} K={K} is not taken (M <= 64, K % 128 == 0, N % 4 == 0)")
+    _need(M > 0 and (grouped or M <= SKINNY_MAX_ROWS) and K % 128 == 0 and N % 4 == 0,
+          f"gemm_skinny: shape M={M} N={N} K={K} is not taken (M <= 64 unless grouped, K % 128 == 0, N % 4 == 0)")
     pr, pw = skinny_plan(N, K)
     out = torch.empty(M, N, dtype=out_dtype, device=x.device)
     _run("sharpi_gemm_skinny", _ptr(x), _ptr(w), _ptr(out), _code(out_dtype), M, N, K, _ptr(a_rows), _ptr(offsets), E,
-         R or pr, NW or pw, 1 if packed else 0, _stream())
+         R or pr, NW or pw, 1 if packed else 0, _row_blocks(group_rows) if grouped else 0, _stream())
     return out
 
 
 def gemm_skinny_swiglu(x: torch.Tensor, w, offsets: torch.Tensor, a_rows: Optional[torch.Tensor],
                        n_rows: int, scale: Optional[torch.Tensor], R: Optional[int] = None,
-                       NW: Optional[int] = None) -> torch.Tensor:
+                       NW: Optional[int] = None, group_rows: Optional[int] = None) -> torch.Tensor:
     """Per expert, silu(s g) * (s u) with (g | u) = x @ w[e]^T rounded to bfloat16, w [E, 2I, K]
     holding gate rows then up rows: the product and the activation in one kernel, for at most
     64 rows.  Returns [n_rows, I] bfloat16."""
@@ -437,15 +446,15 @@ def gemm_skinny_swiglu(x: torch.Tensor, w, offsets: torch.Tensor, a_rows: Option
     else:
         _need(x.shape[0] == M, "gemm_skinny_swiglu: x must have n_rows rows when not gathered")
     _need(x.dim() == 2 and x.shape[1] == K, f"gemm_skinny_swiglu: x {tuple(x.shape)} vs w {tuple(w.shape)}")
-    _need(0 < M <= SKINNY_MAX_ROWS and K % 128 == 0 and N % 8 == 0,
-          f"gemm_skinny_swiglu: shape M={M} N={N} K={K} is not taken (M <= 64, K % 128 == 0, N % 8 == 0)")
+    _need(M > 0 and K % 128 == 0 and N % 8 == 0,
+          f"gemm_skinny_swiglu: shape M={M} N={N} K={K} is not taken (K % 128 == 0, N % 8 == 0)")
     _need(not packed or N % 32 == 0, "gemm_skinny_swiglu: packed weights need gate and up rows in whole 16-row tiles")
     if scale is not None:
         _need(scale.dtype == torch.float32 and scale.shape == (M,), "gemm_skinny_swiglu: scale must be float32 [n_rows]")
     pr, pw = skinny_plan(N, K)
     out = torch.empty(M, N // 2, dtype=torch.bfloat16, device=x.device)
     _run("sharpi_gemm_skinny_swiglu", _ptr(x), _ptr(w), _ptr(out), M, N, K, _ptr(a_rows), _ptr(offsets), E,
-         _ptr(scale), R or pr, NW or pw, 1 if packed else 0, _stream())
+         _ptr(scale), R or pr, NW or pw, 1 if packed else 0, _row_blocks(group_rows), _stream())
     return out
 
 
@@ -657,8 +666,9 @@ def grouped_swiglu(x: torch.Tensor, w_gate_up, rt: Routing, out_dtype: torch.dty
     take one kernel; otherwise the product and the activation are two."""
     N, K = w_gate_up.shape[1], w_gate_up.shape[2]
     if (x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16 and out_dtype == torch.bfloat16
-            and rt.n_rows <= SKINNY_MAX_ROWS and K % 128 == 0 and N % (32 if isinstance(w_gate_up, PackedWeight) else 8) == 0):
-        return gemm_skinny_swiglu(x, w_gate_up, rt.offsets, rt.sorted_token, rt.n_rows, rt.sorted_w)
+            and rt.n_tokens <= SKINNY_MAX_ROWS and K % 128 == 0 and N % (32 if isinstance(w_gate_up, PackedWeight) else 8) == 0):
+        return gemm_skinny_swiglu(x, w_gate_up, rt.offsets, rt.sorted_token, rt.n_rows, rt.sorted_w,
+                                  group_rows=rt.n_tokens)
     return silu_mul(grouped_linear(x, w_gate_up, rt, True, out_dtype), rt.sorted_w)
 
 
@@ -671,8 +681,9 @@ def grouped_linear(x: torch.Tensor, w, rt: Routing, gather: bool, out_dtype: tor
     N, K = w.shape[1], w.shape[2]
     a_rows = rt.sorted_token if gather else None
     if w.dtype == torch.bfloat16 and K % 128 == 0 and N % 4 == 0:
-        if rt.n_rows <= SKINNY_MAX_ROWS:
-            return gemm_skinny(x, w, out_dtype, a_rows=a_rows, offsets=rt.offsets, n_rows=rt.n_rows)
+        if rt.n_tokens <= SKINNY_MAX_ROWS:   # no expert has more rows than there are tokens
+            return gemm_skinny(x, w, out_dtype, a_rows=a_rows, offsets=rt.offsets, n_rows=rt.n_rows,
+                               group_rows=rt.n_tokens)
         return gemm_grouped(x, w, rt, gather, out_dtype)
     y = grouped_gemm(x, w, rt.offsets, a_rows, rt.n_rows)
     return y if y.dtype == out_dtype else cast(y, out_dtype)

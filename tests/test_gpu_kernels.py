@@ -53,7 +53,7 @@ def test_gemm_skinny_rows_do_not_depend_on_the_batch():
             assert torch.equal(part, full[:m]), m
 
 
-@pytest.mark.parametrize("rows,E", [(8, 4), (64, 16), (33, 5), (1, 3)])
+@pytest.mark.parametrize("rows,E", [(8, 4), (64, 16), (33, 5), (1, 3), (100, 3), (150, 2)])
 @pytest.mark.parametrize("N", [264, 272])
 def test_gemm_skinny_grouped(rows, E, N):
     ops = _ops()
@@ -69,9 +69,12 @@ def test_gemm_skinny_grouped(rows, E, N):
     ref = torch.stack([x[int(a_rows[i])].float() @ w[int(expert[i])].float().T for i in range(rows)])
     for form in ([w, ops.pack_weight(w, keep_rows=False)] if ops.can_pack(w) else [w]):
         for R, NW in ((1, 16), (2, 8), (4, 4)):
-            got = ops.gemm_skinny(x, form, torch.float32, a_rows=a_rows.to(DEV), offsets=offsets.to(DEV), n_rows=rows,
-                                  R=R, NW=NW)
-            assert float((got - ref).abs().max()) <= 1e-3 * float(ref.abs().max()), (R, NW, form is w)
+            # the bound on an expert's rows chooses how many 16-row blocks are multiplied at a time;
+            # a bound that is too small (or none) only costs more passes over the weights
+            for bound in (None, int((offsets[1:] - offsets[:-1]).max()), 20):
+                got = ops.gemm_skinny(x, form, torch.float32, a_rows=a_rows.to(DEV), offsets=offsets.to(DEV), n_rows=rows,
+                                      R=R, NW=NW, group_rows=bound)
+                assert float((got - ref).abs().max()) <= 1e-3 * float(ref.abs().max()), (R, NW, form is w, bound)
 
 
 # ---------------------------------------------------------------------------
@@ -269,7 +272,7 @@ def test_router_ties_pick_the_lowest_index():
 
 
 @pytest.mark.parametrize("M,E,I,K", [(8, 4, 40, 128), (64, 16, 264, 256), (33, 5, 8192, 384), (1, 3, 20, 640),
-                                     (16, 3, 48, 256)])
+                                     (16, 3, 48, 256), (70, 2, 48, 256)])
 def test_gemm_skinny_swiglu_equals_product_then_activation(M, E, I, K):
     """The product with the activation in its epilogue gives the bits of the two kernels in a row."""
     ops = _ops()
@@ -286,8 +289,9 @@ def test_gemm_skinny_swiglu_equals_product_then_activation(M, E, I, K):
         for R, NW in ((2, 4), (2, 8), (4, 4), (4, 8)):
             gu = ops.gemm_skinny(x, w, torch.bfloat16, a_rows=a_rows, offsets=offsets.to(DEV), n_rows=M, R=R, NW=NW)
             want = ops.silu_mul(gu, sc)
-            got = ops.gemm_skinny_swiglu(x, w, offsets.to(DEV), a_rows, M, sc, R=R, NW=NW)
-            assert torch.equal(got, want), (R, NW, sc is None)
+            for bound in (None, 32, M):
+                got = ops.gemm_skinny_swiglu(x, w, offsets.to(DEV), a_rows, M, sc, R=R, NW=NW, group_rows=bound)
+                assert torch.equal(got, want), (R, NW, sc is None, bound)
     # and against the formula
     xs = x[a_rows.long()].float().cpu()
     ref = torch.zeros(M, I)
