@@ -188,7 +188,7 @@ def main() -> int:
             log(f"decode b{pb}: {pdt / k * 1e3:.2f} ms/step, {points[f'decode_b{pb}']:.1f} tok/s")
 
     out = {
-        "metric": "decode tok/s at batch 8 (Scout-shaped, 2,048-token prompts)",
+        "metric": f"decode tok/s at batch {args.batch} (Scout-shaped, 2,048-token prompts)",
         "value": value, "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",

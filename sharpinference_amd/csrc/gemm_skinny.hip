@@ -127,18 +127,22 @@ __global__ __launch_bounds__(NW* kWave) void skinny_gemm_kernel(
           else xf[mb][j] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
         }
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
+      for (int mb = 0; mb < MB; ++mb) {
+        // a row block beyond the group's rows is not multiplied (the same for every lane of the block)
+        if (mb > 0 && (rb0 + mb) * 16 >= n_rows) continue;
 #pragma unroll
-        for (int t = 0; t < R; ++t)
+        for (int j = 0; j < 4; ++j)
 #pragma unroll
-          for (int mb = 0; mb < MB; ++mb)
+          for (int t = 0; t < R; ++t)
             acc[t][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[t][j], xf[mb][j], acc[t][mb], 0, 0, 0);
+      }
     }
 
     if constexpr (ACT) {
       // per row block all tiles meet at once; wave t < TG adds up gate tile t and up tile t + TG in wave order
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
+        if (mb > 0 && (rb0 + mb) * 16 >= n_rows) continue;   // uniform over the block
         __syncthreads();
 #pragma unroll
         for (int t = 0; t < R; ++t) red[w][t][lane] = acc[t][mb];
@@ -168,6 +172,11 @@ __global__ __launch_bounds__(NW* kWave) void skinny_gemm_kernel(
     // pair p of a round is summed and stored by wave p
 #pragma unroll
     for (int p0 = 0; p0 < R * MB; p0 += kRedTiles) {
+      // a round whose pairs all lie in row blocks beyond the group's rows is skipped (uniform over the block)
+      bool any = false;
+#pragma unroll
+      for (int p = 0; p < kRedTiles; ++p) any = any || (p0 + p < R * MB && ((p0 + p) % MB == 0 || (rb0 + (p0 + p) % MB) * 16 < n_rows));
+      if (!any) continue;
       __syncthreads();
 #pragma unroll
       for (int p = 0; p < kRedTiles; ++p)

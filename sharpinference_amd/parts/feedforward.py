@@ -64,7 +64,8 @@ class MoESwiGLU(Part):
     (2060-2066); the outputs are summed (2096-2097).  ``gate`` is "sigmoid" or "softmax"
     (2031-2034); ``renormalise`` divides the k scores by their sum (2156-2162)."""
 
-    MERGE_MAX_TOKENS = 64   # the shared group's rows: what the few-rows kernel multiplies against one stream of a tile
+    MERGE_MAX_TOKENS = 16   # one row block of the few-rows kernel for the shared group (measured: up to 64 tokens
+                            # the merged launches and the library's product for the shared expert are as fast)
 
     def __init__(self, hidden: int, num_experts: int, top_k: int, expert_intermediate: int,
                  shared_intermediate: Optional[int] = None, gate: str = "sigmoid", renormalise: bool = False,
