@@ -114,11 +114,22 @@ __global__ __launch_bounds__(256) void rope_kv_vec_kernel(
   const T* src = qkv + (size_t)t * (nh + 2 * nkv) * hd;
   float post = 1.0f;
   if (temp_tuning) post = 1.0f + attn_scale * logf(floorf(((float)pos + 1.0f) / floor_scale) + 1.0f);
+  // a thread's run within a head is the same in every turn of the loop (the block size is a multiple
+  // of the lanes per head), and so are its four angles: their sines and cosines are computed once
+  const int run = threadIdx.x % per_head;
+  float cs[4], sn[4];
+  if (inv_freq) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float ang = (float)pos * inv_freq[run * 4 + j];
+      cs[j] = cosf(ang);
+      sn[j] = sinf(ang);
+    }
+  }
   for (int base = blockIdx.y * blockDim.x; base < chunks; base += gridDim.y * blockDim.x) {
     const int ci = base + threadIdx.x;
     const bool valid = ci < chunks;
     const int head = valid ? ci / per_head : 0;
-    const int run = valid ? ci % per_head : 0;
     const bool is_q = head < nh;
     const bool is_k = !is_q && head < nh + nkv;
     float x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -128,11 +139,9 @@ __global__ __launch_bounds__(256) void rope_kv_vec_kernel(
       if (inv_freq) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const float ang = (float)pos * inv_freq[run * 4 + j];
-          const float c = cosf(ang), sn = sinf(ang);
           const float a = x[2 * j], b = x[2 * j + 1];
-          x[2 * j] = a * c - b * sn;
-          x[2 * j + 1] = a * sn + b * c;
+          x[2 * j] = a * cs[j] - b * sn[j];
+          x[2 * j + 1] = a * sn[j] + b * cs[j];
         }
       }
 #pragma unroll
@@ -178,7 +187,9 @@ SHARPI_EXPORT int sharpi_rope_kv(const void* qkv, void* q_out, void* k_cache, vo
   dim3 grid(n_tokens, nh + 2 * nkv), block(kWave);
   if (dtype != DT_F32 && dtype != DT_BF16) return SHARPI_ERR_ARG;
   if (hd == 32 || hd == 64 || hd == 128 || hd == 256) {
-    const dim3 vgrid(n_tokens, ceil_div((nh + 2 * nkv) * (hd >> 3), 256));
+    // a few tokens (decode): a token's heads over several blocks, for the compute units' sake;
+    // many tokens: one block per token, which then computes its angles once for all heads
+    const dim3 vgrid(n_tokens, n_tokens <= 64 ? ceil_div((nh + 2 * nkv) * (hd >> 3), 256) : 1);
     if (dtype == DT_F32)
       rope_kv_vec_kernel<float><<<vgrid, 256, 0, stream>>>((const float*)qkv, (float*)q_out, (float*)k_cache,
                                                              (float*)v_cache, slot_mapping, positions, inv_freq,

@@ -55,55 +55,79 @@ __device__ void gate_and_pick(float* g, int n_experts, int k, int gate, int reno
     for (int j = 0; j < k; ++j) w[j] /= wsum;
 }
 
-template <typename T, typename TW>
+template <typename T, typename TW, int TT>
 __global__ __launch_bounds__(1024) void router_topk_kernel(const T* __restrict__ x, const TW* __restrict__ wr,
                                                            int* __restrict__ topk_ids,
                                                            float* __restrict__ topk_w,
-                                                           float* __restrict__ gate_out, int hidden,
+                                                           float* __restrict__ gate_out, int n_tokens, int hidden,
                                                            int n_experts, int k, int gate, int renorm) {
-  __shared__ float g[kMaxExperts];
-  const int t = blockIdx.x;
+  // TT tokens per block: a router row is fetched once for all of them.  A token's logit is the same
+  // chain of additions whatever TT is (each token has its own accumulator), so how many tokens
+  // share a block never shows in the result.
+  __shared__ float g[TT][kMaxExperts];
+  const int t0 = blockIdx.x * TT;
   const int lane = threadIdx.x & (kWave - 1);
   const int w = threadIdx.x >> 6;
   const int nw = blockDim.x >> 6;
-  const T* xr = x + (size_t)t * hidden;
+  const T* xr[TT];
+#pragma unroll
+  for (int i = 0; i < TT; ++i) xr[i] = x + (size_t)min(t0 + i, n_tokens - 1) * hidden;   // beyond the last: computed, not kept
   const bool vec = (hidden & 7) == 0;
   for (int e = w; e < n_experts; e += nw) {
     const TW* wrow = wr + (size_t)e * hidden;
-    float s = 0.f;
+    float s[TT];
+#pragma unroll
+    for (int i = 0; i < TT; ++i) s[i] = 0.f;
     if (vec) {  // lane-strided runs of 8: the order of the additions depends on the width only
       // four runs are fetched before the first is added: a row is a dozen dependent round trips
       // to the cache otherwise, and the kernel is nothing but their latency
+      constexpr int Q = TT == 1 ? 4 : 2;
       int c = lane * 8;
-      for (; c + 3 * kWave * 8 < hidden; c += 4 * kWave * 8) {
-        float a[4][8], b[4][8];
+      for (; c + (Q - 1) * kWave * 8 < hidden; c += Q * kWave * 8) {
+        float a[TT][Q][8], b[Q][8];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          load8(xr + c + q * kWave * 8, a[q]);
+        for (int q = 0; q < Q; ++q) {
           load8(wrow + c + q * kWave * 8, b[q]);
+#pragma unroll
+          for (int i = 0; i < TT; ++i) load8(xr[i] + c + q * kWave * 8, a[i][q]);
         }
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
+        for (int i = 0; i < TT; ++i)
 #pragma unroll
-          for (int i = 0; i < 8; ++i) s = fmaf(a[q][i], b[q][i], s);
+          for (int q = 0; q < Q; ++q)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) s[i] = fmaf(a[i][q][j], b[q][j], s[i]);
       }
       for (; c < hidden; c += kWave * 8) {
-        float a[8], b[8];
-        load8(xr + c, a);
+        float b[8];
         load8(wrow + c, b);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) s = fmaf(a[i], b[i], s);
+        for (int i = 0; i < TT; ++i) {
+          float a[8];
+          load8(xr[i] + c, a);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) s[i] = fmaf(a[j], b[j], s[i]);
+        }
       }
     } else {
-      for (int c = lane; c < hidden; c += kWave) s = fmaf(to_f32<T>(xr[c]), to_f32<TW>(wrow[c]), s);
+      for (int c = lane; c < hidden; c += kWave) {
+        const float b = to_f32<TW>(wrow[c]);
+#pragma unroll
+        for (int i = 0; i < TT; ++i) s[i] = fmaf(to_f32<T>(xr[i][c]), b, s[i]);
+      }
     }
-    s = wave_sum(s);
-    if (lane == 0) g[e] = s;
+#pragma unroll
+    for (int i = 0; i < TT; ++i) {
+      const float v = wave_sum(s[i]);
+      if (lane == 0) g[i][e] = v;
+    }
   }
   __syncthreads();
-  if (threadIdx.x == 0)
-    gate_and_pick(g, n_experts, k, gate, renorm, topk_ids + (size_t)t * k, topk_w + (size_t)t * k,
+  if (threadIdx.x < TT && t0 + threadIdx.x < n_tokens) {
+    const int t = t0 + threadIdx.x;
+    gate_and_pick(g[threadIdx.x], n_experts, k, gate, renorm, topk_ids + (size_t)t * k, topk_w + (size_t)t * k,
                   gate_out ? gate_out + (size_t)t * n_experts : nullptr);
+  }
 }
 
 SHARPI_EXPORT int sharpi_router_topk(const void* x, int x_dtype, const void* wr, int w_dtype, int* topk_ids,
@@ -112,11 +136,21 @@ SHARPI_EXPORT int sharpi_router_topk(const void* x, int x_dtype, const void* wr,
   if (n_tokens <= 0) return SHARPI_OK;
   if (hidden <= 0 || n_experts <= 0 || n_experts > kMaxExperts || k <= 0 || k > n_experts) return SHARPI_ERR_ARG;
   if (gate < 0 || gate > 1) return SHARPI_ERR_ARG;
-  // one wave per expert at a time: enough waves for the experts, at most 16
-  dim3 grid(n_tokens), block(kWave * (n_experts >= 16 ? 16 : n_experts >= 8 ? 8 : 4));
-#define ROUTER_LAUNCH(TX, TWT)                                                                              \
-  router_topk_kernel<TX, TWT><<<grid, block, 0, stream>>>((const TX*)x, (const TWT*)wr, topk_ids, topk_w,   \
-                                                          gate_out, hidden, n_experts, k, gate, renorm)
+  // one wave per expert at a time: enough waves for the experts, at most 16; with many tokens four
+  // share a block (and each fetch of a router row)
+  const int tt = n_tokens >= 64 ? 4 : 1;
+  dim3 grid(ceil_div(n_tokens, tt)), block(kWave * (n_experts >= 16 ? 16 : n_experts >= 8 ? 8 : 4));
+#define ROUTER_LAUNCH(TX, TWT)                                                                                   \
+  do {                                                                                                           \
+    if (tt == 4)                                                                                                 \
+      router_topk_kernel<TX, TWT, 4><<<grid, block, 0, stream>>>((const TX*)x, (const TWT*)wr, topk_ids, topk_w, \
+                                                                 gate_out, n_tokens, hidden, n_experts, k, gate, \
+                                                                 renorm);                                        \
+    else                                                                                                         \
+      router_topk_kernel<TX, TWT, 1><<<grid, block, 0, stream>>>((const TX*)x, (const TWT*)wr, topk_ids, topk_w, \
+                                                                 gate_out, n_tokens, hidden, n_experts, k, gate, \
+                                                                 renorm);                                        \
+  } while (0)
   if (x_dtype == DT_F32 && w_dtype == DT_F32) ROUTER_LAUNCH(float, float);
   else if (x_dtype == DT_BF16 && w_dtype == DT_BF16) ROUTER_LAUNCH(bf16_t, bf16_t);
   else if (x_dtype == DT_BF16 && w_dtype == DT_F32) ROUTER_LAUNCH(bf16_t, float);

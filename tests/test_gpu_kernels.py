@@ -263,6 +263,20 @@ def test_router_and_permute(T, E, k, H, dtype):
     assert tiles == want
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H", [5120, 136, 75])
+def test_router_rows_do_not_depend_on_the_batch(dtype, H):
+    """Many tokens share a block of the router kernel (and its fetches of the router's rows); a
+    token's gate values are the same bits as when it is routed alone."""
+    ops = _ops()
+    x = _rand(70, H, dtype=dtype, seed=H)
+    wr = _rand(16, H, dtype=dtype, scale=0.3, seed=H + 1)
+    ids, wts, gates = ops.router_topk(x, wr, 2, want_gates=True)
+    for i in (0, 3, 37, 68, 69):
+        ids1, wts1, gates1 = ops.router_topk(x[i:i + 1].contiguous(), wr, 2, want_gates=True)
+        assert torch.equal(gates1[0], gates[i]) and torch.equal(ids1[0], ids[i]) and torch.equal(wts1[0], wts[i]), i
+
+
 def test_router_ties_pick_the_lowest_index():
     ops = _ops()
     x = _rand(4, 64)
