@@ -1,6 +1,6 @@
 // MoE routing on the device: router logits, gate, top-k, and the expert-sorted row list.
 //
-// router_topk: one block per token. logits[e] = Wr[e, :] . x[t, :] in float (each wave owns
+// router_topk: one block per token, or per four tokens when there are many. logits[e] = Wr[e, :] . x[t, :] in float (each wave owns
 // experts e = wave, wave + nwaves, ...; lanes stride over the hidden width, so the order of
 // the additions depends on the width only).  gate 0 = sigmoid over every expert, gate 1 =
 // softmax over every expert.  The k picks scan ascending with a strict >, so the lowest index
@@ -79,7 +79,7 @@ __global__ __launch_bounds__(1024) void router_topk_kernel(const T* __restrict__
 #pragma unroll
     for (int i = 0; i < TT; ++i) s[i] = 0.f;
     if (vec) {  // lane-strided runs of 8: the order of the additions depends on the width only
-      // four runs are fetched before the first is added: a row is a dozen dependent round trips
+      // Q runs are fetched before the first is added: a row is a dozen dependent round trips
       // to the cache otherwise, and the kernel is nothing but their latency
       constexpr int Q = TT == 1 ? 4 : 2;
       int c = lane * 8;
