@@ -103,3 +103,45 @@ def test_other_page_sizes(model_dir, page_size, dtype):
     for g in eng.cache.groups:
         assert g.pool.num_free == g.pool.num_pages
 
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_graph_replays_equal_eager_steps(model_dir, dtype):
+    """Decode-only steps replay a captured graph per batch size.  Every replay (the first and later
+    ones, with prefill steps, mixed steps, other graphs and a freed request in between) must give
+    the bits of the same step launched kernel by kernel."""
+    which, d = model_dir
+    if which not in ("B", "D"):
+        pytest.skip("two configurations are enough here")
+    vocab = CONFIGS[which]["vocab_size"]
+    toks = {r: H.random_tokens(n, vocab, 900 + i) for i, (r, n) in enumerate((("a", 40), ("b", 30), ("c", 33)))}
+    at = {r: 0 for r in toks}
+
+    def take(r, n, want_last=True):
+        e = {"id": r, "tokens": toks[r][at[r]:at[r] + n], "want": [n - 1] if want_last else []}
+        at[r] += n
+        return e
+
+    steps = [{"entries": [take("a", 20)], "end": []}]
+    steps += [{"entries": [take("a", 1)], "end": []} for _ in range(3)]                       # batch 1, three replays
+    steps += [{"entries": [take("a", 1), take("b", 15)], "end": []}]                           # mixed: launched eagerly
+    steps += [{"entries": [take("a", 1), take("b", 1)], "end": []} for _ in range(3)]          # batch 2
+    steps += [{"entries": [take("c", 18)], "end": []}]                                         # a prompt alone in between
+    steps += [{"entries": [take("a", 1), take("b", 1), take("c", 1)], "end": []} for _ in range(2)]   # batch 3
+    steps[-1]["end"] = ["a"]
+    steps += [{"entries": [take("c", 1), take("b", 1)], "end": []} for _ in range(2)]          # batch 2 again, other requests
+    steps += [{"entries": [take("b", 1)], "end": []} for _ in range(2)]                        # batch 1 again
+    steps[-1]["end"] = ["b", "c"]
+    for i, st in enumerate(steps):
+        st["step"] = i
+    out = {}
+    for graphs in (True, False):
+        eng = H.make_engine(d, dtype, kv_tokens=256, max_num_seqs=4, decode_graphs=graphs)
+        out[graphs] = H.replay(eng, steps)
+        if graphs:
+            graphs_made = eng.runner._graphs
+            assert sorted(graphs_made) == [1, 2, 3] and all(g is not False for g in graphs_made.values()), \
+                "decode steps of batch 1, 2 and 3 should each have captured a graph"
+            assert eng.runner.graph_replays == 12
+    for r in toks:
+        assert torch.equal(out[True][r], out[False][r]), r
+
