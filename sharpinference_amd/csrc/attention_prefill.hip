@@ -11,8 +11,8 @@
 //                                               inside a page), B = P^T
 // and the S^T accumulator of a lane is the B operand of the second product once exponentiated
 // and split into a bfloat16 pair hi + lo.  In LDS the value columns are permuted so that the
-// eight keys a lane needs (4 of each 16-key block) sit side by side; rows are padded so that the
-// 16 lanes of a quarter-wave hit 16 different bank groups.  Softmax state (a reference maximum and
+// eight keys a lane needs (4 of each 16-key block) sit side by side; the 16-byte chunks of a row are
+// swizzled so that reads are free of bank conflicts (see the layouts below).  Softmax state (a reference maximum and
 // the sum per query) is float, kept in base-2 units (scores times log2 e, the hardware's exp2).
 // The keys of a query are always visited in the same blocks, whatever the portion it arrived in,
 // so its sums do not depend on how the prompt was cut.
@@ -26,22 +26,36 @@ constexpr int kPreWaves = 4;
 constexpr int kQT = 2;                               // 16-token column tiles per wave
 constexpr int kWaveTokens = 16 * kQT;
 constexpr int kTileTokens = kWaveTokens * kPreWaves; // 128 tokens per block
-constexpr int kVPad = 40;                            // LDS row of the value tile: 32 keys + 8
+constexpr int kVRow = 32;                            // LDS row of the value tile: 32 keys, no pad (chunks swizzled)
+
+// LDS layouts.  The LDS serves a 16-byte read of a wave in four turns of two octets of lanes: one
+// octet holding operand rows 0..7 and one holding rows 8..15 of the neighbouring lane group (measured
+// with the bank-conflict counter).  The 16 chunks of 16 bytes that a turn reads must fall into the 16
+// different 16-byte groups of the 256-byte bank space; the chunk index is XORed with row bits so that
+// they do, for rows of 256 bytes (keys, head size 128), 128 bytes (head size 64) and 64 bytes
+// (values: 32 keys).  Other head sizes keep rows padded by 16 bytes (two-way conflicts).
+template <int HD> __device__ __forceinline__ constexpr int k_row_elems() { return (HD == 128 || HD == 64) ? HD : HD + 8; }
+template <int HD> __device__ __forceinline__ int k_col(int row, int col) {   // col a multiple of 8 elements
+  if constexpr (HD == 128) return col ^ ((row & 15) << 3);
+  else if constexpr (HD == 64) return col ^ (((row >> 1) & 7) << 3);
+  else return col;
+}
+__device__ __forceinline__ int v_col(int row, int col) { return col ^ (((row >> 2) & 3) << 3); }   // 4 chunks a row
 constexpr float kLazyMax = 8.0f;                     // how far the row maximum may outgrow its reference
 
 template <int HD>
-__global__ __launch_bounds__(kPreWaves* kWave) void attn_prefill_kernel(
+__global__ __launch_bounds__(kPreWaves* kWave, HD <= 128 ? 2 : 1) void attn_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ block_table, const int* __restrict__ positions, const int* __restrict__ tiles,
     bf16_t* __restrict__ out, int window_kind, int window, float scale, int nh, int nkv, int page_size,
     int max_blocks, int num_pages) {
   constexpr int NJ = HD / 32;
   constexpr int ND = HD / 16;
-  constexpr int KPAD = HD + 8;
+  constexpr int KPAD = k_row_elems<HD>();
   constexpr int PIECES = 4 * HD;                                   // 16-byte pieces of a K (or V) chunk
   constexpr int NST = (PIECES + kPreWaves * kWave - 1) / (kPreWaves * kWave);
   __shared__ __attribute__((aligned(16))) bf16_t Ks[2][32][KPAD];
-  __shared__ __attribute__((aligned(16))) bf16_t Vs[2][HD][kVPad];
+  __shared__ __attribute__((aligned(16))) bf16_t Vs[2][HD][kVRow];
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
@@ -149,12 +163,12 @@ __global__ __launch_bounds__(kPreWaves* kWave) void attn_prefill_kernel(
       const int piece = tid + i * kPreWaves * kWave;
       if (piece < PIECES) {
         const int key = piece / (HD / 8), dcol = (piece % (HD / 8)) * 8;
-        *reinterpret_cast<u32x4*>(&Ks[buf][key][dcol]) = kst[i];
+        *reinterpret_cast<u32x4*>(&Ks[buf][key][k_col<HD>(key, dcol)]) = kst[i];
         // keys 8*half .. 8*half+7 of block blk: groups g = 2*half and 2*half + 1, four keys each;
         // column of (g, blk) = g*8 + blk*4
         const int d = piece >> 2, blk = (piece >> 1) & 1, half = piece & 1;
-        *reinterpret_cast<uint2*>(&Vs[buf][d][(2 * half) * 8 + blk * 4]) = uint2{vst[i].x, vst[i].y};
-        *reinterpret_cast<uint2*>(&Vs[buf][d][(2 * half + 1) * 8 + blk * 4]) = uint2{vst[i].z, vst[i].w};
+        *reinterpret_cast<uint2*>(&Vs[buf][d][v_col(d, (2 * half) * 8) + blk * 4]) = uint2{vst[i].x, vst[i].y};
+        *reinterpret_cast<uint2*>(&Vs[buf][d][v_col(d, (2 * half + 1) * 8) + blk * 4]) = uint2{vst[i].z, vst[i].w};
       }
     }
   };
@@ -186,7 +200,7 @@ __global__ __launch_bounds__(kPreWaves* kWave) void attn_prefill_kernel(
         if (have[u]) {
 #pragma unroll
           for (int j = 0; j < NJ; ++j) {
-            const bf16x8 kf = *reinterpret_cast<const bf16x8*>(&Ks[buf][u * 16 + r][j * 32 + g * 8]);
+            const bf16x8 kf = *reinterpret_cast<const bf16x8*>(&Ks[buf][u * 16 + r][k_col<HD>(u * 16 + r, j * 32 + g * 8)]);
 #pragma unroll
             for (int c = 0; c < kQT; ++c) s[c][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[c][j], s[c][u], 0, 0, 0);
           }
@@ -249,7 +263,7 @@ __global__ __launch_bounds__(kPreWaves* kWave) void attn_prefill_kernel(
 #pragma unroll
       for (int d = 0; d < ND; ++d) {
         // lane (d row r, group g): keys 4g..4g+3 of block b, then of block b + 1, side by side in LDS
-        const bf16x8 vf = *reinterpret_cast<const bf16x8*>(&Vs[buf][d * 16 + r][g * 8]);
+        const bf16x8 vf = *reinterpret_cast<const bf16x8*>(&Vs[buf][d * 16 + r][v_col(d * 16 + r, g * 8)]);
 #pragma unroll
         for (int c = 0; c < kQT; ++c) {
           if (rescale[c]) acc[c][d] *= corr[c];
