@@ -42,6 +42,9 @@ template <int HD> __device__ __forceinline__ int k_col(int row, int col) {   // 
 }
 __device__ __forceinline__ int v_col(int row, int col) { return col ^ (((row >> 2) & 3) << 3); }   // 4 chunks a row
 constexpr float kLazyMax = 8.0f;                     // how far the row maximum may outgrow its reference
+// the reference before a row has seen a key: finite, so that a masked score (-inf) minus it is
+// -inf and its probability 0, and far below any score, so that the first key moves it
+constexpr float kNoMax = -1.0e30f;
 
 template <int HD>
 __global__ __launch_bounds__(kPreWaves* kWave, HD <= 128 ? 2 : 1) void attn_prefill_kernel(
@@ -114,7 +117,7 @@ __global__ __launch_bounds__(kPreWaves* kWave, HD <= 128 ? 2 : 1) void attn_pref
   f32x4 acc[kQT][ND];
 #pragma unroll
   for (int c = 0; c < kQT; ++c) {
-    m[c] = -INFINITY;
+    m[c] = kNoMax;
     l[c] = 0.f;
 #pragma unroll
     for (int d = 0; d < ND; ++d) acc[c][d] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -207,13 +210,14 @@ __global__ __launch_bounds__(kPreWaves* kWave, HD <= 128 ? 2 : 1) void attn_pref
         }
       }
       bf16x8 pf[kQT], pf_lo[kQT];
-      float corr[kQT];
       // a chunk that every row of the wave sees whole needs no mask
       const bool whole = wave_full && have[1] && ((b + 2) << 4) - 1 <= wave_first_pos && (b << 4) >= wave_last_start;
+      // lane holds S^T[key = 16*(b+u) + 4g + i][query row c*16 + r]; scores go to base-2 units
+      float lmax[kQT];
+      bool grown = false;
 #pragma unroll
       for (int c = 0; c < kQT; ++c) {
-        // lane holds S^T[key = 16*(b+u) + 4g + i][query row c*16 + r]; scores go to base-2 units
-        float cm = -INFINITY;
+        float lm = -INFINITY;   // the largest score this lane holds of the row
 #pragma unroll
         for (int u = 0; u < 2; ++u)
 #pragma unroll
@@ -225,48 +229,64 @@ __global__ __launch_bounds__(kPreWaves* kWave, HD <= 128 ? 2 : 1) void attn_pref
               t = ok ? t : -INFINITY;
             }
             s[c][u][i] = t;
-            cm = fmaxf(cm, t);
+            lm = fmaxf(lm, t);
           }
-        cm = fmaxf(cm, __shfl_xor(cm, 16, kWave));
-        cm = fmaxf(cm, __shfl_xor(cm, 32, kWave));
-        // m is a reference, not the exact running maximum: it moves only when the maximum has grown
-        // past it by more than kLazyMax (base-2 units), so probabilities reach 2^kLazyMax at most, which
-        // float sums carry easily, and the accumulators are rescaled in few chunks.  The decision
-        // is the row's own (its four lanes hold the same m and cm), so what a row ends up with does
-        // not depend on the rows it shares a wave with.
-        const float m_true = fmaxf(m[c], cm);
-        const float m_new = (m_true - m[c] > kLazyMax) ? m_true : m[c];   // from -inf: inf > kLazyMax; all masked: NaN, stays
-        corr[c] = 1.0f;
-        if (m_new == -INFINITY) {
-          pf[c] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
-          pf_lo[c] = pf[c];
-        } else {
-          corr[c] = __builtin_amdgcn_exp2f(m[c] - m_new);
-          float ls = 0.f;
-#pragma unroll
-          for (int u = 0; u < 2; ++u)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              const float e = __builtin_amdgcn_exp2f(s[c][u][i] - m_new);   // masked: 2^-inf = 0
-              ls += e;
-              const __bf16 hi = (__bf16)e;                                   // round to nearest even
-              pf[c][u * 4 + i] = hi;
-              pf_lo[c][u * 4 + i] = (__bf16)(e - (float)hi);
-            }
-          l[c] = l[c] * corr[c] + ls;
-          m[c] = m_new;
-        }
+        lmax[c] = lm;
+        grown = grown || lm - m[c] > kLazyMax;
       }
+      // m is a reference, not the running maximum: a row moves it only when the chunk's largest
+      // score lies more than kLazyMax (base-2 units) above it.  Probabilities then reach 2^kLazyMax
+      // at most, which float sums carry easily.  Most chunks move no row of the wave: they need
+      // no exchange between lanes and no rescaling.  The rule is the row's own (its four lanes
+      // hold the same m and, once exchanged, the same maximum), so what a row ends up with does
+      // not depend on the rows it shares a wave with.
+      float corr[kQT];
       bool rescale[kQT];
 #pragma unroll
-      for (int c = 0; c < kQT; ++c) rescale[c] = __builtin_amdgcn_ballot_w64(corr[c] != 1.0f) != 0;   // wave-uniform
+      for (int c = 0; c < kQT; ++c) {
+        corr[c] = 1.0f;
+        rescale[c] = false;
+      }
+      if (__builtin_amdgcn_ballot_w64(grown) != 0) {   // wave-uniform
+#pragma unroll
+        for (int c = 0; c < kQT; ++c) {
+          float cm = lmax[c];
+          cm = fmaxf(cm, __shfl_xor(cm, 16, kWave));
+          cm = fmaxf(cm, __shfl_xor(cm, 32, kWave));
+          const bool move = cm - m[c] > kLazyMax;
+          corr[c] = move ? __builtin_amdgcn_exp2f(m[c] - cm) : 1.0f;
+          m[c] = move ? cm : m[c];
+          l[c] *= corr[c];
+          rescale[c] = __builtin_amdgcn_ballot_w64(move) != 0;
+        }
+      }
+#pragma unroll
+      for (int c = 0; c < kQT; ++c) {
+        float ls = 0.f;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float e = __builtin_amdgcn_exp2f(s[c][u][i] - m[c]);   // masked: 2^-inf = 0
+            ls += e;
+            const __bf16 hi = (__bf16)e;                                   // round to nearest even
+            pf[c][u * 4 + i] = hi;
+            pf_lo[c][u * 4 + i] = (__bf16)(e - (float)hi);
+          }
+        l[c] += ls;
+      }
 #pragma unroll
       for (int d = 0; d < ND; ++d) {
         // lane (d row r, group g): keys 4g..4g+3 of block b, then of block b + 1, side by side in LDS
         const bf16x8 vf = *reinterpret_cast<const bf16x8*>(&Vs[buf][d * 16 + r][v_col(d * 16 + r, g * 8)]);
 #pragma unroll
         for (int c = 0; c < kQT; ++c) {
-          if (rescale[c]) acc[c][d] *= corr[c];
+          if (rescale[c]) {
+            // rare, and to stay a branch: the empty statement keeps the compiler from turning it into
+            // a multiplication by one in every chunk
+            asm volatile("");
+            acc[c][d] *= corr[c];
+          }
           acc[c][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[c], acc[c][d], 0, 0, 0);
           acc[c][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf_lo[c], acc[c][d], 0, 0, 0);
         }
