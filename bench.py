@@ -44,13 +44,13 @@ def log(msg: str) -> None:
     print(f"[bench] {msg}", file=sys.stderr, flush=True)
 
 
-def build_engine(layers: int, max_batch: int, page_size: int, graphs: bool = True):
+def build_engine(layers: int, max_batch: int, page_size: int, graphs: bool = True, gen_len: int = GEN_LEN):
     from sharpinference_amd.engine import Engine
 
     cfg = dict(SCOUT)
     cfg["num_hidden_layers"] = layers
     cfg["no_rope_layers"] = [0 if (l + 1) % 4 == 0 else 1 for l in range(layers)]
-    per_req = (PROMPT_LEN + GEN_LEN + page_size - 1) // page_size * page_size
+    per_req = (PROMPT_LEN + gen_len + page_size - 1) // page_size * page_size
     t0 = time.time()
     eng = Engine(config=cfg, weight_seed=2, dtype="bfloat16", device="cuda:0", max_model_len=CONTEXT,
                  max_num_seqs=max_batch, max_tokens_per_step=8192, kv_tokens=max_batch * per_req,
@@ -138,7 +138,7 @@ def decode_run(eng, batch: int, steps: int, warmup: int, rng: random.Random, cou
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--steps", type=int, default=GEN_LEN - 8, help="timed decode steps (default: with the warm-up, the 256 generated tokens of the baseline's run)")
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--layers", type=int, default=FULL_LAYERS)
     ap.add_argument("--batch", type=int, default=8)
@@ -154,7 +154,8 @@ def main() -> int:
 
     rng = random.Random(2)
     max_batch = args.batch if args.no_points else max(args.batch, 64)
-    eng = build_engine(args.layers, max_batch, args.page_size, graphs=not args.no_graphs)
+    gen_len = max(GEN_LEN, args.warmup + args.steps + 2)      # warm-up, timed steps and the one traced step
+    eng = build_engine(args.layers, max_batch, args.page_size, graphs=not args.no_graphs, gen_len=gen_len)
     cfg = eng.config
 
     # prefill: one 2,048-token prompt alone, once to warm up, once timed
@@ -198,7 +199,7 @@ def main() -> int:
             "hidden_size": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
             "head_dim": cfg.head_dim, "experts": cfg.num_local_experts, "experts_per_tok": cfg.num_experts_per_tok,
             "expert_ffn": cfg.intermediate_size, "shared_ffn": cfg.intermediate_size, "vocab": cfg.vocab_size,
-            "attention_chunk": cfg.attention_chunk_size, "prompt_len": PROMPT_LEN, "generated": GEN_LEN,
+            "attention_chunk": cfg.attention_chunk_size, "prompt_len": PROMPT_LEN, "generated": args.warmup + args.steps,
             "page_size": args.page_size,
         },
         "prefill": prefill,
