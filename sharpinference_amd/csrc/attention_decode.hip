@@ -195,11 +195,18 @@ __global__ __launch_bounds__(kDecWaves* kWave) void attn_decode_kernel(
   }
 }
 
-// merge the runs of one (token, head): out = sum_s O_s e^(m_s - M) / sum_s l_s e^(m_s - M)
-__global__ void attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                         const int* __restrict__ positions, const int* __restrict__ token_list,
-                                         bf16_t* __restrict__ out, int window_kind, int window, int nh, int hd,
-                                         int max_splits) {
+// merge the runs of one (token, head): out = sum_s O_s e^(m_s - M) / sum_s l_s e^(m_s - M).
+// A block's threads are (run lane, 4-wide column of d): the run lanes walk the runs side by side
+// with independent loads and meet in LDS, in an order that depends on the number of runs only.
+constexpr int kMergeThreads = 256;
+
+__global__ __launch_bounds__(kMergeThreads) void attn_decode_merge_kernel(
+    const float* __restrict__ part_o, const float* __restrict__ part_ml, const int* __restrict__ positions,
+    const int* __restrict__ token_list, bf16_t* __restrict__ out, int window_kind, int window, int nh, int hd,
+    int max_splits) {
+  __shared__ float red_s[kMergeThreads / kWave];
+  __shared__ f32x4 o_s[kMergeThreads];
+  __shared__ float l_s[kMergeThreads];
   const int li = blockIdx.x;
   const int h = blockIdx.y;
   const int t = token_list ? token_list[li] : li;
@@ -209,21 +216,47 @@ __global__ void attn_decode_merge_kernel(const float* __restrict__ part_o, const
   else if (window_kind == 2) start = p - window + 1 > 0 ? p - window + 1 : 0;
   const int n_runs = ((p >> 4) - (start >> 4)) / kSplitBlocks + 1;
   const size_t base = ((size_t)li * nh + h) * max_splits;
+
   float M = -INFINITY;
-  for (int s = 0; s < n_runs; ++s) M = fmaxf(M, part_ml[(base + s) * 2]);
+  for (int s = threadIdx.x; s < n_runs; s += kMergeThreads) M = fmaxf(M, part_ml[(base + s) * 2]);
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) M = fmaxf(M, __shfl_xor(M, o, kWave));
+  if ((threadIdx.x & (kWave - 1)) == 0) red_s[threadIdx.x >> 6] = M;
+  __syncthreads();
+  M = red_s[0];
+#pragma unroll
+  for (int ww = 1; ww < kMergeThreads / kWave; ++ww) M = fmaxf(M, red_s[ww]);
+
+  const int ncol = hd >> 2;                      // 4-wide columns of a head
+  const int lanes = kMergeThreads / ncol;        // run lanes (hd <= 256: at least 4)
+  const int col = threadIdx.x % ncol, rl = threadIdx.x / ncol;
+  f32x4 o = f32x4{0.f, 0.f, 0.f, 0.f};
   float L = 0.f;
-  for (int s = 0; s < n_runs; ++s) {
-    const float ms = part_ml[(base + s) * 2];
-    L += ms == -INFINITY ? 0.f : part_ml[(base + s) * 2 + 1] * expf(ms - M);
-  }
-  for (int d = threadIdx.x; d < hd; d += blockDim.x) {
-    float o = 0.f;
-    for (int s = 0; s < n_runs; ++s) {
+  if (rl < lanes) {
+    for (int s = rl; s < n_runs; s += lanes) {
       const float ms = part_ml[(base + s) * 2];
-      if (ms != -INFINITY) o += part_o[(base + s) * hd + d] * expf(ms - M);
+      const float f = ms == -INFINITY ? 0.f : expf(ms - M);
+      const f32x4 po = *reinterpret_cast<const f32x4*>(part_o + (base + s) * hd + col * 4);
+      L += part_ml[(base + s) * 2 + 1] * f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[i] += f > 0.f ? po[i] * f : 0.f;
     }
-    out[((size_t)t * nh + h) * hd + d] = f32_to_bf16(L > 0.f ? o / L : 0.f);
   }
+  o_s[threadIdx.x] = o;
+  l_s[threadIdx.x] = L;
+  __syncthreads();
+  if (rl != 0) return;
+  for (int x = 1; x < lanes; ++x) {
+    o += o_s[x * ncol + col];
+    L += l_s[x * ncol + col];
+  }
+  unsigned short b[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) b[i] = f32_to_bf16(L > 0.f ? o[i] / L : 0.f).bits;
+  uint2 pk;
+  pk.x = b[0] | ((unsigned)b[1] << 16);
+  pk.y = b[2] | ((unsigned)b[3] << 16);
+  *reinterpret_cast<uint2*>(out + ((size_t)t * nh + h) * hd + col * 4) = pk;
 }
 
 template <int HD>
@@ -238,7 +271,7 @@ static int launch_decode(const void* q, const void* k_cache, const void* v_cache
                                                     part_ml, window_kind, window, scale, nh, nkv, page_size,
                                                     max_blocks, num_pages, max_splits);
   SHARPI_CHECK_LAUNCH();
-  dim3 mgrid(n_list, nh), mblock(HD >= 128 ? 128 : 64);
+  dim3 mgrid(n_list, nh), mblock(kMergeThreads);
   attn_decode_merge_kernel<<<mgrid, mblock, 0, stream>>>(part_o, part_ml, positions, token_list, (bf16_t*)out,
                                                          window_kind, window, nh, HD, max_splits);
   SHARPI_CHECK_LAUNCH();
