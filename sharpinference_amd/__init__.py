@@ -10,7 +10,7 @@ from .sampling.params import SamplingParams  # noqa: F401
 
 
 def __getattr__(name):
-    if name in ("Engine", "GenerationResult", "StepEntry"):
+    if name in ("Engine", "GenerateChunk", "GenerationResult", "StepEntry"):
         from . import engine as _e
 
         return getattr(_e, name)

@@ -100,10 +100,18 @@ def main(argv: Optional[List[str]] = None) -> int:
         print(f"prompt tokens ({len(prompt)}): {prompt}")
     elif not args.no_display_prompt:
         print(" ".join(str(t) for t in prompt))
-    results = eng.generate([prompt] * args.parallel, params)
-    for i, r in enumerate(results):
-        head = f"[{i}] " if args.parallel > 1 else ""
-        print(f"{head}{' '.join(str(t) for t in r.token_ids)}  ({r.finish_reason})")
+    if args.parallel == 1:
+        # one request: its tokens are printed as they come (the reference streams its chunks the same way)
+        first = True
+        for c in eng.generate_chunks([prompt], params):
+            if c.kind == "token":
+                print(("" if first else " ") + str(c.token_id), end="", flush=True)
+                first = False
+            elif c.kind == "stop":
+                print(f"  ({c.finish_reason})", flush=True)
+    else:
+        for i, r in enumerate(eng.generate([prompt] * args.parallel, params)):
+            print(f"[{i}] {' '.join(str(t) for t in r.token_ids)}  ({r.finish_reason})")
     st = eng.last_stats
     pre = st.prefill_tokens / st.prefill_seconds if st.prefill_seconds > 0 else 0.0
     dec = st.decode_tokens / st.decode_seconds if st.decode_seconds > 0 else 0.0

@@ -10,7 +10,7 @@ from __future__ import annotations
 
 import time
 from dataclasses import dataclass, field
-from typing import Dict, Hashable, List, Optional, Sequence, Union
+from typing import Callable, Dict, Hashable, Iterator, List, Optional, Sequence, Union
 
 import torch
 
@@ -39,6 +39,17 @@ class GenerationResult:
     token_ids: List[int]
     finish_reason: str
     prompt_tokens: int
+
+
+@dataclass
+class GenerateChunk:
+    """One event of a generation (reference: src/SharpInference.Engine/GenerateChunk.cs:52-53)."""
+    kind: str                         # "usage" | "token" | "stop"
+    index: int                        # which prompt of the call
+    token_id: int = -1
+    prompt_tokens: int = 0
+    finish_reason: Optional[str] = None
+    truncated_by_max_tokens: bool = False
 
 
 @dataclass
@@ -105,6 +116,7 @@ class Engine:
                                   max_context=self.max_model_len)
         self.sampler = Sampler(self.device)
         self.last_stats = GenerationStats()
+        self._sched: Optional[Scheduler] = None            # the generation that is running, if one is
 
     # -- the low level: requests and steps ------------------------------------
     def add_request(self, req_id: Hashable) -> None:
@@ -117,12 +129,9 @@ class Engine:
         return self.runner.step(entries, router_trace)
 
     # -- generation -------------------------------------------------------------
-    def generate(self, prompts: Sequence[Sequence[int]], params: Union[SamplingParams, Sequence[SamplingParams], None] = None,
-                 *, max_new_tokens: Optional[int] = None, temperature: Optional[float] = None,
-                 seeds: Optional[Sequence[int]] = None, stop_token_ids: Sequence[int] = ()) -> List[GenerationResult]:
-        """Generate for a list of prompts (token ids) under continuous batching."""
+    def _sampling_params(self, n: int, params, max_new_tokens, temperature, seeds, stop_token_ids) -> List[SamplingParams]:
         plist: List[SamplingParams] = []
-        for i in range(len(prompts)):
+        for i in range(n):
             if isinstance(params, SamplingParams):
                 p = SamplingParams(**{**params.__dict__})
             elif params is not None:
@@ -138,45 +147,105 @@ class Engine:
             if stop_token_ids:
                 p.stop_token_ids = tuple(int(t) for t in stop_token_ids)
             plist.append(p)
+        return plist
+
+    @property
+    def queue_depth(self) -> int:
+        """Requests waiting to be admitted (reference: IInferenceEngine.cs:15)."""
+        return len(self._sched.waiting) if self._sched is not None else 0
+
+    @property
+    def active_requests(self) -> int:
+        """Requests being generated (reference: IInferenceEngine.cs:18)."""
+        return len(self._sched.running) if self._sched is not None else 0
+
+    def generate_chunks(self, prompts: Sequence[Sequence[int]],
+                        params: Union[SamplingParams, Sequence[SamplingParams], None] = None, *,
+                        max_new_tokens: Optional[int] = None, temperature: Optional[float] = None,
+                        seeds: Optional[Sequence[int]] = None, stop_token_ids: Sequence[int] = (),
+                        should_cancel: Optional[Callable[[int], bool]] = None) -> Iterator[GenerateChunk]:
+        """Generate for a list of prompts (token ids) under continuous batching and yield what
+        happens as it happens, in the reference's typed chunks
+        (reference: src/SharpInference.Engine/GenerateChunk.cs:9-53): per prompt one ``usage``
+        chunk with its number of prompt tokens before anything else of it, a ``token`` chunk per
+        generated token (the reference's text chunk; there is no tokenizer here), and one ``stop``
+        chunk when it ends.  ``should_cancel(index)`` is asked before every step, as the
+        reference's cancellation token is; a cancelled prompt ends with reason "abort".  Closing
+        the generator early gives every page back."""
+        if self._sched is not None:
+            raise RuntimeError("a generation is running on this engine: requests are admitted by one loop at a time")
+        plist = self._sampling_params(len(prompts), params, max_new_tokens, temperature, seeds, stop_token_ids)
         sched = Scheduler(self.cache, self.max_num_seqs, self.max_tokens_per_step, self.max_model_len)
         reqs = [Request(("gen", i), [int(t) for t in prompt], plist[i]) for i, prompt in enumerate(prompts)]
         for r in reqs:
             sched.add(r)
         stats = GenerationStats()
+        self.last_stats = stats
+        self._sched = sched
+        reported = 0                                       # finished requests already told of
         try:
+            for i, r in enumerate(reqs):
+                yield GenerateChunk("usage", i, prompt_tokens=len(r.prompt))
             while sched.has_work():
+                if should_cancel is not None:
+                    for i, r in enumerate(reqs):
+                        if not r.finished and not r.cancelled and should_cancel(i):
+                            r.cancelled = True
                 batch = sched.schedule()
-                if not batch:
-                    if sched.has_work():
-                        raise RuntimeError("scheduler has work but nothing can run")
-                    break
-                t0 = time.perf_counter()
-                entries = [StepEntry(s.request.req_id, s.tokens, (len(s.tokens) - 1,) if s.samples else ())
-                           for s in batch]
-                logits = self.runner.step(entries)
-                sampling = [s for s in batch if s.samples]
-                tokens: List[Optional[int]] = [None] * len(batch)
-                if sampling:
-                    hist = [penalty_window(s.request.params, s.request.prompt, s.request.output)
-                            if s.request.params.edits_logits else () for s in sampling]
-                    picked = self.sampler.sample(logits, [s.request.params for s in sampling],
-                                                 [s.request.draws for s in sampling], hist)
-                    it = iter(picked)
-                    tokens = [next(it) if s.samples else None for s in batch]
-                dt = time.perf_counter() - t0
-                n_prefill = sum(len(s.tokens) for s in batch if s.request.in_prefill)
-                n_decode = sum(1 for s in batch if not s.request.in_prefill)
-                if n_prefill:
-                    stats.prefill_tokens += n_prefill
-                    stats.prefill_seconds += dt * n_prefill / (n_prefill + n_decode)
-                if n_decode:
-                    stats.decode_tokens += n_decode
-                    stats.decode_seconds += dt * n_decode / (n_prefill + n_decode)
-                stats.steps += 1
-                sched.update(batch, tokens)
+                if batch:
+                    t0 = time.perf_counter()
+                    entries = [StepEntry(s.request.req_id, s.tokens, (len(s.tokens) - 1,) if s.samples else ())
+                               for s in batch]
+                    logits = self.runner.step(entries)
+                    sampling = [s for s in batch if s.samples]
+                    tokens: List[Optional[int]] = [None] * len(batch)
+                    if sampling:
+                        hist = [penalty_window(s.request.params, s.request.prompt, s.request.output)
+                                if s.request.params.edits_logits else () for s in sampling]
+                        picked = self.sampler.sample(logits, [s.request.params for s in sampling],
+                                                     [s.request.draws for s in sampling], hist)
+                        it = iter(picked)
+                        tokens = [next(it) if s.samples else None for s in batch]
+                    dt = time.perf_counter() - t0
+                    n_prefill = sum(len(s.tokens) for s in batch if s.request.in_prefill)
+                    n_decode = sum(1 for s in batch if not s.request.in_prefill)
+                    if n_prefill:
+                        stats.prefill_tokens += n_prefill
+                        stats.prefill_seconds += dt * n_prefill / (n_prefill + n_decode)
+                    if n_decode:
+                        stats.decode_tokens += n_decode
+                        stats.decode_seconds += dt * n_decode / (n_prefill + n_decode)
+                    stats.steps += 1
+                    had = [len(s.request.output) for s in batch]
+                    sched.update(batch, tokens)
+                    for s, n0 in zip(batch, had):
+                        if len(s.request.output) > n0:
+                            yield GenerateChunk("token", s.request.req_id[1], token_id=s.request.output[-1])
+                elif sched.has_work() and len(sched.finished) == reported:
+                    raise RuntimeError("scheduler has work but nothing can run")
+                for r in sched.finished[reported:]:
+                    yield GenerateChunk("stop", r.req_id[1], finish_reason=r.finish_reason,
+                                        truncated_by_max_tokens=r.finish_reason == "length")
+                reported = len(sched.finished)
+            for r in sched.finished[reported:]:            # what the last scheduling pass ended without a step
+                yield GenerateChunk("stop", r.req_id[1], finish_reason=r.finish_reason,
+                                    truncated_by_max_tokens=r.finish_reason == "length")
         finally:
-            for r in list(sched.running):                  # an error mid-way: give everything back
+            self._sched = None
+            for r in list(sched.running):                  # an error or an early close: give everything back
                 if self.cache.has_request(r.req_id):
                     self.cache.free_request(r.req_id)
-        self.last_stats = stats
-        return [GenerationResult(r.output, r.finish_reason or "abort", len(r.prompt)) for r in reqs]
+
+    def generate(self, prompts: Sequence[Sequence[int]], params: Union[SamplingParams, Sequence[SamplingParams], None] = None,
+                 *, max_new_tokens: Optional[int] = None, temperature: Optional[float] = None,
+                 seeds: Optional[Sequence[int]] = None, stop_token_ids: Sequence[int] = ()) -> List[GenerationResult]:
+        """Generate for a list of prompts (token ids) under continuous batching; the chunks of
+        ``generate_chunks`` gathered per prompt."""
+        out = [GenerationResult([], "abort", len(p)) for p in prompts]
+        for c in self.generate_chunks(prompts, params, max_new_tokens=max_new_tokens, temperature=temperature,
+                                      seeds=seeds, stop_token_ids=stop_token_ids):
+            if c.kind == "token":
+                out[c.index].token_ids.append(c.token_id)
+            elif c.kind == "stop":
+                out[c.index].finish_reason = c.finish_reason
+        return out

@@ -65,6 +65,50 @@ def test_stop_tokens_and_tiny_pool(tmp_path):
     assert all(g.pool.total_allocs > g.pool.num_pages for g in eng.cache.groups)
 
 
+def test_chunks_stream_in_order_and_cancelling_gives_pages_back(tmp_path):
+    """The typed chunks of a generation: per prompt one usage chunk first, its tokens in order,
+    one stop chunk last; the tokens are those of generate().  A prompt cancelled half-way ends
+    with "abort" while the others go on unchanged, a prompt too long for the pool ends at once,
+    and closing the generator early leaves no page held."""
+    d = make_model_dir(tmp_path, "A", std=0.1)
+    prompts = [H.random_tokens(n, 256, 90 + n) for n in (7, 21, 33)]
+    eng = H.make_engine(d, "float32", kv_tokens=256, max_num_seqs=3, max_tokens_per_step=16)
+    want = [r.token_ids for r in eng.generate(prompts, max_new_tokens=10)]
+    seen = {i: [] for i in range(3)}
+    for c in eng.generate_chunks(prompts, max_new_tokens=10):
+        seen[c.index].append(c)
+        if c.kind == "usage":
+            assert eng.queue_depth == 3 and eng.active_requests == 0     # nothing is admitted before the first step
+        elif sum(len(v) for v in seen.values()) == 4:                    # the first token: the others still run
+            assert c.kind == "token" and eng.active_requests >= 2
+    for i, p in enumerate(prompts):
+        kinds = [c.kind for c in seen[i]]
+        assert kinds == ["usage"] + ["token"] * 10 + ["stop"]
+        assert seen[i][0].prompt_tokens == len(p) and [c.token_id for c in seen[i][1:-1]] == want[i]
+        assert seen[i][-1].finish_reason == "length" and seen[i][-1].truncated_by_max_tokens
+    assert eng.active_requests == 0 and eng.queue_depth == 0
+    # prompt 1 is cancelled once it has 4 tokens; a 300-token prompt can never fit into 256
+    got = {i: [] for i in range(4)}
+    reasons = {}
+    for c in eng.generate_chunks(prompts + [H.random_tokens(300, 256, 1)], max_new_tokens=10,
+                                 should_cancel=lambda i: i == 1 and len(got[1]) >= 4):
+        if c.kind == "token":
+            got[c.index].append(c.token_id)
+        elif c.kind == "stop":
+            reasons[c.index] = c.finish_reason
+    assert reasons == {0: "length", 1: "abort", 2: "length", 3: "too_long"}
+    assert got[0] == want[0] and got[2] == want[2] and got[1] == want[1][:4] and got[3] == []
+    # closed early
+    gen = eng.generate_chunks(prompts, max_new_tokens=10)
+    for c in gen:
+        if c.kind == "token":
+            break
+    gen.close()
+    eng.cache.check_invariants()
+    assert all(g.pool.num_free == g.pool.num_pages for g in eng.cache.groups) and not eng.cache.requests
+    assert [r.token_ids for r in eng.generate(prompts, max_new_tokens=10)] == want
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding(tmp_path, dtype):
     """Hundreds of single-token steps: windows slide over many pages that are released and reused."""
