@@ -8,6 +8,7 @@ prompts are lists of token ids and results are lists of token ids.
 """
 from __future__ import annotations
 
+import sys
 import time
 from dataclasses import dataclass, field
 from typing import Callable, Dict, Hashable, Iterator, List, Optional, Sequence, Union
@@ -99,7 +100,7 @@ class Engine:
         t0 = time.time()
         load_model_weights(self.model, source)
         if verbose:
-            print(f"[engine] weights ready in {time.time() - t0:.1f}s", flush=True)
+            print(f"[engine] weights ready in {time.time() - t0:.1f}s", file=sys.stderr, flush=True)
         limit = getattr(self.config, "max_position_embeddings", 0) or 0
         self.max_model_len = int(max_model_len or limit or 4096)
         if limit and self.max_model_len > limit:

@@ -10,6 +10,7 @@ in the same way, src/SharpInference.Engine/CudaForwardPass.cs:4894, 4985-4986).
 """
 from __future__ import annotations
 
+import sys
 from dataclasses import dataclass, field
 from typing import Hashable, List, Optional, Sequence
 
@@ -188,7 +189,7 @@ class ModelRunner:
                 graph = _DecodeGraph(self, pieces, info)
             except Exception as e:  # noqa: BLE001 - capture is an optimisation: report once, go on eagerly
                 print(f"[sharpi] decode graph for batch {n} not captured ({type(e).__name__}: {e}); running eagerly",
-                      flush=True)
+                      file=sys.stderr, flush=True)
                 self._graphs[n] = False
                 return None
             self._graphs[n] = graph
