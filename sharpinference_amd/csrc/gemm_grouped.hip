@@ -4,16 +4,18 @@
 //
 // The product is bound by reading the experts' weights, so a block takes ALL rows of its expert
 // that fit one tile (192, about one and a half times the mean load of 2,048 tokens over 16
-// experts) against 128 weight rows: a typical expert's weights are then read once.  Tiles are
+// experts) against 256 weight rows: a typical expert's weights are then read once.  Tiles are
 // listed on the device by the routing kernel (tile_expert, tile_row0, n_tiles); the host never
 // learns the routing.  The tile's work is compiled three times, for 64, 128 and 192 rows, and a
 // block takes the smallest that holds its rows: no branch inside a K stage, nothing multiplied or
 // staged for 64-row quarters that hold no row.
-//  * Each of the 4 waves owns 32 weight rows (2 MFMA tiles) and reads them straight from global
+//  * Each of the 8 waves owns 32 weight rows (2 MFMA tiles) and reads them straight from global
 //    memory into registers, a ring of 64-wide K stages ahead: a weight element is used by one wave only.
 //  * The x rows (gathered through a_rows) are shared by the waves and staged through LDS, 64
 //    columns of K at a time, double-buffered and fetched two stages ahead; the 16-byte chunks of
-//    a row are swizzled so that reads and stores are free of bank conflicts.
+//    a row are swizzled so that reads and stores are free of bank conflicts.  Eight waves rather
+//    than four share a staged tile (measured: 8 % faster): the x rows come from L2 once per 256
+//    weight rows instead of once per 128, and a lane stages half as many of them.
 //  * W is the A operand (rows = n), x the B operand: a lane ends up with 4 consecutive n of one
 //    row, stored as one 8-byte write.  Each output is one chain over k in ascending order, so a
 //    row's result does not depend on which other rows share its tile.
@@ -41,7 +43,7 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 constexpr int GM = SHARPI_GM;  // rows per tile (the routing kernel lists tiles of this height)
 constexpr int GMT = GM / 16;  // 16-row groups per tile
 #ifndef SHARPI_GW
-#define SHARPI_GW 4
+#define SHARPI_GW 8
 #endif
 #ifndef SHARPI_GNT
 #define SHARPI_GNT 2

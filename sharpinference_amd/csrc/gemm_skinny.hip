@@ -1,5 +1,6 @@
 // Weight-streaming matrix product for few rows (decode): out[M, N] = x[M, K] * W[N, K]^T, bfloat16
-// inputs, float accumulation on the matrix cores (v_mfma_f32_16x16x32_bf16), M <= 64.
+// inputs, float accumulation on the matrix cores (v_mfma_f32_16x16x32_bf16); M <= 64, or any number
+// of rows in the grouped form as long as an expert has few.
 //
 // The weights are read from HBM exactly once; everything else is arranged around that.
 //  * A block owns R tiles of 16 weight rows; its NW waves split K into contiguous slices.  Per
@@ -11,8 +12,9 @@
 //    the weight's shape alone and the x rows never mix, so a row's result does not depend on
 //    the batch around it.
 //  * Grouped form (routed experts): block (tile, expert e) handles rows
-//    [offsets[e], offsets[e + 1]) of the expert-sorted row list with W[e], sixteen at a time;
-//    x rows are gathered through a_rows.  Experts without rows return at once.
+//    [offsets[e], offsets[e + 1]) of the expert-sorted row list with W[e], MB blocks of sixteen at
+//    a time (an expert with more is walked in turns and its weights read again for each); x rows
+//    are gathered through a_rows.  Experts without rows return at once.
 //
 //  * Packed weights (PACKED): the matrix is stored tile by tile instead of row by row, the 4 KB
 //    of a (16-row tile, 128-wide K unit) contiguous and in the order the lanes want them, and
@@ -23,7 +25,7 @@
 //    rounds both to bfloat16 (what a separate activation kernel would have read) and stores
 //    silu(s g) * (s u), s the row's score: out is [M, N/2] and the gate|up rows never go to memory.
 //
-// Limits (the caller falls back to other kernels otherwise): K % 128 == 0, N % 4 == 0, M <= 64.
+// Limits (the caller falls back to other kernels otherwise): K % 128 == 0, N % 4 == 0, M <= 64 (plain form).
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;

@@ -1,10 +1,11 @@
 // MoE routing on the device: router logits, gate, top-k, and the expert-sorted row list.
 //
-// router_topk: one block per token, or per four tokens when there are many. logits[e] = Wr[e, :] . x[t, :] in float (each wave owns
-// experts e = wave, wave + nwaves, ...; lanes stride over the hidden width, so the order of
-// the additions depends on the width only).  gate 0 = sigmoid over every expert, gate 1 =
-// softmax over every expert.  The k picks scan ascending with a strict >, so the lowest index
-// wins a tie; the weight of a pick is its gate value; renorm divides the k weights by their sum.
+// router_topk: one block per token, or per four tokens when there are many.
+// logits[e] = Wr[e, :] . x[t, :] in float (each wave owns experts e = wave, wave + nwaves, ...;
+// lanes stride over the hidden width, so the order of the additions depends on the width only).
+// gate 0 = sigmoid over every expert, gate 1 = softmax over every expert.  The k picks scan
+// ascending with a strict >, so the lowest index wins a tie; the weight of a pick is its gate
+// value; renorm divides the k weights by their sum.
 //
 // moe_permute: one block. Counts rows per expert, prefix-sums them into offsets[E + 1] and
 // writes, in expert order, the token and weight of every (token, pick) pair plus the inverse
