@@ -19,7 +19,12 @@
 //  * W is the A operand (rows = n), x the B operand: a lane ends up with 4 consecutive n of one
 //    row, stored as one 8-byte write.  Each output is one chain over k in ascending order, so a
 //    row's result does not depend on which other rows share its tile.
-// Limits: K % 64 == 0, N % 4 == 0.
+//  * SwiGLU form (ACT): W holds gate rows [0, N/2) and up rows [N/2, N) of every expert; a wave's two
+//    tiles are the gate tile and the up tile of the same 16 columns, so a lane ends up with both
+//    products of its outputs, rounds them to bfloat16 (what a separate activation kernel would have
+//    read) and stores silu(s g) * (s u), s the row's score: out is [rows, N/2] and the gate|up
+//    rows never go to memory.
+// Limits: K % 64 == 0, N % 4 == 0 (N % 32 == 0 in the SwiGLU form).
 #include <type_traits>
 
 #include "common.h"
@@ -71,10 +76,13 @@ static_assert(GK == 64, "the swizzle assumes rows of eight 16-byte chunks");
 __device__ __forceinline__ int xs_col(int row, int col) { return col ^ (((row >> 1) & 7) << 3); }
 
 // The work of one tile of NQ * 64 rows (the block's rows, rounded up) against GN weight rows.
-template <typename TO, int NQ, bool PACKED>
+template <typename TO, int NQ, bool PACKED, bool ACT>
 __device__ __forceinline__ void grouped_tile(const bf16_t* __restrict__ x, const bf16_t* __restrict__ We,
                                              TO* __restrict__ out, int N, int K, const int* __restrict__ a_rows,
-                                             int row0, int row_end, int n_base, bf16_t (*xs)[GM][GPAD]) {
+                                             const float* __restrict__ act_scale, int row0, int row_end, int n_base,
+                                             bf16_t (*xs)[GM][GPAD]) {
+  static_assert(!ACT || NT == 2, "the SwiGLU form pairs one gate tile with one up tile");
+  const int n_out = ACT ? N / 2 : N;            // output columns
   constexpr int MT = NQ * 4;                    // 16-row groups
   constexpr int PASS = NQ * 64 / GROWS;         // staging passes
   const int lane = threadIdx.x & (kWave - 1);
@@ -90,13 +98,16 @@ __device__ __forceinline__ void grouped_tile(const bf16_t* __restrict__ x, const
   uint32_t woff[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
+    // ACT: tile 0 is the gate tile of the wave's 16 columns, tile 1 the up tile of the same columns
     if constexpr (PACKED) {
-      int n = n_base + t * 16;
-      if (n >= N) n = N - 16;  // loaded, never stored
+      int n = ACT ? n_base : n_base + t * 16;
+      if (n >= n_out) n = n_out - 16;  // loaded, never stored
+      if (ACT && t == 1) n += n_out;
       woff[t] = (uint32_t)n * (uint32_t)K + lane * 8;
     } else {
-      int n = n_base + t * 16 + r;
-      if (n >= N) n = N - 1;  // loaded, never stored
+      int n = (ACT ? n_base : n_base + t * 16) + r;
+      if (n >= n_out) n = n_out - 1;  // loaded, never stored
+      if (ACT && t == 1) n += n_out;
       woff[t] = (uint32_t)n * (uint32_t)K + g * 8;
     }
   }
@@ -208,33 +219,50 @@ __device__ __forceinline__ void grouped_tile(const bf16_t* __restrict__ x, const
   for (; c < chunks; c += kUnroll) stage_group(c, std::false_type{});                      // the last stages check each fetch
 
   // lane holds out[row0 + mb*16 + r][n_base + t*16 + 4g + 0..3]
+  auto store = [&](TO* dst, const f32x4& v) {
+    if constexpr (sizeof(TO) == 4) {
+      *reinterpret_cast<f32x4*>(dst) = v;
+    } else {
+      uint2 packed;
+      packed.x = (uint32_t)f32_to_bf16(v[0]).bits | ((uint32_t)f32_to_bf16(v[1]).bits << 16);
+      packed.y = (uint32_t)f32_to_bf16(v[2]).bits | ((uint32_t)f32_to_bf16(v[3]).bits << 16);
+      *reinterpret_cast<uint2*>(dst) = packed;
+    }
+  };
 #pragma unroll
   for (int mb = 0; mb < MT; ++mb) {
     const int row = row0 + mb * 16 + r;
     if (row >= row_end) continue;
+    if constexpr (ACT) {
+      const int n = n_base + 4 * g;
+      if (n >= n_out) continue;
+      const float sc = act_scale ? act_scale[row] : 1.0f;
+      f32x4 o;
 #pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      const int n = n_base + t * 16 + 4 * g;
-      if (n >= N) continue;
-      TO* dst = out + (size_t)row * N + n;
-      if constexpr (sizeof(TO) == 4) {
-        *reinterpret_cast<f32x4*>(dst) = acc[t][mb];
-      } else {
-        uint2 packed;
-        packed.x = (uint32_t)f32_to_bf16(acc[t][mb][0]).bits | ((uint32_t)f32_to_bf16(acc[t][mb][1]).bits << 16);
-        packed.y = (uint32_t)f32_to_bf16(acc[t][mb][2]).bits | ((uint32_t)f32_to_bf16(acc[t][mb][3]).bits << 16);
-        *reinterpret_cast<uint2*>(dst) = packed;
+      for (int i = 0; i < 4; ++i)
+        o[i] = swiglu_f32(bf16_to_f32(f32_to_bf16(acc[0][mb][i])), bf16_to_f32(f32_to_bf16(acc[1][mb][i])), sc,
+                          act_scale != nullptr);
+      store(out + (size_t)row * n_out + n, o);
+    } else {
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        const int n = n_base + t * 16 + 4 * g;
+        if (n >= N) continue;
+        store(out + (size_t)row * N + n, acc[t][mb]);
       }
     }
   }
 }
 
-template <typename TO, bool PACKED>
+template <typename TO, bool PACKED, bool ACT>
 __global__ __launch_bounds__(GW* kWave, 2) void grouped_gemm_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ W, TO* __restrict__ out, int N, int K,
-    const int* __restrict__ a_rows, const int* __restrict__ group_offsets, const int* __restrict__ tile_expert,
-    const int* __restrict__ tile_row0, const int* __restrict__ n_tiles, int nb_per_unit) {
+    const int* __restrict__ a_rows, const float* __restrict__ act_scale, const int* __restrict__ group_offsets,
+    const int* __restrict__ tile_expert, const int* __restrict__ tile_row0, const int* __restrict__ n_tiles,
+    int nb_per_unit) {
   __shared__ __attribute__((aligned(16))) bf16_t xs[2][GM][GPAD];
+  constexpr int kCols = ACT ? GN / 2 : GN;   // output columns of a block
+  const int n_out = ACT ? N / 2 : N;
   // Workgroups go to the 8 XCDs round-robin by their linear id, and each XCD has an L2 of its
   // own.  All column blocks of one (tile, half of the columns) unit are therefore given ids that
   // are equal modulo 8: the unit's x rows are fetched into one L2 and stay there.
@@ -243,26 +271,35 @@ __global__ __launch_bounds__(GW* kWave, 2) void grouped_gemm_kernel(
   const int unit = (slot / nb_per_unit) * kXcds + xcd;
   const int tile = unit / kHalves;
   const int nblock = (unit % kHalves) * nb_per_unit + slot % nb_per_unit;
-  if (tile >= n_tiles[0] || nblock * GN >= N) return;
+  if (tile >= n_tiles[0] || nblock * kCols >= n_out) return;
   const int e = tile_expert[tile];
   const int row0 = tile_row0[tile];
   const int row_end = min(group_offsets[e + 1], row0 + GM);   // the tile's rows end here; later ones are another tile's
   const int n_rows = row_end - row0;
   if (n_rows <= 0) return;
-  const int n_base = nblock * GN + (threadIdx.x >> 6) * 16 * NT;
+  const int n_base = nblock * kCols + (threadIdx.x >> 6) * (ACT ? 16 : 16 * NT);
   const bf16_t* We = W + (size_t)e * N * K;
   static_assert(GM % 64 == 0 && GM >= 128 && GM <= 256, "tile heights are compiled in steps of 64 rows, up to GM");
   if (n_rows <= 64) {
-    grouped_tile<TO, 1, PACKED>(x, We, out, N, K, a_rows, row0, row_end, n_base, xs);
+    grouped_tile<TO, 1, PACKED, ACT>(x, We, out, N, K, a_rows, act_scale, row0, row_end, n_base, xs);
   } else if (n_rows <= 128) {
-    grouped_tile<TO, 2, PACKED>(x, We, out, N, K, a_rows, row0, row_end, n_base, xs);
+    grouped_tile<TO, 2, PACKED, ACT>(x, We, out, N, K, a_rows, act_scale, row0, row_end, n_base, xs);
   } else if constexpr (GM >= 192) {
     if (GM == 192 || n_rows <= 192) {
-      grouped_tile<TO, 3, PACKED>(x, We, out, N, K, a_rows, row0, row_end, n_base, xs);
+      grouped_tile<TO, 3, PACKED, ACT>(x, We, out, N, K, a_rows, act_scale, row0, row_end, n_base, xs);
     } else if constexpr (GM >= 256) {
-      grouped_tile<TO, 4, PACKED>(x, We, out, N, K, a_rows, row0, row_end, n_base, xs);
+      grouped_tile<TO, 4, PACKED, ACT>(x, We, out, N, K, a_rows, act_scale, row0, row_end, n_base, xs);
     }
   }
+}
+
+static bool grouped_args_ok(int x_rows, int N, int K, int max_tiles, int packed, const int* group_offsets,
+                            const int* tile_expert, const int* tile_row0, const int* n_tiles) {
+  if (N <= 0 || (N & 3) || K <= 0 || K % GK != 0 || max_tiles <= 0) return false;
+  if (packed && ((N & 15) || (K & 127))) return false;
+  if (!group_offsets || !tile_expert || !tile_row0 || !n_tiles) return false;
+  // the kernel addresses x and one expert's weights with 32-bit element offsets
+  return (long long)N * K <= 0x7fffffffLL && x_rows > 0 && (long long)x_rows * K <= 0x7fffffffLL;
 }
 
 // x [x_rows, K] bf16 (rows gathered through a_rows if given), W [E, N, K] bf16, out [n_rows, N];
@@ -274,18 +311,14 @@ SHARPI_EXPORT int sharpi_gemm_grouped(const void* x, int x_rows, const void* W, 
                                       const int* tile_row0, const int* n_tiles, int max_tiles, int packed,
                                       hipStream_t stream) {
   if (n_rows <= 0) return SHARPI_OK;
-  if (N <= 0 || (N & 3) || K <= 0 || K % GK != 0 || max_tiles <= 0) return SHARPI_ERR_ARG;
-  if (packed && ((N & 15) || (K & 127))) return SHARPI_ERR_ARG;
-  if (!group_offsets || !tile_expert || !tile_row0 || !n_tiles) return SHARPI_ERR_ARG;
-  // the kernel addresses x and one expert's weights with 32-bit element offsets
-  if ((long long)N * K > 0x7fffffffLL || x_rows <= 0 || (long long)x_rows * K > 0x7fffffffLL) return SHARPI_ERR_ARG;
+  if (!grouped_args_ok(x_rows, N, K, max_tiles, packed, group_offsets, tile_expert, tile_row0, n_tiles)) return SHARPI_ERR_ARG;
   const int nb_per_unit = ceil_div(ceil_div(N, GN), kHalves);
   const int units = ceil_div(max_tiles * kHalves, kXcds) * kXcds;
   dim3 grid(units * nb_per_unit), block(GW * kWave);
-#define GG_LAUNCH(TOV, PK)                                                                                        \
-  grouped_gemm_kernel<TOV, PK><<<grid, block, 0, stream>>>((const bf16_t*)x, (const bf16_t*)W, (TOV*)out, N, K,    \
-                                                          a_rows, group_offsets, tile_expert, tile_row0, n_tiles,  \
-                                                          nb_per_unit)
+#define GG_LAUNCH(TOV, PK)                                                                                          \
+  grouped_gemm_kernel<TOV, PK, false><<<grid, block, 0, stream>>>((const bf16_t*)x, (const bf16_t*)W, (TOV*)out, N, \
+                                                                 K, a_rows, nullptr, group_offsets, tile_expert,    \
+                                                                 tile_row0, n_tiles, nb_per_unit)
   if (out_dtype == DT_BF16) {
     if (packed) GG_LAUNCH(bf16_t, true); else GG_LAUNCH(bf16_t, false);
   } else if (out_dtype == DT_F32) {
@@ -294,6 +327,31 @@ SHARPI_EXPORT int sharpi_gemm_grouped(const void* x, int x_rows, const void* W, 
     return SHARPI_ERR_ARG;
   }
 #undef GG_LAUNCH
+  SHARPI_CHECK_LAUNCH();
+  return SHARPI_OK;
+}
+
+// The grouped product with SwiGLU in its epilogue: W [E, N, K] holds gate rows [0, N/2) then up rows
+// of every expert; out [n_rows, N/2] bf16 = silu(s g) * (s u) with g, u the two products rounded
+// to bfloat16 and s = act_scale[row] (null: 1).  N % 32 == 0; the rest as above.
+SHARPI_EXPORT int sharpi_gemm_grouped_swiglu(const void* x, int x_rows, const void* W, void* out, int n_rows, int N,
+                                             int K, const int* a_rows, const int* group_offsets,
+                                             const int* tile_expert, const int* tile_row0, const int* n_tiles,
+                                             int max_tiles, const float* act_scale, int packed, hipStream_t stream) {
+  if (n_rows <= 0) return SHARPI_OK;
+  if ((N & 31) || !grouped_args_ok(x_rows, N, K, max_tiles, packed, group_offsets, tile_expert, tile_row0, n_tiles))
+    return SHARPI_ERR_ARG;
+  const int nb_per_unit = ceil_div(ceil_div(N / 2, GN / 2), kHalves);
+  const int units = ceil_div(max_tiles * kHalves, kXcds) * kXcds;
+  dim3 grid(units * nb_per_unit), block(GW * kWave);
+  if (packed)
+    grouped_gemm_kernel<bf16_t, true, true><<<grid, block, 0, stream>>>(
+        (const bf16_t*)x, (const bf16_t*)W, (bf16_t*)out, N, K, a_rows, act_scale, group_offsets, tile_expert,
+        tile_row0, n_tiles, nb_per_unit);
+  else
+    grouped_gemm_kernel<bf16_t, false, true><<<grid, block, 0, stream>>>(
+        (const bf16_t*)x, (const bf16_t*)W, (bf16_t*)out, N, K, a_rows, act_scale, group_offsets, tile_expert,
+        tile_row0, n_tiles, nb_per_unit);
   SHARPI_CHECK_LAUNCH();
   return SHARPI_OK;
 }

@@ -598,6 +598,27 @@ def gemm_grouped(x: torch.Tensor, w, rt: Routing, gather: bool, out_dtype: torch
     return out
 
 
+def gemm_grouped_swiglu(x: torch.Tensor, w, rt: Routing, scale: Optional[torch.Tensor]) -> torch.Tensor:
+    """Per expert, silu(s g) * (s u) with (g | u) = x @ w[e]^T rounded to bfloat16, for many rows: the
+    grouped product with the activation in its epilogue.  x rows are read through the routing's
+    token list; w [E, 2I, K] holds gate rows then up rows.  Returns [n_rows, I] bfloat16."""
+    w, packed = _unwrap(w)
+    _dev(x, w, scale)
+    _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_grouped_swiglu: bfloat16 operands only")
+    _need(w.dim() == 3 and w.shape[0] >= rt.n_experts and rt.n_groups == rt.n_experts and x.dim() == 2
+          and x.shape[1] == w.shape[2], f"gemm_grouped_swiglu: x {tuple(x.shape)} vs w {tuple(w.shape)}")
+    E, N, K = w.shape
+    _need(K % 64 == 0 and N % 32 == 0, "gemm_grouped_swiglu: K % 64 == 0 and N % 32 == 0 wanted")
+    _need(x.shape[0] == rt.n_tokens, "gemm_grouped_swiglu: x has the wrong number of rows")
+    if scale is not None:
+        _need(scale.dtype == torch.float32 and scale.shape == (rt.n_rows,), "gemm_grouped_swiglu: scale must be float32 [n_rows]")
+    out = torch.empty(rt.n_rows, N // 2, dtype=torch.bfloat16, device=x.device)
+    _run("sharpi_gemm_grouped_swiglu", _ptr(x), x.shape[0], _ptr(w), _ptr(out), rt.n_rows, N, K, _ptr(rt.sorted_token),
+         _ptr(rt.offsets), _ptr(rt.tile_expert), _ptr(rt.tile_row0), _ptr(rt.n_tiles), rt.max_tiles, _ptr(scale),
+         1 if packed else 0, _stream())
+    return out
+
+
 # ---------------------------------------------------------------------------
 def argmax_rows(logits: torch.Tensor) -> torch.Tensor:
     _dev(logits)
@@ -662,13 +683,16 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, gro
 
 def grouped_swiglu(x: torch.Tensor, w_gate_up, rt: Routing, out_dtype: torch.dtype) -> torch.Tensor:
     """The experts' gate|up products of the routed tokens and their activation,
-    silu(s g) * (s u) with s the pick's weight: [n_rows, I] in expert-sorted order.  A few rows
-    take one kernel; otherwise the product and the activation are two."""
+    silu(s g) * (s u) with s the pick's weight: [n_rows, I] in expert-sorted order.  On the
+    matrix cores the activation is the product's epilogue (the few-rows kernel or the many-rows
+    one); otherwise the product and the activation are two kernels."""
     N, K = w_gate_up.shape[1], w_gate_up.shape[2]
-    if (x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16 and out_dtype == torch.bfloat16
-            and rt.n_tokens <= SKINNY_MAX_ROWS and K % 128 == 0 and N % (32 if isinstance(w_gate_up, PackedWeight) else 8) == 0):
-        return gemm_skinny_swiglu(x, w_gate_up, rt.offsets, rt.sorted_token, rt.n_rows, rt.sorted_w,
-                                  group_rows=rt.n_tokens)
+    if x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16 and out_dtype == torch.bfloat16 and K % 128 == 0:
+        if rt.n_tokens <= SKINNY_MAX_ROWS and N % (32 if isinstance(w_gate_up, PackedWeight) else 8) == 0:
+            return gemm_skinny_swiglu(x, w_gate_up, rt.offsets, rt.sorted_token, rt.n_rows, rt.sorted_w,
+                                      group_rows=rt.n_tokens)
+        if rt.n_tokens > SKINNY_MAX_ROWS and N % 32 == 0 and rt.n_groups == rt.n_experts:
+            return gemm_grouped_swiglu(x, w_gate_up, rt, rt.sorted_w)
     return silu_mul(grouped_linear(x, w_gate_up, rt, True, out_dtype), rt.sorted_w)
 
 

@@ -356,6 +356,35 @@ def test_gemm_grouped(T, E, k, N, K):
         assert torch.equal(ops.gemm_grouped(x, pw, rt, True, torch.float32).cpu(), got)
 
 
+@pytest.mark.parametrize("T,E,k,I,K", [(300, 4, 1, 128, 256), (700, 16, 2, 272, 128), (65, 3, 1, 16, 384),
+                                       (500, 5, 1, 112, 640), (260, 2, 2, 80, 1216), (430, 3, 1, 8192, 128)])
+def test_gemm_grouped_swiglu_equals_product_then_activation(T, E, k, I, K):
+    """The many-rows product with the activation in its epilogue gives the bits of the two kernels
+    in a row, from weights stored row by row and tile by tile (column blocks that end inside a
+    block of the kernel, experts with no row, with one tile and with several)."""
+    ops = _ops()
+    x = _rand(T, K, dtype=torch.bfloat16, seed=3)
+    w = _rand(E, 2 * I, K, dtype=torch.bfloat16, scale=0.1, seed=4)
+    g = torch.Generator().manual_seed(T)
+    ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32).to(DEV)
+    if E == 4:
+        ids[:] = 2
+    wts = torch.rand(T, k, generator=g).to(DEV)
+    rt = ops.moe_permute(ids, wts, E)
+    for scale in (rt.sorted_w, None):
+        want = ops.silu_mul(ops.gemm_grouped(x, w, rt, True, torch.bfloat16), scale)
+        got = ops.gemm_grouped_swiglu(x, w, rt, scale)
+        assert got.shape == (T * k, I) and torch.equal(got, want)
+        if ops.can_pack(w):
+            assert torch.equal(ops.gemm_grouped_swiglu(x, ops.pack_weight(w, keep_rows=False), rt, scale), want)
+    # the same numbers as the float product followed by the activation, to bfloat16's rounding
+    gu = ops.gemm_grouped(x, w, rt, True, torch.float32).cpu()
+    s = rt.sorted_w.cpu()[:, None]
+    ga, up = (gu[:, :I] * s), (gu[:, I:] * s)
+    ref = ga / (1 + torch.exp(-ga)) * up
+    assert float((ops.gemm_grouped_swiglu(x, w, rt, rt.sorted_w).float().cpu() - ref).abs().max()) <= 3e-2 * float(ref.abs().max() + 1e-6)
+
+
 @pytest.mark.parametrize("nh,nkv,hd", [(8, 2, 64), (5, 5, 32), (40, 8, 128), (3, 1, 96)])
 @pytest.mark.parametrize("kind,window", [(0, 0), (1, 24), (1, 100), (2, 50)])
 @pytest.mark.parametrize("ps", [16, 32])
