@@ -22,6 +22,7 @@ from ..parts.base import GroupView, LayerCache, StepContext
 
 
 MAX_GRAPH_BATCH = 16   # decode steps of up to this many requests are replayed from a HIP graph (beyond, launches no longer bound the step and the fixed maxima cost more than they save)
+GRAPH_CONTEXT_MIN = 4096   # a graph is captured for a bound on the contexts of its requests: this, or 4, 16, 64 ... times it
 TILE = 128   # tokens per attention tile of multi-token entries (ops.PREFILL_TILE_TOKENS)
 
 
@@ -174,25 +175,34 @@ class ModelRunner:
         n = len(entries)
         if not self.decode_graphs or n > MAX_GRAPH_BATCH:
             return None
+        longest = 0
         for e in entries:
             if len(e.tokens) != 1 or len(e.want) != 1 or int(e.want[0]) != 0:
                 return None
-            if self.cache.length(e.req_id) + 1 > self.max_context:
-                return None
-        graph = self._graphs.get(n)
+            longest = max(longest, self.cache.length(e.req_id) + 1)
+        if longest > self.max_context:
+            return None
+        # The graph's shapes are fixed at a bound on the contexts (block table width, runs of the
+        # decode kernel); a bound far above the contexts costs time, so bounds grow in steps of 4
+        bound = GRAPH_CONTEXT_MIN
+        while bound < longest:
+            bound *= 4
+        bound = min(bound, self.max_context)
+        key = (n, bound)
+        graph = self._graphs.get(key)
         if graph is False:
             return None
-        static_blocks = (self.max_context + self.cache.page_size - 1) // self.cache.page_size
+        static_blocks = (bound + self.cache.page_size - 1) // self.cache.page_size
         pieces, info = self._host_arrays(entries, static_blocks=static_blocks)
         if graph is None:
             try:
-                graph = _DecodeGraph(self, pieces, info)
+                graph = _DecodeGraph(self, pieces, info, bound)
             except Exception as e:  # noqa: BLE001 - capture is an optimisation: report once, go on eagerly
-                print(f"[sharpi] decode graph for batch {n} not captured ({type(e).__name__}: {e}); running eagerly",
-                      file=sys.stderr, flush=True)
-                self._graphs[n] = False
+                print(f"[sharpi] decode graph for batch {n}, contexts to {bound} not captured ({type(e).__name__}: {e}); "
+                      "running eagerly", file=sys.stderr, flush=True)
+                self._graphs[key] = False
                 return None
-            self._graphs[n] = graph
+            self._graphs[key] = graph
         self.graph_replays += 1
         return graph.replay(pieces)
 
@@ -231,10 +241,10 @@ class _DecodeGraph:
 
     The index arrays of a step are written into a pinned host buffer, copied into the device
     buffer the graph was captured over, and the graph is replayed; shapes that vary from step to
-    step (block table width, context bound of the decode kernel) are fixed at their maxima.
+    step (block table width, context bound of the decode kernel) are fixed at ``max_context``.
     The logits tensor belongs to the graph: the caller gets a copy."""
 
-    def __init__(self, runner: ModelRunner, pieces, info: dict):
+    def __init__(self, runner: ModelRunner, pieces, info: dict, max_context: int):
         self.runner = runner
         self.sizes = [p.size for p in pieces]
         total = sum(self.sizes)
@@ -242,7 +252,7 @@ class _DecodeGraph:
         self.host_np = self.host.numpy()
         self.dev = torch.empty(total, dtype=torch.int32, device=runner.device)
         self.copied = torch.cuda.Event()
-        info = dict(info, max_context=runner.max_context)
+        info = dict(info, max_context=max_context)
         # capture over harmless contents: nothing is stored (slots -1) and no key is visible (tables -1)
         null = [np.zeros_like(p) for p in pieces]
         n = info["n"]

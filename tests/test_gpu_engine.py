@@ -139,9 +139,38 @@ def test_decode_graph_replays_equal_eager_steps(model_dir, dtype):
         out[graphs] = H.replay(eng, steps)
         if graphs:
             graphs_made = eng.runner._graphs
-            assert sorted(graphs_made) == [1, 2, 3] and all(g is not False for g in graphs_made.values()), \
+            assert sorted(n for n, _ in graphs_made) == [1, 2, 3] and all(g is not False for g in graphs_made.values()), \
                 "decode steps of batch 1, 2 and 3 should each have captured a graph"
             assert eng.runner.graph_replays == 12
+    for r in toks:
+        assert torch.equal(out[True][r], out[False][r]), r
+
+
+def test_decode_graphs_follow_the_context(tmp_path):
+    """A graph's shapes are fixed at a bound on its requests' contexts, and bounds grow in steps
+    of four: a request that decodes across a bound moves on to the next graph, a short one beside
+    it is carried along, and every step gives the bits of the same step launched kernel by kernel."""
+    from sharpinference_amd.engine import runner as R
+
+    d = make_model_dir(tmp_path, "D", std=0.06, max_position_embeddings=20000)
+    first = R.GRAPH_CONTEXT_MIN
+    toks = {"long": H.random_tokens(first + 8, 500, 1), "short": H.random_tokens(40, 500, 2)}
+    steps = [{"entries": [{"id": "long", "tokens": toks["long"][:first - 6], "want": [first - 7]}], "end": []},
+             {"entries": [{"id": "short", "tokens": toks["short"][:30], "want": [29]}], "end": []}]
+    for i in range(10):     # contexts first - 5 ... first + 4: the bound is crossed half-way
+        steps.append({"entries": [{"id": "long", "tokens": [toks["long"][first - 6 + i]], "want": [0]},
+                                  {"id": "short", "tokens": [toks["short"][30 + i]], "want": [0]}], "end": []})
+    steps[-1]["end"] = ["long"]
+    steps += [{"entries": [{"id": "short", "tokens": [toks["short"][40 - 1]], "want": [0]}], "end": ["short"]}]
+    for i, st in enumerate(steps):
+        st["step"] = i
+    out = {}
+    for graphs in (True, False):
+        eng = H.make_engine(d, "bfloat16", kv_tokens=first + 128, max_num_seqs=2, decode_graphs=graphs)
+        out[graphs] = H.replay(eng, steps)
+        if graphs:
+            assert sorted(eng.runner._graphs) == [(1, first), (2, first), (2, 4 * first)]
+            assert eng.runner.graph_replays == 11
     for r in toks:
         assert torch.equal(out[True][r], out[False][r]), r
 
