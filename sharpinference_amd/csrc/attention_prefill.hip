@@ -11,9 +11,10 @@
 //                                               inside a page), B = P^T
 // and the S^T accumulator of a lane is the B operand of the second product once exponentiated
 // and split into a bfloat16 pair hi + lo.  In LDS the value columns are permuted so that the
-// eight keys a lane needs (4 of each 16-key block) sit side by side; the 16-byte chunks of a row are
-// swizzled so that reads are free of bank conflicts (see the layouts below).  Softmax state (a reference maximum and
-// the sum per query) is float, kept in base-2 units (scores times log2 e, the hardware's exp2).
+// eight keys a lane needs (4 of each 16-key block) sit side by side; rows and their 16-byte chunks
+// are placed so that reads and stores are free of bank conflicts (see the layouts below).  Softmax
+// state (a reference maximum and the sum per query) is float, kept in base-2 units (scores times
+// log2 e, the hardware's exp2).
 // The keys of a query are always visited in the same blocks, whatever the portion it arrived in,
 // so its sums do not depend on how the prompt was cut.
 #include "common.h"
@@ -33,14 +34,21 @@ constexpr int kVRow = 32;                            // LDS row of the value til
 // with the bank-conflict counter).  The 16 chunks of 16 bytes that a turn reads must fall into the 16
 // different 16-byte groups of the 256-byte bank space; the chunk index is XORed with row bits so that
 // they do, for rows of 256 bytes (keys, head size 128), 128 bytes (head size 64) and 64 bytes
-// (values: 32 keys).  Other head sizes keep rows padded by 16 bytes (two-way conflicts).
+// (values: 32 keys, see v_row).  Other head sizes keep key rows padded by 16 bytes (two-way conflicts).
 template <int HD> __device__ __forceinline__ constexpr int k_row_elems() { return (HD == 128 || HD == 64) ? HD : HD + 8; }
 template <int HD> __device__ __forceinline__ int k_col(int row, int col) {   // col a multiple of 8 elements
   if constexpr (HD == 128) return col ^ ((row & 15) << 3);
   else if constexpr (HD == 64) return col ^ (((row >> 1) & 7) << 3);
   else return col;
 }
-__device__ __forceinline__ int v_col(int row, int col) { return col ^ (((row >> 2) & 3) << 3); }   // 4 chunks a row
+// values: rows of 64 bytes (32 keys), sixteen to a 1 KB tile.  Within a tile the rows are kept in the
+// order 0 1 8 9 | 2 3 10 11 | 4 5 12 13 | 6 7 14 15 (rows 0..7 in one half of the bank space, 8..15 in
+// the other) and a row's four chunks are XORed with bits 1..2 of the row: an octet of lanes (rows
+// r..r+7 of a tile, one chunk column) then reads eight different 16-byte groups of one half, and
+// the stores (a lane per row and half row) are as free of conflicts (both measured with the counter;
+// XORing the chunk alone left every read and store two-way conflicted).
+__device__ __forceinline__ int v_row(int d) { return (d & ~15) | (d & 1) | (((d >> 3) & 1) << 1) | (((d >> 1) & 3) << 2); }
+__device__ __forceinline__ int v_col(int d, int col) { return col ^ (((d >> 1) & 3) << 3); }   // 4 chunks a row
 constexpr float kLazyMax = 8.0f;                     // how far the row maximum may outgrow its reference
 // the reference before a row has seen a key: finite, so that a masked score (-inf) minus it is
 // -inf and its probability 0, and far below any score, so that the first key moves it
@@ -57,6 +65,8 @@ __global__ __launch_bounds__(kPreWaves* kWave, HD <= 128 ? 2 : 1) void attn_pref
   constexpr int KPAD = k_row_elems<HD>();
   constexpr int PIECES = 4 * HD;                                   // 16-byte pieces of a K (or V) chunk
   constexpr int NST = (PIECES + kPreWaves * kWave - 1) / (kPreWaves * kWave);
+  constexpr int VPAIRS = 2 * HD;                                   // (value row, half of its 16 keys per block) pairs of a chunk
+  constexpr int NSV = (VPAIRS + kPreWaves * kWave - 1) / (kPreWaves * kWave);
   __shared__ __attribute__((aligned(16))) bf16_t Ks[2][32][KPAD];
   __shared__ __attribute__((aligned(16))) bf16_t Vs[2][HD][kVRow];
 
@@ -140,7 +150,7 @@ __global__ __launch_bounds__(kPreWaves* kWave, HD <= 128 ? 2 : 1) void attn_pref
   // keys are masked, its values are finite and meet probabilities of zero).  The compiler counts
   // outstanding loads statically; one load behind a branch and every wait in the loop becomes a
   // wait for all loads, the chunk in flight included.
-  u32x4 kst[NST], vst[NST];
+  u32x4 kst[NST], vst[NSV][2];
   auto fetch = [&](int b) {
     long long kbase[2], vbase[2];
 #pragma unroll
@@ -156,8 +166,15 @@ __global__ __launch_bounds__(kPreWaves* kWave, HD <= 128 ? 2 : 1) void attn_pref
       const int piece = min(tid + i * kPreWaves * kWave, PIECES - 1);
       const int key = piece / (HD / 8), dcol = (piece % (HD / 8)) * 8;     // K: 32 keys x HD
       kst[i] = *reinterpret_cast<const u32x4*>(k_cache + kbase[key >> 4] + (size_t)(key & 15) * HD + dcol);
-      const int d = piece >> 2, blk = (piece >> 1) & 1, half = piece & 1;  // V^T: HD rows x 2 blocks x 2 halves
-      vst[i] = *reinterpret_cast<const u32x4*>(v_cache + vbase[blk] + (size_t)d * page_size + half * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < NSV; ++i) {
+      // V^T: a thread takes keys 8*half .. 8*half+7 of both 16-key blocks for one value row
+      const int pair = min(tid + i * kPreWaves * kWave, VPAIRS - 1);
+      const int d = pair >> 1, half = pair & 1;
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk)
+        vst[i][blk] = *reinterpret_cast<const u32x4*>(v_cache + vbase[blk] + (size_t)d * page_size + half * 8);
     }
   };
   auto stash = [&](int buf) {
@@ -167,11 +184,19 @@ __global__ __launch_bounds__(kPreWaves* kWave, HD <= 128 ? 2 : 1) void attn_pref
       if (piece < PIECES) {
         const int key = piece / (HD / 8), dcol = (piece % (HD / 8)) * 8;
         *reinterpret_cast<u32x4*>(&Ks[buf][key][k_col<HD>(key, dcol)]) = kst[i];
-        // keys 8*half .. 8*half+7 of block blk: groups g = 2*half and 2*half + 1, four keys each;
-        // column of (g, blk) = g*8 + blk*4
-        const int d = piece >> 2, blk = (piece >> 1) & 1, half = piece & 1;
-        *reinterpret_cast<uint2*>(&Vs[buf][d][v_col(d, (2 * half) * 8) + blk * 4]) = uint2{vst[i].x, vst[i].y};
-        *reinterpret_cast<uint2*>(&Vs[buf][d][v_col(d, (2 * half + 1) * 8) + blk * 4]) = uint2{vst[i].z, vst[i].w};
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < NSV; ++i) {
+      const int pair = tid + i * kPreWaves * kWave;
+      if (pair < VPAIRS) {
+        // chunk g of a row holds keys 4g .. 4g+3 of the first block, then of the second: what lane
+        // group g of the second product wants side by side.  The thread's keys are those of the
+        // groups g = 2*half and 2*half + 1.
+        const int d = pair >> 1, half = pair & 1;
+        const u32x4 a = vst[i][0], b = vst[i][1];
+        *reinterpret_cast<u32x4*>(&Vs[buf][v_row(d)][v_col(d, (2 * half) * 8)]) = u32x4{a[0], a[1], b[0], b[1]};
+        *reinterpret_cast<u32x4*>(&Vs[buf][v_row(d)][v_col(d, (2 * half + 1) * 8)]) = u32x4{a[2], a[3], b[2], b[3]};
       }
     }
   };
@@ -278,7 +303,7 @@ __global__ __launch_bounds__(kPreWaves* kWave, HD <= 128 ? 2 : 1) void attn_pref
 #pragma unroll
       for (int d = 0; d < ND; ++d) {
         // lane (d row r, group g): keys 4g..4g+3 of block b, then of block b + 1, side by side in LDS
-        const bf16x8 vf = *reinterpret_cast<const bf16x8*>(&Vs[buf][d * 16 + r][v_col(d * 16 + r, g * 8)]);
+        const bf16x8 vf = *reinterpret_cast<const bf16x8*>(&Vs[buf][v_row(d * 16 + r)][v_col(d * 16 + r, g * 8)]);
 #pragma unroll
         for (int c = 0; c < kQT; ++c) {
           if (rescale[c]) {

@@ -16,6 +16,7 @@ from typing import Callable, Dict, Hashable, Iterator, List, Optional, Sequence,
 import torch
 
 from ..cache.manager import CacheManager
+from ..cache.spec import KVSpec
 from ..config.base import ModelConfig, load_config
 from ..registry import build_model
 from ..sampling.params import SamplingParams
@@ -108,11 +109,16 @@ class Engine:
         self.max_num_seqs = int(max_num_seqs)
         self.max_tokens_per_step = int(max_tokens_per_step)
         self.page_size = int(page_size)
+        specs = self.model.cache_specs()
         if kv_tokens is None:
+            # every request at full length, or what four fifths of the free memory hold if that is less
             kv_tokens = self.max_num_seqs * ((self.max_model_len + page_size - 1) // page_size * page_size)
+            width = torch.empty(0, dtype=self.dtype).element_size()
+            per_token = sum(2 * s.num_kv_heads * s.head_dim * width for s in specs if isinstance(s, KVSpec))
+            free = torch.cuda.mem_get_info(self.device)[0]
+            kv_tokens = max(page_size, min(kv_tokens, int(free * 0.8) // max(1, per_token)))
         num_pages = max(1, (int(kv_tokens) + page_size - 1) // page_size)
-        self.cache = CacheManager(self.model.cache_specs(), page_size, num_pages, self.max_num_seqs, self.dtype,
-                                  self.device)
+        self.cache = CacheManager(specs, page_size, num_pages, self.max_num_seqs, self.dtype, self.device)
         self.runner = ModelRunner(self.model, self.cache, self.dtype, self.device, decode_graphs=decode_graphs,
                                   max_context=self.max_model_len)
         self.sampler = Sampler(self.device)
