@@ -229,6 +229,69 @@ def test_attention_sees_one_key_at_every_edge(kind, window, ps):
             assert (near <= 2e-2) == (st <= j <= p), ("prefill", j, p, near)
 
 
+@pytest.mark.parametrize("kind,window", [(0, 0), (1, 2048), (2, 3000)])
+@pytest.mark.parametrize("ps", [16, 64])
+def test_attention_over_thousands_of_keys(kind, window, ps):
+    """Contexts of thousands of keys: the prefill kernel holds 128 entries of the block table in
+    registers and moves on by 64 as it walks (several times here), the decode kernel splits the keys
+    into many runs and the merge kernel adds them.  One key at a time carries all the weight: the
+    first, one just before and after each place where the held pages run out, one in the middle
+    of nowhere, the last.  Whichever is visible must come back as the value; a key outside the
+    window must not."""
+    ops = _ops()
+    nh, nkv, hd, L = 4, 2, 64, 4300
+    scale = 1.0 / math.sqrt(hd)
+    g = torch.Generator().manual_seed(ps + kind)
+    u = torch.randn(hd, generator=g)
+    u = (u / u.norm() * math.sqrt(hd)).to(torch.bfloat16).float()
+    q1 = (2.0 * u).expand(nh, hd)
+    portion = 130                                   # prefill: a full tile and a partial one at the end
+    p_last = L - 1
+    edges = [0, 1, 64 * ps - 1, 64 * ps, 128 * ps - 1, 128 * ps, 128 * ps + 1, 192 * ps, 3001, p_last - 2048, p_last - 2999,
+             p_last - 3000, L - portion - 1, L - portion, p_last]
+    edges = sorted({e for e in edges if 0 <= e < L})
+    k0 = torch.randn(L, nkv, hd, generator=g) * 0.05
+    v0 = torch.randn(L, nkv, hd, generator=g)
+    n = len(edges)
+    ks, vs = [], []
+    for j in edges:
+        k = k0.clone()
+        k[j] = 4.0 * u                              # score 8 * hd * scale against ~0: all the weight
+        ks.append(k.to(torch.bfloat16).float())
+        vs.append(v0.to(torch.bfloat16).float())
+    bt, kc, vc = _pages_from(ks, vs, ps, torch.bfloat16, 7)
+    bt, kc, vc = bt.to(DEV), kc.to(DEV), vc.to(DEV)
+    # decode: one query per request at the last position
+    q = q1.to(torch.bfloat16).reshape(1, nh * hd).expand(n, nh * hd).contiguous().to(DEV)
+    pos = torch.full((n,), p_last, dtype=torch.int32, device=DEV)
+    ent = torch.arange(n, dtype=torch.int32, device=DEV)
+    dec = ops.attention_decode(q, kc, vc, bt, ent, pos, None, L, kind, window, scale, nh, nkv, hd).float().cpu().view(n, nh, hd)
+    st = _start(p_last, kind, window)
+    for i, j in enumerate(edges):
+        ref = _ref_attention(q1, ks[i], vs[i], p_last, st, scale)
+        assert float((dec[i] - ref).abs().max()) <= 2e-2, ("decode", j)
+        near = float((dec[i] - vs[i][j].repeat_interleave(nh // nkv, 0)).abs().max())
+        assert (near <= 2e-2) == (st <= j <= p_last), ("decode", j, near)
+    # prefill: the last `portion` positions of every request are queries (first and last row checked)
+    T = n * portion
+    qp = q1.to(torch.bfloat16).reshape(1, nh * hd).expand(T, nh * hd).contiguous().to(DEV)
+    ppos = torch.cat([torch.arange(L - portion, L, dtype=torch.int32) for _ in range(n)]).to(DEV)
+    tiles = []
+    for i in range(n):
+        for o in range(0, portion, ops.PREFILL_TILE_TOKENS):
+            tiles.append((i, i * portion + o, min(ops.PREFILL_TILE_TOKENS, portion - o)))
+    pre = ops.attention_prefill(qp, kc, vc, bt, ppos, torch.tensor(tiles, dtype=torch.int32, device=DEV), kind, window,
+                                scale, nh, nkv, hd).float().cpu().view(n, portion, nh, hd)
+    for i, j in enumerate(edges):
+        for row in (0, 77, portion - 1):
+            p = L - portion + row
+            stp = _start(p, kind, window)
+            ref = _ref_attention(q1, ks[i], vs[i], p, stp, scale)
+            assert float((pre[i, row] - ref).abs().max()) <= 2e-2, ("prefill", j, p)
+            near = float((pre[i, row] - vs[i][j].repeat_interleave(nh // nkv, 0)).abs().max())
+            assert (near <= 2e-2) == (stp <= j <= p), ("prefill", j, p, near)
+
+
 # ---------------------------------------------------------------------------
 # routing and the grouped product for many rows
 # ---------------------------------------------------------------------------
