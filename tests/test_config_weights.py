@@ -139,3 +139,41 @@ def test_random_source_is_order_independent():
     assert torch.equal(a.get(names[-1]), b.get(names[-1]))
     assert not torch.equal(RandomSource(specs, 4, torch.float32, "cpu").get(names[0]), b.get(names[0]))
     check_specs(specs, a.available())
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The benchmark measures one GPU: for N > 1 it says so in one line and exits with 2, before
+    anything touches a device."""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    p = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2", "--steps", "1", "--warmup", "0"],
+                       capture_output=True, text=True, timeout=60)
+    assert p.returncode == 2 and len(p.stdout.strip().splitlines()) == 1 and "one GPU" in p.stdout
+
+
+def test_bench_counts_what_a_chunked_layer_sees():
+    """The roofline's bytes and the prefill's flops follow the layer kinds: a chunked layer sees
+    the keys of its chunk only."""
+    import os
+    import sys
+
+    sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    import bench
+    from sharpinference_amd.config.base import load_config
+
+    d = dict(bench.SCOUT)
+    d["num_hidden_layers"] = 4
+    d["no_rope_layers"] = [1, 1, 1, 0]
+    cfg = load_config(d)
+    C = cfg.attention_chunk_size
+    assert bench.visible_keys(cfg, 0, C - 1) == C and bench.visible_keys(cfg, 0, C) == 1
+    assert bench.visible_keys(cfg, 3, C) == C + 1
+    # twice the chunk: chunked layers do the work of two chunks, the global layer of one long prompt
+    lin = bench.prefill_flops(cfg, 2 * C, 4) - bench.prefill_flops(cfg, 2 * C, 0)
+    per_pair = 4 * cfg.num_attention_heads * cfg.head_dim
+    pairs = 3 * 2 * (C * (C + 1) // 2) + (2 * C) * (2 * C + 1) // 2
+    dense = bench.prefill_flops(cfg, 1, 4) - bench.prefill_flops(cfg, 1, 0) - 4 * per_pair   # the linear part of one token
+    assert abs(lin - (2 * C * dense + per_pair * pairs)) <= 1e-6 * lin
