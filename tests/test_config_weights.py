@@ -177,3 +177,39 @@ def test_bench_counts_what_a_chunked_layer_sees():
     pairs = 3 * 2 * (C * (C + 1) // 2) + (2 * C) * (2 * C + 1) // 2
     dense = bench.prefill_flops(cfg, 1, 4) - bench.prefill_flops(cfg, 1, 0) - 4 * per_pair   # the linear part of one token
     assert abs(lin - (2 * C * dense + per_pair * pairs)) <= 1e-6 * lin
+
+
+def test_random_model_command_writes_a_folder_that_loads(tmp_path):
+    """bin/sharpi-random-model: a configuration and a seed give a model folder, the same bytes
+    each time, whose tensors are those the model asks for (32-bit where asked)."""
+    import json
+    import os
+    import subprocess
+    import sys
+
+    from tiny_configs import TINY_C
+
+    from sharpinference_amd.config.base import load_config
+    from sharpinference_amd.registry import build_model
+    from sharpinference_amd.weights import safetensors_io as st
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cfg_path = tmp_path / "config.json"
+    cfg_path.write_text(json.dumps(TINY_C))
+    outs = []
+    for name in ("m1", "m2"):
+        p = subprocess.run([sys.executable, os.path.join(root, "bin", "sharpi-random-model"), "--config", str(cfg_path),
+                            "--seed", "4", "--out", str(tmp_path / name), "--float32", "norm.weight"],
+                           capture_output=True, text=True, timeout=120)
+        assert p.returncode == 0, p.stderr
+        outs.append(tmp_path / name)
+    a, b = [(o / "model.safetensors").read_bytes() for o in outs]
+    assert a == b
+    cfg = load_config(str(outs[0]))
+    assert cfg.to_dict() == load_config(dict(TINY_C)).to_dict()
+    index = st.index_folder(str(outs[0]))
+    specs = build_model(cfg).param_specs()
+    assert set(index) == set(specs)
+    for n, info in index.items():
+        assert tuple(info.shape) == tuple(specs[n].shape), n
+        assert info.dtype == (torch.float32 if n.endswith("norm.weight") else torch.bfloat16), n
