@@ -68,8 +68,8 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__
 }
 
 // The same with rows a multiple of 8 wide: 16-byte accesses, the row kept in registers between
-// the two passes (up to kNormKeep runs of 8 per thread; wider rows are read again).
-constexpr int kNormKeep = 4;
+// the two passes (up to kNormKeep runs of 8 per thread, of up to 1,024 threads; wider rows are read again).
+constexpr int kNormKeep = 2;
 
 // delta of row r, columns c .. c + 7, as floats.  Plain: delta[r].  As an expert sum (sum_pos
 // given): the rows sum_pos[r*k .. r*k + k) of delta plus sum_shared[r], added in that order in
@@ -102,20 +102,47 @@ __device__ __forceinline__ void load_delta8(const TD* __restrict__ delta, const 
 }
 
 template <typename TD, typename TW, typename TO>
-__global__ void add_rmsnorm_vec_kernel(float* __restrict__ h, const TD* __restrict__ delta,
-                                       const TW* __restrict__ w, TO* __restrict__ out,
-                                       const int* __restrict__ rows, int hidden, float eps, int write_back,
-                                       const int* __restrict__ sum_pos, const TD* __restrict__ sum_shared,
-                                       int sum_k) {
+__global__ __launch_bounds__(1024) void add_rmsnorm_vec_kernel(float* __restrict__ h, const TD* __restrict__ delta,
+                                                               const TW* __restrict__ w, TO* __restrict__ out,
+                                                               const int* __restrict__ rows, int hidden, float eps,
+                                                               int write_back, const int* __restrict__ sum_pos,
+                                                               const TD* __restrict__ sum_shared, int sum_k) {
   __shared__ float red[16];
   const int i = blockIdx.x;
   const int r = rows ? rows[i] : i;
   float* hr = h + (size_t)r * hidden;
   const bool dr = delta != nullptr;
-  float keep[kNormKeep][8];
+  // A block has a thread per run of 8 where the row allows it (the launch sees to that): the row,
+  // its delta and the norm's weights are then requested in one go, the kernel is one trip to
+  // memory, the reduction and one store.  With a handful of rows (decode) that latency is all
+  // the kernel costs.
+  float keep[kNormKeep][8], wk[kNormKeep][8];
   float ss = 0.f;
-  int n = 0;
-  for (int c = threadIdx.x * 8; c < hidden; c += blockDim.x * 8, ++n) {
+#pragma unroll
+  for (int n = 0; n < kNormKeep; ++n) {
+    const int c = (threadIdx.x + n * blockDim.x) * 8;
+    if (c < hidden) {
+      load8(hr + c, keep[n]);
+      if (w) load8(w + c, wk[n]);
+    }
+  }
+#pragma unroll
+  for (int n = 0; n < kNormKeep; ++n) {
+    const int c = (threadIdx.x + n * blockDim.x) * 8;
+    if (c < hidden) {
+      if (dr) {
+        float d[8];
+        load_delta8<TD>(delta, sum_pos, sum_shared, sum_k, r, hidden, c, d);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) keep[n][j] += d[j];
+        if (write_back) store8(hr + c, keep[n]);
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ss += keep[n][j] * keep[n][j];
+    }
+  }
+  // rows wider than the registers hold: the rest is read again in the second pass
+  for (int c = (threadIdx.x + kNormKeep * blockDim.x) * 8; c < hidden; c += blockDim.x * 8) {
     float x[8];
     load8(hr + c, x);
     if (dr) {
@@ -127,28 +154,28 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ h, const TD* __restri
     }
 #pragma unroll
     for (int j = 0; j < 8; ++j) ss += x[j] * x[j];
-    if (n < kNormKeep) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) keep[n][j] = x[j];
-    }
   }
   const float total = block_sum(ss, red);
   const float s = 1.0f / sqrtf(total / (float)hidden + eps);
   TO* o = out + (size_t)i * hidden;
-  n = 0;
-  for (int c = threadIdx.x * 8; c < hidden; c += blockDim.x * 8, ++n) {
+#pragma unroll
+  for (int n = 0; n < kNormKeep; ++n) {
+    const int c = (threadIdx.x + n * blockDim.x) * 8;
+    if (c < hidden) {
+      float y[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) y[j] = w ? (keep[n][j] * s) * wk[n][j] : keep[n][j] * s;
+      store8(o + c, y);
+    }
+  }
+  for (int c = (threadIdx.x + kNormKeep * blockDim.x) * 8; c < hidden; c += blockDim.x * 8) {
     float x[8];
-    if (n < kNormKeep) {
+    load8(hr + c, x);
+    if (dr && !write_back) {
+      float d[8];
+      load_delta8<TD>(delta, sum_pos, sum_shared, sum_k, r, hidden, c, d);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) x[j] = keep[n][j];
-    } else {
-      load8(hr + c, x);
-      if (dr && !write_back) {
-        float d[8];
-        load_delta8<TD>(delta, sum_pos, sum_shared, sum_k, r, hidden, c, d);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) x[j] += d[j];
-      }
+      for (int j = 0; j < 8; ++j) x[j] += d[j];
     }
     float y[8];
     if (w) {
@@ -171,7 +198,9 @@ static int launch_add_rmsnorm_o(float* h, const void* delta, const void* w, void
   dim3 grid(n_out), block(hidden >= 2048 ? 512 : 256);
   if (out_dtype != DT_F32 && out_dtype != DT_BF16) return SHARPI_ERR_ARG;
   if ((hidden & 7) == 0) {
-    dim3 vblock(hidden >= 4096 ? 256 : hidden >= 1024 ? 128 : 64);
+    // a thread per run of 8, in whole waves, up to 1,024: the same for every number of rows, so
+    // that a row's statistics are the same sums however many rows share the launch
+    dim3 vblock(min(1024, ceil_div(hidden / 8, kWave) * kWave));
     if (out_dtype == DT_F32)
       add_rmsnorm_vec_kernel<TD, TW, float><<<grid, vblock, 0, stream>>>(h, (const TD*)delta, (const TW*)w,
                                                                         (float*)out, rows, hidden, eps, write_back,
