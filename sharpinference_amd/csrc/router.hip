@@ -10,12 +10,13 @@
 // moe_permute: one block. Counts rows per expert, prefix-sums them into offsets[E + 1] and
 // writes, in expert order, the token and weight of every (token, pick) pair plus the inverse
 // map inv_pos[t * k + j] = row in that order, and the list of (expert, first row) tiles of
-// tile_rows rows that the grouped product of many rows walks.  With shared_group the list gets one
+// tile_rows rows that the grouped product of many rows walks (tallest tiles first).  With shared_group the list gets one
 // more group after the experts: every token once, weight 1 (an always-on expert that shares the
 // experts' weight tensor); offsets then has n_experts + 2 entries and the row arrays n_tokens more.
 #include "common.h"
 
 constexpr int kMaxExperts = 1024;
+constexpr int kSortTiles = 512;   // tile lists up to this long are ordered tallest first
 
 // One thread: gate the logits g[0 .. n_experts) in place, pick k of them (ascending scan with a
 // strict >, so the lowest index wins a tie) into ids / w.
@@ -170,6 +171,11 @@ __device__ void permute_block(const int* __restrict__ topk_ids, const float* __r
                               int* __restrict__ tile_expert, int* __restrict__ tile_row0, int* __restrict__ n_tiles,
                               int n_pairs, int k, int n_experts, int tile_rows, int max_tiles, int shared_group,
                               int* count, int* cursor) {
+  // Tallest tiles first: a block's time grows with its tile's rows, and the blocks that start
+  // last should be the short ones.  (Only lists that fit the LDS arrays are put in order.)
+  __shared__ int s_expert[kSortTiles], s_row0[kSortTiles], s_rows[kSortTiles];
+  __shared__ int s_nt;
+  const bool sort_tiles = max_tiles <= kSortTiles;
   for (int e = threadIdx.x; e < n_experts; e += blockDim.x) count[e] = 0;
   __syncthreads();
   for (int i = threadIdx.x; i < n_pairs; i += blockDim.x) atomicAdd(&count[topk_ids[i]], 1);
@@ -182,20 +188,28 @@ __device__ void permute_block(const int* __restrict__ topk_ids, const float* __r
       run += count[e];
     }
     offsets[n_experts] = run;
-    // row tiles of the experts that have rows, for the grouped product of many rows
+    // row tiles of the experts that have rows, for the grouped product of many rows; up to
+    // kSortTiles of them are listed in LDS first and put in order below
     int nt = 0;
     run = 0;
     for (int e = 0; e < n_experts; ++e) {
       for (int r0 = run; r0 < run + count[e]; r0 += tile_rows) {
         if (nt < max_tiles) {
-          tile_expert[nt] = e;
-          tile_row0[nt] = r0;
+          if (sort_tiles) {
+            s_expert[nt] = e;
+            s_row0[nt] = r0;
+            s_rows[nt] = min(tile_rows, run + count[e] - r0);
+          } else {
+            tile_expert[nt] = e;
+            tile_row0[nt] = r0;
+          }
           ++nt;
         }
       }
       run += count[e];
     }
     n_tiles[0] = nt;
+    s_nt = nt;
     // an always-on expert as one more group: every token once, in token order, with weight 1
     if (shared_group) offsets[n_experts + 1] = run + n_pairs / k;
   }
@@ -206,6 +220,15 @@ __device__ void permute_block(const int* __restrict__ topk_ids, const float* __r
     }
   }
   __syncthreads();
+  if (sort_tiles) {
+    // a tile's place = the number of tiles that are taller, or as tall and listed before it
+    for (int i = threadIdx.x; i < s_nt; i += blockDim.x) {
+      int place = 0;
+      for (int j = 0; j < s_nt; ++j) place += (s_rows[j] > s_rows[i] || (s_rows[j] == s_rows[i] && j < i)) ? 1 : 0;
+      tile_expert[place] = s_expert[i];
+      tile_row0[place] = s_row0[i];
+    }
+  }
   for (int i = threadIdx.x; i < n_pairs; i += blockDim.x) {
     const int e = topk_ids[i];
     const int r = atomicAdd(&cursor[e], 1);

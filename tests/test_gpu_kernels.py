@@ -323,6 +323,8 @@ def test_router_and_permute(T, E, k, H, dtype):
     nt = int(rt.n_tiles.cpu())
     tiles = list(zip(rt.tile_expert.cpu().tolist()[:nt], rt.tile_row0.cpu().tolist()[:nt]))
     want = [(e, r0) for e in range(E) for r0 in range(off[e], off[e + 1], ops.GROUPED_TILE_ROWS)]
+    # tallest tiles first (the blocks that start last should be the short ones), otherwise in expert order
+    want.sort(key=lambda t: -min(ops.GROUPED_TILE_ROWS, off[t[0] + 1] - t[1]))
     assert tiles == want
 
 
