@@ -526,6 +526,7 @@ def router_topk(x: torch.Tensor, wr: torch.Tensor, k: int, gate: int = GATE_SIGM
 
 
 GROUPED_TILE_ROWS = 192   # rows per tile of the grouped product (csrc/gemm_grouped.hip GM)
+SORTED_TILE_LISTS = 512   # tile lists up to this long come tallest first (csrc/router.hip kSortTiles)
 
 
 class Routing:
