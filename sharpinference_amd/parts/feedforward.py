@@ -154,4 +154,4 @@ class MoESwiGLU(Part):
         shared = self.shared.forward(x, ctx) if self.shared is not None else None
         act = ops.grouped_swiglu(x, self.w_gate_up, rt, ctx.act_dtype)
         y = ops.grouped_linear(act, self.w_down, rt, False, ctx.act_dtype)
-        return ops.moe_combine(y, rt.inv_pos, shared, T, self.k)
+        return ops.ExpertSum(y, rt.inv_pos, shared, T, self.k)   # formed by the next norm (or by whoever asks for a tensor)
