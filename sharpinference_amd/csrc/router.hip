@@ -268,3 +268,5 @@ SHARPI_EXPORT int sharpi_moe_permute(const int* topk_ids, const float* topk_w, i
   SHARPI_CHECK_LAUNCH();
   return SHARPI_OK;
 }
+
+SHARPI_EXPORT int sharpi_router_sorted_tiles() { return kSortTiles; }

@@ -18,12 +18,13 @@ import numpy as np
 import torch
 
 from ..cache.manager import CacheError, CacheManager
+from ..ops.lib import PREFILL_TILE_TOKENS
 from ..parts.base import GroupView, LayerCache, StepContext
 
 
 MAX_GRAPH_BATCH = 16   # decode steps of up to this many requests are replayed from a HIP graph (beyond, launches no longer bound the step and the fixed maxima cost more than they save)
 GRAPH_CONTEXT_MIN = 4096   # a graph is captured for a bound on the contexts of its requests: this, or 4, 16, 64 ... times it
-TILE = 128   # tokens per attention tile of multi-token entries (ops.PREFILL_TILE_TOKENS)
+TILE = PREFILL_TILE_TOKENS   # tokens per attention tile of multi-token entries
 
 
 class CacheExhausted(CacheError):

@@ -217,7 +217,7 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     return out
 
 
-DECODE_RUN_KEYS = 256   # keys per block of the decode kernel (fixed: sums must not depend on the batch)
+DECODE_RUN_KEYS = _lib.DECODE_RUN_KEYS   # keys per block of the decode kernel (fixed: sums must not depend on the batch)
 
 
 def decode_attention_ok(dtype: torch.dtype, hd: int) -> bool:
@@ -255,7 +255,7 @@ def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     return out
 
 
-PREFILL_TILE_TOKENS = 128   # tokens per block of the prefill kernel (32 per wave)
+PREFILL_TILE_TOKENS = _lib.PREFILL_TILE_TOKENS   # tokens per block of the prefill kernel (32 per wave)
 
 
 def prefill_attention_ok(dtype: torch.dtype, hd: int) -> bool:
@@ -528,8 +528,8 @@ def router_topk(x: torch.Tensor, wr: torch.Tensor, k: int, gate: int = GATE_SIGM
     return (ids, wts, gates) if want_gates else (ids, wts)
 
 
-GROUPED_TILE_ROWS = 192   # rows per tile of the grouped product (csrc/gemm_grouped.hip GM)
-SORTED_TILE_LISTS = 512   # tile lists up to this long come tallest first (csrc/router.hip kSortTiles)
+GROUPED_TILE_ROWS = _lib.GROUPED_TILE_ROWS   # rows per tile of the grouped product (csrc/gemm_grouped.hip GM)
+SORTED_TILE_LISTS = _lib.SORTED_TILE_LISTS   # tile lists up to this long come tallest first (csrc/router.hip kSortTiles)
 
 
 class Routing:

@@ -41,6 +41,19 @@ _SIGNATURES = {
 # entry points that newer sources add; bound when present
 _OPTIONAL_SIGNATURES: dict = {}
 
+# Sizes that the host code lays work out by and the kernels are compiled for: the library says what
+# it was built with, and a build with other sizes is refused at load (it would compute wrong results).
+DECODE_RUN_KEYS = 256       # keys per block of the decode attention kernel
+PREFILL_TILE_TOKENS = 128   # tokens per block of the prefill attention kernel
+GROUPED_TILE_ROWS = 192     # rows per tile of the grouped product for many rows
+SORTED_TILE_LISTS = 512     # tile lists up to this long come tallest first
+_BUILT_WITH = {
+    "sharpi_attention_decode_split_keys": DECODE_RUN_KEYS,
+    "sharpi_attention_prefill_tile_tokens": PREFILL_TILE_TOKENS,
+    "sharpi_gemm_grouped_tile_rows": GROUPED_TILE_ROWS,
+    "sharpi_router_sorted_tiles": SORTED_TILE_LISTS,
+}
+
 
 class KernelLibraryError(RuntimeError):
     pass
@@ -74,6 +87,15 @@ def load(verbose: bool = True) -> ctypes.CDLL:
             continue
         fn.argtypes = args
         fn.restype = c_int
+    for name, want in _BUILT_WITH.items():
+        try:
+            fn = getattr(lib, name)
+        except AttributeError:
+            raise KernelLibraryError(f"{path} lacks entry point {name}: rebuild the kernels") from None
+        fn.argtypes, fn.restype = [], c_int
+        got = fn()
+        if got != want:
+            raise KernelLibraryError(f"{path} was built with {name}() = {got}, the host code lays work out for {want}")
     _lib, _lib_path = lib, path
     return lib
 
