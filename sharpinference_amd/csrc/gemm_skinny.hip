@@ -16,6 +16,12 @@
 //    a time (an expert with more is walked in turns and its weights read again for each); x rows
 //    are gathered through a_rows.  Experts without rows return at once.
 //
+//  * Picked form (a few decode tokens): instead of a sorted row list the kernel is given the
+//    router's picks themselves.  Row i of the output is pair i = (token i / k, its pick i % k), in
+//    that order, followed by one row per token for an always-on expert that shares the tensor; a
+//    block finds the rows of its expert with one ballot over the picks.  No kernel has to sort
+//    the pairs first, and the x rows wait for one index load instead of two.
+//
 //  * Packed weights (PACKED): the matrix is stored tile by tile instead of row by row, the 4 KB
 //    of a (16-row tile, 128-wide K unit) contiguous and in the order the lanes want them, and
 //    the K units are dealt to the waves in turn: a block's reads are contiguous runs of NW * 4 KB
@@ -43,28 +49,60 @@ template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, f32x4 v) {
 }
 
 constexpr int kRedTiles = 2;  // (tile, row block) pairs summed per LDS round
+constexpr int kMaxPicked = 64;  // pairs (and tokens) of the picked form: one ballot of a wave
+
+// The picked form's arguments (ids null: the other forms).
+struct Picks {
+  const int* ids;      // [n_pairs] expert of pair i
+  const float* w;      // [n_pairs] its score (the SwiGLU form scales by it), or null
+  int n_pairs, k, n_experts;
+  int gather;          // x rows are tokens (pair i reads row i / k); otherwise x is in the output's row order
+};
 
 template <int R, int MB, int NW, typename TO, bool ACT, bool PACKED>
 __global__ __launch_bounds__(NW* kWave) void skinny_gemm_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ W, TO* __restrict__ out, int M, int N, int K,
-    const int* __restrict__ a_rows, const int* __restrict__ group_offsets, const float* __restrict__ act_scale) {
+    const int* __restrict__ a_rows, const int* __restrict__ group_offsets, const float* __restrict__ act_scale,
+    Picks pk) {
   static_assert(!ACT || R % 2 == 0, "the SwiGLU form pairs gate and up tiles");
   constexpr int RT = ACT ? R : kRedTiles;   // tiles that meet in LDS per round
   constexpr int TG = ACT ? R / 2 : R;       // tiles of distinct output columns per block
   __shared__ f32x4 red[NW][RT][kWave];
+  __shared__ int members[kMaxPicked];       // picked form: the output rows of this block's expert
+  __shared__ int n_members;
   const int lane = threadIdx.x & (kWave - 1);
   const int w = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
   const int nb = blockIdx.x;
   const int e = blockIdx.y;
+  const bool picked = pk.ids != nullptr;
   int row_begin = 0, row_end = M;
-  if (group_offsets) {
+  if (picked) {
+    if (w == 0) {
+      // expert e < n_experts: the pairs that picked it; e == n_experts: every token once
+      const bool routed = e < pk.n_experts;
+      const bool mine = routed ? (lane < pk.n_pairs && pk.ids[lane] == e) : lane < pk.n_pairs / pk.k;
+      const unsigned long long mask = __builtin_amdgcn_ballot_w64(mine);
+      if (mine) members[__popcll(mask & ((1ull << lane) - 1ull))] = routed ? lane : pk.n_pairs + lane;
+      if (lane == 0) n_members = __popcll(mask);
+    }
+    __syncthreads();
+    row_end = n_members;
+    W += (size_t)e * N * K;
+  } else if (group_offsets) {
     row_begin = group_offsets[e];
     row_end = group_offsets[e + 1];
     W += (size_t)e * N * K;
   }
   const int n_rows = row_end - row_begin;
   if (n_rows <= 0) return;
+  // where row m of the block's list reads x, and where it is stored
+  auto out_row = [&](int m) { return picked ? members[m] : m; };
+  auto x_row = [&](int m) {
+    if (!picked) return a_rows ? a_rows[m] : m;
+    const int i = members[m];
+    return pk.gather ? (i < pk.n_pairs ? i / pk.k : i - pk.n_pairs) : i;
+  };
   const int n_base = nb * 16 * TG;
   const int n_out = ACT ? N / 2 : N;        // output columns
 
@@ -102,7 +140,7 @@ __global__ __launch_bounds__(NW* kWave) void skinny_gemm_kernel(
     for (int mb = 0; mb < MB; ++mb) {
       const int m = row_begin + (rb0 + mb) * 16 + r;
       xvalid[mb] = m < row_end;
-      const int src = xvalid[mb] ? (a_rows ? a_rows[m] : m) : 0;
+      const int src = xvalid[mb] ? x_row(m) : 0;
       xrow[mb] = x + (size_t)src * K + g * XG;
     }
     f32x4 acc[R][MB];
@@ -159,12 +197,20 @@ __global__ __launch_bounds__(NW* kWave) void skinny_gemm_kernel(
           const int row = row_begin + (rb0 + mb) * 16 + r;
           const int n = n_base + w * 16 + g * 4;
           if (row < row_end && n < n_out) {
-            const float sc = act_scale ? act_scale[row] : 1.0f;
+            const int orow = out_row(row);
+            float sc = 1.0f;
+            bool scaled = act_scale != nullptr;
+            if (picked) {            // a pair's score; the always-on expert's rows are not scaled
+              scaled = pk.w != nullptr;
+              if (scaled) sc = orow < pk.n_pairs ? pk.w[orow] : 1.0f;
+            } else if (scaled) {
+              sc = act_scale[row];
+            }
             f32x4 o;
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-              o[i] = swiglu_f32(bf16_to_f32(f32_to_bf16(gv[i])), bf16_to_f32(f32_to_bf16(uv[i])), sc, act_scale != nullptr);
-            store4<TO>(out + (size_t)row * n_out + n, o);
+              o[i] = swiglu_f32(bf16_to_f32(f32_to_bf16(gv[i])), bf16_to_f32(f32_to_bf16(uv[i])), sc, scaled);
+            store4<TO>(out + (size_t)orow * n_out + n, o);
           }
         }
       }
@@ -192,7 +238,7 @@ __global__ __launch_bounds__(NW* kWave) void skinny_gemm_kernel(
         // lane holds out[row = ... + r][n = n_base + t*16 + g*4 + 0..3]
         const int row = row_begin + (rb0 + mb) * 16 + r;
         const int n = n_base + t * 16 + g * 4;
-        if (row < row_end && n < N) store4<TO>(out + (size_t)row * N + n, v);
+        if (row < row_end && n < N) store4<TO>(out + (size_t)out_row(row) * N + n, v);
       }
     }
   }
@@ -201,15 +247,15 @@ __global__ __launch_bounds__(NW* kWave) void skinny_gemm_kernel(
 template <int R, int MB, int NW, bool ACT, bool PACKED>
 static int launch_skinny(const void* x, const void* W, void* out, int out_dtype, int M, int N, int K,
                          const int* a_rows, const int* group_offsets, int groups, const float* act_scale,
-                         hipStream_t stream) {
+                         hipStream_t stream, Picks pk = Picks{}) {
   dim3 grid(ceil_div(ACT ? N / 2 : N, 16 * (ACT ? R / 2 : R)), groups > 0 ? groups : 1), block(NW * kWave);
   const int* go = groups > 0 ? group_offsets : nullptr;
   if (out_dtype == DT_F32)
     skinny_gemm_kernel<R, MB, NW, float, ACT, PACKED><<<grid, block, 0, stream>>>(
-        (const bf16_t*)x, (const bf16_t*)W, (float*)out, M, N, K, a_rows, go, act_scale);
+        (const bf16_t*)x, (const bf16_t*)W, (float*)out, M, N, K, a_rows, go, act_scale, pk);
   else
     skinny_gemm_kernel<R, MB, NW, bf16_t, ACT, PACKED><<<grid, block, 0, stream>>>(
-        (const bf16_t*)x, (const bf16_t*)W, (bf16_t*)out, M, N, K, a_rows, go, act_scale);
+        (const bf16_t*)x, (const bf16_t*)W, (bf16_t*)out, M, N, K, a_rows, go, act_scale, pk);
   SHARPI_CHECK_LAUNCH();
   return SHARPI_OK;
 }
@@ -279,5 +325,41 @@ SHARPI_EXPORT int sharpi_gemm_skinny_swiglu(const void* x, const void* W, void* 
   SKA(4, 4); SKA(4, 8);
 #undef SKA
 #undef SKA1
+  return SHARPI_ERR_ARG;
+}
+
+// The picked form: per-expert products of a few decode tokens straight from the router's picks.
+// ids [n_pairs] (pair i = token i / k, pick i % k), W [n_experts (+ 1 if shared), N, K]; out row i is
+// pair i, rows n_pairs .. n_pairs + n_pairs / k - 1 are the tokens through expert n_experts (shared != 0).
+// gather: x [tokens, K] is read by token; otherwise x rows are in the output's order.  With act != 0
+// W holds gate then up rows and out [rows, N/2] bf16 = silu(s g) * (s u), s = w[i] for pair i (w may
+// be null: no scaling) and 1 for the shared rows.  n_pairs and the tokens fit one wave's ballot (<= 64).
+SHARPI_EXPORT int sharpi_gemm_skinny_picked(const void* x, const void* W, void* out, int out_dtype, int N, int K,
+                                            const int* ids, const float* w, int n_pairs, int k, int n_experts,
+                                            int shared, int gather, int act, int R, int NW, int packed,
+                                            hipStream_t stream) {
+  if (n_pairs <= 0) return SHARPI_OK;
+  if (ids == nullptr || k <= 0 || n_pairs % k != 0 || n_pairs > kMaxPicked || n_experts <= 0) return SHARPI_ERR_ARG;
+  if (N <= 0 || (N & (act ? 7 : 3)) || K <= 0 || (K & 127)) return SHARPI_ERR_ARG;
+  if (packed && (N & (act ? 31 : 15))) return SHARPI_ERR_ARG;
+  if (out_dtype != DT_F32 && out_dtype != DT_BF16) return SHARPI_ERR_ARG;
+  if (act && out_dtype != DT_BF16) return SHARPI_ERR_ARG;
+  const int groups = n_experts + (shared ? 1 : 0);
+  if (groups > 65535) return SHARPI_ERR_ARG;
+  const int M = n_pairs + (shared ? n_pairs / k : 0);
+  const Picks pk = {ids, w, n_pairs, k, n_experts, gather};
+  // group_offsets is not read in this form; the pointer only has to be non-null for the grid's sake
+#define SKP(RR, WW, ACTV)                                                                                       \
+  if (R == RR && NW == WW && (act != 0) == ACTV)                                                                \
+  return packed ? launch_skinny<RR, 1, WW, ACTV, true>(x, W, out, out_dtype, M, N, K, nullptr, ids, groups,     \
+                                                       nullptr, stream, pk)                                     \
+                : launch_skinny<RR, 1, WW, ACTV, false>(x, W, out, out_dtype, M, N, K, nullptr, ids, groups,    \
+                                                        nullptr, stream, pk)
+  SKP(1, 4, false); SKP(1, 8, false); SKP(1, 16, false);
+  SKP(2, 4, false); SKP(2, 8, false);
+  SKP(4, 4, false); SKP(4, 8, false);
+  SKP(2, 4, true); SKP(2, 8, true);
+  SKP(4, 4, true); SKP(4, 8, true);
+#undef SKP
   return SHARPI_ERR_ARG;
 }

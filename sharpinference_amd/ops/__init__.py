@@ -461,6 +461,58 @@ def gemm_skinny_swiglu(x: torch.Tensor, w, offsets: torch.Tensor, a_rows: Option
     return out
 
 
+PICKED_MAX_PAIRS = 64   # (token, pick) pairs of the picked form: one ballot of a wave (csrc/gemm_skinny.hip kMaxPicked)
+
+_COUNTING: dict = {}    # per device: 0, 1, 2, ... (the places of pairs that are stored in their own order)
+
+
+def counting(n: int, dev: torch.device) -> torch.Tensor:
+    """int32 [n] = 0 .. n-1 on the device, from one tensor per device that is made once (outside
+    any graph capture)."""
+    c = _COUNTING.get(dev)
+    if c is None or c.numel() < n:
+        _need(not torch.cuda.is_current_stream_capturing(), "counting: the first call on a device must not be captured")
+        c = _COUNTING[dev] = torch.arange(max(n, 4096), dtype=torch.int32, device=dev)
+    return c[:n]
+
+
+def picked_ok(n_tokens: int, k: int, N: int, K: int, act: bool, packed: bool) -> bool:
+    return (0 < n_tokens * k <= PICKED_MAX_PAIRS and K % 128 == 0
+            and N % ((32 if packed else 8) if act else (16 if packed else 4)) == 0)
+
+
+def gemm_skinny_picked(x: torch.Tensor, w, ids: torch.Tensor, wts: Optional[torch.Tensor], shared: bool, gather: bool,
+                       act: bool, out_dtype: torch.dtype) -> torch.Tensor:
+    """Per-expert products of a few decode tokens straight from the router's picks ids [T, k]:
+    row i of the result is pair i = (token i // k, pick i % k), followed (shared) by one row per
+    token through expert E of w [E + 1, N, K].  gather: x [T, K] is read by token, otherwise x is in
+    the result's row order.  act: w holds gate rows then up rows and the result is
+    silu(s g) * (s u) [rows, N/2] with s the pair's weight (wts; 1 for the shared rows)."""
+    w, packed = _unwrap(w)
+    _dev(x, w, ids, wts)
+    _i32(ids, "ids")
+    _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_skinny_picked: bfloat16 operands only")
+    _need(ids.dim() == 2 and ids.is_contiguous(), "gemm_skinny_picked: ids [T, k]")
+    T, k = ids.shape
+    E = w.shape[0] - (1 if shared else 0)
+    _need(w.dim() == 3 and E >= 1, "gemm_skinny_picked: w [E (+ 1), N, K]")
+    N, K = w.shape[1], w.shape[2]
+    _need(picked_ok(T, k, N, K, act, packed), f"gemm_skinny_picked: T={T} k={k} N={N} K={K} is not taken")
+    rows = T * k + (T if shared else 0)
+    _need(x.dim() == 2 and x.shape[1] == K and x.shape[0] == (T if gather else rows),
+          f"gemm_skinny_picked: x {tuple(x.shape)} has the wrong shape")
+    if wts is not None:
+        _need(act and wts.dtype == torch.float32 and wts.shape == ids.shape and wts.is_contiguous(),
+              "gemm_skinny_picked: weights are float32 [T, k] and belong to the activation form")
+    if act:
+        _need(out_dtype == torch.bfloat16, "gemm_skinny_picked: the activation form stores bfloat16")
+    pr, pw = skinny_plan(N, K)
+    out = torch.empty(rows, N // 2 if act else N, dtype=out_dtype, device=x.device)
+    _run("sharpi_gemm_skinny_picked", _ptr(x), _ptr(w), _ptr(out), _code(out_dtype), N, K, _ptr(ids), _ptr(wts), T * k, k, E,
+         1 if shared else 0, 1 if gather else 0, 1 if act else 0, pr, pw, 1 if packed else 0, _stream())
+    return out
+
+
 def linear(x: torch.Tensor, w, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """y = x W^T.  float32 weights: the float FMA kernel (true 32-bit, whatever x was stored
     as).  bfloat16 weights: the weight-streaming kernel for a few rows (over the packed form if w

@@ -141,8 +141,19 @@ class MoESwiGLU(Part):
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         T = x.shape[0]
         merge = self.merged and T <= self.MERGE_MAX_TOKENS and ctx.act_dtype == torch.bfloat16
-        ids, wts, rt = ops.route(x, self.w_router, self.k, self.gate, self.renormalise, shared_group=merge)
         trace = ctx.extras.get("router_trace")
+        packed = isinstance(self.w_gate_up, ops.PackedWeight)
+        if (merge and ops.picked_ok(T, self.k, 2 * self.inter, self.hidden, True, packed)
+                and ops.picked_ok(T, self.k, self.hidden, self.inter, False, packed)):
+            # a few decode tokens: the two products find their rows from the picks themselves (no
+            # sorting kernel), pair by pair in the picks' own order, the shared expert's rows after them
+            ids, wts = ops.router_topk(x, self.w_router, self.k, self.gate, self.renormalise)
+            if trace is not None:
+                trace.append((ids, wts))
+            act = ops.gemm_skinny_picked(x, self.w_gate_up, ids, wts, True, True, True, ctx.act_dtype)
+            y = ops.gemm_skinny_picked(act, self.w_down, ids, None, True, False, False, ctx.act_dtype)
+            return ops.ExpertSum(y, ops.counting(T * self.k, x.device), y[T * self.k:], T, self.k)
+        ids, wts, rt = ops.route(x, self.w_router, self.k, self.gate, self.renormalise, shared_group=merge)
         if trace is not None:      # the picks of this step, layer by layer (reference: ForwardPass.cs:2042-2056)
             trace.append((ids, wts))
         if merge:

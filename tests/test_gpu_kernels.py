@@ -422,6 +422,49 @@ def test_gemm_grouped(T, E, k, N, K):
         assert torch.equal(ops.gemm_grouped(x, pw, rt, True, torch.float32).cpu(), got)
 
 
+@pytest.mark.parametrize("T,E,k,I,K", [(1, 16, 1, 256, 256), (8, 16, 1, 8192, 640), (16, 4, 4, 128, 384), (5, 3, 2, 128, 128),
+                                       (16, 2, 1, 384, 256)])
+@pytest.mark.parametrize("packed", [False, True])
+def test_picked_products_equal_the_sorted_ones(T, E, k, I, K, packed):
+    """The few-rows products that find their rows from the router's picks give, pair by pair, the
+    bits of the products over the sorted row list (an expert with every pair, experts with none,
+    the always-on expert's rows at the end)."""
+    ops = _ops()
+    H = K
+    x = _rand(T, H, dtype=torch.bfloat16, seed=T)
+    wgu = _rand(E + 1, 2 * I, H, dtype=torch.bfloat16, scale=0.1, seed=I)
+    wdn = _rand(E + 1, H, I, dtype=torch.bfloat16, scale=0.1, seed=I + 1)
+    if packed:
+        if not (ops.can_pack(wgu) and ops.can_pack(wdn) and (2 * I) % 32 == 0):
+            pytest.skip("sizes that are not stored tile by tile")
+        wgu_f, wdn_f = ops.pack_weight(wgu, keep_rows=False), ops.pack_weight(wdn, keep_rows=False)
+    else:
+        wgu_f, wdn_f = wgu, wdn
+    g = torch.Generator().manual_seed(T + E)
+    ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32)
+    if E == 2:
+        ids[:] = 1                                         # one expert takes every pair
+    ids = ids.to(DEV)
+    wts = torch.rand(T, k, generator=g).to(DEV)
+    rt = ops.moe_permute(ids, wts, E, True)
+    act_s = ops.gemm_skinny_swiglu(x, wgu_f, rt.offsets, rt.sorted_token, rt.n_rows, rt.sorted_w, group_rows=T)
+    y_s = ops.gemm_skinny(act_s, wdn_f, torch.bfloat16, offsets=rt.offsets, n_rows=rt.n_rows, group_rows=T)
+    act_p = ops.gemm_skinny_picked(x, wgu_f, ids, wts, True, True, True, torch.bfloat16)
+    y_p = ops.gemm_skinny_picked(act_p, wdn_f, ids, None, True, False, False, torch.bfloat16)
+    inv = rt.inv_pos.long()
+    assert torch.equal(act_p[:T * k], act_s[inv]) and torch.equal(act_p[T * k:], act_s[T * k:])
+    assert torch.equal(y_p[:T * k], y_s[inv]) and torch.equal(y_p[T * k:], y_s[T * k:])
+    # and the sums the next norm forms from either are the same
+    a = ops.ExpertSum(y_p, ops.counting(T * k, y_p.device), y_p[T * k:], T, k).tensor()
+    b = ops.ExpertSum(y_s, rt.inv_pos, y_s[T * k:], T, k).tensor()
+    assert torch.equal(a, b)
+    # without the always-on expert
+    y1 = ops.gemm_skinny_picked(x, ops.PackedWeight(wgu_f.packed[:E], None) if packed else wgu[:E], ids, None, False, True, False,
+                                torch.float32)
+    ref = torch.stack([x[i // k].float() @ wgu[int(ids.flatten()[i])].float().T for i in range(T * k)])
+    assert float((y1 - ref).abs().max()) <= 1e-3 * float(ref.abs().max())
+
+
 @pytest.mark.parametrize("T,E,k,I,K", [(300, 4, 1, 128, 256), (700, 16, 2, 272, 128), (65, 3, 1, 16, 384),
                                        (500, 5, 1, 112, 640), (260, 2, 2, 80, 1216), (430, 3, 1, 8192, 128)])
 def test_gemm_grouped_swiglu_equals_product_then_activation(T, E, k, I, K):
