@@ -57,15 +57,65 @@ __device__ void gate_and_pick(float* g, int n_experts, int k, int gate, int reno
     for (int j = 0; j < k; ++j) w[j] /= wsum;
 }
 
+// One wave: s[i] = wrow . xr[i] for TT rows, in float.  Lanes stride over the width in runs of 8
+// (one fused multiply-add chain per lane and row, in ascending order), then the lanes are summed:
+// the order of the additions depends on the width only, and each row has its own accumulator, so
+// a token's logit is the same bits whatever TT is and whichever kernel calls this.
+template <typename T, typename TW, int TT>
+__device__ __forceinline__ void wave_dot_rows(const T* const (&xr)[TT], const TW* __restrict__ wrow, int hidden,
+                                              int lane, float (&out)[TT]) {
+  float s[TT];
+#pragma unroll
+  for (int i = 0; i < TT; ++i) s[i] = 0.f;
+  if ((hidden & 7) == 0) {
+    // Q runs are fetched before the first is added: a row is a dozen dependent round trips
+    // to the cache otherwise, and the kernel is nothing but their latency
+    constexpr int Q = TT == 1 ? 4 : 2;
+    int c = lane * 8;
+    for (; c + (Q - 1) * kWave * 8 < hidden; c += Q * kWave * 8) {
+      float a[TT][Q][8], b[Q][8];
+#pragma unroll
+      for (int q = 0; q < Q; ++q) {
+        load8(wrow + c + q * kWave * 8, b[q]);
+#pragma unroll
+        for (int i = 0; i < TT; ++i) load8(xr[i] + c + q * kWave * 8, a[i][q]);
+      }
+#pragma unroll
+      for (int i = 0; i < TT; ++i)
+#pragma unroll
+        for (int q = 0; q < Q; ++q)
+#pragma unroll
+          for (int j = 0; j < 8; ++j) s[i] = fmaf(a[i][q][j], b[q][j], s[i]);
+    }
+    for (; c < hidden; c += kWave * 8) {
+      float b[8];
+      load8(wrow + c, b);
+#pragma unroll
+      for (int i = 0; i < TT; ++i) {
+        float a[8];
+        load8(xr[i] + c, a);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s[i] = fmaf(a[j], b[j], s[i]);
+      }
+    }
+  } else {
+    for (int c = lane; c < hidden; c += kWave) {
+      const float b = to_f32<TW>(wrow[c]);
+#pragma unroll
+      for (int i = 0; i < TT; ++i) s[i] = fmaf(to_f32<T>(xr[i][c]), b, s[i]);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < TT; ++i) out[i] = wave_sum(s[i]);
+}
+
 template <typename T, typename TW, int TT>
 __global__ __launch_bounds__(1024) void router_topk_kernel(const T* __restrict__ x, const TW* __restrict__ wr,
                                                            int* __restrict__ topk_ids,
                                                            float* __restrict__ topk_w,
                                                            float* __restrict__ gate_out, int n_tokens, int hidden,
                                                            int n_experts, int k, int gate, int renorm) {
-  // TT tokens per block: a router row is fetched once for all of them.  A token's logit is the same
-  // chain of additions whatever TT is (each token has its own accumulator), so how many tokens
-  // share a block never shows in the result.
+  // TT tokens per block: a router row is fetched once for all of them.
   __shared__ float g[TT][kMaxExperts];
   const int t0 = blockIdx.x * TT;
   const int lane = threadIdx.x & (kWave - 1);
@@ -74,54 +124,12 @@ __global__ __launch_bounds__(1024) void router_topk_kernel(const T* __restrict__
   const T* xr[TT];
 #pragma unroll
   for (int i = 0; i < TT; ++i) xr[i] = x + (size_t)min(t0 + i, n_tokens - 1) * hidden;   // beyond the last: computed, not kept
-  const bool vec = (hidden & 7) == 0;
   for (int e = w; e < n_experts; e += nw) {
-    const TW* wrow = wr + (size_t)e * hidden;
-    float s[TT];
+    float v[TT];
+    wave_dot_rows<T, TW, TT>(xr, wr + (size_t)e * hidden, hidden, lane, v);
+    if (lane == 0) {
 #pragma unroll
-    for (int i = 0; i < TT; ++i) s[i] = 0.f;
-    if (vec) {  // lane-strided runs of 8: the order of the additions depends on the width only
-      // Q runs are fetched before the first is added: a row is a dozen dependent round trips
-      // to the cache otherwise, and the kernel is nothing but their latency
-      constexpr int Q = TT == 1 ? 4 : 2;
-      int c = lane * 8;
-      for (; c + (Q - 1) * kWave * 8 < hidden; c += Q * kWave * 8) {
-        float a[TT][Q][8], b[Q][8];
-#pragma unroll
-        for (int q = 0; q < Q; ++q) {
-          load8(wrow + c + q * kWave * 8, b[q]);
-#pragma unroll
-          for (int i = 0; i < TT; ++i) load8(xr[i] + c + q * kWave * 8, a[i][q]);
-        }
-#pragma unroll
-        for (int i = 0; i < TT; ++i)
-#pragma unroll
-          for (int q = 0; q < Q; ++q)
-#pragma unroll
-            for (int j = 0; j < 8; ++j) s[i] = fmaf(a[i][q][j], b[q][j], s[i]);
-      }
-      for (; c < hidden; c += kWave * 8) {
-        float b[8];
-        load8(wrow + c, b);
-#pragma unroll
-        for (int i = 0; i < TT; ++i) {
-          float a[8];
-          load8(xr[i] + c, a);
-#pragma unroll
-          for (int j = 0; j < 8; ++j) s[i] = fmaf(a[j], b[j], s[i]);
-        }
-      }
-    } else {
-      for (int c = lane; c < hidden; c += kWave) {
-        const float b = to_f32<TW>(wrow[c]);
-#pragma unroll
-        for (int i = 0; i < TT; ++i) s[i] = fmaf(to_f32<T>(xr[i][c]), b, s[i]);
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < TT; ++i) {
-      const float v = wave_sum(s[i]);
-      if (lane == 0) g[i][e] = v;
+      for (int i = 0; i < TT; ++i) g[i][e] = v[i];
     }
   }
   __syncthreads();
@@ -130,6 +138,92 @@ __global__ __launch_bounds__(1024) void router_topk_kernel(const T* __restrict__
     gate_and_pick(g[threadIdx.x], n_experts, k, gate, renorm, topk_ids + (size_t)t * k, topk_w + (size_t)t * k,
                   gate_out ? gate_out + (size_t)t * n_experts : nullptr);
   }
+}
+
+// Residual add + RMSNorm + router in one launch, for a few decode tokens: one block per token
+// forms h += delta, normalises it (the arithmetic of the norm kernel: a thread per run of 8, the
+// same statistics), stores the normalised row in `out` for the experts and keeps a copy in LDS,
+// from which its waves then compute the router's logits (wave_dot_rows over the stored, rounded
+// values: the bits of the router kernel) and one thread picks.  hidden % 8 == 0, hidden <= 8192.
+constexpr int kFusedMaxHidden = 8192;
+
+template <typename TW, typename TWR>
+__global__ __launch_bounds__(1024) void add_rmsnorm_router_kernel(
+    float* __restrict__ h, const bf16_t* __restrict__ delta, const TW* __restrict__ w, bf16_t* __restrict__ out,
+    int hidden, float eps, const TWR* __restrict__ wr, int* __restrict__ topk_ids, float* __restrict__ topk_w,
+    int n_experts, int k, int gate, int renorm) {
+  __shared__ float red[16];
+  __shared__ float g[1][kMaxExperts];
+  __shared__ __attribute__((aligned(16))) bf16_t row[kFusedMaxHidden];
+  const int t = blockIdx.x;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wv = threadIdx.x >> 6;
+  const int nw = blockDim.x >> 6;
+  float* hr = h + (size_t)t * hidden;
+  const int c = threadIdx.x * 8;
+  float x[8], wk[8];
+  float ss = 0.f;
+  if (c < hidden) {
+    load8(hr + c, x);
+    if (w) load8(w + c, wk);
+    if (delta) {
+      float d[8];
+      load8(delta + (size_t)t * hidden + c, d);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) x[j] += d[j];
+      store8(hr + c, x);
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ss += x[j] * x[j];
+  }
+  const float total = block_sum(ss, red);
+  const float s = 1.0f / sqrtf(total / (float)hidden + eps);
+  if (c < hidden) {
+    float y[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) y[j] = w ? (x[j] * s) * wk[j] : x[j] * s;
+    store8(out + (size_t)t * hidden + c, y);
+    store8(row + c, y);            // the same rounding: what the router would read back from memory
+  }
+  __syncthreads();
+  const bf16_t* xr[1] = {row};
+  for (int e = wv; e < n_experts; e += nw) {
+    float v[1];
+    wave_dot_rows<bf16_t, TWR, 1>(xr, wr + (size_t)e * hidden, hidden, lane, v);
+    if (lane == 0) g[0][e] = v[0];
+  }
+  __syncthreads();
+  if (threadIdx.x == 0)
+    gate_and_pick(g[0], n_experts, k, gate, renorm, topk_ids + (size_t)t * k, topk_w + (size_t)t * k, nullptr);
+}
+
+// h [T, hidden] float (updated), delta [T, hidden] bf16 or null, w the norm's weights (bf16 or float, or
+// null), out [T, hidden] bf16, wr [n_experts, hidden] (bf16 or float): what sharpi_add_rmsnorm then
+// sharpi_router_topk give, in one launch.
+SHARPI_EXPORT int sharpi_add_rmsnorm_router(float* h, const void* delta, const void* w, int w_dtype, void* out,
+                                            int n_tokens, int hidden, float eps, const void* wr, int wr_dtype,
+                                            int* topk_ids, float* topk_w, int n_experts, int k, int gate,
+                                            int renorm, hipStream_t stream) {
+  if (n_tokens <= 0) return SHARPI_OK;
+  if (hidden <= 0 || (hidden & 7) || hidden > kFusedMaxHidden || !(eps > 0.f)) return SHARPI_ERR_ARG;
+  if (n_experts <= 0 || n_experts > kMaxExperts || k <= 0 || k > n_experts || gate < 0 || gate > 1) return SHARPI_ERR_ARG;
+  dim3 grid(n_tokens), block(1024);
+#define FUSED_LAUNCH(TWV, TWRV)                                                                                  \
+  add_rmsnorm_router_kernel<TWV, TWRV><<<grid, block, 0, stream>>>(h, (const bf16_t*)delta, (const TWV*)w,      \
+                                                                   (bf16_t*)out, hidden, eps, (const TWRV*)wr,  \
+                                                                   topk_ids, topk_w, n_experts, k, gate, renorm)
+  const bool wf = w == nullptr || w_dtype == DT_F32;
+  if (!wf && w_dtype != DT_BF16) return SHARPI_ERR_ARG;
+  if (wr_dtype == DT_BF16) {
+    if (wf) FUSED_LAUNCH(float, bf16_t); else FUSED_LAUNCH(bf16_t, bf16_t);
+  } else if (wr_dtype == DT_F32) {
+    if (wf) FUSED_LAUNCH(float, float); else FUSED_LAUNCH(bf16_t, float);
+  } else {
+    return SHARPI_ERR_ARG;
+  }
+#undef FUSED_LAUNCH
+  SHARPI_CHECK_LAUNCH();
+  return SHARPI_OK;
 }
 
 SHARPI_EXPORT int sharpi_router_topk(const void* x, int x_dtype, const void* wr, int w_dtype, int* topk_ids,

@@ -580,6 +580,40 @@ def router_topk(x: torch.Tensor, wr: torch.Tensor, k: int, gate: int = GATE_SIGM
     return (ids, wts, gates) if want_gates else (ids, wts)
 
 
+FUSED_NORM_ROUTER_MAX_HIDDEN = 8192   # csrc/router.hip kFusedMaxHidden
+
+
+def norm_router_ok(h: torch.Tensor, delta, out_dtype: torch.dtype) -> bool:
+    """Can add_rmsnorm_router take this step?  (a plain bfloat16 delta or none, a width the
+    kernel's LDS row holds)"""
+    return (out_dtype == torch.bfloat16 and h.shape[1] % 8 == 0 and h.shape[1] <= FUSED_NORM_ROUTER_MAX_HIDDEN
+            and (delta is None or (isinstance(delta, torch.Tensor) and delta.dtype == torch.bfloat16)))
+
+
+def add_rmsnorm_router(h: torch.Tensor, delta: Optional[torch.Tensor], weight: Optional[torch.Tensor], eps: float,
+                       wr: torch.Tensor, k: int, gate: int = GATE_SIGMOID, renorm: bool = False):
+    """add_rmsnorm (the sum goes back into h) and router_topk on its output in one launch, for a
+    few tokens: returns (normalised rows bfloat16 [T, H], ids [T, k], weights [T, k]), the bits
+    of the two kernels in a row."""
+    _dev(h, delta, weight, wr)
+    _need(h.dim() == 2 and h.dtype == torch.float32, "add_rmsnorm_router: h must be float32 [T, H]")
+    T, H = h.shape
+    _need(norm_router_ok(h, delta, torch.bfloat16), "add_rmsnorm_router: bfloat16 rows of a width the kernel holds only")
+    if delta is not None:
+        _need(tuple(delta.shape) == (T, H) and delta.is_contiguous(), "add_rmsnorm_router: delta must be [T, H]")
+    if weight is not None:
+        _need(weight.shape == (H,), f"add_rmsnorm_router: weight {tuple(weight.shape)} vs width {H}")
+    _need(wr.dim() == 2 and wr.shape[1] == H, "add_rmsnorm_router: wr [E, H]")
+    E = wr.shape[0]
+    out = torch.empty(T, H, dtype=torch.bfloat16, device=h.device)
+    ids = torch.empty(T, k, dtype=torch.int32, device=h.device)
+    wts = torch.empty(T, k, dtype=torch.float32, device=h.device)
+    _run("sharpi_add_rmsnorm_router", _ptr(h), _ptr(delta), _ptr(weight), _code(weight.dtype) if weight is not None else 0,
+         _ptr(out), T, H, float(eps), _ptr(wr), _code(wr.dtype), _ptr(ids), _ptr(wts), E, k, gate, 1 if renorm else 0,
+         _stream())
+    return out, ids, wts
+
+
 GROUPED_TILE_ROWS = _lib.GROUPED_TILE_ROWS   # rows per tile of the grouped product (csrc/gemm_grouped.hip GM)
 SORTED_TILE_LISTS = _lib.SORTED_TILE_LISTS   # tile lists up to this long come tallest first (csrc/router.hip kSortTiles)
 

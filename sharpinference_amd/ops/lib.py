@@ -30,6 +30,7 @@ _SIGNATURES = {
     "sharpi_gemm_skinny": [P, P, P, I, I, I, I, P, P, I, I, I, I, I, P],
     "sharpi_gemm_skinny_swiglu": [P, P, P, I, I, I, P, P, I, P, I, I, I, I, P],
     "sharpi_gemm_skinny_picked": [P, P, P, I, I, I, P, P, I, I, I, I, I, I, I, I, I, P],
+    "sharpi_add_rmsnorm_router": [P, P, P, I, P, I, I, F, P, I, P, P, I, I, I, I, P],
     "sharpi_router_topk": [P, I, P, I, P, P, P, I, I, I, I, I, I, P],
     "sharpi_moe_permute": [P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, P],
     "sharpi_gemm_grouped": [P, I, P, P, I, I, I, I, P, P, P, P, P, I, I, P],

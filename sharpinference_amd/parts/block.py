@@ -11,7 +11,9 @@ class PreNormBlock(Part):
     (reference: src/SharpInference.Engine/ForwardPass.cs:1557-1561, 1690-1714).
 
     The additions are folded into the norm that follows them (see ResidualStream), so a block
-    leaves its feed-forward output pending for the next block's first norm.  Names of the four
+    leaves its feed-forward output pending for the next block's first norm.  A feed-forward that
+    has ``forward_from_stream(stream, norm, ctx)`` is handed the stream and the second norm instead
+    of normalised rows (it must leave the stream as the norm would have).  Names of the four
     parts in the weight file are arguments."""
 
     def __init__(self, norm1: Part, mixer: Part, norm2: Part, ffn: Part, names=None):
@@ -40,5 +42,9 @@ class PreNormBlock(Part):
     def forward(self, stream: ResidualStream, ctx: StepContext, cache: LayerCache) -> None:
         n = self.norm1.forward(stream, ctx.act_dtype)
         stream.pending = self.mixer.forward(n, ctx, cache)
-        n = self.norm2.forward(stream, ctx.act_dtype)
-        stream.pending = self.ffn.forward(n, ctx)
+        from_stream = getattr(self.ffn, "forward_from_stream", None)
+        if from_stream is not None:    # a feed-forward that may fuse the norm with work of its own
+            stream.pending = from_stream(stream, self.norm2, ctx)
+        else:
+            n = self.norm2.forward(stream, ctx.act_dtype)
+            stream.pending = self.ffn.forward(n, ctx)

@@ -6,7 +6,8 @@ from typing import Dict, Optional
 import torch
 
 from .. import ops
-from .base import ParamSpec, Part, StepContext, TensorSource
+from .base import ParamSpec, Part, ResidualStream, StepContext, TensorSource
+from .norm import RMSNorm
 
 
 def _fuse_rows(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
@@ -138,21 +139,43 @@ class MoESwiGLU(Part):
         self.w_gate_up = ops.PackedWeight(gu, None) if pack else gu
         self.w_down = ops.PackedWeight(dn, None) if pack else dn
 
+    def _few_tokens(self, T: int, ctx: StepContext) -> bool:
+        """A few decode tokens in bfloat16 with the shared expert in the experts' tensors: the
+        two products find their rows from the picks themselves."""
+        packed = isinstance(self.w_gate_up, ops.PackedWeight)
+        return (self.merged and T <= self.MERGE_MAX_TOKENS and ctx.act_dtype == torch.bfloat16
+                and ops.picked_ok(T, self.k, 2 * self.inter, self.hidden, True, packed)
+                and ops.picked_ok(T, self.k, self.hidden, self.inter, False, packed))
+
+    def _picked(self, x: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, ctx: StepContext):
+        """No sorting kernel: pair by pair in the picks' own order, the shared expert's rows after them."""
+        T = x.shape[0]
+        trace = ctx.extras.get("router_trace")
+        if trace is not None:
+            trace.append((ids, wts))
+        act = ops.gemm_skinny_picked(x, self.w_gate_up, ids, wts, True, True, True, ctx.act_dtype)
+        y = ops.gemm_skinny_picked(act, self.w_down, ids, None, True, False, False, ctx.act_dtype)
+        return ops.ExpertSum(y, ops.counting(T * self.k, x.device), y[T * self.k:], T, self.k)
+
+    def forward_from_stream(self, stream: ResidualStream, norm: Part, ctx: StepContext):
+        """The block's second half from the residual stream: normalise and feed forward.  With a
+        few decode tokens the norm and the router are one launch (the bits of the two)."""
+        T = stream.h.shape[0]
+        if (self._few_tokens(T, ctx) and isinstance(norm, RMSNorm)
+                and ops.norm_router_ok(stream.h, stream.pending, ctx.act_dtype)):
+            x, ids, wts = ops.add_rmsnorm_router(stream.h, stream.pending, norm.weight, norm.eps, self.w_router, self.k,
+                                                 self.gate, self.renormalise)
+            stream.pending = None
+            return self._picked(x, ids, wts, ctx)
+        return self.forward(norm.forward(stream, ctx.act_dtype), ctx)
+
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         T = x.shape[0]
         merge = self.merged and T <= self.MERGE_MAX_TOKENS and ctx.act_dtype == torch.bfloat16
         trace = ctx.extras.get("router_trace")
-        packed = isinstance(self.w_gate_up, ops.PackedWeight)
-        if (merge and ops.picked_ok(T, self.k, 2 * self.inter, self.hidden, True, packed)
-                and ops.picked_ok(T, self.k, self.hidden, self.inter, False, packed)):
-            # a few decode tokens: the two products find their rows from the picks themselves (no
-            # sorting kernel), pair by pair in the picks' own order, the shared expert's rows after them
+        if self._few_tokens(T, ctx):
             ids, wts = ops.router_topk(x, self.w_router, self.k, self.gate, self.renormalise)
-            if trace is not None:
-                trace.append((ids, wts))
-            act = ops.gemm_skinny_picked(x, self.w_gate_up, ids, wts, True, True, True, ctx.act_dtype)
-            y = ops.gemm_skinny_picked(act, self.w_down, ids, None, True, False, False, ctx.act_dtype)
-            return ops.ExpertSum(y, ops.counting(T * self.k, x.device), y[T * self.k:], T, self.k)
+            return self._picked(x, ids, wts, ctx)
         ids, wts, rt = ops.route(x, self.w_router, self.k, self.gate, self.renormalise, shared_group=merge)
         if trace is not None:      # the picks of this step, layer by layer (reference: ForwardPass.cs:2042-2056)
             trace.append((ids, wts))

@@ -329,6 +329,27 @@ def test_router_and_permute(T, E, k, H, dtype):
     assert tiles == want
 
 
+@pytest.mark.parametrize("T,H,E,k", [(1, 5120, 16, 1), (8, 5120, 16, 1), (16, 256, 5, 2), (3, 8192, 128, 4), (5, 136, 3, 3)])
+@pytest.mark.parametrize("w_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("with_delta", [True, False])
+def test_norm_and_router_in_one_launch_equal_the_two_kernels(T, H, E, k, w_dtype, with_delta):
+    """Residual add + RMSNorm + router for a few tokens in one launch: the residual stream, the
+    normalised rows, the picks and their weights are the bits of the two kernels in a row."""
+    ops = _ops()
+    h0 = _rand(T, H, seed=T + H)
+    delta = _rand(T, H, dtype=torch.bfloat16, scale=0.5, seed=H) if with_delta else None
+    wn = (torch.rand(H, generator=torch.Generator().manual_seed(E)) + 0.5).to(w_dtype).to(DEV)
+    wr = _rand(E, H, dtype=w_dtype, scale=0.3, seed=E + 1)
+    for gate, renorm in ((ops.GATE_SIGMOID, False), (ops.GATE_SOFTMAX, True)):
+        ha, hb = h0.clone(), h0.clone()
+        xa = ops.add_rmsnorm(ha, delta, wn, 1e-5, torch.bfloat16)
+        ia, wa = ops.router_topk(xa, wr, k, gate, renorm)
+        xb, ib, wb = ops.add_rmsnorm_router(hb, delta, wn, 1e-5, wr, k, gate, renorm)
+        assert torch.equal(ha, hb) and torch.equal(xa, xb) and torch.equal(ia, ib) and torch.equal(wa, wb)
+    if with_delta:
+        assert not torch.equal(ha, h0)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H", [5120, 136, 75])
 def test_router_rows_do_not_depend_on_the_batch(dtype, H):
