@@ -140,22 +140,26 @@ class MoESwiGLU(Part):
         self.w_down = ops.PackedWeight(dn, None) if pack else dn
 
     def _few_tokens(self, T: int, ctx: StepContext) -> bool:
-        """A few decode tokens in bfloat16 with the shared expert in the experts' tensors: the
-        two products find their rows from the picks themselves."""
+        """A few decode tokens in bfloat16 (at most 64 picks): the experts' two products find their
+        rows from the picks themselves."""
         packed = isinstance(self.w_gate_up, ops.PackedWeight)
-        return (self.merged and T <= self.MERGE_MAX_TOKENS and ctx.act_dtype == torch.bfloat16
+        return (ctx.act_dtype == torch.bfloat16 and self.w_gate_up.dtype == torch.bfloat16
                 and ops.picked_ok(T, self.k, 2 * self.inter, self.hidden, True, packed)
                 and ops.picked_ok(T, self.k, self.hidden, self.inter, False, packed))
 
     def _picked(self, x: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, ctx: StepContext):
-        """No sorting kernel: pair by pair in the picks' own order, the shared expert's rows after them."""
+        """No sorting kernel: pair by pair in the picks' own order.  With up to MERGE_MAX_TOKENS
+        tokens the shared expert rides along as one more group of the same two launches (its rows
+        after the pairs'); with more it goes through the library."""
         T = x.shape[0]
         trace = ctx.extras.get("router_trace")
-        if trace is not None:
+        if trace is not None:      # the picks of this step, layer by layer (reference: ForwardPass.cs:2042-2056)
             trace.append((ids, wts))
-        act = ops.gemm_skinny_picked(x, self.w_gate_up, ids, wts, True, True, True, ctx.act_dtype)
-        y = ops.gemm_skinny_picked(act, self.w_down, ids, None, True, False, False, ctx.act_dtype)
-        return ops.ExpertSum(y, ops.counting(T * self.k, x.device), y[T * self.k:], T, self.k)
+        along = self.merged and T <= self.MERGE_MAX_TOKENS
+        shared = None if along or self.shared is None else self.shared.forward(x, ctx)
+        act = ops.gemm_skinny_picked(x, self.w_gate_up, ids, wts, along, True, True, ctx.act_dtype)
+        y = ops.gemm_skinny_picked(act, self.w_down, ids, None, along, False, False, ctx.act_dtype)
+        return ops.ExpertSum(y, ops.counting(T * self.k, x.device), y[T * self.k:] if along else shared, T, self.k)
 
     def forward_from_stream(self, stream: ResidualStream, norm: Part, ctx: StepContext):
         """The block's second half from the residual stream: normalise and feed forward.  With a
@@ -171,11 +175,11 @@ class MoESwiGLU(Part):
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         T = x.shape[0]
-        merge = self.merged and T <= self.MERGE_MAX_TOKENS and ctx.act_dtype == torch.bfloat16
         trace = ctx.extras.get("router_trace")
         if self._few_tokens(T, ctx):
             ids, wts = ops.router_topk(x, self.w_router, self.k, self.gate, self.renormalise)
             return self._picked(x, ids, wts, ctx)
+        merge = self.merged and T <= self.MERGE_MAX_TOKENS and ctx.act_dtype == torch.bfloat16
         ids, wts, rt = ops.route(x, self.w_router, self.k, self.gate, self.renormalise, shared_group=merge)
         if trace is not None:      # the picks of this step, layer by layer (reference: ForwardPass.cs:2042-2056)
             trace.append((ids, wts))
