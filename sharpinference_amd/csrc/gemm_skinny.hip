@@ -348,18 +348,23 @@ SHARPI_EXPORT int sharpi_gemm_skinny_picked(const void* x, const void* W, void* 
   if (groups > 65535) return SHARPI_ERR_ARG;
   const int M = n_pairs + (shared ? n_pairs / k : 0);
   const Picks pk = {ids, w, n_pairs, k, n_experts, gather};
+  // an expert has at most n_pairs rows: one, two or four blocks of sixteen rows against one stream of its weights
+  const int MB = n_pairs <= 16 ? 1 : n_pairs <= 32 ? 2 : 4;
   // group_offsets is not read in this form; the pointer only has to be non-null for the grid's sake
-#define SKP(RR, WW, ACTV)                                                                                       \
-  if (R == RR && NW == WW && (act != 0) == ACTV)                                                                \
-  return packed ? launch_skinny<RR, 1, WW, ACTV, true>(x, W, out, out_dtype, M, N, K, nullptr, ids, groups,     \
-                                                       nullptr, stream, pk)                                     \
-                : launch_skinny<RR, 1, WW, ACTV, false>(x, W, out, out_dtype, M, N, K, nullptr, ids, groups,    \
-                                                        nullptr, stream, pk)
+#define SKP1(RR, WW, ACTV, MBV, PK) \
+  return launch_skinny<RR, MBV, WW, ACTV, PK>(x, W, out, out_dtype, M, N, K, nullptr, ids, groups, nullptr, stream, pk)
+#define SKP(RR, WW, ACTV)                                                      \
+  if (R == RR && NW == WW && (act != 0) == ACTV) {                             \
+    if (MB == 1) { if (packed) SKP1(RR, WW, ACTV, 1, true); else SKP1(RR, WW, ACTV, 1, false); } \
+    if (MB == 2) { if (packed) SKP1(RR, WW, ACTV, 2, true); else SKP1(RR, WW, ACTV, 2, false); } \
+    if (packed) SKP1(RR, WW, ACTV, 4, true); else SKP1(RR, WW, ACTV, 4, false); \
+  }
   SKP(1, 4, false); SKP(1, 8, false); SKP(1, 16, false);
   SKP(2, 4, false); SKP(2, 8, false);
   SKP(4, 4, false); SKP(4, 8, false);
   SKP(2, 4, true); SKP(2, 8, true);
   SKP(4, 4, true); SKP(4, 8, true);
+#undef SKP1
 #undef SKP
   return SHARPI_ERR_ARG;
 }

@@ -444,7 +444,7 @@ def test_gemm_grouped(T, E, k, N, K):
 
 
 @pytest.mark.parametrize("T,E,k,I,K", [(1, 16, 1, 256, 256), (8, 16, 1, 8192, 640), (16, 4, 4, 128, 384), (5, 3, 2, 128, 128),
-                                       (16, 2, 1, 384, 256)])
+                                       (16, 2, 1, 384, 256), (48, 2, 1, 128, 128), (64, 16, 1, 256, 256), (27, 5, 1, 128, 256)])
 @pytest.mark.parametrize("packed", [False, True])
 def test_picked_products_equal_the_sorted_ones(T, E, k, I, K, packed):
     """The few-rows products that find their rows from the router's picks give, pair by pair, the
