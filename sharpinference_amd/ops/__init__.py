@@ -587,7 +587,8 @@ def norm_router_ok(h: torch.Tensor, delta, out_dtype: torch.dtype) -> bool:
     """Can add_rmsnorm_router take this step?  (a plain bfloat16 delta or none, a width the
     kernel's LDS row holds)"""
     return (out_dtype == torch.bfloat16 and h.shape[1] % 8 == 0 and h.shape[1] <= FUSED_NORM_ROUTER_MAX_HIDDEN
-            and (delta is None or (isinstance(delta, torch.Tensor) and delta.dtype == torch.bfloat16)))
+            and (delta is None or (isinstance(delta, torch.Tensor) and delta.dtype == torch.bfloat16
+                                   and delta.is_contiguous() and tuple(delta.shape) == tuple(h.shape))))
 
 
 def add_rmsnorm_router(h: torch.Tensor, delta: Optional[torch.Tensor], weight: Optional[torch.Tensor], eps: float,
