@@ -5,8 +5,9 @@ src/SharpInference.Cli/RunCommand.cs:23-300 for the options, 1907-1911 for the c
 Options keep the reference's names and meanings where it has them: -m/--model, -p/--prompt,
 -f/--file, -n/--n-predict (512), --temp (0.7; 0 = greedy), --top-k (40), --top-p (0.95),
 --min-p (0.05), -s/--seed (-1 = from the clock), -c/--ctx-size (0 = the model's), --kv-type,
---repeat-penalty (1.1), --repeat-last-n, --frequency-penalty, --presence-penalty,
---verbose-prompt.  There is no tokenizer in this engine: a prompt is a list of token ids
+--repeat-penalty/--rep-penalty (1.1), --repeat-last-n, --frequency-penalty, --presence-penalty,
+--verbose-prompt, --no-display-prompt, --device (an index or a name), -g/--ngl (accepted: every
+layer is on the GPU), --backend (auto).  There is no tokenizer in this engine: a prompt is a list of token ids
 (``--prompt-ids 1,2,3``; -p/-f take the same comma- or space-separated ids) or ``--prompt-len N``
 random ids.  ``-m`` names a model folder (config.json + model.safetensors); with
 ``--random-weights`` the folder needs only config.json.
@@ -29,6 +30,20 @@ def _ids(text: str) -> List[int]:
         raise SystemExit("this engine has no tokenizer: give the prompt as token ids, e.g. -p '1,2,3'") from None
 
 
+def parse_device(text: Optional[str]) -> str:
+    """--device as the reference takes it (an index or a name, reference:
+    src/SharpInference.Cli/RunCommand.cs:99-102) -> a torch device string; 'none' (the CPU) is refused."""
+    if text is None or text == "" or text.lower() == "auto":
+        return "cuda:0"
+    t = text.strip().lower()
+    if t == "none" or t == "cpu":
+        raise SystemExit("--device none asks for the CPU: this engine has no CPU path")
+    m = re.fullmatch(r"(?:cuda:?|hip:?|gpu:?)?(\d+)", t)
+    if not m:
+        raise SystemExit(f"--device {text!r}: give an index (0, 1, ...) or a name such as cuda:0")
+    return f"cuda:{int(m.group(1))}"
+
+
 def build_parser() -> argparse.ArgumentParser:
     ap = argparse.ArgumentParser(prog="sharpi-cli", description="Generate with a Llama 4 model folder on one MI355X.")
     ap.add_argument("-m", "--model", required=True, help="model folder (config.json, model.safetensors)")
@@ -44,13 +59,17 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("-s", "--seed", type=int, default=-1, help="sampling seed; -1 = from the clock")
     ap.add_argument("-c", "--ctx-size", type=int, default=0, help="longest sequence; 0 = the model's")
     ap.add_argument("--kv-type", default=None, choices=["fp32", "bf16"], help="cache dtype (follows --dtype)")
-    ap.add_argument("--repeat-penalty", type=float, default=1.1)
+    ap.add_argument("--repeat-penalty", "--rep-penalty", dest="repeat_penalty", type=float, default=1.1)
     ap.add_argument("--repeat-last-n", type=int, default=256)
     ap.add_argument("--frequency-penalty", type=float, default=0.0)
     ap.add_argument("--presence-penalty", type=float, default=0.0)
     ap.add_argument("--verbose-prompt", action="store_true", help="print the prompt's token ids")
     ap.add_argument("--no-display-prompt", action="store_true")
     ap.add_argument("--stop-ids", default="", help="token ids that end generation")
+    ap.add_argument("-g", "--ngl", "--n-gpu-layers", "--gpu-layers", dest="n_gpu_layers", type=int, default=-1,
+                    help="accepted for the reference's sake: every layer runs on the GPU (-1 or any count > 0; 0 is refused)")
+    ap.add_argument("--device", default=None, help="GPU to run on: an index (0, 1, ...) or a name (cuda:0); default 0")
+    ap.add_argument("--backend", default="auto", choices=["auto", "hip"], help="there is one backend: HIP on gfx950")
     # this engine's own
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32", "bfloat16", "float32"])
     ap.add_argument("--random-weights", action="store_true", help="seeded random weights (folder needs config.json only)")
@@ -70,6 +89,9 @@ def main(argv: Optional[List[str]] = None) -> int:
     from .sampling.params import SamplingParams
 
     dtype = {"bf16": "bfloat16", "fp32": "float32"}.get(args.dtype, args.dtype)
+    device = parse_device(args.device)
+    if args.n_gpu_layers == 0:
+        raise SystemExit("-g 0 asks for the CPU: this engine has no CPU path (leave -g out, or give -1)")
     if args.kv_type and {"bf16": "bfloat16", "fp32": "float32"}[args.kv_type] != dtype:
         raise SystemExit("--kv-type must equal --dtype: the cache is stored in the compute dtype")
     cfg = load_config(args.model)
@@ -84,7 +106,7 @@ def main(argv: Optional[List[str]] = None) -> int:
     else:
         raise SystemExit("no prompt: give -p / --prompt-ids / -f / --prompt-len (there is no interactive mode)")
     ctx = args.ctx_size or None
-    common = dict(dtype=dtype, device="cuda:0", max_model_len=ctx, max_num_seqs=max(args.max_num_seqs, args.parallel),
+    common = dict(dtype=dtype, device=device, max_model_len=ctx, max_num_seqs=max(args.max_num_seqs, args.parallel),
                   max_tokens_per_step=args.max_tokens_per_step, kv_tokens=args.kv_tokens, page_size=args.page_size)
     if args.random_weights:
         eng = Engine(config=cfg, weight_seed=args.weight_seed, **common)

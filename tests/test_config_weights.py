@@ -213,3 +213,23 @@ def test_random_model_command_writes_a_folder_that_loads(tmp_path):
     for n, info in index.items():
         assert tuple(info.shape) == tuple(specs[n].shape), n
         assert info.dtype == (torch.float32 if n.endswith("norm.weight") else torch.bfloat16), n
+
+
+def test_command_line_takes_the_reference_s_option_names():
+    """Names and defaults of the reference's options (src/SharpInference.Cli/RunCommand.cs:50-210)."""
+    from sharpinference_amd.cli import build_parser, parse_device
+
+    a = build_parser().parse_args(["-m", "X", "-p", "1 2"])
+    assert (a.temp, a.top_k, a.top_p, a.min_p, a.n_predict, a.seed, a.ctx_size) == (0.7, 40, 0.95, 0.05, 512, -1, 0)
+    assert (a.repeat_penalty, a.frequency_penalty, a.presence_penalty, a.backend, a.n_gpu_layers) == (1.1, 0.0, 0.0, "auto", -1)
+    b = build_parser().parse_args(["--model", "X", "--prompt", "1", "--rep-penalty", "1.3", "--ngl", "99", "--device", "CUDA0",
+                                   "--n-predict", "7", "--ctx-size", "256", "--no-display-prompt", "--verbose-prompt"])
+    assert b.repeat_penalty == 1.3 and b.n_gpu_layers == 99 and b.n_predict == 7 and b.ctx_size == 256
+    assert parse_device(b.device) == "cuda:0" and parse_device("1") == "cuda:1" and parse_device(None) == "cuda:0"
+    for bad in ("none", "Vulkan1x"):
+        try:
+            parse_device(bad)
+        except SystemExit:
+            pass
+        else:
+            raise AssertionError(bad)
