@@ -83,3 +83,5 @@ SHARPI_EXPORT int sharpi_gemm_skinny_picked(const void* x, const void* W, void* 
 #undef SKP
   return SHARPI_ERR_ARG;
 }
+
+SHARPI_EXPORT int sharpi_gemm_skinny_max_picked() { return kMaxPicked; }

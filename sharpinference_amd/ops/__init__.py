@@ -461,7 +461,7 @@ def gemm_skinny_swiglu(x: torch.Tensor, w, offsets: torch.Tensor, a_rows: Option
     return out
 
 
-PICKED_MAX_PAIRS = 64   # (token, pick) pairs of the picked form: one ballot of a wave (csrc/gemm_skinny_kernel.h kMaxPicked)
+PICKED_MAX_PAIRS = _lib.PICKED_MAX_PAIRS   # (token, pick) pairs of the picked form: one ballot of a wave (csrc/gemm_skinny_kernel.h kMaxPicked)
 
 _COUNTING: dict = {}    # per device: 0, 1, 2, ... (the places of pairs that are stored in their own order)
 
@@ -580,7 +580,7 @@ def router_topk(x: torch.Tensor, wr: torch.Tensor, k: int, gate: int = GATE_SIGM
     return (ids, wts, gates) if want_gates else (ids, wts)
 
 
-FUSED_NORM_ROUTER_MAX_HIDDEN = 8192   # csrc/router.hip kFusedMaxHidden
+FUSED_NORM_ROUTER_MAX_HIDDEN = _lib.FUSED_NORM_ROUTER_MAX_HIDDEN   # csrc/router.hip kFusedMaxHidden
 
 
 def norm_router_ok(h: torch.Tensor, delta, out_dtype: torch.dtype) -> bool:
