@@ -4,8 +4,8 @@
 // A block owns a tile of up to 128 consecutive tokens of one entry and one query head; each of its
 // four waves takes 32 of the tokens.  The block walks the keys its rows can see in 32-key chunks
 // (two 16-key blocks aligned to absolute positions, so a block never straddles a page); a chunk's
-// keys and values are fetched from the cache once, staged in LDS (double-buffered, one chunk
-// ahead) and read from there by all four waves.  As in the decode kernel everything is transposed:
+// keys and values are fetched from the cache once, staged in LDS (double-buffered; two chunks
+// are on their way through registers) and read from there by all four waves.  As in the decode kernel everything is transposed:
 //   S^T[key, q]  = K[key, :] . Q[q, :]          A = K block, B = Q^T
 //   O^T[d, q]   += V^T[d, key] * P^T[key, q]    A = V^T block (values are stored transposed
 //                                               inside a page), B = P^T
@@ -17,6 +17,8 @@
 // log2 e, the hardware's exp2).
 // The keys of a query are always visited in the same blocks, whatever the portion it arrived in,
 // so its sums do not depend on how the prompt was cut.
+#include <type_traits>
+
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -150,8 +152,9 @@ __global__ __launch_bounds__(kPreWaves* kWave, HD <= 128 ? 2 : 1) void attn_pref
   // keys are masked, its values are finite and meet probabilities of zero).  The compiler counts
   // outstanding loads statically; one load behind a branch and every wait in the loop becomes a
   // wait for all loads, the chunk in flight included.
-  u32x4 kst[NST], vst[NSV][2];
-  auto fetch = [&](int b) {
+  u32x4 kst[2][NST], vst[2][NSV][2];   // two chunks on their way
+  auto fetch = [&](int b, auto set_tag) {
+    constexpr int set = decltype(set_tag)::value;
     long long kbase[2], vbase[2];
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
@@ -165,7 +168,7 @@ __global__ __launch_bounds__(kPreWaves* kWave, HD <= 128 ? 2 : 1) void attn_pref
     for (int i = 0; i < NST; ++i) {
       const int piece = min(tid + i * kPreWaves * kWave, PIECES - 1);
       const int key = piece / (HD / 8), dcol = (piece % (HD / 8)) * 8;     // K: 32 keys x HD
-      kst[i] = *reinterpret_cast<const u32x4*>(k_cache + kbase[key >> 4] + (size_t)(key & 15) * HD + dcol);
+      kst[set][i] = *reinterpret_cast<const u32x4*>(k_cache + kbase[key >> 4] + (size_t)(key & 15) * HD + dcol);
     }
 #pragma unroll
     for (int i = 0; i < NSV; ++i) {
@@ -174,16 +177,18 @@ __global__ __launch_bounds__(kPreWaves* kWave, HD <= 128 ? 2 : 1) void attn_pref
       const int d = pair >> 1, half = pair & 1;
 #pragma unroll
       for (int blk = 0; blk < 2; ++blk)
-        vst[i][blk] = *reinterpret_cast<const u32x4*>(v_cache + vbase[blk] + (size_t)d * page_size + half * 8);
+        vst[set][i][blk] = *reinterpret_cast<const u32x4*>(v_cache + vbase[blk] + (size_t)d * page_size + half * 8);
     }
   };
-  auto stash = [&](int buf) {
+  auto stash = [&](auto set_tag) {   // register set `set` goes to LDS buffer `set`
+    constexpr int set = decltype(set_tag)::value;
+    constexpr int buf = set;
 #pragma unroll
     for (int i = 0; i < NST; ++i) {
       const int piece = tid + i * kPreWaves * kWave;
       if (piece < PIECES) {
         const int key = piece / (HD / 8), dcol = (piece % (HD / 8)) * 8;
-        *reinterpret_cast<u32x4*>(&Ks[buf][key][k_col<HD>(key, dcol)]) = kst[i];
+        *reinterpret_cast<u32x4*>(&Ks[buf][key][k_col<HD>(key, dcol)]) = kst[set][i];
       }
     }
 #pragma unroll
@@ -194,26 +199,32 @@ __global__ __launch_bounds__(kPreWaves* kWave, HD <= 128 ? 2 : 1) void attn_pref
         // group g of the second product wants side by side.  The thread's keys are those of the
         // groups g = 2*half and 2*half + 1.
         const int d = pair >> 1, half = pair & 1;
-        const u32x4 a = vst[i][0], b = vst[i][1];
+        const u32x4 a = vst[set][i][0], b = vst[set][i][1];
         *reinterpret_cast<u32x4*>(&Vs[buf][v_row(d)][v_col(d, (2 * half) * 8)]) = u32x4{a[0], a[1], b[0], b[1]};
         *reinterpret_cast<u32x4*>(&Vs[buf][v_row(d)][v_col(d, (2 * half + 1) * 8)]) = u32x4{a[2], a[3], b[2], b[3]};
       }
     }
   };
 
-  fetch(b_first);
-  stash(0);
+  using Set0 = std::integral_constant<int, 0>;
+  using Set1 = std::integral_constant<int, 1>;
+  fetch(b_first, Set0{});
+  fetch(b_first + 2 <= b_last ? b_first + 2 : b_first, Set1{});
+  stash(Set0{});
   __syncthreads();
-  int buf = 0;
-  for (int b = b_first; b <= b_last; b += 2, buf ^= 1) {
-    const bool more = b + 2 <= b_last;
-    const int b_next = more ? b + 2 : b;                     // after the last chunk: the same one again, unused
-    if ((((b_next + 1) << 4) / page_size) - pv_base >= 2 * kWave - 1) {   // the pages held run out: move on by 64
+  // One chunk: the chunk in LDS buffer `par` is multiplied while the chunk after it waits in register set
+  // par ^ 1 and the one after that is requested into set par (two chunks on their way: the keys
+  // and values of a prompt were just written by another kernel and come from memory, not from cache).
+  auto one_chunk = [&](int b, auto par_tag) {
+    constexpr int par = decltype(par_tag)::value;
+    constexpr int buf = par;
+    const int b_fetch = b + 4 <= b_last ? b + 4 : b;            // beyond the last chunk: this one again, unused
+    if ((((b_fetch + 1) << 4) / page_size) - pv_base >= 2 * kWave - 1) {   // the pages held run out: move on by 64
       pv = pv_next;
       pv_base += kWave;
       pv_next = load_pages(pv_base + kWave);
     }
-    fetch(b_next);
+    fetch(b_fetch, par_tag);
     __builtin_amdgcn_sched_barrier(0);                       // the loads are issued here, not where they are used
     // does any row of this wave see a key of this chunk?
     const bool active = wave_has_rows && (b << 4) <= wave_last && ((b + 2) << 4) > wave_first;
@@ -318,8 +329,13 @@ __global__ __launch_bounds__(kPreWaves* kWave, HD <= 128 ? 2 : 1) void attn_pref
       }
     }
     __builtin_amdgcn_sched_barrier(0);
-    stash(buf ^ 1);
+    stash(std::integral_constant<int, par ^ 1>{});
     __syncthreads();
+  };
+  for (int b = b_first; b <= b_last; b += 4) {
+    one_chunk(b, Set0{});
+    if (b + 2 > b_last) break;
+    one_chunk(b + 2, Set1{});
   }
 
 #pragma unroll
