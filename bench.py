@@ -175,12 +175,16 @@ def main() -> int:
     eng = build_engine(args.layers, max_batch, args.page_size, graphs=not args.no_graphs, gen_len=gen_len, prompt_len=P)
     cfg = eng.config
 
-    # prefill: one prompt (2,048 tokens) alone, once to warm up, once timed
+    # prefill: one prompt (2,048 tokens) alone, once to warm up, then three times timed
     prompt = [rng.randrange(cfg.vocab_size) for _ in range(P)]
     run_prefill(eng, "warm", prompt)
     eng.free_request("warm")
-    pre_s, _ = run_prefill(eng, "timed", prompt)
-    eng.free_request("timed")
+    times = []
+    for i in range(3):                                   # the median of three: a single run varies by a per cent or two
+        t, _ = run_prefill(eng, f"timed{i}", prompt)
+        eng.free_request(f"timed{i}")
+        times.append(t)
+    pre_s = sorted(times)[1]
     log(f"prefill {P} tokens: {pre_s * 1e3:.1f} ms")
     flops = prefill_flops(cfg, P, args.layers)
     prefill = {"value": P / pre_s, "tokens": P, "ms": pre_s * 1e3,
