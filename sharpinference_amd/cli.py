@@ -7,10 +7,13 @@ Options keep the reference's names and meanings where it has them: -m/--model, -
 --min-p (0.05), -s/--seed (-1 = from the clock), -c/--ctx-size (0 = the model's), --kv-type,
 --repeat-penalty/--rep-penalty (1.1), --repeat-last-n, --frequency-penalty, --presence-penalty,
 --verbose-prompt, --no-display-prompt, --device (an index or a name), -g/--ngl (accepted: every
-layer is on the GPU), --backend (auto).  There is no tokenizer in this engine: a prompt is a list of token ids
-(``--prompt-ids 1,2,3``; -p/-f take the same comma- or space-separated ids) or ``--prompt-len N``
-random ids.  ``-m`` names a model folder (config.json + model.safetensors); with
-``--random-weights`` the folder needs only config.json.
+layer is on the GPU), --backend (auto).  -p and -f take text if the model folder has a
+``tokenizer.json`` (the generated text is then printed as it comes); a prompt that is nothing
+but numbers, ``--prompt-ids 1,2,3``, and every prompt for a folder without a tokenizer, are
+token ids, and ``--prompt-len N`` makes N random ids.  Generation stops at the configuration's
+``eos_token_id`` (``--ignore-eos`` switches that off; ``--stop-ids`` adds more).  ``-m`` names
+a model folder (config.json + model.safetensors); with ``--random-weights`` the folder needs
+only config.json.
 """
 from __future__ import annotations
 
@@ -27,7 +30,17 @@ def _ids(text: str) -> List[int]:
     try:
         return [int(p) for p in parts]
     except ValueError:
-        raise SystemExit("this engine has no tokenizer: give the prompt as token ids, e.g. -p '1,2,3'") from None
+        raise SystemExit(f"token ids expected (comma or space separated numbers), got {text[:40]!r}") from None
+
+
+def prompt_ids(text: str, codec) -> List[int]:
+    """A prompt from the command line: numbers are token ids; anything else is text for the
+    folder's tokenizer."""
+    if re.fullmatch(r"[\d,\s]+", text) and re.search(r"\d", text):
+        return _ids(text)
+    if codec is None:
+        raise SystemExit("the model folder has no tokenizer.json: give the prompt as token ids, e.g. -p '1,2,3'")
+    return codec.encode(text)
 
 
 def parse_device(text: Optional[str]) -> str:
@@ -47,8 +60,9 @@ def parse_device(text: Optional[str]) -> str:
 def build_parser() -> argparse.ArgumentParser:
     ap = argparse.ArgumentParser(prog="sharpi-cli", description="Generate with a Llama 4 model folder on one MI355X.")
     ap.add_argument("-m", "--model", required=True, help="model folder (config.json, model.safetensors)")
-    ap.add_argument("-p", "--prompt", help="prompt as token ids (comma or space separated)")
-    ap.add_argument("-f", "--file", help="read the prompt's token ids from a file")
+    ap.add_argument("-p", "--prompt", help="prompt: text (the folder's tokenizer.json encodes it) or token ids "
+                                           "(comma or space separated numbers)")
+    ap.add_argument("-f", "--file", help="read the prompt (text or token ids) from a file")
     ap.add_argument("--prompt-ids", help="prompt as token ids (same as -p)")
     ap.add_argument("--prompt-len", type=int, help="a prompt of N random token ids")
     ap.add_argument("-n", "--n-predict", type=int, default=512, help="tokens to generate")
@@ -65,7 +79,8 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--presence-penalty", type=float, default=0.0)
     ap.add_argument("--verbose-prompt", action="store_true", help="print the prompt's token ids")
     ap.add_argument("--no-display-prompt", action="store_true")
-    ap.add_argument("--stop-ids", default="", help="token ids that end generation")
+    ap.add_argument("--stop-ids", default="", help="token ids that end generation, beside the model's eos_token_id")
+    ap.add_argument("--ignore-eos", action="store_true", help="do not stop at the model's eos_token_id")
     ap.add_argument("-g", "--ngl", "--n-gpu-layers", "--gpu-layers", dest="n_gpu_layers", type=int, default=-1,
                     help="accepted for the reference's sake: every layer runs on the GPU (-1 or any count > 0; 0 is refused)")
     ap.add_argument("--device", default=None, help="GPU to run on: an index (0, 1, ...) or a name (cuda:0); default 0")
@@ -95,11 +110,15 @@ def main(argv: Optional[List[str]] = None) -> int:
     if args.kv_type and {"bf16": "bfloat16", "fp32": "float32"}[args.kv_type] != dtype:
         raise SystemExit("--kv-type must equal --dtype: the cache is stored in the compute dtype")
     cfg = load_config(args.model)
+    from .text import TextCodec
+    codec = TextCodec.from_folder(args.model, cfg.bos_token_id)
     if args.file:
         with open(args.file) as f:
-            prompt = _ids(f.read())
-    elif args.prompt_ids or args.prompt:
-        prompt = _ids(args.prompt_ids or args.prompt)
+            prompt = prompt_ids(f.read(), codec)
+    elif args.prompt_ids:
+        prompt = _ids(args.prompt_ids)
+    elif args.prompt:
+        prompt = prompt_ids(args.prompt, codec)
     elif args.prompt_len:
         rng = random.Random(args.weight_seed)
         prompt = [rng.randrange(cfg.vocab_size) for _ in range(args.prompt_len)]
@@ -116,24 +135,28 @@ def main(argv: Optional[List[str]] = None) -> int:
     params = [SamplingParams(temperature=args.temp, top_k=args.top_k, top_p=args.top_p, min_p=args.min_p,
                              repetition_penalty=args.repeat_penalty, penalty_last_n=args.repeat_last_n,
                              frequency_penalty=args.frequency_penalty, presence_penalty=args.presence_penalty,
-                             max_new_tokens=args.n_predict, stop_token_ids=tuple(_ids(args.stop_ids)) if args.stop_ids else (),
+                             max_new_tokens=args.n_predict, stop_token_ids=() if args.ignore_eos else None,
+                             additional_stop_token_ids=tuple(_ids(args.stop_ids)) if args.stop_ids else (),
                              seed=seed + i) for i in range(args.parallel)]
     if args.verbose_prompt:
         print(f"prompt tokens ({len(prompt)}): {prompt}")
     elif not args.no_display_prompt:
-        print(" ".join(str(t) for t in prompt))
+        print(codec.decode(prompt) if codec else " ".join(str(t) for t in prompt))
     if args.parallel == 1:
         # one request: its tokens are printed as they come (the reference streams its chunks the same way)
         first = True
+        stream = codec.streamer() if codec else None
         for c in eng.generate_chunks([prompt], params):
             if c.kind == "token":
-                print(("" if first else " ") + str(c.token_id), end="", flush=True)
+                piece = stream.push(c.token_id) if stream else ("" if first else " ") + str(c.token_id)
+                print(piece, end="", flush=True)
                 first = False
             elif c.kind == "stop":
-                print(f"  ({c.finish_reason})", flush=True)
+                print((stream.flush() if stream else "") + f"  ({c.finish_reason})", flush=True)
     else:
         for i, r in enumerate(eng.generate([prompt] * args.parallel, params)):
-            print(f"[{i}] {' '.join(str(t) for t in r.token_ids)}  ({r.finish_reason})")
+            shown = codec.decode(r.token_ids) if codec else " ".join(str(t) for t in r.token_ids)
+            print(f"[{i}] {shown}  ({r.finish_reason})")
     st = eng.last_stats
     pre = st.prefill_tokens / st.prefill_seconds if st.prefill_seconds > 0 else 0.0
     dec = st.decode_tokens / st.decode_seconds if st.decode_seconds > 0 else 0.0

@@ -11,11 +11,23 @@ from __future__ import annotations
 import json
 import os
 from dataclasses import dataclass, fields
-from typing import Any, Dict
+from typing import Any, Dict, Optional, Tuple
 
 
 class ConfigError(ValueError):
     """A config.json that cannot describe a model: the message names the key."""
+
+
+def special_tokens_from(src: Dict[str, Any]) -> Dict[str, Any]:
+    """eos_token_id (absent, one id or a list of ids) and bos_token_id of a config.json, as the
+    keyword arguments of a configuration class."""
+    eos = src.get("eos_token_id")
+    try:
+        ids = () if eos is None else tuple(int(t) for t in eos) if isinstance(eos, (list, tuple)) else (int(eos),)
+        bos = None if src.get("bos_token_id") is None else int(src["bos_token_id"])
+    except (TypeError, ValueError):
+        raise ConfigError(f"eos_token_id / bos_token_id must be token ids (got {eos!r}, {src.get('bos_token_id')!r})") from None
+    return {"eos_token_ids": ids, "bos_token_id": bos}
 
 
 @dataclass
@@ -23,6 +35,9 @@ class ModelConfig:
     """Base of all architecture configurations."""
 
     architecture: str = ""
+    # what ends a generation (config.json's eos_token_id: one id or a list) and what starts a prompt
+    eos_token_ids: Tuple[int, ...] = ()
+    bos_token_id: Optional[int] = None
 
     # -- reading ---------------------------------------------------------
     @classmethod
@@ -34,6 +49,15 @@ class ModelConfig:
 
     def validate(self) -> None:
         """Raise ConfigError when sizes or options contradict each other."""
+
+    def special_tokens_dict(self) -> Dict[str, Any]:
+        """The token keys as config.json writes them (absent where the configuration has none)."""
+        out: Dict[str, Any] = {}
+        if self.eos_token_ids:
+            out["eos_token_id"] = list(self.eos_token_ids) if len(self.eos_token_ids) > 1 else self.eos_token_ids[0]
+        if self.bos_token_id is not None:
+            out["bos_token_id"] = self.bos_token_id
+        return out
 
     # -- helpers ---------------------------------------------------------
     def replace(self, **changes) -> "ModelConfig":

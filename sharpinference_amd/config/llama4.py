@@ -11,7 +11,7 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Any, Dict, List, Optional
 
-from .base import ConfigError, ModelConfig
+from .base import ConfigError, ModelConfig, special_tokens_from
 
 
 @dataclass
@@ -140,6 +140,7 @@ class Llama4TextConfig(ModelConfig):
             tie_word_embeddings=bool(src.get("tie_word_embeddings", False)),
             max_position_embeddings=int(src.get("max_position_embeddings", 0)),
             torch_dtype=str(src.get("torch_dtype", "bfloat16")),
+            **special_tokens_from(src),
         )
 
     def to_dict(self) -> Dict[str, Any]:
@@ -172,6 +173,7 @@ class Llama4TextConfig(ModelConfig):
         }
         if self.moe_layers is not None:
             out["moe_layers"] = list(self.moe_layers)
+        out.update(self.special_tokens_dict())
         return out
 
     # ------------------------------------------------------------------

@@ -151,7 +151,7 @@ class Engine:
                 p.temperature = float(temperature)
             if seeds is not None:
                 p.seed = int(seeds[i])
-            if stop_token_ids:
+            if stop_token_ids is not None:
                 p.stop_token_ids = tuple(int(t) for t in stop_token_ids)
             plist.append(p)
         return plist
@@ -169,7 +169,7 @@ class Engine:
     def generate_chunks(self, prompts: Sequence[Sequence[int]],
                         params: Union[SamplingParams, Sequence[SamplingParams], None] = None, *,
                         max_new_tokens: Optional[int] = None, temperature: Optional[float] = None,
-                        seeds: Optional[Sequence[int]] = None, stop_token_ids: Sequence[int] = (),
+                        seeds: Optional[Sequence[int]] = None, stop_token_ids: Optional[Sequence[int]] = None,
                         should_cancel: Optional[Callable[[int], bool]] = None) -> Iterator[GenerateChunk]:
         """Generate for a list of prompts (token ids) under continuous batching and yield what
         happens as it happens, in the reference's typed chunks
@@ -177,12 +177,15 @@ class Engine:
         chunk with its number of prompt tokens before anything else of it, a ``token`` chunk per
         generated token (the reference's text chunk; there is no tokenizer here), and one ``stop``
         chunk when it ends.  ``should_cancel(index)`` is asked before every step, as the
-        reference's cancellation token is; a cancelled prompt ends with reason "abort".  Closing
+        reference's cancellation token is; a cancelled prompt ends with reason "abort".  A request
+        stops at the configuration's end-of-generation tokens unless its ``stop_token_ids``
+        (or the argument here) replace them, as in the reference (Sampler.cs:724-741).  Closing
         the generator early gives every page back."""
         if self._sched is not None:
             raise RuntimeError("a generation is running on this engine: requests are admitted by one loop at a time")
         plist = self._sampling_params(len(prompts), params, max_new_tokens, temperature, seeds, stop_token_ids)
-        sched = Scheduler(self.cache, self.max_num_seqs, self.max_tokens_per_step, self.max_model_len)
+        sched = Scheduler(self.cache, self.max_num_seqs, self.max_tokens_per_step, self.max_model_len,
+                          end_of_generation=self.config.eos_token_ids)
         reqs = [Request(("gen", i), [int(t) for t in prompt], plist[i]) for i, prompt in enumerate(prompts)]
         for r in reqs:
             sched.add(r)
@@ -245,7 +248,7 @@ class Engine:
 
     def generate(self, prompts: Sequence[Sequence[int]], params: Union[SamplingParams, Sequence[SamplingParams], None] = None,
                  *, max_new_tokens: Optional[int] = None, temperature: Optional[float] = None,
-                 seeds: Optional[Sequence[int]] = None, stop_token_ids: Sequence[int] = ()) -> List[GenerationResult]:
+                 seeds: Optional[Sequence[int]] = None, stop_token_ids: Optional[Sequence[int]] = None) -> List[GenerationResult]:
         """Generate for a list of prompts (token ids) under continuous batching; the chunks of
         ``generate_chunks`` gathered per prompt."""
         out = [GenerationResult([], "abort", len(p)) for p in prompts]

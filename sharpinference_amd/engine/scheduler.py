@@ -43,6 +43,7 @@ class Request:
     finish_reason: Optional[str] = None
     cancelled: bool = False
     draws: int = 0                    # uniforms used so far
+    stops: frozenset = frozenset()    # tokens that end it (its own and the model's), set on admission to the queue
 
     @property
     def finished(self) -> bool:
@@ -61,7 +62,8 @@ class Scheduled:
 
 
 class Scheduler:
-    def __init__(self, cache: CacheManager, max_num_seqs: int, max_tokens_per_step: int, max_model_len: int):
+    def __init__(self, cache: CacheManager, max_num_seqs: int, max_tokens_per_step: int, max_model_len: int,
+                 end_of_generation: Sequence[int] = ()):
         if max_tokens_per_step < 1 or max_num_seqs < 1:
             raise ValueError("max_tokens_per_step and max_num_seqs must be positive")
         if max_num_seqs > cache.max_requests:
@@ -70,6 +72,7 @@ class Scheduler:
         self.max_num_seqs = max_num_seqs
         self.max_tokens_per_step = max_tokens_per_step
         self.max_model_len = max_model_len
+        self.end_of_generation = tuple(int(t) for t in end_of_generation)   # the model's own stop tokens
         self.waiting: Deque[Request] = deque()
         self.running: List[Request] = []
         self.finished: List[Request] = []
@@ -78,6 +81,7 @@ class Scheduler:
     def add(self, request: Request) -> None:
         if not request.prompt:
             raise ValueError(f"request {request.req_id!r} has an empty prompt")
+        request.stops = request.params.stop_set(self.end_of_generation)
         self.waiting.append(request)
 
     def has_work(self) -> bool:
@@ -145,7 +149,7 @@ class Scheduler:
                 continue
             assert tok is not None
             r.draws += 0 if r.params.greedy else 1
-            if tok in r.params.stop_token_ids:
+            if tok in r.stops:
                 self._finish(r, FINISH_STOP, held=True)   # the stop token is not emitted
                 done.append(r)
                 continue

@@ -233,3 +233,44 @@ def test_command_line_takes_the_reference_s_option_names():
             pass
         else:
             raise AssertionError(bad)
+
+
+def test_end_and_begin_tokens_of_config_json():
+    base = dict(TINY_A)
+    assert load_config(base).eos_token_ids == () and load_config(base).bos_token_id is None
+    one = load_config({**base, "eos_token_id": 7, "bos_token_id": 3})
+    assert one.eos_token_ids == (7,) and one.bos_token_id == 3 and one.to_dict()["eos_token_id"] == 7
+    many = load_config({**base, "eos_token_id": [7, 9, 11]})
+    assert many.eos_token_ids == (7, 9, 11) and load_config(many.to_dict()) == many
+    nested = load_config({"architectures": base["architectures"], "text_config": {k: v for k, v in base.items() if k != "architectures"},
+                          "eos_token_id": [5]})
+    assert nested.eos_token_ids == (5,)
+    with pytest.raises(ConfigError, match="eos_token_id"):
+        load_config({**base, "eos_token_id": "</s>"})
+
+
+def _word_tokenizer(folder):
+    """A tokenizer.json of whole words, made with the tokenizers package."""
+    from tokenizers import Tokenizer, models, pre_tokenizers
+
+    vocab = {"<unk>": 0, "<s>": 1, "the": 2, "cat": 3, "sat": 4, "on": 5, "mat": 6}
+    tok = Tokenizer(models.WordLevel(vocab, unk_token="<unk>"))
+    tok.pre_tokenizer = pre_tokenizers.Whitespace()
+    tok.save(os.path.join(folder, "tokenizer.json"))
+
+
+def test_prompts_as_text_or_ids(tmp_path):
+    from sharpinference_amd.cli import prompt_ids
+    from sharpinference_amd.text import TextCodec
+
+    assert TextCodec.from_folder(str(tmp_path)) is None
+    assert prompt_ids("1, 2 3", None) == [1, 2, 3]
+    with pytest.raises(SystemExit, match="tokenizer.json"):
+        prompt_ids("the cat", None)
+    _word_tokenizer(str(tmp_path))
+    codec = TextCodec.from_folder(str(tmp_path), bos_token_id=1)
+    assert prompt_ids("the cat sat", codec) == [1, 2, 3, 4]            # the begin token leads, once
+    assert prompt_ids("4 5 6", codec) == [4, 5, 6]                     # numbers stay token ids
+    assert TextCodec.from_folder(str(tmp_path)).encode("on the mat") == [5, 2, 6]
+    s = codec.streamer()
+    assert [s.push(t) for t in (2, 3, 6)] == ["the", " cat", " mat"] and s.flush() == ""

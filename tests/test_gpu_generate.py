@@ -187,3 +187,37 @@ def test_command_line(tmp_path):
     assert lines[0] == " ".join(map(str, prompt))
     assert lines[1].startswith(" ".join(map(str, want))) and lines[1].endswith("(length)")
     assert lines[-1].startswith("Prefill: 12 tokens, ") and "| Decode: 7 tokens, " in lines[-1] and lines[-1].endswith("t/s")
+
+
+def test_command_line_with_text_and_the_model_s_end_token(tmp_path):
+    """A folder with a tokenizer.json takes a text prompt and prints text; generation ends at the
+    configuration's eos_token_id unless --ignore-eos is given."""
+    import json
+
+    from tokenizers import Tokenizer, models, pre_tokenizers
+
+    d = make_model_dir(tmp_path, "A", std=0.1)
+    c, W = P.read_config(d), P.load_weights(d)
+    prompt = H.random_tokens(12, 256, 2)
+    want = P.generate(c, W, prompt, 8)
+    end = want[4]
+    cut = want.index(end)                                    # the end token's first appearance
+    with open(os.path.join(d, "config.json")) as f:
+        cfg = json.load(f)
+    cfg["eos_token_id"] = [end, 255]
+    with open(os.path.join(d, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    tok = Tokenizer(models.WordLevel({f"w{i}": i for i in range(256)}, unk_token="w0"))
+    tok.pre_tokenizer = pre_tokenizers.Whitespace()
+    tok.save(os.path.join(d, "tokenizer.json"))
+    text = " ".join(f"w{t}" for t in prompt)
+    base = [sys.executable, os.path.join(ROOT, "bin", "sharpi-cli"), "-m", d, "-p", text, "-n", "8", "--temp", "0",
+            "--dtype", "fp32", "--kv-tokens", "128"]
+    out = subprocess.run(base, capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stderr
+    lines = out.stdout.strip().splitlines()
+    assert lines[0] == text
+    assert lines[1] == " ".join(f"w{t}" for t in want[:cut]) + "  (stop)", lines[1]
+    out = subprocess.run(base + ["--ignore-eos"], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stderr
+    assert out.stdout.strip().splitlines()[1] == " ".join(f"w{t}" for t in want) + "  (length)"

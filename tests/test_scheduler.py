@@ -130,3 +130,24 @@ def test_max_num_seqs_bounds_the_batch():
     batches = _run(sched, lambda r: 1)
     assert max(len(b) for b in batches) == 2
     assert all(r.finish_reason == "length" for r in reqs)
+
+
+def test_the_model_s_end_tokens_stop_a_request_unless_it_replaces_them():
+    """None = the model's end-of-generation tokens, a tuple replaces them, additional ones are added to
+    either (reference: src/SharpInference.Engine/Sampler.cs:724-741)."""
+    assert SamplingParams().stop_set((5, 6)) == {5, 6}
+    assert SamplingParams(stop_token_ids=()).stop_set((5, 6)) == set()
+    assert SamplingParams(stop_token_ids=(9,)).stop_set((5, 6)) == {9}
+    assert SamplingParams(additional_stop_token_ids=(9,)).stop_set((5, 6)) == {5, 6, 9}
+    assert SamplingParams(stop_token_ids=(1,), additional_stop_token_ids=(9,)).stop_set((5, 6)) == {1, 9}
+
+    sched = Scheduler(_cache(64), 4, 64, 256, end_of_generation=(7, 8))
+    plain = Request("plain", [1, 2, 3], SamplingParams(temperature=0.0, max_new_tokens=6))
+    deaf = Request("deaf", [1, 2, 3], SamplingParams(temperature=0.0, max_new_tokens=6, stop_token_ids=()))
+    more = Request("more", [1, 2, 3], SamplingParams(temperature=0.0, max_new_tokens=6, additional_stop_token_ids=(50,)))
+    for r in (plain, deaf, more):
+        sched.add(r)
+    _run(sched, lambda r: 8 if len(r.output) == 2 else 50)
+    assert plain.output == [50, 50] and plain.finish_reason == "stop"
+    assert deaf.output == [50, 50, 8, 50, 50, 50] and deaf.finish_reason == "length"
+    assert more.output == [] and more.finish_reason == "stop"
