@@ -19,6 +19,9 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
+// the head sizes the kernel is compiled for
+#define SHARPI_DECODE_HEAD_SIZES(X) X(32) X(64) X(96) X(128) X(160) X(192) X(224) X(256)
+
 constexpr int kDecWaves = 4;
 constexpr int kSplitBlocks = 16;  // 16-key blocks per run: 256 keys
 
@@ -295,12 +298,20 @@ SHARPI_EXPORT int sharpi_attention_decode(const void* q, const void* k_cache, co
   if (nkv * ((nh / nkv + 15) / 16) > 65535) return SHARPI_ERR_ARG;
 #define DEC(HDV)                                                                                                  \
   if (hd == HDV)                                                                                                  \
-  return launch_decode<HDV>(q, k_cache, v_cache, block_table, entry_of_token, positions, token_list, part_o,      \
-                            part_ml, out, window_kind, window, scale, n_list, nh, nkv, page_size, max_blocks,     \
-                            num_pages, max_splits, stream)
-  DEC(32); DEC(64); DEC(96); DEC(128); DEC(192); DEC(256);
+    return launch_decode<HDV>(q, k_cache, v_cache, block_table, entry_of_token, positions, token_list, part_o,    \
+                              part_ml, out, window_kind, window, scale, n_list, nh, nkv, page_size, max_blocks,   \
+                              num_pages, max_splits, stream);
+  SHARPI_DECODE_HEAD_SIZES(DEC)
 #undef DEC
-  return SHARPI_ERR_ARG;  // head sizes that are no multiple of 32 go to the generic kernel
+  return SHARPI_ERR_ARG;  // other head sizes go to the generic kernel
+}
+
+// 1 if the kernel is compiled for this head size (the caller's choice of kernel asks here).
+SHARPI_EXPORT int sharpi_attention_decode_takes(int hd) {
+#define DEC(HDV) if (hd == HDV) return 1;
+  SHARPI_DECODE_HEAD_SIZES(DEC)
+#undef DEC
+  return 0;
 }
 
 SHARPI_EXPORT int sharpi_attention_decode_split_keys() { return kSplitBlocks * 16; }

@@ -25,6 +25,9 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
+// the head sizes the kernel is compiled for
+#define SHARPI_PREFILL_HEAD_SIZES(X) X(32) X(64) X(96) X(128) X(160) X(192)
+
 constexpr int kPreWaves = 4;
 constexpr int kQT = 2;                               // 16-token column tiles per wave
 constexpr int kWaveTokens = 16 * kQT;
@@ -380,9 +383,17 @@ SHARPI_EXPORT int sharpi_attention_prefill(const void* q, const void* k_cache, c
     SHARPI_CHECK_LAUNCH();                                                                                    \
     return SHARPI_OK;                                                                                         \
   }
-  PRE(32) PRE(64) PRE(96) PRE(128) PRE(192)
+  SHARPI_PREFILL_HEAD_SIZES(PRE)
 #undef PRE
   return SHARPI_ERR_ARG;  // other head sizes go to the generic kernel
+}
+
+// 1 if the kernel is compiled for this head size (the caller's choice of kernel asks here).
+SHARPI_EXPORT int sharpi_attention_prefill_takes(int hd) {
+#define PRE(HDV) if (hd == HDV) return 1;
+  SHARPI_PREFILL_HEAD_SIZES(PRE)
+#undef PRE
+  return 0;
 }
 
 SHARPI_EXPORT int sharpi_attention_prefill_tile_tokens() { return kTileTokens; }

@@ -221,7 +221,7 @@ DECODE_RUN_KEYS = _lib.DECODE_RUN_KEYS   # keys per block of the decode kernel (
 
 
 def decode_attention_ok(dtype: torch.dtype, hd: int) -> bool:
-    return dtype == torch.bfloat16 and hd % 32 == 0 and 32 <= hd <= 256
+    return dtype == torch.bfloat16 and _lib.attention_takes("decode", hd)
 
 
 def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
@@ -236,7 +236,7 @@ def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     _i32(positions, "positions")
     _i32(token_list, "token_list")
     T = q.shape[0]
-    _need(q.shape == (T, nh * hd) and decode_attention_ok(q.dtype, hd), "attention_decode: q must be bfloat16 [T, nh*hd], hd a multiple of 32")
+    _need(q.shape == (T, nh * hd) and decode_attention_ok(q.dtype, hd), "attention_decode: q must be bfloat16 [T, nh*hd], hd a head size the kernel is compiled for")
     _need(_cache_shapes_ok(k_cache, v_cache, nkv, hd) and k_cache.dtype == q.dtype and v_cache.dtype == q.dtype,
           "attention_decode: caches must be K [pages, nkv, page_size, hd], V [pages, nkv, hd, page_size] bfloat16")
     _need(block_table.dim() == 2 and entry_of_token.shape == (T,) and positions.shape == (T,),
@@ -259,7 +259,7 @@ PREFILL_TILE_TOKENS = _lib.PREFILL_TILE_TOKENS   # tokens per block of the prefi
 
 
 def prefill_attention_ok(dtype: torch.dtype, hd: int) -> bool:
-    return dtype == torch.bfloat16 and hd % 32 == 0 and 32 <= hd <= 192
+    return dtype == torch.bfloat16 and _lib.attention_takes("prefill", hd)
 
 
 def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
@@ -273,7 +273,7 @@ def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     _i32(tiles, "tiles")
     T = q.shape[0]
     _need(q.shape == (T, nh * hd) and prefill_attention_ok(q.dtype, hd),
-          "attention_prefill: q must be bfloat16 [T, nh*hd], hd a multiple of 32 up to 192")
+          "attention_prefill: q must be bfloat16 [T, nh*hd], hd a head size the kernel is compiled for")
     _need(_cache_shapes_ok(k_cache, v_cache, nkv, hd) and k_cache.dtype == q.dtype and v_cache.dtype == q.dtype,
           "attention_prefill: caches must be K [pages, nkv, page_size, hd], V [pages, nkv, hd, page_size] bfloat16")
     _need(block_table.dim() == 2 and positions.shape == (T,) and tiles.dim() == 2 and tiles.shape[1] == 3,

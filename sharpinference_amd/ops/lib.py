@@ -106,6 +106,20 @@ def load(verbose: bool = True) -> ctypes.CDLL:
     return lib
 
 
+_takes: dict = {}
+
+
+def attention_takes(kind: str, hd: int) -> bool:
+    """Whether the matrix-core attention kernel of this kind ('decode' or 'prefill') is compiled for
+    head size hd: the library is asked, so that the choice of kernel cannot drift from the build."""
+    key = (kind, int(hd))
+    if key not in _takes:
+        fn = getattr(load(), f"sharpi_attention_{kind}_takes")
+        fn.argtypes, fn.restype = [c_int], c_int
+        _takes[key] = bool(fn(int(hd)))
+    return _takes[key]
+
+
 def register_signature(name: str, argtypes) -> None:
     """Used by op modules that bind further entry points of the library."""
     _SIGNATURES[name] = list(argtypes)

@@ -274,3 +274,10 @@ def test_prompts_as_text_or_ids(tmp_path):
     assert TextCodec.from_folder(str(tmp_path)).encode("on the mat") == [5, 2, 6]
     s = codec.streamer()
     assert [s.push(t) for t in (2, 3, 6)] == ["the", " cat", " mat"] and s.flush() == ""
+
+
+def test_a_head_size_no_kernel_takes_is_refused_when_the_model_is_built():
+    for hd in (272, 24):
+        cfg = load_config({**TINY_A, "head_dim": hd})
+        with pytest.raises(ValueError, match=f"head_dim {hd}"):
+            build_model(cfg)

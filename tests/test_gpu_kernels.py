@@ -148,11 +148,18 @@ def _start(p, kind, window):
     return (p // window) * window if kind == 1 else max(0, p - window + 1) if kind == 2 else 0
 
 
-@pytest.mark.parametrize("nh,nkv,hd", [(8, 2, 64), (5, 5, 32), (40, 8, 128), (3, 1, 96), (34, 2, 32)])
-@pytest.mark.parametrize("kind,window", [(0, 0), (1, 24), (1, 300), (2, 50)])
-@pytest.mark.parametrize("ps", [16, 64])
+_DECODE_CASES = [(nh, nkv, hd, kind, window, ps)
+                 for nh, nkv, hd in [(8, 2, 64), (5, 5, 32), (40, 8, 128), (3, 1, 96), (34, 2, 32)]
+                 for kind, window in [(0, 0), (1, 24), (1, 300), (2, 50)] for ps in (16, 64)]
+# every other head size the kernel is compiled for, each with one kind of window
+_DECODE_CASES += [(2, 1, 160, 1, 300, 16), (6, 2, 192, 0, 0, 64), (3, 3, 224, 2, 50, 16), (4, 2, 256, 1, 24, 16),
+                  (4, 2, 256, 0, 0, 64)]
+
+
+@pytest.mark.parametrize("nh,nkv,hd,kind,window,ps", _DECODE_CASES)
 def test_attention_decode_kernel(nh, nkv, hd, kind, window, ps):
     ops = _ops()
+    assert ops.decode_attention_ok(torch.bfloat16, hd)
     lens = [1, 17, 300, 1000, 257, 512]
     bt, kc, vc, ks, vs = _paged_case(lens, nh, nkv, hd, ps, torch.bfloat16, seed=nh * 7 + hd, strong_key=3)
     n = len(lens)
@@ -515,12 +522,17 @@ def test_gemm_grouped_swiglu_equals_product_then_activation(T, E, k, I, K):
     assert float((ops.gemm_grouped_swiglu(x, w, rt, rt.sorted_w).float().cpu() - ref).abs().max()) <= 3e-2 * float(ref.abs().max() + 1e-6)
 
 
-@pytest.mark.parametrize("nh,nkv,hd", [(8, 2, 64), (5, 5, 32), (40, 8, 128), (3, 1, 96)])
-@pytest.mark.parametrize("kind,window", [(0, 0), (1, 24), (1, 100), (2, 50)])
-@pytest.mark.parametrize("ps", [16, 32])
+_PREFILL_CASES = [(nh, nkv, hd, kind, window, ps)
+                  for nh, nkv, hd in [(8, 2, 64), (5, 5, 32), (40, 8, 128), (3, 1, 96)]
+                  for kind, window in [(0, 0), (1, 24), (1, 100), (2, 50)] for ps in (16, 32)]
+_PREFILL_CASES += [(2, 1, 160, 1, 100, 16), (3, 3, 160, 0, 0, 32), (6, 2, 192, 2, 50, 16), (2, 2, 192, 1, 24, 32)]
+
+
+@pytest.mark.parametrize("nh,nkv,hd,kind,window,ps", _PREFILL_CASES)
 def test_attention_prefill_kernel(nh, nkv, hd, kind, window, ps):
     """Portions of several requests at different starting positions, against dense softmax."""
     ops = _ops()
+    assert ops.prefill_attention_ok(torch.bfloat16, hd)
     ctx_lens = [70, 300, 33, 129]          # context after the portion
     portion = [70, 45, 2, 100]             # the last `portion` tokens are this step's queries
     bt, kc, vc, ks, vs = _paged_case(ctx_lens, nh, nkv, hd, ps, torch.bfloat16, seed=nh + hd + ps, strong_key=5)
@@ -654,3 +666,12 @@ def test_gemm_tiled_is_a_true_float_product_and_batch_invariant(M, N, K):
     if M > 1:
         assert torch.equal(ops.gemm_tiled(x[:1].contiguous(), w), got[:1])
         assert torch.equal(ops.gemm_tiled(x[M // 2:].contiguous(), w), got[M // 2:])
+
+
+def test_the_library_says_which_head_sizes_its_attention_kernels_take():
+    """The choice between the matrix-core kernels and the generic one asks the library: a head size is
+    either compiled or goes to the generic kernel, which takes every size up to 256."""
+    ops = _ops()
+    assert [hd for hd in range(16, 273, 16) if ops.decode_attention_ok(torch.bfloat16, hd)] == [32, 64, 96, 128, 160, 192, 224, 256]
+    assert [hd for hd in range(16, 273, 16) if ops.prefill_attention_ok(torch.bfloat16, hd)] == [32, 64, 96, 128, 160, 192]
+    assert not ops.decode_attention_ok(torch.float32, 128) and not ops.prefill_attention_ok(torch.float32, 128)

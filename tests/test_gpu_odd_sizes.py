@@ -26,6 +26,12 @@ CASES = {
     # no layer routed at all (the step is larger than the model), and many experts, no power of two, four picked
     "dense_only": ("B", dict(interleave_moe_layer_step=7, vocab_size=384)),
     "e130_k4": ("A", dict(num_local_experts=130, num_experts_per_tok=4, vocab_size=256)),
+    # head sizes 160 and 256: the decode attention's matrix-core kernel with one chunk in flight, prompts through
+    # the generic kernel; 256 is the largest head size taken
+    "hd160": ("B", dict(hidden_size=96, num_attention_heads=3, num_key_value_heads=1, head_dim=160, vocab_size=311,
+                        attention_chunk_size=20)),
+    "hd256": ("D", dict(hidden_size=128, num_attention_heads=2, num_key_value_heads=2, head_dim=256, vocab_size=499,
+                        intermediate_size=128, num_local_experts=3, num_experts_per_tok=2, attention_chunk_size=56)),
     "hd192": ("D", dict(hidden_size=384, num_attention_heads=2, num_key_value_heads=2, head_dim=192, vocab_size=333,
                         intermediate_size=128, num_local_experts=4, num_experts_per_tok=2, attention_chunk_size=40)),
 }
