@@ -364,4 +364,5 @@ SHARPI_EXPORT int sharpi_moe_permute(const int* topk_ids, const float* topk_w, i
 }
 
 SHARPI_EXPORT int sharpi_router_sorted_tiles() { return kSortTiles; }
+SHARPI_EXPORT int sharpi_router_max_experts() { return kMaxExperts; }
 SHARPI_EXPORT int sharpi_add_rmsnorm_router_max_hidden() { return kFusedMaxHidden; }

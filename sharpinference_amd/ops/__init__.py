@@ -461,6 +461,7 @@ def gemm_skinny_swiglu(x: torch.Tensor, w, offsets: torch.Tensor, a_rows: Option
     return out
 
 
+ROUTER_MAX_EXPERTS = _lib.ROUTER_MAX_EXPERTS   # experts the routing kernels hold scores for (csrc/router.hip kMaxExperts)
 PICKED_MAX_PAIRS = _lib.PICKED_MAX_PAIRS   # (token, pick) pairs of the picked form: one ballot of a wave (csrc/gemm_skinny_kernel.h kMaxPicked)
 
 _COUNTING: dict = {}    # per device: 0, 1, 2, ... (the places of pairs that are stored in their own order)

@@ -51,11 +51,13 @@ GROUPED_TILE_ROWS = 192     # rows per tile of the grouped product for many rows
 SORTED_TILE_LISTS = 512     # tile lists up to this long come tallest first
 PICKED_MAX_PAIRS = 64       # (token, pick) pairs the few-rows product takes straight from the router's picks
 FUSED_NORM_ROUTER_MAX_HIDDEN = 8192   # widest row of the norm + router kernel
+ROUTER_MAX_EXPERTS = 1024   # experts the routing kernels hold scores for
 _BUILT_WITH = {
     "sharpi_attention_decode_split_keys": DECODE_RUN_KEYS,
     "sharpi_attention_prefill_tile_tokens": PREFILL_TILE_TOKENS,
     "sharpi_gemm_grouped_tile_rows": GROUPED_TILE_ROWS,
     "sharpi_router_sorted_tiles": SORTED_TILE_LISTS,
+    "sharpi_router_max_experts": ROUTER_MAX_EXPERTS,
     "sharpi_gemm_skinny_max_picked": PICKED_MAX_PAIRS,
     "sharpi_add_rmsnorm_router_max_hidden": FUSED_NORM_ROUTER_MAX_HIDDEN,
 }

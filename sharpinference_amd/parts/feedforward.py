@@ -73,6 +73,8 @@ class MoESwiGLU(Part):
                  score_on_input: bool = True):
         if not 1 <= top_k <= num_experts:
             raise ValueError(f"top_k {top_k} must lie in 1..{num_experts}")
+        if num_experts > ops.ROUTER_MAX_EXPERTS:
+            raise ValueError(f"{num_experts} experts are not taken: the routing kernels hold scores for {ops.ROUTER_MAX_EXPERTS}")
         if gate not in ("sigmoid", "softmax"):
             raise ValueError(f"router gate {gate!r} is not known (sigmoid, softmax)")
         if not score_on_input:

@@ -281,3 +281,5 @@ def test_a_head_size_no_kernel_takes_is_refused_when_the_model_is_built():
         cfg = load_config({**TINY_A, "head_dim": hd})
         with pytest.raises(ValueError, match=f"head_dim {hd}"):
             build_model(cfg)
+    with pytest.raises(ValueError, match="1025 experts"):
+        build_model(load_config({**TINY_A, "num_local_experts": 1025}))
