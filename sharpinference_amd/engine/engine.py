@@ -69,7 +69,10 @@ class Engine:
                  max_model_len: Optional[int] = None, max_num_seqs: int = 8, max_tokens_per_step: int = 2048,
                  kv_tokens: Optional[int] = None, page_size: int = 16, weight_std: float = 0.02,
                  weight_std_by_suffix: Optional[Dict[str, float]] = None, verbose: bool = False,
-                 decode_graphs: bool = True):
+                 decode_graphs: bool = True, past_position_limit: bool = False):
+        """max_model_len: the longest sequence a request may reach (default: the configuration's
+        max_position_embeddings, 4096 if it names none); beyond max_position_embeddings only with
+        past_position_limit (replaying given tokens needs no trained positions)."""
         self.dtype = parse_dtype(dtype)
         self.device = torch.device(device)
         if self.device.type != "cuda":
@@ -104,7 +107,7 @@ class Engine:
             print(f"[engine] weights ready in {time.time() - t0:.1f}s", file=sys.stderr, flush=True)
         limit = getattr(self.config, "max_position_embeddings", 0) or 0
         self.max_model_len = int(max_model_len or limit or 4096)
-        if limit and self.max_model_len > limit:
+        if limit and self.max_model_len > limit and not past_position_limit:
             raise ValueError(f"max_model_len {self.max_model_len} exceeds the model's max_position_embeddings {limit}")
         self.max_num_seqs = int(max_num_seqs)
         self.max_tokens_per_step = int(max_tokens_per_step)

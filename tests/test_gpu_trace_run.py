@@ -72,3 +72,17 @@ def test_trace_run_mixed(which, dtype, tmp_path):
             H.assert_close_fp32(got[rid], H.plain_logits(d, toks)[places], f"trace_run {which} {rid}")
         else:   # configuration C uses every expert for every token: no route can flip
             H.assert_close_bf16(got[rid], H.plain_logits(d, toks, bf16_storage=True)[places], f"trace_run {which} {rid}")
+
+
+def test_trace_run_past_the_length_config_json_names(tmp_path):
+    """A replay is bounded by --max-tokens, not by max_position_embeddings: given tokens need no trained positions."""
+    d = make_model_dir(tmp_path, "A", std=0.1, max_position_embeddings=32)
+    vocab = CONFIGS["A"]["vocab_size"]
+    toks = H.random_tokens(100, vocab, 77)
+    steps = [{"step": 0, "entries": [{"id": "x", "tokens": toks[:61], "want": [0, 31, 60]}], "end": []},
+             {"step": 1, "entries": [{"id": "x", "tokens": toks[61:99], "want": [37]}], "end": []},
+             {"step": 2, "entries": [{"id": "x", "tokens": toks[99:], "want": [0]}], "end": ["x"]}]
+    out = str(tmp_path / "out")
+    _run_trace(d, "float32", steps, out, 128)
+    got = _collect(steps, out, vocab)["x"]
+    H.assert_close_fp32(got, H.plain_logits(d, toks)[[0, 31, 60, 98, 99]], "trace_run past the named length")
