@@ -139,6 +139,133 @@ __device__ __forceinline__ void renormalise(float* p, int vocab, float* red) {
   __syncthreads();
 }
 
+
+// Rows with a small top-k (the usual case: 40 of 200,000) need the whole vocabulary three times
+// only: for the maximum, for the softmax sum, and to collect the few entries that can survive.
+// Every thread's largest probability is one element, so the k-th largest of those 1,024 values is a
+// lower bound of the k-th largest probability: entries at or above it (a few more than k) go to
+// LDS, one per thread, and top-k, min-p, top-p, both renormalisations and the inverse CDF run
+// there, with the same definitions as the full path below (ties at a cut are all kept; the CDF
+// walks ascending indices).  The probabilities have the same bits as the full path's.  Returns
+// false, with nothing written, if more entries than threads reach the bound: the caller then
+// takes the full path.  Every thread of the block returns the same value.
+constexpr int kFastMaxK = 256;
+
+__device__ __forceinline__ bool sample_few_survivors(const float* __restrict__ x, int vocab, float T, int k, float mp,
+                                                     float tp, float u, int* __restrict__ out_r, float* red) {
+  __shared__ float a_p[kSampThreads];
+  __shared__ int a_i[kSampThreads];
+  __shared__ float b_p[kSampThreads];
+  __shared__ int b_i[kSampThreads];
+  __shared__ float s_bound;
+  __shared__ int s_count, s_win;
+  const int t = threadIdx.x;
+  const int nt = blockDim.x;
+  const float invT = 1.0f / T;
+  const bool scaled = T != 1.0f;
+
+  float vmax = -INFINITY;
+  for (int i = t; i < vocab; i += nt) vmax = fmaxf(vmax, scaled ? x[i] * invT : x[i]);
+  const float mx = block_max(vmax, red);
+  float s = 0.f;
+  for (int i = t; i < vocab; i += nt) s += expf((scaled ? x[i] * invT : x[i]) - mx);
+  const float inv_sum = 1.0f / block_sum(s, red);
+
+  // the k-th largest of the threads' largest probabilities (a thread without an element holds -1)
+  const float lm = vmax == -INFINITY ? -1.f : expf(vmax - mx) * inv_sum;
+  a_p[t] = lm;
+  if (t == 0) {
+    s_count = 0;
+    s_win = 0x7fffffff;
+  }
+  __syncthreads();
+  int rank = 0;
+  for (int j = 0; j < nt; ++j) {
+    const float o = a_p[j];
+    rank += (o > lm || (o == lm && j < t)) ? 1 : 0;
+  }
+  if (rank == k - 1) s_bound = lm;   // ranks are a permutation: one thread has this one
+  __syncthreads();
+  const float bound = s_bound;
+  for (int i = t; i < vocab; i += nt) {
+    const float p = expf((scaled ? x[i] * invT : x[i]) - mx) * inv_sum;
+    if (p >= bound) {
+      const int slot = atomicAdd(&s_count, 1);
+      if (slot < kSampThreads) {
+        b_p[slot] = p;
+        b_i[slot] = i;
+      }
+    }
+  }
+  __syncthreads();
+  const int c = s_count;
+  if (c > kSampThreads || c > nt) return false;
+
+  // top-k with ties: an entry stays if fewer than k entries are strictly larger
+  const bool have = t < c;
+  const float p0 = have ? b_p[t] : -1.f;
+  const int idx = have ? b_i[t] : 0x7fffffff;
+  int larger = 0;
+  for (int j = 0; j < c; ++j) larger += b_p[j] > p0 ? 1 : 0;
+  const bool kept = have && larger < k;
+  a_i[t] = kept ? idx : 0x7fffffff;
+  __syncthreads();
+  // in ascending index order: a_p / a_i [0, n)
+  int pos = 0, n = 0;
+  for (int j = 0; j < c; ++j) {
+    const int o = a_i[j];
+    pos += o < idx ? 1 : 0;
+    n += o != 0x7fffffff ? 1 : 0;
+  }
+  __syncthreads();
+  if (kept) {
+    a_p[pos] = p0;
+    a_i[pos] = idx;
+  }
+  __syncthreads();
+  const bool mine = t < n;
+  float q = mine ? a_p[t] : 0.f;
+  float total = 0.f;
+  for (int j = 0; j < n; ++j) total += a_p[j];
+  if (total > 0.f && total != 1.0f) q *= 1.0f / total;
+  b_p[t] = q;
+  __syncthreads();
+  if (mp > 0.f) {
+    float pm = 0.f;
+    for (int j = 0; j < n; ++j) pm = fmaxf(pm, b_p[j]);
+    if (q < mp * pm) q = 0.f;
+    __syncthreads();
+    b_p[t] = q;
+    __syncthreads();
+  }
+  if (tp > 0.f && tp < 1.0f) {
+    // the descending running sum reaches top_p at some value: an entry stays if what is strictly
+    // larger than it has not reached top_p yet
+    float above = 0.f;
+    for (int j = 0; j < n; ++j) {
+      const float o = b_p[j];
+      above += o > q ? o : 0.f;
+    }
+    if (!(above < tp)) q = 0.f;
+    __syncthreads();
+    b_p[t] = q;
+    __syncthreads();
+  }
+  total = 0.f;
+  for (int j = 0; j < n; ++j) total += b_p[j];
+  const float inv = (total > 0.f && total != 1.0f) ? 1.0f / total : 1.0f;
+  const bool rescale = total > 0.f && total != 1.0f;
+  if (mine) {
+    float run = 0.f;
+    for (int j = 0; j <= t; ++j) run += rescale ? b_p[j] * inv : b_p[j];
+    if (u <= run) atomicMin(&s_win, t);
+  }
+  __syncthreads();
+  // (a uniform of exactly 0 is reached by the running sum at index 0 already, whatever lies there)
+  if (t == 0) *out_r = u <= 0.f ? 0 : s_win < n ? a_i[s_win] : vocab - 1;
+  return true;
+}
+
 __global__ __launch_bounds__(kSampThreads) void sample_rows_kernel(
     const float* __restrict__ logits, float* __restrict__ probs, const float* __restrict__ temperature,
     const float* __restrict__ uniform, const int* __restrict__ top_k, const float* __restrict__ top_p,
@@ -152,6 +279,11 @@ __global__ __launch_bounds__(kSampThreads) void sample_rows_kernel(
   float* p = probs + (size_t)r * vocab;
   const float T = temperature[r];
   const float invT = 1.0f / T;
+  const int k = top_k ? top_k[r] : 0;
+  if (k > 0 && k <= kFastMaxK && k < vocab) {
+    if (sample_few_survivors(x, vocab, T, k, min_p ? min_p[r] : 0.f, top_p ? top_p[r] : 1.0f, uniform[r], out + r, red))
+      return;
+  }
 
   // softmax(logits / T)
   float mx = -INFINITY;
@@ -172,7 +304,6 @@ __global__ __launch_bounds__(kSampThreads) void sample_rows_kernel(
   __syncthreads();
 
   // top-k: largest threshold whose count of p >= threshold is still >= k
-  const int k = top_k ? top_k[r] : 0;
   if (k > 0 && k < vocab) {
     uint32_t lo = 0u, hi = 0x7f800000u;  // invariant: count(>= lo) >= k, count(>= hi + 1) < k
     while (lo < hi) {

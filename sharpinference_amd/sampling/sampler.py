@@ -15,7 +15,6 @@ src/SharpInference.Engine/ContinuousBatchingEngine.cs:732.)
 """
 from __future__ import annotations
 
-from collections import Counter
 from typing import List, Optional, Sequence
 
 import numpy as np
@@ -41,9 +40,14 @@ def uniform(seed: int, index: int) -> float:
 def penalty_window(params: SamplingParams, prompt: Sequence[int], generated: Sequence[int]) -> List[int]:
     """The tokens the penalties look at (reference: src/SharpInference.Engine/PenaltyWindow.cs;
     Sampler.cs:690-741)."""
-    hist = (list(prompt) if params.penalty_seed_from_prompt else []) + list(generated)
     n = params.penalty_last_n
-    return hist[-n:] if n > 0 else hist
+    if n > 0 and len(generated) >= n:
+        return list(generated[-n:])
+    if not params.penalty_seed_from_prompt:
+        return list(generated)
+    if n <= 0:
+        return list(prompt) + list(generated)
+    return list(prompt[len(prompt) - min(len(prompt), n - len(generated)):]) + list(generated)
 
 
 class Sampler:
@@ -72,33 +76,55 @@ class Sampler:
                 sub = ops.cast(logits, torch.float32)   # a copy: the caller's logits stay as they are
             self._edit(sub, ps, [histories[r] if histories is not None else () for r in rows], V)
         dev = self.device
-        temp = torch.tensor([p.temperature for p in ps], dtype=torch.float32, device=dev)
-        u = torch.tensor([uniform(p.seed, draw_index[r]) for p, r in zip(ps, rows)], dtype=torch.float32, device=dev)
-        top_k = torch.tensor([p.top_k for p in ps], dtype=torch.int32, device=dev) if any(p.top_k > 0 for p in ps) else None
-        top_p = torch.tensor([p.top_p for p in ps], dtype=torch.float32, device=dev) if any(0 < p.top_p < 1 for p in ps) else None
-        min_p = torch.tensor([p.min_p for p in ps], dtype=torch.float32, device=dev) if any(p.min_p > 0 for p in ps) else None
-        ids = ops.sample_rows(sub, temp, u, top_k, top_p, min_p).cpu().tolist()
+        n = len(ps)
+        # temperature, uniform, top-p and min-p of the rows in one copy, top-k in another
+        f = torch.tensor([[p.temperature for p in ps], [uniform(p.seed, draw_index[r]) for p, r in zip(ps, rows)],
+                          [p.top_p for p in ps], [p.min_p for p in ps]], dtype=torch.float32).to(dev)
+        top_k = torch.tensor([p.top_k for p in ps], dtype=torch.int32).to(dev) if any(p.top_k > 0 for p in ps) else None
+        top_p = f[2] if any(0 < p.top_p < 1 for p in ps) else None
+        min_p = f[3] if any(p.min_p > 0 for p in ps) else None
+        assert f.shape == (4, n)
+        ids = ops.sample_rows(sub, f[0], f[1], top_k, top_p, min_p).cpu().tolist()
         for r, t in zip(rows, ids):
             out[r] = t
         return out
 
     def _edit(self, logits: torch.Tensor, ps: Sequence[SamplingParams], hists, vocab: int) -> None:
-        offs, ids, counts, bias = [0], [], [], []
+        """The rows' sparse edits (distinct tokens of the window with their counts, biased tokens), laid
+        out on the host as one integer and one float array: two copies to the device, one launch."""
+        R = len(ps)
+        row_ids, row_counts, row_bias = [], [], []
         for p, h in zip(ps, hists):
-            cnt = Counter(int(t) for t in h) if p.has_penalties else Counter()
-            b = dict(p.logit_bias or {})
-            for t in sorted(set(cnt) | set(b)):
-                if 0 <= t < vocab:
-                    ids.append(t)
-                    counts.append(cnt.get(t, 0))
-                    bias.append(float(b.get(t, 0.0)))
-            offs.append(len(ids))
-        dev = self.device
-        i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)  # noqa: E731
-        f32 = lambda x: torch.tensor(x, dtype=torch.float32, device=dev)  # noqa: E731
-        ops.edit_logits(logits, i32(offs), i32(ids), i32(counts), f32(bias),
-                        f32([p.repetition_penalty for p in ps]), f32([p.frequency_penalty for p in ps]),
-                        f32([p.presence_penalty for p in ps]))
+            if p.has_penalties and len(h):
+                ids, cnt = np.unique(np.asarray(h, dtype=np.int64), return_counts=True)   # ascending ids
+            else:
+                ids, cnt = np.empty(0, np.int64), np.empty(0, np.int64)
+            b = np.zeros(ids.shape[0], np.float32)
+            if p.logit_bias:
+                extra = np.asarray(sorted(int(t) for t in p.logit_bias if int(t) not in set(ids.tolist())), dtype=np.int64)
+                ids = np.concatenate([ids, extra])
+                cnt = np.concatenate([cnt, np.zeros(extra.shape[0], np.int64)])
+                order = np.argsort(ids, kind="stable")
+                ids, cnt = ids[order], cnt[order]
+                b = np.asarray([float(p.logit_bias.get(int(t), 0.0)) for t in ids], dtype=np.float32)
+            ok = (ids >= 0) & (ids < vocab)
+            row_ids.append(ids[ok]); row_counts.append(cnt[ok]); row_bias.append(b[ok])
+        lens = [a.shape[0] for a in row_ids]
+        n = int(sum(lens))
+        ints = np.empty(R + 1 + 2 * n, np.int32)
+        ints[0] = 0
+        np.cumsum(lens, out=ints[1:R + 1])
+        ints[R + 1:R + 1 + n] = np.concatenate(row_ids) if n else 0
+        ints[R + 1 + n:] = np.concatenate(row_counts) if n else 0
+        flts = np.empty(n + 3 * R, np.float32)
+        flts[:n] = np.concatenate(row_bias) if n else 0
+        flts[n:n + R] = [p.repetition_penalty for p in ps]
+        flts[n + R:n + 2 * R] = [p.frequency_penalty for p in ps]
+        flts[n + 2 * R:] = [p.presence_penalty for p in ps]
+        di = torch.from_numpy(ints).to(self.device)
+        df = torch.from_numpy(flts).to(self.device)
+        ops.edit_logits(logits, di[:R + 1], di[R + 1:R + 1 + n], di[R + 1 + n:], df[:n], df[n:n + R],
+                        df[n + R:n + 2 * R], df[n + 2 * R:])
 
 
 def _gather_rows(logits: torch.Tensor, rows: Sequence[int]) -> torch.Tensor:

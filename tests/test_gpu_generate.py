@@ -155,6 +155,43 @@ def test_sampling_kernels_against_plain():
         assert got == want, case
 
 
+def test_sampling_with_a_small_top_k_over_a_large_vocabulary():
+    """Rows with a small top-k gather the few entries that can survive and finish in LDS; larger k, and
+    rows where too many entries tie at the cut, take the full path: both against the plain implementation,
+    over many uniforms (also at the ends of [0, 1)), with ties at the k-th value."""
+    from sharpinference_amd import ops
+
+    g = torch.Generator().manual_seed(4)
+    V = 50021
+    R = 8
+    logits = torch.randn(R, V, generator=g) * 2.5
+    logits[1, 40000] = logits[1, 7] = logits[1, 123]                      # ties somewhere
+    top = torch.topk(logits[2], 5).values[-1].item()
+    logits[2, 11] = logits[2, 30011] = top                               # three entries tie at the 5th value
+    logits[3] = 0.25                                                     # all equal: every entry survives any k
+    logits[4] *= 0.01                                                    # nearly flat
+    logits[5, 49999] = 30.0                                              # one entry holds all the mass
+    logits = logits.to(DEV)
+    cases = [dict(temperature=1.0, top_k=5), dict(temperature=0.7, top_k=40, top_p=0.95, min_p=0.05),
+             dict(temperature=1.5, top_k=256, top_p=0.9), dict(temperature=0.8, top_k=300, min_p=0.02),
+             dict(temperature=1.1, top_k=1), dict(temperature=0.9, top_k=64, top_p=0.5)]
+    for case in cases:
+        for draw in range(3):
+            us = P.uniform_stream(11 + draw, R)
+            us[0], us[7] = (0.0, 1.0 - 2.0 ** -24) if draw == 0 else (us[0], us[7])
+            temp = torch.full((R,), case["temperature"], device=DEV)
+            tk = torch.full((R,), case.get("top_k", 0), dtype=torch.int32, device=DEV)
+            tp = torch.full((R,), case.get("top_p", 1.0), device=DEV)
+            mp = torch.full((R,), case.get("min_p", 0.0), device=DEV)
+            got = ops.sample_rows(logits, temp, torch.tensor(us, device=DEV), tk, tp, mp).cpu().tolist()
+            want = [P.sample(logits[i].cpu(), us[i], **case) for i in range(R)]
+            # row 3 is 50,021 equal probabilities: where their running sum passes u depends on the order of
+            # the additions to the last bit, and which of equal values the nucleus keeps is left open
+            assert "top_p" in case or abs(got[3] - want[3]) <= 2, (case, draw, got[3], want[3])
+            got[3] = want[3] = -1
+            assert got == want, (case, draw, got, want)
+
+
 def test_penalties_and_bias_follow_the_reference_order():
     """reference: src/SharpInference.Engine/Sampler.cs:52-69, 414-433: bias, then the repetition
     penalty once per distinct token (divide if positive, multiply if negative), then

@@ -151,3 +151,19 @@ def test_the_model_s_end_tokens_stop_a_request_unless_it_replaces_them():
     assert plain.output == [50, 50] and plain.finish_reason == "stop"
     assert deaf.output == [50, 50, 8, 50, 50, 50] and deaf.finish_reason == "length"
     assert more.output == [] and more.finish_reason == "stop"
+
+
+def test_the_penalty_window_is_the_tail_of_prompt_and_output():
+    """The last penalty_last_n tokens of prompt + output (0 = all), the prompt left out if it is not to
+    seed the window (reference: src/SharpInference.Engine/Sampler.cs:764-798)."""
+    import random
+
+    from sharpinference_amd.sampling.sampler import penalty_window
+
+    rng = random.Random(0)
+    for _ in range(2000):
+        p = SamplingParams(penalty_last_n=rng.choice([0, 1, 3, 5, 8, 100]), penalty_seed_from_prompt=rng.random() < 0.5)
+        prompt = [rng.randrange(50) for _ in range(rng.randrange(0, 9))]
+        out = [rng.randrange(50) for _ in range(rng.randrange(0, 9))]
+        whole = (prompt if p.penalty_seed_from_prompt else []) + out
+        assert penalty_window(p, prompt, out) == (whole[-p.penalty_last_n:] if p.penalty_last_n > 0 else whole)
