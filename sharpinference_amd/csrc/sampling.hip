@@ -146,9 +146,13 @@ __device__ __forceinline__ void renormalise(float* p, int vocab, float* red) {
 // lower bound of the k-th largest probability: entries at or above it (a few more than k) go to
 // LDS, one per thread, and top-k, min-p, top-p, both renormalisations and the inverse CDF run
 // there, with the same definitions as the full path below (ties at a cut are all kept; the CDF
-// walks ascending indices).  The probabilities have the same bits as the full path's.  Returns
-// false, with nothing written, if more entries than threads reach the bound: the caller then
-// takes the full path.  Every thread of the block returns the same value.
+// walks ascending indices).  The probabilities have the same bits as the full path's.
+// Without a top-k (k = 0) the 256 largest-or-so entries are gathered the same way, and the result
+// stands if nothing else can survive: the gathered entries that pass min-p already hold top_p of
+// the mass (a peaked distribution), or min-p's cut lies at or above the gathering bound.
+// Returns false, with nothing written, if more entries than threads reach the bound or that
+// cannot be shown: the caller then takes the full path.  Every thread of the block returns the
+// same value.
 constexpr int kFastMaxK = 256;
 
 __device__ __forceinline__ bool sample_few_survivors(const float* __restrict__ x, int vocab, float T, int k, float mp,
@@ -184,7 +188,7 @@ __device__ __forceinline__ bool sample_few_survivors(const float* __restrict__ x
     const float o = a_p[j];
     rank += (o > lm || (o == lm && j < t)) ? 1 : 0;
   }
-  if (rank == k - 1) s_bound = lm;   // ranks are a permutation: one thread has this one
+  if (rank == (k > 0 ? k : kFastMaxK) - 1) s_bound = lm;   // ranks are a permutation: one thread has this one
   __syncthreads();
   const float bound = s_bound;
   for (int i = t; i < vocab; i += nt) {
@@ -207,7 +211,7 @@ __device__ __forceinline__ bool sample_few_survivors(const float* __restrict__ x
   const int idx = have ? b_i[t] : 0x7fffffff;
   int larger = 0;
   for (int j = 0; j < c; ++j) larger += b_p[j] > p0 ? 1 : 0;
-  const bool kept = have && larger < k;
+  const bool kept = have && (k > 0 ? larger < k : true);
   a_i[t] = kept ? idx : 0x7fffffff;
   __syncthreads();
   // in ascending index order: a_p / a_i [0, n)
@@ -227,16 +231,24 @@ __device__ __forceinline__ bool sample_few_survivors(const float* __restrict__ x
   float q = mine ? a_p[t] : 0.f;
   float total = 0.f;
   for (int j = 0; j < n; ++j) total += a_p[j];
-  if (total > 0.f && total != 1.0f) q *= 1.0f / total;
+  if (k > 0 && total > 0.f && total != 1.0f) q *= 1.0f / total;   // top-k renormalises; without it nothing has gone
   b_p[t] = q;
   __syncthreads();
+  float pm = 0.f;
+  for (int j = 0; j < n; ++j) pm = fmaxf(pm, b_p[j]);
   if (mp > 0.f) {
-    float pm = 0.f;
-    for (int j = 0; j < n; ++j) pm = fmaxf(pm, b_p[j]);
     if (q < mp * pm) q = 0.f;
     __syncthreads();
     b_p[t] = q;
     __syncthreads();
+  }
+  if (k <= 0) {
+    // what was not gathered lies below the bound: it is out if min-p cuts there or higher, or if the
+    // gathered entries alone reach top_p (then the descending sum stops among them)
+    float held = 0.f;
+    for (int j = 0; j < n; ++j) held += b_p[j];
+    const bool shown = (mp > 0.f && mp * pm >= bound) || (tp > 0.f && tp < 1.0f && held >= tp);
+    if (!shown) return false;
   }
   if (tp > 0.f && tp < 1.0f) {
     // the descending running sum reaches top_p at some value: an entry stays if what is strictly
@@ -280,7 +292,9 @@ __global__ __launch_bounds__(kSampThreads) void sample_rows_kernel(
   const float T = temperature[r];
   const float invT = 1.0f / T;
   const int k = top_k ? top_k[r] : 0;
-  if (k > 0 && k <= kFastMaxK && k < vocab) {
+  const float tp0 = top_p ? top_p[r] : 1.0f, mp0 = min_p ? min_p[r] : 0.f;
+  if ((k > 0 && k <= kFastMaxK && k < vocab) ||
+      (k <= 0 && vocab > kFastMaxK && (mp0 > 0.f || (tp0 > 0.f && tp0 < 1.0f)))) {
     if (sample_few_survivors(x, vocab, T, k, min_p ? min_p[r] : 0.f, top_p ? top_p[r] : 1.0f, uniform[r], out + r, red))
       return;
   }

@@ -171,14 +171,23 @@ def test_sampling_with_a_small_top_k_over_a_large_vocabulary():
     logits[3] = 0.25                                                     # all equal: every entry survives any k
     logits[4] *= 0.01                                                    # nearly flat
     logits[5, 49999] = 30.0                                              # one entry holds all the mass
+    logits[6] *= 3.0                                                     # peaked: a few hundred entries hold nearly all
+    logits[7] *= 2.0
     logits = logits.to(DEV)
+    # (without a top-k the few-entries path stands only where it can show that nothing else survives: the
+    # peaked rows; the flat ones go on to the full path)
     cases = [dict(temperature=1.0, top_k=5), dict(temperature=0.7, top_k=40, top_p=0.95, min_p=0.05),
              dict(temperature=1.5, top_k=256, top_p=0.9), dict(temperature=0.8, top_k=300, min_p=0.02),
-             dict(temperature=1.1, top_k=1), dict(temperature=0.9, top_k=64, top_p=0.5)]
+             dict(temperature=1.1, top_k=1), dict(temperature=0.9, top_k=64, top_p=0.5),
+             dict(temperature=1.0, top_p=0.9), dict(temperature=0.8, min_p=0.05),
+             dict(temperature=1.2, top_p=0.6, min_p=0.01), dict(temperature=0.6, top_p=0.99)]
     for case in cases:
         for draw in range(3):
             us = P.uniform_stream(11 + draw, R)
-            us[0], us[7] = (0.0, 1.0 - 2.0 ** -24) if draw == 0 else (us[0], us[7])
+            if draw == 0:
+                us[0] = 0.0
+                if "top_k" in case:      # (over thousands of entries it is the order of the additions that decides
+                    us[7] = 1.0 - 2.0 ** -24   # whether the running sum reaches the largest uniform at all)
             temp = torch.full((R,), case["temperature"], device=DEV)
             tk = torch.full((R,), case.get("top_k", 0), dtype=torch.int32, device=DEV)
             tp = torch.full((R,), case.get("top_p", 1.0), device=DEV)
