@@ -112,6 +112,104 @@ class SafetensorsSource(TensorSource):
         return host.to(self.device)
 
 
+class LayoutAdapter(TensorSource):
+    """Presents a checkpoint that is laid out otherwise under the names and shapes the model asks
+    for.  Nothing here knows a model: the adaptations are found from the names and shapes alone.
+
+    * A container prefix: a multimodal file keeps the text decoder under a prefix (for instance
+      ``language_model.``).  If a wanted name is absent but ``prefix + name`` exists for one common
+      prefix, names are read through it, and tensors outside the prefix (another tower's) are not
+      the decoder's business: they are neither loaded nor reported as unexpected.
+    * Fused expert matrices: ``X.gate_up_proj`` in place of ``X.gate_proj`` and ``X.up_proj``, split
+      along the axis that is twice the wanted one; stacked matrices stored ``[E, in, out]`` where
+      ``[E, out, in]`` is wanted are transposed (only where the two sizes differ, so that the shape
+      tells).
+    The reference does the like when it slices an expert out of a packed tensor and ties a missing
+    head to the embedding (reference: src/SharpInference.Engine/ForwardPass.cs:2105-2113, 410-413).
+    No published checkpoint could be read where this was written: the adaptations are tested on
+    files written in those layouts by the tests."""
+
+    def __init__(self, inner: TensorSource, specs: Dict[str, ParamSpec]):
+        self.inner = inner
+        self.where = inner.where
+        have = inner.available()
+        self.prefix = self._find_prefix(specs, have)
+        self._plan: Dict[str, tuple] = {}
+        self._avail: Dict[str, Tuple[Tuple[int, ...], torch.dtype]] = {}
+        used = set()
+        for name, spec in specs.items():
+            src = self.prefix + name
+            want = tuple(spec.shape)
+            if src in have:
+                shape, dtype = have[src]
+                if tuple(shape) != want and len(want) == 3 and tuple(shape) == (want[0], want[2], want[1]) and want[1] != want[2]:
+                    self._plan[name] = ("transpose", src)
+                    self._avail[name] = (want, dtype)
+                else:
+                    self._plan[name] = ("plain", src)
+                    self._avail[name] = (tuple(shape), dtype)
+                used.add(src)
+                continue
+            fused = self._fused_source(name)
+            if fused and self.prefix + fused[0] in have:
+                fsrc, half = self.prefix + fused[0], fused[1]
+                shape, dtype = have[fsrc]
+                how = self._split_plan(tuple(shape), want)
+                if how is not None:
+                    self._plan[name] = ("split", fsrc, half, how)
+                    self._avail[name] = (want, dtype)
+                    used.add(fsrc)
+        for n, v in have.items():
+            if n not in used and n.startswith(self.prefix):
+                self._avail.setdefault(n[len(self.prefix):], v)     # shown so that check_specs can call it unexpected
+
+    @staticmethod
+    def _find_prefix(specs, have) -> str:
+        if any(n in have for n in specs):
+            return ""
+        first = next(iter(specs), None)
+        if first is None:
+            return ""
+        found = {n[:-len(first)] for n in have if n.endswith(first) and len(n) > len(first)}
+        good = [p for p in found if sum(1 for n in specs if p + n in have) * 2 >= len(specs)]
+        return sorted(good, key=len)[0] if good else ""
+
+    @staticmethod
+    def _fused_source(name: str):
+        for part, half in (("gate_proj", 0), ("up_proj", 1)):
+            head, sep, tail = name.rpartition(part)
+            if sep and not head.endswith("gate_"):
+                return head + "gate_up_proj" + tail, half
+        return None
+
+    @staticmethod
+    def _split_plan(shape, want):
+        """(axis to split, transpose afterwards) for a fused tensor of `shape` giving `want`, or None."""
+        if len(shape) != len(want):
+            return None
+        if shape[:-2] == want[:-2]:
+            if shape[-2] == 2 * want[-2] and shape[-1] == want[-1]:
+                return (len(shape) - 2, False)
+            if shape[-1] == 2 * want[-2] and shape[-2] == want[-1]:
+                return (len(shape) - 1, True)
+        return None
+
+    def available(self):
+        return dict(self._avail)
+
+    def get(self, name: str) -> torch.Tensor:
+        plan = self._plan[name]
+        if plan[0] == "plain":
+            return self.inner.get(plan[1])
+        if plan[0] == "transpose":
+            return self.inner.get(plan[1]).transpose(1, 2).contiguous()
+        _, src, half, (axis, transpose) = plan
+        t = self.inner.get(src)
+        n = t.shape[axis] // 2
+        t = t.narrow(axis, half * n, n)
+        return (t.transpose(-1, -2) if transpose else t).contiguous()
+
+
 def _name_seed(seed: int, name: str) -> int:
     h = hashlib.sha256(f"{seed}:{name}".encode()).digest()
     return int.from_bytes(h[:8], "little") & ((1 << 63) - 1)
@@ -192,6 +290,8 @@ class RandomSource(TensorSource):
 def load_model_weights(model, source: TensorSource) -> None:
     """Check the source against the model's request, then let the parts take their tensors."""
     specs = model.param_specs()
+    if isinstance(source, SafetensorsSource):
+        source = LayoutAdapter(source, specs)        # other layouts of the same tensors (prefix, fused experts)
     check_specs(specs, source.available(), source.where)
     model.load_weights(source)
 
