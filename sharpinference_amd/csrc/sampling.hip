@@ -108,6 +108,7 @@ __device__ __forceinline__ void count_sum_ge(const float* p, int vocab, uint32_t
                                              int* red_i, int& count, float& sum) {
   int c = 0;
   float s = 0.f;
+  #pragma unroll 8
   for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
     const float v = p[i];
     if (__float_as_uint(v) >= thr_bits) {
@@ -130,10 +131,12 @@ __device__ __forceinline__ void count_sum_ge(const float* p, int vocab, uint32_t
 
 __device__ __forceinline__ void renormalise(float* p, int vocab, float* red) {
   float s = 0.f;
+  #pragma unroll 8
   for (int i = threadIdx.x; i < vocab; i += blockDim.x) s += p[i];
   const float total = block_sum(s, red);
   if (total > 0.f && total != 1.0f) {
     const float inv = 1.0f / total;
+    #pragma unroll 8
     for (int i = threadIdx.x; i < vocab; i += blockDim.x) p[i] *= inv;
   }
   __syncthreads();
@@ -169,9 +172,11 @@ __device__ __forceinline__ bool sample_few_survivors(const float* __restrict__ x
   const bool scaled = T != 1.0f;
 
   float vmax = -INFINITY;
+  #pragma unroll 8
   for (int i = t; i < vocab; i += nt) vmax = fmaxf(vmax, scaled ? x[i] * invT : x[i]);
   const float mx = block_max(vmax, red);
   float s = 0.f;
+  #pragma unroll 8
   for (int i = t; i < vocab; i += nt) s += expf((scaled ? x[i] * invT : x[i]) - mx);
   const float inv_sum = 1.0f / block_sum(s, red);
 
@@ -191,6 +196,7 @@ __device__ __forceinline__ bool sample_few_survivors(const float* __restrict__ x
   if (rank == (k > 0 ? k : kFastMaxK) - 1) s_bound = lm;   // ranks are a permutation: one thread has this one
   __syncthreads();
   const float bound = s_bound;
+  #pragma unroll 8
   for (int i = t; i < vocab; i += nt) {
     const float p = expf((scaled ? x[i] * invT : x[i]) - mx) * inv_sum;
     if (p >= bound) {
@@ -301,6 +307,7 @@ __global__ __launch_bounds__(kSampThreads) void sample_rows_kernel(
 
   // softmax(logits / T)
   float mx = -INFINITY;
+  #pragma unroll 8
   for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
     const float v = (T != 1.0f) ? x[i] * invT : x[i];
     p[i] = v;
@@ -308,12 +315,14 @@ __global__ __launch_bounds__(kSampThreads) void sample_rows_kernel(
   }
   mx = block_max(mx, red);
   float s = 0.f;
+  #pragma unroll 8
   for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
     const float e = expf(p[i] - mx);
     p[i] = e;
     s += e;
   }
   const float inv_sum = 1.0f / block_sum(s, red);
+  #pragma unroll 8
   for (int i = threadIdx.x; i < vocab; i += blockDim.x) p[i] *= inv_sum;
   __syncthreads();
 
@@ -327,6 +336,7 @@ __global__ __launch_bounds__(kSampThreads) void sample_rows_kernel(
       count_sum_ge(p, vocab, mid, red, red_i, c, sm);
       if (c >= k) lo = mid; else hi = mid - 1;
     }
+    #pragma unroll 8
     for (int i = threadIdx.x; i < vocab; i += blockDim.x)
       if (__float_as_uint(p[i]) < lo) p[i] = 0.f;
     __syncthreads();
@@ -336,9 +346,11 @@ __global__ __launch_bounds__(kSampThreads) void sample_rows_kernel(
   const float mp = min_p ? min_p[r] : 0.f;
   if (mp > 0.f) {
     float pm = 0.f;
+    #pragma unroll 8
     for (int i = threadIdx.x; i < vocab; i += blockDim.x) pm = fmaxf(pm, p[i]);
     pm = block_max(pm, red);
     const float thr = mp * pm;
+    #pragma unroll 8
     for (int i = threadIdx.x; i < vocab; i += blockDim.x)
       if (p[i] < thr) p[i] = 0.f;
     __syncthreads();
@@ -354,6 +366,7 @@ __global__ __launch_bounds__(kSampThreads) void sample_rows_kernel(
       count_sum_ge(p, vocab, mid, red, red_i, c, sm);
       if (sm >= tp) lo = mid; else hi = mid - 1;
     }
+    #pragma unroll 8
     for (int i = threadIdx.x; i < vocab; i += blockDim.x)
       if (__float_as_uint(p[i]) < lo) p[i] = 0.f;
     __syncthreads();
