@@ -10,7 +10,7 @@ from sharpinference_amd.config.llama4 import Llama4TextConfig
 from sharpinference_amd.weights import safetensors_io as st
 from sharpinference_amd.weights.loader import (RandomSource, SafetensorsSource, WeightError, check_specs,
                                                load_model_weights, storage_dtype, write_random_model)
-from tiny_configs import CONFIGS, TINY_A, TINY_B, make_model_dir
+from tiny_configs import CONFIGS, TINY_A, TINY_B, make_model_dir, write_other_layout
 
 
 def test_every_key_is_read_and_round_trips():
@@ -285,30 +285,6 @@ def test_a_head_size_no_kernel_takes_is_refused_when_the_model_is_built():
         build_model(load_config({**TINY_A, "num_local_experts": 1025}))
 
 
-def _write_other_layout(src_dir, out_dir, prefix, extra=()):
-    """The tensors of a model folder under a container prefix, the experts' gate and up fused as
-    [E, in, 2 * out] and their down stored [E, in, out]; `extra` tensors are added as they are."""
-    entries = st.index_folder(src_dir)
-    tensors = {n: st.read_tensor(e) for n, e in entries.items()}
-    out = {}
-    for n, t in tensors.items():
-        if n.endswith("experts.gate_proj"):
-            up = tensors[n[:-len("gate_proj")] + "up_proj"]
-            out[prefix + n[:-len("gate_proj")] + "gate_up_proj"] = torch.cat([t, up], 1).transpose(1, 2).contiguous()
-        elif n.endswith("experts.up_proj"):
-            continue
-        elif n.endswith("experts.down_proj"):
-            out[prefix + n] = t.transpose(1, 2).contiguous()
-        else:
-            out[prefix + n] = t
-    out.update(extra)
-    os.makedirs(out_dir, exist_ok=True)
-    with open(os.path.join(src_dir, "config.json")) as f, open(os.path.join(out_dir, "config.json"), "w") as g:
-        g.write(f.read())
-    st.write_file(os.path.join(out_dir, "model.safetensors"), sorted(out.items()))
-    return out_dir
-
-
 def test_other_layouts_of_the_same_tensors_are_read(tmp_path):
     """A container prefix, fused gate|up and [E, in, out] experts are found from names and shapes."""
     from sharpinference_amd.weights.loader import LayoutAdapter
@@ -316,7 +292,7 @@ def test_other_layouts_of_the_same_tensors_are_read(tmp_path):
     d = make_model_dir(tmp_path, "B")
     cfg = load_config(d)
     specs = build_model(cfg).param_specs()
-    other = _write_other_layout(d, str(tmp_path / "other"), "language_model.",
+    other = write_other_layout(d, str(tmp_path / "other"), "language_model.",
                                 extra={"vision_model.patch.weight": torch.zeros(3, 5, dtype=torch.bfloat16)})
     plain = SafetensorsSource(d, torch.bfloat16, "cpu")
     adapted = LayoutAdapter(SafetensorsSource(other, torch.bfloat16, "cpu"), specs)
@@ -327,7 +303,7 @@ def test_other_layouts_of_the_same_tensors_are_read(tmp_path):
     # a canonical folder passes through untouched, and faults are still told in one error
     same = LayoutAdapter(SafetensorsSource(d, torch.bfloat16, "cpu"), specs)
     assert same.prefix == "" and all(torch.equal(same.get(n), plain.get(n)) for n in list(specs)[:5])
-    broken = _write_other_layout(d, str(tmp_path / "broken"), "language_model.",
+    broken = write_other_layout(d, str(tmp_path / "broken"), "language_model.",
                                  extra={"language_model.model.layers.9.extra.weight": torch.zeros(2, dtype=torch.bfloat16)})
     with pytest.raises(WeightError) as e:
         check_specs(specs, LayoutAdapter(SafetensorsSource(broken, torch.bfloat16, "cpu"), specs).available(), broken)

@@ -3,7 +3,7 @@ import pytest
 import torch
 
 import helpers as H
-from tiny_configs import CONFIGS, make_model_dir
+from tiny_configs import CONFIGS, make_model_dir, write_other_layout
 
 pytestmark = pytest.mark.gpu
 
@@ -178,10 +178,8 @@ def test_decode_graphs_follow_the_context(tmp_path):
 
 def test_a_checkpoint_in_another_layout_gives_the_same_logits(tmp_path):
     """A container prefix, fused gate|up and [E, in, out] experts: the engine reads the same model."""
-    from test_config_weights import _write_other_layout
-
     d = make_model_dir(tmp_path, "B", std=0.1)
-    other = _write_other_layout(d, str(tmp_path / "other"), "language_model.")
+    other = write_other_layout(d, str(tmp_path / "other"), "language_model.")
     toks = H.random_tokens(40, 384, 3)
     a = H.run_cut(H.make_engine(d, "float32"), "a", toks, H.whole(len(toks)))
     b = H.run_cut(H.make_engine(other, "float32"), "b", toks, H.whole(len(toks)))

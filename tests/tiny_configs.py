@@ -71,3 +71,33 @@ def make_model_dir(tmp_path, which: str, std: float = 0.02, **overrides) -> str:
     out = str(tmp_path / f"tiny_{which}")
     write_random_model(cfg, out, SEEDS[which], std=std, float32_names=FLOAT32_NAMES[which])
     return out
+
+
+def write_other_layout(src_dir, out_dir, prefix, extra=()):
+    """The tensors of a model folder under a container prefix, the experts' gate and up fused as
+    [E, in, 2 * out] and their down stored [E, in, out]; `extra` tensors are added as they are."""
+    import os
+
+    import torch
+
+    from sharpinference_amd.weights import safetensors_io as st
+
+    entries = st.index_folder(src_dir)
+    tensors = {n: st.read_tensor(e) for n, e in entries.items()}
+    out = {}
+    for n, t in tensors.items():
+        if n.endswith("experts.gate_proj"):
+            up = tensors[n[:-len("gate_proj")] + "up_proj"]
+            out[prefix + n[:-len("gate_proj")] + "gate_up_proj"] = torch.cat([t, up], 1).transpose(1, 2).contiguous()
+        elif n.endswith("experts.up_proj"):
+            continue
+        elif n.endswith("experts.down_proj"):
+            out[prefix + n] = t.transpose(1, 2).contiguous()
+        else:
+            out[prefix + n] = t
+    out.update(extra)
+    os.makedirs(out_dir, exist_ok=True)
+    with open(os.path.join(src_dir, "config.json")) as f, open(os.path.join(out_dir, "config.json"), "w") as g:
+        g.write(f.read())
+    st.write_file(os.path.join(out_dir, "model.safetensors"), sorted(out.items()))
+    return out_dir
