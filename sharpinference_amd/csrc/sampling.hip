@@ -284,6 +284,57 @@ __device__ __forceinline__ bool sample_few_survivors(const float* __restrict__ x
   return true;
 }
 
+// Rows without any filter: token i has probability e_i / S with e_i = exp(v_i - max), so the first
+// index whose running sum of e reaches u * S is the one whose running sum of e / S reaches u.
+// No probability is written: one pass for the maximum, one in which every thread adds up its
+// contiguous piece of the row, and the thread whose piece holds the target walks it once more.
+// S is the running sum at the last entry, so the target (u < 1) always lies inside the row.
+__device__ __forceinline__ void sample_unfiltered(const float* __restrict__ x, int vocab, float T, float u,
+                                                  int* __restrict__ out_r, float* red) {
+  __shared__ double piece[kSampThreads];
+  const int t = threadIdx.x;
+  const int nt = blockDim.x;
+  const float invT = 1.0f / T;
+  const bool scaled = T != 1.0f;
+  float vmax = -INFINITY;
+#pragma unroll 8
+  for (int i = t; i < vocab; i += nt) vmax = fmaxf(vmax, scaled ? x[i] * invT : x[i]);
+  const float mx = block_max(vmax, red);
+  const int chunk = (vocab + nt - 1) / nt;
+  const int b = min(t * chunk, vocab), e = min(b + chunk, vocab);
+  double cs = 0.0;   // the running sums are kept in double: where the target falls is then decided by the
+                     // terms themselves, not by the rounding of sums of thousands of them
+#pragma unroll 4
+  for (int i = b; i < e; ++i) cs += (double)expf((scaled ? x[i] * invT : x[i]) - mx);
+  piece[t] = cs;
+  __syncthreads();
+  // running sums before and after this thread's piece, and the whole, each added up in the same
+  // ascending order by every thread that needs them
+  double before = 0.0, total = 0.0;
+  for (int j = 0; j < nt; ++j) {
+    if (j == t) before = total;
+    total += piece[j];
+  }
+  const double target = (double)u * total;
+  if (u <= 0.f) {
+    if (t == 0) *out_r = 0;   // a uniform of exactly 0 is reached at index 0 already
+    return;
+  }
+  // exactly one piece has before < target <= before + piece (the sums are the same numbers in every thread)
+  if (b < e && before < target && target <= before + cs) {
+    double run = before;
+    int pick = e - 1;
+    for (int i = b; i < e; ++i) {
+      run += (double)expf((scaled ? x[i] * invT : x[i]) - mx);
+      if (target <= run) {
+        pick = i;
+        break;
+      }
+    }
+    *out_r = pick;
+  }
+}
+
 __global__ __launch_bounds__(kSampThreads) void sample_rows_kernel(
     const float* __restrict__ logits, float* __restrict__ probs, const float* __restrict__ temperature,
     const float* __restrict__ uniform, const int* __restrict__ top_k, const float* __restrict__ top_p,
@@ -299,6 +350,10 @@ __global__ __launch_bounds__(kSampThreads) void sample_rows_kernel(
   const float invT = 1.0f / T;
   const int k = top_k ? top_k[r] : 0;
   const float tp0 = top_p ? top_p[r] : 1.0f, mp0 = min_p ? min_p[r] : 0.f;
+  if ((k <= 0 || k >= vocab) && mp0 <= 0.f && !(tp0 > 0.f && tp0 < 1.0f)) {
+    sample_unfiltered(x, vocab, T, uniform[r], out + r, red);
+    return;
+  }
   if ((k > 0 && k <= kFastMaxK && k < vocab) ||
       (k <= 0 && vocab > kFastMaxK && (mp0 > 0.f || (tp0 > 0.f && tp0 < 1.0f)))) {
     if (sample_few_survivors(x, vocab, T, k, min_p ? min_p[r] : 0.f, top_p ? top_p[r] : 1.0f, uniform[r], out + r, red))
