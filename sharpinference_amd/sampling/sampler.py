@@ -93,6 +93,28 @@ class Sampler:
         """The rows' sparse edits (distinct tokens of the window with their counts, biased tokens), laid
         out on the host as one integer and one float array: two copies to the device, one launch."""
         R = len(ps)
+        if not any(p.logit_bias for p in ps):
+            # penalties only (the usual case): the distinct (row, token) pairs of all windows in one sort
+            wins = [(r, np.asarray(h, dtype=np.int64)) for r, (p, h) in enumerate(zip(ps, hists))
+                    if p.has_penalties and len(h)]
+            if all(int(w.min()) >= 0 and int(w.max()) < vocab for _, w in wins):   # (else the careful path drops them)
+                flat = np.concatenate([w + r * vocab for r, w in wins]) if wins else np.empty(0, np.int64)
+                uniq, cnt = np.unique(flat, return_counts=True)           # ascending by row, then by token
+                n = uniq.shape[0]
+                ints = np.empty(R + 1 + 2 * n, np.int32)
+                ints[0] = 0
+                np.cumsum(np.bincount(uniq // vocab, minlength=R)[:R], out=ints[1:R + 1])
+                ints[R + 1:R + 1 + n] = uniq % vocab
+                ints[R + 1 + n:] = cnt
+                flts = np.zeros(n + 3 * R, np.float32)
+                flts[n:n + R] = [p.repetition_penalty for p in ps]
+                flts[n + R:n + 2 * R] = [p.frequency_penalty for p in ps]
+                flts[n + 2 * R:] = [p.presence_penalty for p in ps]
+                di = torch.from_numpy(ints).to(self.device)
+                df = torch.from_numpy(flts).to(self.device)
+                ops.edit_logits(logits, di[:R + 1], di[R + 1:R + 1 + n], di[R + 1 + n:], df[:n], df[n:n + R],
+                                df[n + R:n + 2 * R], df[n + 2 * R:])
+                return
         row_ids, row_counts, row_bias = [], [], []
         for p, h in zip(ps, hists):
             if p.has_penalties and len(h):
