@@ -143,7 +143,7 @@ def decode_run(eng, batch: int, steps: int, warmup: int, rng: random.Random, cou
     if count_experts:
         trace: list = []
         last = one_step(last, trace)
-        distinct = sum(len(set(p.flatten().cpu().tolist())) for p, _ in trace) / max(1, len(trace))
+        distinct = sum(len(set(p.flatten().cpu().tolist())) for p, _, _ in trace) / max(1, len(trace))
     ctx = eng.cache.length(ids[0])
     for r in ids:
         eng.free_request(r)

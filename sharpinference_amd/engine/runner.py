@@ -170,7 +170,7 @@ class ModelRunner:
         return out
 
     # ------------------------------------------------------------------
-    def _decode_graph_step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+    def _decode_graph_step(self, entries: Sequence[StepEntry], router_trace: Optional[list] = None) -> Optional[torch.Tensor]:
         """Replay the captured graph of this batch size if the step qualifies: every entry one
         token whose logits are wanted, all contexts within the captured bound.  None otherwise."""
         n = len(entries)
@@ -205,13 +205,13 @@ class ModelRunner:
                 return None
             self._graphs[key] = graph
         self.graph_replays += 1
-        return graph.replay(pieces)
+        return graph.replay(pieces, router_trace)
 
     def step(self, entries: Sequence[StepEntry], router_trace: Optional[list] = None) -> Optional[torch.Tensor]:
         """Run one batch.  Returns float32 logits [wanted, vocab] in the order of the entries and
         of their ``want`` lists, or None when nothing is wanted.  A list given as ``router_trace``
-        receives, per routed layer run, the (expert ids, weights) of the step's tokens, as the
-        reference can print its router picks (src/SharpInference.Engine/ForwardPass.cs:2042-2056)."""
+        receives, per routed layer run, the (expert ids, weights, router input) of the step's tokens,
+        as the reference can print its router picks (src/SharpInference.Engine/ForwardPass.cs:2042-2056)."""
         if not entries:
             return None
         self._validate(entries)
@@ -221,7 +221,7 @@ class ModelRunner:
                 if not self.cache.append(e.req_id, len(e.tokens)):
                     raise CacheExhausted(f"no pages left for request {e.req_id!r} ({len(e.tokens)} more tokens)")
                 appended.append(e.req_id)
-            logits = self._decode_graph_step(entries) if router_trace is None else None
+            logits = self._decode_graph_step(entries, router_trace)
             if logits is None:
                 ctx, rows = self.build_context(entries)
                 if router_trace is not None:
@@ -274,6 +274,10 @@ class _DecodeGraph:
             runner.model.forward(ctx, caches, rows)
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
+        # the captured run also notes where its router picks lie (tensors of the graph's own memory,
+        # filled anew by every replay), so that a replayed step can be traced like a launched one
+        self.trace: list = []
+        ctx.extras["router_trace"] = self.trace
         self.graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(self.graph):
             self.logits = runner.model.forward(ctx, caches, rows)
@@ -288,7 +292,9 @@ class _DecodeGraph:
         self.dev.copy_(self.host, non_blocking=True)
         self.copied.record()
 
-    def replay(self, pieces) -> torch.Tensor:
+    def replay(self, pieces, router_trace: Optional[list] = None) -> torch.Tensor:
         self._upload(pieces)
         self.graph.replay()
+        if router_trace is not None:
+            router_trace.extend(tuple(t.clone() for t in item) for item in self.trace)
         return self.logits.clone()

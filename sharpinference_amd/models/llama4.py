@@ -53,3 +53,7 @@ def build_llama4(cfg: Llama4TextConfig) -> DecoderModel:
 
 
 register_architecture("Llama4ForCausalLM", Llama4TextConfig, build_llama4)
+# A multimodal folder names the container class; of it this engine runs the text decoder alone
+# (its keys sit under text_config, its tensors under a prefix that the loader strips; the other
+# towers' tensors are passed over).
+register_architecture("Llama4ForConditionalGeneration", Llama4TextConfig, build_llama4)

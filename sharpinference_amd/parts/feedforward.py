@@ -156,7 +156,7 @@ class MoESwiGLU(Part):
         T = x.shape[0]
         trace = ctx.extras.get("router_trace")
         if trace is not None:      # the picks of this step, layer by layer (reference: ForwardPass.cs:2042-2056)
-            trace.append((ids, wts))
+            trace.append((ids, wts, x))
         along = self.merged and T <= self.MERGE_MAX_TOKENS
         shared = None if along or self.shared is None else self.shared.forward(x, ctx)
         act = ops.gemm_skinny_picked(x, self.w_gate_up, ids, wts, along, True, True, ctx.act_dtype)
@@ -184,7 +184,7 @@ class MoESwiGLU(Part):
         merge = self.merged and T <= self.MERGE_MAX_TOKENS and ctx.act_dtype == torch.bfloat16
         ids, wts, rt = ops.route(x, self.w_router, self.k, self.gate, self.renormalise, shared_group=merge)
         if trace is not None:      # the picks of this step, layer by layer (reference: ForwardPass.cs:2042-2056)
-            trace.append((ids, wts))
+            trace.append((ids, wts, x))
         if merge:
             # few rows: the shared expert rides along as one more group of the same two launches
             act = ops.grouped_swiglu(x, self.w_gate_up, rt, ctx.act_dtype)

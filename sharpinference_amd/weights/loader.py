@@ -120,10 +120,12 @@ class LayoutAdapter(TensorSource):
       ``language_model.``).  If a wanted name is absent but ``prefix + name`` exists for one common
       prefix, names are read through it, and tensors outside the prefix (another tower's) are not
       the decoder's business: they are neither loaded nor reported as unexpected.
-    * Fused expert matrices: ``X.gate_up_proj`` in place of ``X.gate_proj`` and ``X.up_proj``, split
-      along the axis that is twice the wanted one; stacked matrices stored ``[E, in, out]`` where
-      ``[E, out, in]`` is wanted are transposed (only where the two sizes differ, so that the shape
-      tells).
+    * Fused expert matrices: ``X.gate_up_proj`` in place of ``X.gate_proj`` and ``X.up_proj``.  The
+      name decides the order of the axes: a stacked tensor without a ``.weight`` suffix holds
+      ``[E, in, 2 * out]`` (gate columns first), and the ``down_proj`` stored beside it holds
+      ``[E, in, out]``; a fused ``….weight`` holds ``[2 * out, in]`` as a linear layer does.  Where
+      the name does not decide, the shape may (a transposed stack whose two sizes differ); where
+      neither does, the tensor is left as it is and reported with its shape.
     The reference does the like when it slices an expert out of a packed tensor and ties a missing
     head to the embedding (reference: src/SharpInference.Engine/ForwardPass.cs:2105-2113, 410-413).
     No published checkpoint could be read where this was written: the adaptations are tested on
@@ -141,20 +143,22 @@ class LayoutAdapter(TensorSource):
             src = self.prefix + name
             want = tuple(spec.shape)
             if src in have:
-                shape, dtype = have[src]
-                if tuple(shape) != want and len(want) == 3 and tuple(shape) == (want[0], want[2], want[1]) and want[1] != want[2]:
+                shape, dtype = tuple(have[src][0]), have[src][1]
+                swapped = len(want) == 3 and shape == (want[0], want[2], want[1])
+                beside_fused = self._fused_sibling(name) is not None and self.prefix + self._fused_sibling(name) in have
+                if swapped and (beside_fused or want[1] != want[2]):
                     self._plan[name] = ("transpose", src)
                     self._avail[name] = (want, dtype)
                 else:
                     self._plan[name] = ("plain", src)
-                    self._avail[name] = (tuple(shape), dtype)
+                    self._avail[name] = (shape, dtype)
                 used.add(src)
                 continue
             fused = self._fused_source(name)
             if fused and self.prefix + fused[0] in have:
                 fsrc, half = self.prefix + fused[0], fused[1]
                 shape, dtype = have[fsrc]
-                how = self._split_plan(tuple(shape), want)
+                how = self._split_plan(tuple(shape), want, stacked_in_out=not fsrc.endswith(".weight"))
                 if how is not None:
                     self._plan[name] = ("split", fsrc, half, how)
                     self._avail[name] = (want, dtype)
@@ -183,15 +187,25 @@ class LayoutAdapter(TensorSource):
         return None
 
     @staticmethod
-    def _split_plan(shape, want):
-        """(axis to split, transpose afterwards) for a fused tensor of `shape` giving `want`, or None."""
-        if len(shape) != len(want):
+    def _fused_sibling(name: str):
+        """The fused gate|up tensor that a stacked ``down_proj`` would be stored beside."""
+        head, sep, tail = name.rpartition("down_proj")
+        return head + "gate_up_proj" + tail if sep and not tail else None
+
+    @staticmethod
+    def _split_plan(shape, want, stacked_in_out: bool):
+        """(axis to split, transpose afterwards) for a fused tensor of `shape` giving `want`, or
+        None.  `stacked_in_out`: the name says [.., in, 2 * out]; otherwise it says [.., 2 * out, in]."""
+        if len(shape) != len(want) or len(shape) < 2 or shape[:-2] != want[:-2]:
             return None
-        if shape[:-2] == want[:-2]:
-            if shape[-2] == 2 * want[-2] and shape[-1] == want[-1]:
-                return (len(shape) - 2, False)
-            if shape[-1] == 2 * want[-2] and shape[-2] == want[-1]:
-                return (len(shape) - 1, True)
+        rows = shape[-2:] == (2 * want[-2], want[-1])          # [.., 2 * out, in]
+        cols = shape[-2:] == (want[-1], 2 * want[-2])          # [.., in, 2 * out]
+        if rows and cols:
+            cols, rows = stacked_in_out, not stacked_in_out
+        if cols:
+            return (len(shape) - 1, True)
+        if rows:
+            return (len(shape) - 2, False)
         return None
 
     def available(self):

@@ -15,6 +15,10 @@ import plain_llama4 as P
 ROUTE_REGRET = 0.02
 
 
+def assert_route_regret(regret: float, what: str) -> None:
+    assert regret <= ROUTE_REGRET, f"{what}: the engine picked an expert {regret:.3f} (relative) below the best"
+
+
 def random_tokens(n: int, vocab: int, seed: int) -> List[int]:
     rng = random.Random(seed)
     return [rng.randrange(vocab) for _ in range(n)]
@@ -69,7 +73,7 @@ def run_cut(engine, rid, tokens: Sequence[int], sizes: Sequence[int], with_route
         trace: list = []
         lg = engine.step([StepEntry(rid, list(tokens[o:o + s]), list(range(s)))], router_trace=trace)
         out.append(lg.float().cpu())
-        picks.append([ids.cpu() for ids, _ in trace])
+        picks.append([ids.cpu() for ids, _, _ in trace])
         o += s
     engine.free_request(rid)
     engine.cache.check_invariants()
@@ -93,7 +97,7 @@ def check_against_plain(engine, model_dir: str, dtype: str, rid, tokens: Sequenc
     got, picks = run_cut(engine, rid, tokens, sizes, with_routes=True)
     routes = dict(zip(moe_layers_of(model_dir), picks))
     ref, regret = plain_logits_routed(model_dir, tokens, routes)
-    assert regret <= ROUTE_REGRET, f"{what}: the engine picked an expert {regret:.3f} (relative) below the best"
+    assert_route_regret(regret, what)
     assert_close_bf16(got, ref, what)
     return got
 
@@ -231,7 +235,7 @@ def replay(engine, steps: List[dict], with_routes: bool = False):
                 logits.setdefault(e["id"], []).append(lg[row:row + n])
                 row += n
             if with_routes:
-                picks.setdefault(e["id"], []).append([ids[tok:tok + len(e["tokens"])].cpu() for ids, _ in trace])
+                picks.setdefault(e["id"], []).append([ids[tok:tok + len(e["tokens"])].cpu() for ids, _, _ in trace])
             tok += len(e["tokens"])
         for rid in st["end"]:
             engine.free_request(rid)
@@ -258,5 +262,5 @@ def check_trace_against_plain(engine, model_dir: str, dtype: str, requests: Dict
     layers = moe_layers_of(model_dir)
     for rid, toks in requests.items():
         ref, regret = plain_logits_routed(model_dir, toks, dict(zip(layers, picks[rid])))
-        assert regret <= ROUTE_REGRET, f"{what} request {rid}: expert pick {regret:.3f} (relative) below the best"
+        assert_route_regret(regret, f"{what} request {rid}")
         assert_close_bf16(got[rid], ref, f"{what} request {rid}")

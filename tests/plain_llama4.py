@@ -3,8 +3,8 @@
 This file is the yardstick of the tests.  It shares no code with the package: it
 reads ``config.json`` as a raw dict, takes weights as a ``{name: tensor}`` dict and
 computes everything with ordinary dense tensor arithmetic on the CPU.  Each function
-cites the place in the reference (paths under /root/reference) whose formula it
-follows; where the reference has no such code the formula is stated in full.
+cites the place in the reference (paths from the root of pekkah/SharpInference) whose
+formula it follows; where the reference has no such code the formula is stated in full.
 """
 from __future__ import annotations
 
@@ -26,6 +26,15 @@ def read_config(model_dir: str) -> dict:
     for k, v in d.items():
         if k != "text_config":
             c.setdefault(k, v)
+    # the rotary base and its scaling may come in one object instead of two keys
+    rp = c.get("rope_parameters")
+    if rp:
+        c["rope_theta"] = rp["rope_theta"]
+        rest = {k: v for k, v in rp.items() if k != "rope_theta"}
+        c["rope_scaling"] = rest if rest.get("rope_type", "default") != "default" else None
+    if not c.get("no_rope_layers") and c.get("no_rope_layer_interval"):
+        step = int(c["no_rope_layer_interval"])
+        c["no_rope_layers"] = [int((l + 1) % step != 0) for l in range(int(c["num_hidden_layers"]))]
     return c
 
 

@@ -10,7 +10,7 @@ from sharpinference_amd.config.llama4 import Llama4TextConfig
 from sharpinference_amd.weights import safetensors_io as st
 from sharpinference_amd.weights.loader import (RandomSource, SafetensorsSource, WeightError, check_specs,
                                                load_model_weights, storage_dtype, write_random_model)
-from tiny_configs import CONFIGS, TINY_A, TINY_B, make_model_dir, write_other_layout
+from tiny_configs import CONFIGS, TINY_A, TINY_B, as_other_tools_write_it, make_model_dir, write_other_layout
 
 
 def test_every_key_is_read_and_round_trips():
@@ -48,6 +48,58 @@ def test_nested_text_config():
 def test_contradictions_are_refused(change, word):
     with pytest.raises(ConfigError, match=word):
         load_config({**TINY_A, **change})
+
+
+def test_the_other_form_of_the_same_config_reads_the_same():
+    """rope_parameters instead of rope_theta + rope_scaling: the base and the llama3 fields must
+    arrive (a reader that only knows the old names would fall back to 500000 and no scaling)."""
+    for d in CONFIGS.values():
+        a, b = load_config(d), load_config(as_other_tools_write_it(d))
+        assert (a.rope_theta, a.rope_scaling) == (b.rope_theta, b.rope_scaling)
+        for f in ("hidden_size", "no_rope_layers", "attention_chunk_size", "floor_scale", "attn_scale", "rms_norm_eps",
+                  "intermediate_size_mlp", "num_experts_per_tok", "tie_word_embeddings", "use_qk_norm"):
+            assert getattr(a, f) == getattr(b, f), f
+        assert [a.is_moe_layer(l) for l in range(a.num_hidden_layers)] == [b.is_moe_layer(l) for l in range(b.num_hidden_layers)]
+        assert b.unread_keys == ()
+    a = load_config(TINY_A)
+    assert a.rope_theta == 10000.0 and a.rope_scaling is None
+    b = load_config(as_other_tools_write_it(TINY_B))
+    assert b.rope_theta == 500000.0 and b.rope_scaling.factor == 8.0 and b.rope_scaling.original_max_position_embeddings == 32
+    assert build_model(b).blocks[0].mixer.rotary.scaling == b.rope_scaling
+
+
+def test_no_rope_layer_interval_fills_the_list():
+    d = {k: v for k, v in TINY_A.items() if k != "no_rope_layers"}
+    d.update(num_hidden_layers=6, no_rope_layer_interval=3)
+    assert load_config(d).no_rope_layers == [1, 1, 0, 1, 1, 0]
+    d["no_rope_layers"] = []                 # an empty list is "not given"
+    assert load_config(d).no_rope_layers == [1, 1, 0, 1, 1, 0]
+
+
+@pytest.mark.parametrize("change,word", [
+    ({"hidden_act": "gelu"}, "hidden_act"), ({"attention_bias": True}, "attention_bias"),
+    ({"layer_types": ["full_attention", "full_attention"]}, "layer_types"),
+    ({"attention_chunk_size": None}, "attention_chunk_size"), ({"attention_chunk_size": "8192"}, "attention_chunk_size"),
+    ({"rope_parameters": {"rope_theta": 5.0}}, "contradicts"),
+    ({"rope_parameters": {"rope_theta": 10000.0, "rope_type": "llama3", "factor": 2.0,
+                          "original_max_position_embeddings": 8}, "rope_scaling": {"rope_type": "llama3", "factor": 4.0,
+                                                                                   "original_max_position_embeddings": 8}}, "contradicts"),
+    ({"rope_parameters": {"rope_theta": 10000.0, "rope_type": "yarn", "factor": 2.0}}, "rope_type"),
+    ({"rope_parameters": {"rope_theta": 10000.0, "beta_fast": 32}}, "beta_fast"),
+    ({"rope_parameters": {"rope_theta": 10000.0, "rope_type": "default", "factor": 2.0}}, "factor"),
+    ({"sliding_window": 128}, "sliding_window"), ({"partial_rotary_factor": 0.5, "logit_cap": 30.0}, "logit_cap.*partial_rotary_factor"),
+    ({"rms_norm_eps": None}, "rms_norm_eps"), ({"num_hidden_layers": "3"}, "num_hidden_layers"),
+    ({"text_config": 3}, "text_config"),
+])
+def test_keys_that_would_change_the_computation_are_not_passed_over(change, word):
+    with pytest.raises(ConfigError, match=word):
+        load_config({**TINY_A, **change})
+
+
+def test_unknown_text_keys_are_listed_not_refused():
+    cfg = load_config({**TINY_A, "some_note": "hello", "another": None})
+    assert cfg.unread_keys == ("another", "some_note")
+    assert load_config({**TINY_A, "rope_scaling": {"rope_type": "default"}}).rope_scaling is None
 
 
 def test_missing_keys_and_unknown_architecture():
@@ -308,3 +360,27 @@ def test_other_layouts_of_the_same_tensors_are_read(tmp_path):
     with pytest.raises(WeightError) as e:
         check_specs(specs, LayoutAdapter(SafetensorsSource(broken, torch.bfloat16, "cpu"), specs).available(), broken)
     assert "model.layers.9.extra.weight" in str(e.value)
+
+
+@pytest.mark.parametrize("hidden,inter", [(64, 64), (64, 32), (64, 128)])
+def test_axis_order_is_decided_by_name_where_the_shape_cannot_tell(tmp_path, hidden, inter):
+    """A stacked expert tensor whose two sizes are equal (down: hidden == width; fused gate|up:
+    hidden == 2 * width) reads the same transposed or not; the name decides: without a
+    ``.weight`` suffix a fused tensor is [E, in, 2 * out] and the down beside it [E, in, out].
+    The tensors are made unsymmetric so that a wrong reading cannot equal the right one."""
+    from sharpinference_amd.weights.loader import LayoutAdapter
+
+    d = make_model_dir(tmp_path, "A", hidden_size=hidden, intermediate_size=inter, head_dim=16)
+    specs = build_model(load_config(d)).param_specs()
+    other = write_other_layout(d, str(tmp_path / "other"), "")
+    plain = SafetensorsSource(d, torch.bfloat16, "cpu")
+    adapted = LayoutAdapter(SafetensorsSource(other, torch.bfloat16, "cpu"), specs)
+    check_specs(specs, adapted.available(), other)
+    for n in specs:
+        got, want = adapted.get(n), plain.get(n)
+        assert torch.equal(got, want), n
+        if want.dim() == 3 and want.shape[1] == want.shape[2]:
+            assert not torch.equal(want, want.transpose(1, 2)), "the test's tensor must tell the two readings apart"
+    # the canonical folder (separate gate and up, down [E, out, in]) with the same sizes is left as it is
+    same = LayoutAdapter(SafetensorsSource(d, torch.bfloat16, "cpu"), specs)
+    assert all(torch.equal(same.get(n), plain.get(n)) for n in specs)

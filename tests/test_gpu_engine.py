@@ -3,7 +3,7 @@ import pytest
 import torch
 
 import helpers as H
-from tiny_configs import CONFIGS, make_model_dir, write_other_layout
+from tiny_configs import CONFIGS, as_other_tools_write_it, make_model_dir, write_other_layout
 
 pytestmark = pytest.mark.gpu
 
@@ -176,11 +176,29 @@ def test_decode_graphs_follow_the_context(tmp_path):
 
 
 
-def test_a_checkpoint_in_another_layout_gives_the_same_logits(tmp_path):
-    """A container prefix, fused gate|up and [E, in, out] experts: the engine reads the same model."""
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("prefix", ["", "language_model."])
+def test_a_folder_in_the_other_form_against_plain(tmp_path, dtype, prefix):
+    """The same model as another tool writes it: text keys nested, rotary base and llama3 scaling
+    in ``rope_parameters``, ``layer_types``, a container prefix, experts fused as [E, in, 2 * out]
+    and stored [E, in, out].  The engine reads that folder; the plain implementation reads the
+    canonical one.  (A reader that dropped ``rope_parameters`` would rotate with another base
+    and no scaling: every rotary layer's logits would differ.)"""
+    import json
+    import os
+
     d = make_model_dir(tmp_path, "B", std=0.1)
-    other = write_other_layout(d, str(tmp_path / "other"), "language_model.")
-    toks = H.random_tokens(40, 384, 3)
-    a = H.run_cut(H.make_engine(d, "float32"), "a", toks, H.whole(len(toks)))
-    b = H.run_cut(H.make_engine(other, "float32"), "b", toks, H.whole(len(toks)))
-    assert torch.equal(a, b)
+    other = write_other_layout(d, str(tmp_path / "other"), prefix,
+                               extra={"vision_model.patch.weight": torch.zeros(3, 5, dtype=torch.bfloat16)} if prefix else ())
+    with open(os.path.join(other, "config.json"), "w") as f:
+        json.dump(as_other_tools_write_it(CONFIGS["B"]), f)
+    toks = H.random_tokens(90, 384, 3)           # crosses three chunk edges of 24
+    eng = H.make_engine(other, dtype)
+    assert eng.config.rope_scaling is not None and eng.config.rope_scaling.factor == 8.0
+    if dtype == "float32":
+        H.assert_close_fp32(H.run_cut(eng, "a", toks, H.changing_portions(len(toks), 1)), H.plain_logits(d, toks), "other form")
+    else:
+        got, picks = H.run_cut(eng, "a", toks, H.last_decoded(len(toks)), with_routes=True)
+        ref, regret = H.plain_logits_routed(d, toks, dict(zip(H.moe_layers_of(d), picks)))
+        H.assert_route_regret(regret, "other form")
+        H.assert_close_bf16(got, ref, "other form")

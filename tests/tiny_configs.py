@@ -61,6 +61,26 @@ CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
 FLOAT32_NAMES = {"A": (), "B": ("layernorm.weight", "model.norm.weight", "router.weight"), "C": (), "D": ()}
 
 
+def as_other_tools_write_it(d):
+    """The same model in the other form a Llama 4 config.json is found in: the text keys nested,
+    the rotary base and scaling in one ``rope_parameters`` object, the window of every layer
+    named in ``layer_types``, and the training / bookkeeping keys such files carry."""
+    text = {k: v for k, v in d.items() if k not in ("architectures", "rope_theta", "rope_scaling", "tie_word_embeddings")}
+    rp = {"rope_theta": d["rope_theta"], "rope_type": "default"}
+    if d.get("rope_scaling"):
+        rp = {"rope_theta": d["rope_theta"], **d["rope_scaling"]}
+    text.update({
+        "rope_parameters": rp, "model_type": "llama4_text", "hidden_act": "silu", "attention_bias": False,
+        "attention_dropout": 0.0, "initializer_range": 0.02, "output_router_logits": False,
+        "router_aux_loss_coef": 0.001, "router_jitter_noise": 0.0, "use_cache": True, "pad_token_id": 0,
+        "layer_types": ["chunked_attention" if r else "full_attention" for r in d["no_rope_layers"]],
+        "no_rope_layer_interval": 4, "for_llm_compressor": False, "cache_implementation": "hybrid",
+    })
+    return {"architectures": ["Llama4ForConditionalGeneration"], "model_type": "llama4", "text_config": text,
+            "tie_word_embeddings": d["tie_word_embeddings"], "transformers_version": "5.0.0",
+            "vision_config": {"hidden_size": 32}, "image_token_index": 7, "boi_token_index": 8, "eoi_token_index": 9}
+
+
 def make_model_dir(tmp_path, which: str, std: float = 0.02, **overrides) -> str:
     from sharpinference_amd.config.base import load_config
     from sharpinference_amd.weights.loader import write_random_model
