@@ -10,6 +10,7 @@ in the same way, src/SharpInference.Engine/CudaForwardPass.cs:4894, 4985-4986).
 """
 from __future__ import annotations
 
+import gc
 import sys
 from dataclasses import dataclass, field
 from typing import Hashable, List, Optional, Sequence
@@ -246,7 +247,6 @@ class _DecodeGraph:
     The logits tensor belongs to the graph: the caller gets a copy."""
 
     def __init__(self, runner: ModelRunner, pieces, info: dict, max_context: int):
-        self.runner = runner
         self.sizes = [p.size for p in pieces]
         total = sum(self.sizes)
         self.host = torch.empty(total, dtype=torch.int32).pin_memory()
@@ -279,8 +279,18 @@ class _DecodeGraph:
         self.trace: list = []
         ctx.extras["router_trace"] = self.trace
         self.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(self.graph):
-            self.logits = runner.model.forward(ctx, caches, rows)
+        # No garbage collection while the stream is capturing: a collector run that frees another
+        # engine's graph (or anything else that calls into the runtime) in the middle of a capture
+        # aborts the process.  (This object holds no reference to the runner, so that an engine
+        # that is dropped frees its graphs at once, by reference count, not in some later collection.)
+        collecting = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.graph(self.graph):
+                self.logits = runner.model.forward(ctx, caches, rows)
+        finally:
+            if collecting:
+                gc.enable()
 
     def _upload(self, pieces) -> None:
         self.copied.synchronize()                         # the previous copy has left the pinned buffer
