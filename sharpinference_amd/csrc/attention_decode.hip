@@ -14,6 +14,8 @@
 // head, and a second kernel merges the runs of a token.  The run length is fixed, so the sums
 // of a query depend on (start, position) only, not on the batch.
 #include "common.h"
+#include "sharpi_noalloc.h"
+#include <mutex>
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
@@ -217,7 +219,8 @@ __global__ __launch_bounds__(kMergeThreads) void attn_decode_merge_kernel(
   int start = 0;
   if (window_kind == 1) start = (p / window) * window;
   else if (window_kind == 2) start = p - window + 1 > 0 ? p - window + 1 : 0;
-  const int n_runs = ((p >> 4) - (start >> 4)) / kSplitBlocks + 1;
+  // (never beyond the runs the workspace holds, whatever the caller's bound was)
+  const int n_runs = min(((p >> 4) - (start >> 4)) / kSplitBlocks + 1, max_splits);
   const size_t base = ((size_t)li * nh + h) * max_splits;
 
   float M = -INFINITY;
@@ -315,3 +318,50 @@ SHARPI_EXPORT int sharpi_attention_decode_takes(int hd) {
 }
 
 SHARPI_EXPORT int sharpi_attention_decode_split_keys() { return kSplitBlocks * 16; }
+
+// ---------------------------------------------------------------------------------------------
+// The same without workspace arguments, for callers that cannot allocate: the partial results go
+// to a file-scope device array.  In host code the array's name is only a stand-in for the symbol,
+// not a device address; each device's address is looked up once, with that device current, and
+// that pointer is what the kernels get.
+static __device__ __align__(256) float scratch[SHARPI_NOALLOC_SCRATCH_FLOATS];
+
+constexpr int kMaxDevices = 64;
+static float* scratch_of_device[kMaxDevices];   // per device: where its copy of `scratch` lies
+static std::mutex scratch_lock;
+
+static int scratch_here(float** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= kMaxDevices) return SHARPI_ERR_ARG;
+  std::lock_guard<std::mutex> guard(scratch_lock);
+  if (!scratch_of_device[dev]) {
+    float* p = nullptr;
+    e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (!p) return SHARPI_ERR_LAUNCH;
+    scratch_of_device[dev] = p;
+  }
+  *out = scratch_of_device[dev];
+  return SHARPI_OK;
+}
+
+int sharpi_attention_decode_noalloc(const void* q, const void* k_cache, const void* v_cache, const int* block_table,
+                                    const int* entry_of_token, const int* positions, const int* token_list, void* out,
+                                    int window_kind, int window, float scale, int n_list, int nh, int nkv, int hd,
+                                    int page_size, int max_blocks, int num_pages, int max_splits, hipStream_t stream) {
+  if (n_list <= 0) return SHARPI_OK;
+  if (nh <= 0 || hd <= 0 || max_splits <= 0) return SHARPI_ERR_ARG;
+  // part_o [n_list, nh, max_splits, hd] then part_ml [n_list, nh, max_splits, 2]
+  const unsigned long long runs = (unsigned long long)n_list * (unsigned long long)nh * (unsigned long long)max_splits;
+  if (runs * (unsigned long long)(hd + 2) > (unsigned long long)SHARPI_NOALLOC_SCRATCH_FLOATS) return SHARPI_ERR_ARG;
+  float* ws = nullptr;
+  const int rc = scratch_here(&ws);
+  if (rc != SHARPI_OK) return rc;
+  float* part_o = ws;
+  float* part_ml = ws + runs * (unsigned long long)hd;   // hd is a multiple of 32: stays 16-byte aligned
+  return sharpi_attention_decode(q, k_cache, v_cache, block_table, entry_of_token, positions, token_list, part_o,
+                                 part_ml, out, window_kind, window, scale, n_list, nh, nkv, hd, page_size, max_blocks,
+                                 num_pages, max_splits, stream);
+}
