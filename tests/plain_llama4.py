@@ -288,19 +288,21 @@ def moe_layer(c: dict, W: Dict[str, torch.Tensor], layer: int, n: torch.Tensor, 
         ids = forced
         wts = torch.gather(router_gates(n, W[p + "router.weight"]), 1, forced)
     if trace is not None:
+        trace.setdefault("picks", {})[layer] = ids      # the picks this run made (or was given), layer by layer
         m = router_margin(n, W[p + "router.weight"], k)
         trace["router_margin"] = torch.minimum(trace["router_margin"], m) if "router_margin" in trace else m
     out = swiglu(n, W[p + "shared_expert.gate_proj.weight"], W[p + "shared_expert.up_proj.weight"],
                  W[p + "shared_expert.down_proj.weight"], store)
     Wg, Wu, Wd = W[p + "experts.gate_proj"], W[p + "experts.up_proj"], W[p + "experts.down_proj"]
     routed = torch.zeros_like(out)
-    for t in range(n.shape[0]):
-        for j in range(k):
-            e = int(ids[t, j])
-            w = wts[t, j]
-            g = store(Wg[e] @ n[t]) * w
-            u = store(Wu[e] @ n[t]) * w
-            routed[t] += store(Wd[e] @ store(silu(g) * u))
+    for e in range(Wg.shape[0]):                 # expert by expert, over the (token, pick) pairs that chose it
+        t_idx, j_idx = (ids == e).nonzero(as_tuple=True)
+        if t_idx.numel() == 0:
+            continue
+        w = wts[t_idx, j_idx][:, None]
+        g = store(n[t_idx] @ Wg[e].T) * w
+        u = store(n[t_idx] @ Wu[e].T) * w
+        routed.index_add_(0, t_idx, store(store(silu(g) * u) @ Wd[e].T))
     return store(routed + out)
 
 

@@ -35,6 +35,37 @@ def test_greedy_generation_matches_plain(tmp_path):
     assert [solo.generate([p], max_new_tokens=16)[0].token_ids for p in prompts] == want
 
 
+@pytest.mark.parametrize("which,std", [("B", 0.1), ("D", 0.06)])
+def test_greedy_generation_in_bfloat16_token_for_token(tmp_path, which, std):
+    """Greedy generation in bfloat16 through the entry point, then every generated token against
+    the plain implementation with bfloat16 storage and the engine's own routes: the token must be
+    the plain implementation's best, or lie below its best by no more than the bound on a
+    bfloat16 logit (two logits, each off by at most the bound).  The generation's steps (prompt
+    whole, then one token a step) are replayed through the step function for the routes, and the
+    replay must give the generated tokens exactly."""
+    d = make_model_dir(tmp_path, which, std=std)
+    vocab = CONFIGS[which]["vocab_size"]
+    tol_max, _ = H.bounds_of(d)
+    n_new = 24
+    strict = 0
+    for i, n in enumerate((6, 30, 50)):
+        prompt = H.random_tokens(n, vocab, 60 + i)
+        eng = H.make_engine(d, "bfloat16", kv_tokens=256, max_num_seqs=2, max_tokens_per_step=64)
+        out = eng.generate([prompt], max_new_tokens=n_new, temperature=0.0)[0].token_ids
+        assert len(out) == n_new
+        toks = prompt + out[:-1]
+        got, picks, seen = H.run_cut(eng, "g", toks, [n] + [1] * (n_new - 1), with_routes=True)
+        assert got[n - 1:].argmax(dim=-1).tolist() == out, "the replayed steps choose other tokens than the generation did"
+        H.assert_routes_are_the_best(d, picks, seen, f"{which} generation {i}")
+        ref = H.plain_logits_routed(d, toks, dict(zip(H.moe_layers_of(d), picks)))[n - 1:]
+        rms = ref.double().pow(2).mean(dim=-1).sqrt()
+        chosen = ref.gather(1, torch.tensor(out)[:, None])[:, 0]
+        below = (ref.max(dim=-1).values - chosen).double() / rms
+        assert float(below.max()) <= 2 * tol_max, f"{which} prompt {i}: a generated token lies {float(below.max()):.3f} row rms below the plain best"
+        strict += int((ref.argmax(dim=-1) == torch.tensor(out)).sum())
+    assert strict >= 3 * n_new - 3, f"only {strict} of {3 * n_new} tokens are the plain implementation's own choice"
+
+
 def test_temperature_generation_matches_plain(tmp_path):
     """Tiny B, 32-bit: prompts of 1 / 17 / 50 / 77 tokens, 24 steps at temperature 0.8 with
     fixed seeds: the same uniforms give the same tokens."""

@@ -42,6 +42,28 @@ def test_gemm_skinny(M, N, K, out_dtype):
                 assert float((got - ref).abs().max()) <= tol * float(ref.abs().max()), (M, N, K, R, NW, form is w)
 
 
+@pytest.mark.parametrize("M", [16, 17, 24, 32, 33])
+def test_linear_against_a_very_tall_matrix(M):
+    """The head's shape class (more than 65,536 rows): the few-rows kernel up to 32 rows, the
+    library beyond; both sides of 16/17 and 32/33 through the dispatcher the model calls, over the
+    packed form and the row form, into float32 (logits) and bfloat16."""
+    ops = _ops()
+    N, K = 65536 + 1024, 256
+    x = _rand(M, K, dtype=torch.bfloat16, seed=M)
+    w = _rand(N, K, dtype=torch.bfloat16, scale=0.1, seed=7)
+    ref = x.float() @ w.float().T
+    assert ops.skinny_ok(M, N, K) == (M <= 32) and ops.skinny_ok(M, 4096, K) == (M <= 16)
+    for form in (w, ops.pack_weight(w)):
+        for out_dtype, tol in ((torch.float32, 1e-3), (torch.bfloat16, 2e-2)):
+            got = ops.linear(x, form, out_dtype)
+            assert got.dtype == out_dtype and got.shape == (M, N)
+            assert float((got.float() - ref).abs().max()) <= tol * float(ref.abs().max()), (M, form is w, out_dtype)
+    # a row's result does not depend on how many rows ride along (within the kernel's reach)
+    if M <= 32:
+        one = ops.linear(x[:1].contiguous(), w, torch.float32)
+        assert torch.equal(one[0], ops.linear(x, w, torch.float32)[0])
+
+
 def test_gemm_skinny_rows_do_not_depend_on_the_batch():
     ops = _ops()
     x = _rand(64, 512, dtype=torch.bfloat16, seed=3)

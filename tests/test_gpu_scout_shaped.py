@@ -62,3 +62,18 @@ def test_scout_shaped_mixed_batches(scout_dir, dtype):
     H.check_trace_against_plain(eng, scout_dir, dtype, reqs, steps, f"scout-shaped {dtype} mixed")
     for g in eng.cache.groups:
         assert g.pool.num_free == g.pool.num_pages
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("width", [8, 17, 33, 65])
+def test_scout_shaped_wide_decode_batches(scout_dir, width, dtype):
+    """The served model's layer sizes with as many live requests as a serving step has, on both
+    sides of the batch sizes at which a step changes kernels."""
+    import random
+
+    rng = random.Random(width)
+    reqs = {f"w{i}": H.random_tokens(rng.randint(4, 12), SCOUT_SHAPED["vocab_size"], 8000 + 100 * width + i)
+            for i in range(width)}
+    steps = H.wide_trace(reqs, tail=2, per_prefill_step=16)
+    eng = H.make_engine(scout_dir, dtype, kv_tokens=H.tokens_held(steps), max_num_seqs=width)
+    H.check_trace_against_plain(eng, scout_dir, dtype, reqs, steps, f"scout-shaped {dtype} {width} live requests")

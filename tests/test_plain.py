@@ -226,3 +226,55 @@ def test_sampling_vectors():
         counts[P.sample(torch.zeros(4), u, 100.0)] += 1
     assert all(850 <= n <= 1150 for n in counts)                       # hot temperature: near uniform
     assert P.uniform_stream(5, 3) == P.uniform_stream(5, 3) and P.uniform_stream(5, 3) != P.uniform_stream(6, 3)
+
+
+@pytest.mark.parametrize("which,std", [("A", 0.1), ("B", 0.08), ("D", 0.06)])
+def test_the_bfloat16_bound_is_what_two_orders_of_summation_differ_by(tmp_path, which, std):
+    """The bound that bfloat16 engine runs are held to (helpers.bf16_bounds) against what it is
+    derived for: two runs of the plain implementation with the same stores and the same routes,
+    one summing in float and one in double.  They must lie within the bound, and not more than
+    twenty times below it (else the bound would be loose enough to hide a fault of the size of a
+    rounding)."""
+    import helpers as H
+
+    d = make_model_dir(tmp_path, which, std=std)
+    c, W = P.read_config(d), P.load_weights(d)
+    tol_max, tol_rms = H.bounds_of(d)
+    worst_rms = worst_max = 0.0
+    for seed in range(2):
+        toks = H.random_tokens(100, c["vocab_size"], 70 + seed)
+        made: dict = {}
+        a = P.forward(c, W, toks, store=P.store_bf16, trace=made)
+        picks = made["picks"]                 # the float run's own picks, given to the other run
+        b = P.forward(c, W, toks, dtype=torch.float64, store=P.store_bf16, routes=picks)
+        err = a.double() - b.double()
+        rms = b.double().pow(2).mean(dim=-1).sqrt()
+        worst_rms = max(worst_rms, float((err.pow(2).mean(dim=-1).sqrt() / rms).max()))
+        worst_max = max(worst_max, float((err.abs().max(dim=-1).values / rms).max()))
+    assert tol_rms / 20 <= worst_rms <= tol_rms, (worst_rms, tol_rms)
+    assert tol_max / 20 <= worst_max <= tol_max, (worst_max, tol_max)
+
+
+def test_the_router_check_tells_a_worse_pick_from_a_rounding():
+    import helpers as H
+
+    torch.manual_seed(0)
+    x = torch.randn(6, 64).to(torch.bfloat16).float()
+    w = torch.randn(8, 64)
+    r = x.double() @ w.double().T
+    best = r.topk(2, dim=1).indices.to(torch.int32)
+    H.assert_picks_are_the_best(x, w, best, "best")
+    H.assert_picks_are_the_best(x, w, best.flip(1), "order does not matter")
+    third = r.topk(3, dim=1).indices[:, [0, 2]].to(torch.int32)
+    with pytest.raises(AssertionError, match="below the best"):
+        H.assert_picks_are_the_best(x, w, third, "third instead of second")
+    twice = best.clone()
+    twice[:, 1] = twice[:, 0]
+    with pytest.raises(AssertionError, match="twice"):
+        H.assert_picks_are_the_best(x, w, twice, "twice")
+    # two experts with the same weights: either is right
+    w[5] = w[2]
+    r = x.double() @ w.double().T
+    top = r.topk(1, dim=1).indices.to(torch.int32)
+    swapped = torch.where(top == 2, torch.full_like(top, 5), top)
+    H.assert_picks_are_the_best(x, w, swapped, "a tie")
