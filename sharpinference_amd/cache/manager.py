@@ -28,6 +28,34 @@ class CacheError(RuntimeError):
     pass
 
 
+def pages_to_hold(spec: KVSpec, page_size: int, total_tokens: int, max_step_tokens: int) -> int:
+    """Upper bound of the pages a request of `total_tokens` holds at once under `spec` when no step
+    brings more than `max_step_tokens` of it: all of them without a window; with one, the window,
+    the step that is being appended before the pages behind the window are given back, and one
+    page for the edges."""
+    full = (total_tokens + page_size - 1) // page_size
+    if spec.window_kind == 0:
+        return full
+    span = spec.window + max(1, max_step_tokens)
+    return min(full, (span + page_size - 1) // page_size + 1)
+
+
+def pool_sizes(slot_specs, page_size: int, max_requests: int, total_tokens: int, max_step_tokens: int,
+               budget_pages: Optional[int] = None) -> Dict[tuple, int]:
+    """Pages per group for `max_requests` requests of up to `total_tokens` each: a group without
+    a window gets them all (or `budget_pages`, if that is less), a windowed group what its window
+    can ever hold, which is what makes its memory bounded however long the requests grow."""
+    out: Dict[tuple, int] = {}
+    for spec in slot_specs:
+        if not isinstance(spec, KVSpec) or spec.group_key() in out:
+            continue
+        n = max_requests * pages_to_hold(spec, page_size, total_tokens, max_step_tokens)
+        if budget_pages is not None:
+            n = min(n, budget_pages)
+        out[spec.group_key()] = max(1, n)
+    return out
+
+
 class PagePool:
     """Free list of page ids 0..n-1; LIFO, so a page just released is the next handed out."""
 
@@ -108,6 +136,9 @@ class CacheManager:
             else:
                 self.group_of_slot.append(-1)
         self._free_state_slots = list(range(max_requests - 1, -1, -1))
+        # one more slot than requests: a slot that belongs to no request, for runs whose effects on
+        # state must not count (the trial run of a graph capture)
+        self.scratch_state_slot = max_requests
         self.requests: Dict[Hashable, RequestCache] = {}
         self._reserved_total = [0] * len(self.groups)
         # device tensors
@@ -125,7 +156,7 @@ class CacheManager:
                     self.v[i] = torch.zeros((n, spec.num_kv_heads, spec.head_dim, page_size), dtype=dtype,
                                             device=self.device)
                 elif isinstance(spec, StateSpec):
-                    self.state[i] = torch.zeros((max_requests, *spec.shape), dtype=spec.dtype, device=self.device)
+                    self.state[i] = torch.zeros((max_requests + 1, *spec.shape), dtype=spec.dtype, device=self.device)
 
     # ------------------------------------------------------------------ sizes
     def bytes_per_page(self) -> List[int]:
@@ -146,12 +177,7 @@ class CacheManager:
     def pages_to_hold(self, group: int, total_tokens: int, max_step_tokens: int) -> int:
         """Upper bound of the pages a request of `total_tokens` holds at once in a group when no
         step brings more than `max_step_tokens` of it."""
-        spec = self.groups[group].spec
-        full = self.blocks_for(total_tokens)
-        if spec.window_kind == 0:
-            return full
-        span = spec.window + max(1, max_step_tokens)
-        return min(full, self.blocks_for(span) + 1)
+        return pages_to_hold(self.groups[group].spec, self.page_size, total_tokens, max_step_tokens)
 
     # ------------------------------------------------------------------ requests
     def has_request(self, req_id) -> bool:

@@ -72,13 +72,14 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__
 constexpr int kNormKeep = 2;
 
 // delta of row r, columns c .. c + 7, as floats.  Plain: delta[r].  As an expert sum (sum_pos
-// given): the rows sum_pos[r*k .. r*k + k) of delta plus sum_shared[r], added in that order in
-// float and rounded to the storage type, which is what the separate combine kernel would have
-// stored for the norm to read.
+// given): the rows sum_pos[r*k .. r*k + k) of delta (each times its weight sum_w[r*k + q], if
+// weights are given: scores applied to the experts' outputs) plus sum_shared[r], added in that
+// order in float and rounded to the storage type, which is what the separate combine kernel
+// would have stored for the norm to read.
 template <typename TD>
 __device__ __forceinline__ void load_delta8(const TD* __restrict__ delta, const int* __restrict__ sum_pos,
-                                            const TD* __restrict__ sum_shared, int sum_k, int r, int hidden,
-                                            int c, float* d) {
+                                            const TD* __restrict__ sum_shared, const float* __restrict__ sum_w,
+                                            int sum_k, int r, int hidden, int c, float* d) {
   if (!sum_pos) {
     load8(delta + (size_t)r * hidden + c, d);
     return;
@@ -88,8 +89,9 @@ __device__ __forceinline__ void load_delta8(const TD* __restrict__ delta, const 
   for (int q = 0; q < sum_k; ++q) {
     float v[8];
     load8(delta + (size_t)sum_pos[r * sum_k + q] * hidden + c, v);
+    const float wq = sum_w ? sum_w[r * sum_k + q] : 1.0f;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) d[j] += v[j];
+    for (int j = 0; j < 8; ++j) d[j] += sum_w ? wq * v[j] : v[j];
   }
   if (sum_shared) {
     float v[8];
@@ -106,7 +108,8 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_vec_kernel(float* __restrict
                                                                const TW* __restrict__ w, TO* __restrict__ out,
                                                                const int* __restrict__ rows, int hidden, float eps,
                                                                int write_back, const int* __restrict__ sum_pos,
-                                                               const TD* __restrict__ sum_shared, int sum_k) {
+                                                               const TD* __restrict__ sum_shared,
+                                                               const float* __restrict__ sum_w, int sum_k) {
   __shared__ float red[16];
   const int i = blockIdx.x;
   const int r = rows ? rows[i] : i;
@@ -132,7 +135,7 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_vec_kernel(float* __restrict
     if (c < hidden) {
       if (dr) {
         float d[8];
-        load_delta8<TD>(delta, sum_pos, sum_shared, sum_k, r, hidden, c, d);
+        load_delta8<TD>(delta, sum_pos, sum_shared, sum_w, sum_k, r, hidden, c, d);
 #pragma unroll
         for (int j = 0; j < 8; ++j) keep[n][j] += d[j];
         if (write_back) store8(hr + c, keep[n]);
@@ -147,7 +150,7 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_vec_kernel(float* __restrict
     load8(hr + c, x);
     if (dr) {
       float d[8];
-      load_delta8<TD>(delta, sum_pos, sum_shared, sum_k, r, hidden, c, d);
+      load_delta8<TD>(delta, sum_pos, sum_shared, sum_w, sum_k, r, hidden, c, d);
 #pragma unroll
       for (int j = 0; j < 8; ++j) x[j] += d[j];
       if (write_back) store8(hr + c, x);
@@ -173,7 +176,7 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_vec_kernel(float* __restrict
     load8(hr + c, x);
     if (dr && !write_back) {
       float d[8];
-      load_delta8<TD>(delta, sum_pos, sum_shared, sum_k, r, hidden, c, d);
+      load_delta8<TD>(delta, sum_pos, sum_shared, sum_w, sum_k, r, hidden, c, d);
 #pragma unroll
       for (int j = 0; j < 8; ++j) x[j] += d[j];
     }
@@ -194,7 +197,7 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_vec_kernel(float* __restrict
 template <typename TD, typename TW>
 static int launch_add_rmsnorm_o(float* h, const void* delta, const void* w, void* out, int out_dtype,
                                 const int* rows, int n_out, int hidden, float eps, int write_back,
-                                const int* sum_pos, const void* sum_shared, int sum_k, hipStream_t stream) {
+                                const int* sum_pos, const void* sum_shared, const float* sum_w, int sum_k, hipStream_t stream) {
   dim3 grid(n_out), block(hidden >= 2048 ? 512 : 256);
   if (out_dtype != DT_F32 && out_dtype != DT_BF16) return SHARPI_ERR_ARG;
   if ((hidden & 7) == 0) {
@@ -204,11 +207,11 @@ static int launch_add_rmsnorm_o(float* h, const void* delta, const void* w, void
     if (out_dtype == DT_F32)
       add_rmsnorm_vec_kernel<TD, TW, float><<<grid, vblock, 0, stream>>>(h, (const TD*)delta, (const TW*)w,
                                                                         (float*)out, rows, hidden, eps, write_back,
-                                                                        sum_pos, (const TD*)sum_shared, sum_k);
+                                                                        sum_pos, (const TD*)sum_shared, sum_w, sum_k);
     else
       add_rmsnorm_vec_kernel<TD, TW, bf16_t><<<grid, vblock, 0, stream>>>(h, (const TD*)delta, (const TW*)w,
                                                                          (bf16_t*)out, rows, hidden, eps, write_back,
-                                                                         sum_pos, (const TD*)sum_shared, sum_k);
+                                                                         sum_pos, (const TD*)sum_shared, sum_w, sum_k);
   } else if (sum_pos)
     return SHARPI_ERR_ARG;   // an expert sum is folded in by the vector kernel only (width % 8 == 0)
   else if (out_dtype == DT_F32)
@@ -224,14 +227,14 @@ static int launch_add_rmsnorm_o(float* h, const void* delta, const void* w, void
 template <typename TD>
 static int launch_add_rmsnorm_w(float* h, const void* delta, const void* w, int w_dtype, void* out,
                                 int out_dtype, const int* rows, int n_out, int hidden, float eps,
-                                int write_back, const int* sum_pos, const void* sum_shared, int sum_k,
-                                hipStream_t stream) {
+                                int write_back, const int* sum_pos, const void* sum_shared, const float* sum_w,
+                                int sum_k, hipStream_t stream) {
   if (w_dtype == DT_F32 || w == nullptr)
     return launch_add_rmsnorm_o<TD, float>(h, delta, w, out, out_dtype, rows, n_out, hidden, eps, write_back,
-                                           sum_pos, sum_shared, sum_k, stream);
+                                           sum_pos, sum_shared, sum_w, sum_k, stream);
   if (w_dtype == DT_BF16)
     return launch_add_rmsnorm_o<TD, bf16_t>(h, delta, w, out, out_dtype, rows, n_out, hidden, eps, write_back,
-                                            sum_pos, sum_shared, sum_k, stream);
+                                            sum_pos, sum_shared, sum_w, sum_k, stream);
   return SHARPI_ERR_ARG;
 }
 
@@ -241,17 +244,17 @@ static int launch_add_rmsnorm_w(float* h, const void* delta, const void* w, int 
 SHARPI_EXPORT int sharpi_add_rmsnorm(float* h, const void* delta, int delta_dtype, const void* w, int w_dtype,
                                      void* out, int out_dtype, const int* rows, int n_out, int hidden,
                                      float eps, int write_back, const int* sum_pos, const void* sum_shared,
-                                     int sum_k, hipStream_t stream) {
+                                     const float* sum_w, int sum_k, hipStream_t stream) {
   if (n_out <= 0) return SHARPI_OK;
   if (hidden <= 0 || !(eps > 0.f)) return SHARPI_ERR_ARG;
   if (rows && write_back) return SHARPI_ERR_ARG;  // gathered rows never write the stream back
   if (sum_pos && (delta == nullptr || sum_k <= 0)) return SHARPI_ERR_ARG;
   if (delta == nullptr || delta_dtype == DT_F32)
     return launch_add_rmsnorm_w<float>(h, delta, w, w_dtype, out, out_dtype, rows, n_out, hidden, eps, write_back,
-                                       sum_pos, sum_shared, sum_k, stream);
+                                       sum_pos, sum_shared, sum_w, sum_k, stream);
   if (delta_dtype == DT_BF16)
     return launch_add_rmsnorm_w<bf16_t>(h, delta, w, w_dtype, out, out_dtype, rows, n_out, hidden, eps, write_back,
-                                        sum_pos, sum_shared, sum_k, stream);
+                                        sum_pos, sum_shared, sum_w, sum_k, stream);
   return SHARPI_ERR_ARG;
 }
 
@@ -308,23 +311,29 @@ SHARPI_EXPORT int sharpi_silu_mul(const void* gu, const float* scale, void* out,
 }
 
 // ---------------------------------------------------------------------------
-// MoE combine: out[t, :] = sum_j y[inv_pos[t*k + j], :] (+ shared[t, :]); float sums, j ascending.
+// MoE combine: out[t, :] = sum_j w[t*k + j] * y[inv_pos[t*k + j], :] (+ shared[t, :]); w null: ones;
+// float sums, j ascending.
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ void moe_combine_kernel(const T* __restrict__ y, const int* __restrict__ inv_pos,
-                                   const T* __restrict__ shared, T* __restrict__ out, int hidden, int k) {
+                                   const T* __restrict__ shared, const float* __restrict__ w,
+                                   T* __restrict__ out, int hidden, int k) {
   const int t = blockIdx.x;
   const int c = blockIdx.y * blockDim.x + threadIdx.x;
   if (c >= hidden) return;
   float acc = 0.f;
-  for (int j = 0; j < k; ++j) acc += to_f32<T>(y[(size_t)inv_pos[t * k + j] * hidden + c]);
+  for (int j = 0; j < k; ++j) {
+    const float v = to_f32<T>(y[(size_t)inv_pos[t * k + j] * hidden + c]);
+    acc += w ? w[t * k + j] * v : v;
+  }
   if (shared) acc += to_f32<T>(shared[(size_t)t * hidden + c]);
   out[(size_t)t * hidden + c] = from_f32<T>(acc);
 }
 
 template <typename T>
 __global__ void moe_combine_vec_kernel(const T* __restrict__ y, const int* __restrict__ inv_pos,
-                                       const T* __restrict__ shared, T* __restrict__ out, int hidden, int k) {
+                                       const T* __restrict__ shared, const float* __restrict__ w,
+                                       T* __restrict__ out, int hidden, int k) {
   const int t = blockIdx.x;
   const int c = (blockIdx.y * blockDim.x + threadIdx.x) * 8;
   if (c >= hidden) return;
@@ -332,8 +341,9 @@ __global__ void moe_combine_vec_kernel(const T* __restrict__ y, const int* __res
   for (int j = 0; j < k; ++j) {
     float v[8];
     load8(y + (size_t)inv_pos[t * k + j] * hidden + c, v);
+    const float wj = w ? w[t * k + j] : 1.0f;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) acc[i] += v[i];
+    for (int i = 0; i < 8; ++i) acc[i] += w ? wj * v[i] : v[i];
   }
   if (shared) {
     float v[8];
@@ -344,7 +354,7 @@ __global__ void moe_combine_vec_kernel(const T* __restrict__ y, const int* __res
   store8(out + (size_t)t * hidden + c, acc);
 }
 
-SHARPI_EXPORT int sharpi_moe_combine(const void* y, const int* inv_pos, const void* shared, void* out, int dtype,
+SHARPI_EXPORT int sharpi_moe_combine(const void* y, const int* inv_pos, const void* shared, const float* w, void* out, int dtype,
                                      int n_tokens, int hidden, int k, hipStream_t stream) {
   if (n_tokens <= 0) return SHARPI_OK;
   if (hidden <= 0 || k <= 0 || ceil_div(hidden, 256) > 65535) return SHARPI_ERR_ARG;
@@ -353,16 +363,16 @@ SHARPI_EXPORT int sharpi_moe_combine(const void* y, const int* inv_pos, const vo
   if ((hidden & 7) == 0) {
     dim3 vblock(128), vgrid(n_tokens, ceil_div(hidden, 128 * 8));
     if (dtype == DT_F32)
-      moe_combine_vec_kernel<float><<<vgrid, vblock, 0, stream>>>((const float*)y, inv_pos, (const float*)shared,
+      moe_combine_vec_kernel<float><<<vgrid, vblock, 0, stream>>>((const float*)y, inv_pos, (const float*)shared, w,
                                                                  (float*)out, hidden, k);
     else
-      moe_combine_vec_kernel<bf16_t><<<vgrid, vblock, 0, stream>>>((const bf16_t*)y, inv_pos, (const bf16_t*)shared,
+      moe_combine_vec_kernel<bf16_t><<<vgrid, vblock, 0, stream>>>((const bf16_t*)y, inv_pos, (const bf16_t*)shared, w,
                                                                   (bf16_t*)out, hidden, k);
   } else if (dtype == DT_F32)
-    moe_combine_kernel<float><<<grid, block, 0, stream>>>((const float*)y, inv_pos, (const float*)shared,
+    moe_combine_kernel<float><<<grid, block, 0, stream>>>((const float*)y, inv_pos, (const float*)shared, w,
                                                          (float*)out, hidden, k);
   else
-    moe_combine_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)y, inv_pos, (const bf16_t*)shared,
+    moe_combine_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)y, inv_pos, (const bf16_t*)shared, w,
                                                           (bf16_t*)out, hidden, k);
   SHARPI_CHECK_LAUNCH();
   return SHARPI_OK;

@@ -4,7 +4,9 @@
 // q head : rotate (if inv_freq) -> norm (if qk_norm) -> * temperature (if temp_tuning) -> q_out
 // k head : rotate (if inv_freq) -> norm (if qk_norm) -> cache K at slot_mapping[t]
 // v head : cache V at slot_mapping[t]
-// Rotation is on interleaved pairs (2i, 2i+1) with angle = float(pos) * inv_freq[i], all in float.
+// Rotation is on the first rotary_dim elements of a head (the rest pass through unrotated), in
+// pairs (2i, 2i+1) (interleaved) or (i, i + rotary_dim/2) (half-split), with
+// angle = float(pos) * inv_freq[i], i < rotary_dim/2, all in float.  The norm runs over the whole head.
 // Cache layout of one layer: keys [page][kv head][page_size][hd], values transposed inside the page,
 // [page][kv head][hd][page_size] (so that the matrix-core kernels read runs of keys for one
 // value column); slot = page * page_size + offset;
@@ -16,7 +18,7 @@ __global__ void rope_kv_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
                                T* __restrict__ v_cache, const int* __restrict__ slot_mapping,
                                const int* __restrict__ positions, const float* __restrict__ inv_freq,
                                int qk_norm, float eps, int temp_tuning, float floor_scale, float attn_scale,
-                               int nh, int nkv, int hd, int page_size) {
+                               int nh, int nkv, int hd, int page_size, int half_split, int rotary_dim) {
   const int t = blockIdx.x;
   const int head = blockIdx.y;            // 0..nh-1 q, nh..nh+nkv-1 k, then v
   const int lane = threadIdx.x;           // one wave
@@ -36,18 +38,33 @@ __global__ void rope_kv_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
   }
   if (is_k && slot < 0) return;
 
-  // pairs handled by this lane: i = lane, lane + 64, ... (hd <= 512)
+  // pairs handled by this lane: i = lane, lane + 64, ... (hd <= 512).  Pair i < rotary_dim/2 is a
+  // rotary pair, at elements (2i, 2i+1) or (i, i + rotary_dim/2); the pairs after them are the
+  // neighbouring elements of the unrotated rest.
+  const int rot_pairs = rotary_dim >> 1;
   float x0[4], x1[4];
+  int e0[4], e1[4];
   float ss = 0.f;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int i = lane + j * kWave;
     x0[j] = 0.f;
     x1[j] = 0.f;
+    e0[j] = e1[j] = 0;
     if (i < half) {
-      float a = to_f32<T>(src[2 * i]);
-      float b = to_f32<T>(src[2 * i + 1]);
-      if (inv_freq) {
+      if (i >= rot_pairs) {
+        e0[j] = 2 * i;
+        e1[j] = 2 * i + 1;
+      } else if (half_split) {
+        e0[j] = i;
+        e1[j] = i + rot_pairs;
+      } else {
+        e0[j] = 2 * i;
+        e1[j] = 2 * i + 1;
+      }
+      float a = to_f32<T>(src[e0[j]]);
+      float b = to_f32<T>(src[e1[j]]);
+      if (inv_freq && i < rot_pairs) {
         const float ang = (float)pos * inv_freq[i];
         const float c = cosf(ang);
         const float s = sinf(ang);
@@ -90,13 +107,14 @@ __global__ void rope_kv_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
         a *= post;
         b *= post;
       }
-      dst[2 * i] = from_f32<T>(a);
-      dst[2 * i + 1] = from_f32<T>(b);
+      dst[e0[j]] = from_f32<T>(a);
+      dst[e1[j]] = from_f32<T>(b);
     }
   }
 }
 
-// The same for head sizes 32, 64, 128, 256: a thread per run of 8 elements (4 rotary pairs),
+// The same for head sizes 32, 64, 128, 256 with interleaved pairs and a rotary width that is a
+// multiple of 8 (runs beyond it pass through): a thread per run of 8 elements (4 rotary pairs),
 // 16-byte accesses; the hd/8 lanes of a head are neighbours in a wave and sum their squares with
 // shuffles.  Blocks (token, y) share a token's heads between them, 256 runs each, so that a
 // handful of decode tokens still spreads over many compute units.
@@ -105,7 +123,7 @@ __global__ __launch_bounds__(256) void rope_kv_vec_kernel(
     const T* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
     const int* __restrict__ slot_mapping, const int* __restrict__ positions, const float* __restrict__ inv_freq,
     int qk_norm, float eps, int temp_tuning, float floor_scale, float attn_scale, int nh, int nkv, int hd,
-    int page_size) {
+    int page_size, int rotary_dim) {
   const int t = blockIdx.x;
   const int per_head = hd >> 3;                    // lanes per head: 4, 8, 16 or 32
   const int chunks = (nh + 2 * nkv) * per_head;
@@ -118,7 +136,8 @@ __global__ __launch_bounds__(256) void rope_kv_vec_kernel(
   // of the lanes per head), and so are its four angles: their sines and cosines are computed once
   const int run = threadIdx.x % per_head;
   float cs[4], sn[4];
-  if (inv_freq) {
+  const bool rotates = inv_freq != nullptr && run * 8 < rotary_dim;
+  if (rotates) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const float ang = (float)pos * inv_freq[run * 4 + j];
@@ -136,7 +155,7 @@ __global__ __launch_bounds__(256) void rope_kv_vec_kernel(
     if (valid) load8(src + (size_t)head * hd + run * 8, x);
     float ss = 0.f;
     if (valid && (is_q || is_k)) {
-      if (inv_freq) {
+      if (rotates) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const float a = x[2 * j], b = x[2 * j + 1];
@@ -179,14 +198,19 @@ __global__ __launch_bounds__(256) void rope_kv_vec_kernel(
 SHARPI_EXPORT int sharpi_rope_kv(const void* qkv, void* q_out, void* k_cache, void* v_cache, int dtype,
                                  const int* slot_mapping, const int* positions, const float* inv_freq,
                                  int qk_norm, float eps, int temp_tuning, float floor_scale, float attn_scale,
-                                 int n_tokens, int nh, int nkv, int hd, int page_size, hipStream_t stream) {
+                                 int n_tokens, int nh, int nkv, int hd, int page_size, int pair_layout,
+                                 int rotary_dim, hipStream_t stream) {
   if (n_tokens <= 0) return SHARPI_OK;
+  // pair_layout: 0 = pairs (2i, 2i+1), 1 = pairs (i, i + rotary_dim/2); rotary_dim even, <= hd
+  if (pair_layout < 0 || pair_layout > 1) return SHARPI_ERR_ARG;
+  if (inv_freq == nullptr) rotary_dim = 0;
+  else if (rotary_dim <= 0 || (rotary_dim & 1) || rotary_dim > hd) return SHARPI_ERR_ARG;
   if (hd <= 0 || (hd & 1) || hd > 512 || nh <= 0 || nkv <= 0 || page_size <= 0) return SHARPI_ERR_ARG;
   if (nh + 2 * nkv > 65535) return SHARPI_ERR_ARG;
   if (temp_tuning && !(floor_scale > 0.f)) return SHARPI_ERR_ARG;
   dim3 grid(n_tokens, nh + 2 * nkv), block(kWave);
   if (dtype != DT_F32 && dtype != DT_BF16) return SHARPI_ERR_ARG;
-  if (hd == 32 || hd == 64 || hd == 128 || hd == 256) {
+  if ((hd == 32 || hd == 64 || hd == 128 || hd == 256) && pair_layout == 0 && (rotary_dim & 7) == 0) {
     // a few tokens (decode): a token's heads over several blocks, for the compute units' sake;
     // many tokens: one block per token, which then computes its angles once for all heads
     const dim3 vgrid(n_tokens, n_tokens <= 64 ? ceil_div((nh + 2 * nkv) * (hd >> 3), 256) : 1);
@@ -194,12 +218,12 @@ SHARPI_EXPORT int sharpi_rope_kv(const void* qkv, void* q_out, void* k_cache, vo
       rope_kv_vec_kernel<float><<<vgrid, 256, 0, stream>>>((const float*)qkv, (float*)q_out, (float*)k_cache,
                                                              (float*)v_cache, slot_mapping, positions, inv_freq,
                                                              qk_norm, eps, temp_tuning, floor_scale, attn_scale,
-                                                             nh, nkv, hd, page_size);
+                                                             nh, nkv, hd, page_size, rotary_dim);
     else
       rope_kv_vec_kernel<bf16_t><<<vgrid, 256, 0, stream>>>((const bf16_t*)qkv, (bf16_t*)q_out,
                                                               (bf16_t*)k_cache, (bf16_t*)v_cache, slot_mapping,
                                                               positions, inv_freq, qk_norm, eps, temp_tuning,
-                                                              floor_scale, attn_scale, nh, nkv, hd, page_size);
+                                                              floor_scale, attn_scale, nh, nkv, hd, page_size, rotary_dim);
     SHARPI_CHECK_LAUNCH();
     return SHARPI_OK;
   }
@@ -207,12 +231,12 @@ SHARPI_EXPORT int sharpi_rope_kv(const void* qkv, void* q_out, void* k_cache, vo
     rope_kv_kernel<float><<<grid, block, 0, stream>>>((const float*)qkv, (float*)q_out, (float*)k_cache,
                                                      (float*)v_cache, slot_mapping, positions, inv_freq, qk_norm,
                                                      eps, temp_tuning, floor_scale, attn_scale, nh, nkv, hd,
-                                                     page_size);
+                                                     page_size, pair_layout, rotary_dim);
   else if (dtype == DT_BF16)
     rope_kv_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)qkv, (bf16_t*)q_out, (bf16_t*)k_cache,
                                                       (bf16_t*)v_cache, slot_mapping, positions, inv_freq,
                                                       qk_norm, eps, temp_tuning, floor_scale, attn_scale, nh, nkv,
-                                                      hd, page_size);
+                                                      hd, page_size, pair_layout, rotary_dim);
   else
     return SHARPI_ERR_ARG;
   SHARPI_CHECK_LAUNCH();

@@ -15,7 +15,7 @@ from typing import Callable, Dict, Hashable, Iterator, List, Optional, Sequence,
 
 import torch
 
-from ..cache.manager import CacheManager
+from ..cache.manager import CacheManager, pool_sizes
 from ..cache.spec import KVSpec
 from ..config.base import ModelConfig, load_config
 from ..registry import build_model
@@ -113,15 +113,23 @@ class Engine:
         self.max_tokens_per_step = int(max_tokens_per_step)
         self.page_size = int(page_size)
         specs = self.model.cache_specs()
-        if kv_tokens is None:
-            # every request at full length, or what four fifths of the free memory hold if that is less
-            kv_tokens = self.max_num_seqs * ((self.max_model_len + page_size - 1) // page_size * page_size)
-            width = torch.empty(0, dtype=self.dtype).element_size()
-            per_token = sum(2 * s.num_kv_heads * s.head_dim * width for s in specs if isinstance(s, KVSpec))
-            free = torch.cuda.mem_get_info(self.device)[0]
-            kv_tokens = max(page_size, min(kv_tokens, int(free * 0.8) // max(1, per_token)))
-        num_pages = max(1, (int(kv_tokens) + page_size - 1) // page_size)
-        self.cache = CacheManager(specs, page_size, num_pages, self.max_num_seqs, self.dtype, self.device)
+        # Pages per group.  kv_tokens is the number of tokens the pools are made for (default: every
+        # request at full length, or what four fifths of the free memory hold if that is less); a
+        # group without a window gets that many, a windowed group only what its windows can ever
+        # hold at once (window + one step, per request), however long the requests grow.
+        width = torch.empty(0, dtype=self.dtype).element_size()
+        kv_specs = [s for s in specs if isinstance(s, KVSpec)]
+        full_len = (self.max_model_len + page_size - 1) // page_size * page_size
+        sizes = pool_sizes(specs, page_size, self.max_num_seqs, full_len, self.max_tokens_per_step,
+                           None if kv_tokens is None else max(1, (int(kv_tokens) + page_size - 1) // page_size))
+        if kv_tokens is None and kv_specs:
+            def total_bytes(sz):
+                return sum(sz[s.group_key()] * 2 * s.num_kv_heads * s.head_dim * page_size * width for s in kv_specs)
+            budget = int(torch.cuda.mem_get_info(self.device)[0] * 0.8)
+            while total_bytes(sizes) > budget and max(sizes.values()) > 1:
+                big = max(sizes, key=lambda k: sizes[k])       # the largest pools give way first
+                sizes[big] = max(1, int(sizes[big] * 0.9))
+        self.cache = CacheManager(specs, page_size, sizes if sizes else 1, self.max_num_seqs, self.dtype, self.device)
         self.runner = ModelRunner(self.model, self.cache, self.dtype, self.device, decode_graphs=decode_graphs,
                                   max_context=self.max_model_len)
         self.sampler = Sampler(self.device)

@@ -48,9 +48,13 @@ class ModelRunner:
         self.device = torch.device(device)
         self.steps_run = 0
         # Steps made of single decoded tokens only are launch-bound: they are captured once per
-        # batch size into a HIP graph over fixed index buffers and replayed.
-        # (not for mixers with state of their own: the capture's trial run would advance it)
-        self.decode_graphs = bool(decode_graphs) and max_context > 0 and all(t is None for t in cache.state)
+        # batch size into a HIP graph over fixed index buffers and replayed.  A mixer with state of
+        # its own must say that its step can be captured (``graph_safe``: it walks the entries
+        # through the context's device tensors, without a copy to the host); the capture's trial
+        # run then works on the cache manager's scratch state slot, so that no request's state moves.
+        safe = getattr(model, "decode_graph_safe", None)
+        self.decode_graphs = bool(decode_graphs) and max_context > 0 and (
+            all(t is None for t in cache.state) or bool(safe and safe()))
         self.max_context = int(max_context)
         self._graphs: dict = {}
         self.graph_replays = 0
@@ -259,7 +263,7 @@ class _DecodeGraph:
         n = info["n"]
         null[2] = np.arange(n, dtype=np.int32)            # entry of token
         null[3] = np.arange(n + 1, dtype=np.int32)        # cu_tokens
-        null[4] = pieces[4]                               # state slots (any valid slot)
+        null[4] = np.full_like(pieces[4], runner.cache.scratch_state_slot)   # state: the slot of no request
         null[5] = np.full(n, -1, dtype=np.int32)
         null[6] = np.arange(n, dtype=np.int32)            # logit rows
         null[7] = np.arange(n, dtype=np.int32)

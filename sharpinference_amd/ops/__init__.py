@@ -75,18 +75,23 @@ def embed_gather(ids: torch.Tensor, table: torch.Tensor, out: Optional[torch.Ten
 
 
 class ExpertSum:
-    """A branch output that is still a sum to be formed: row t = sum_j y[inv_pos[t*k + j]]
-    (+ shared[t]).  ``add_rmsnorm`` forms it on the fly; ``tensor()`` forms it with a kernel of
-    its own.  Either way the sum is rounded once to y's storage type."""
+    """A branch output that is still a sum to be formed: row t = sum_j w[t, j] * y[inv_pos[t*k + j]]
+    (+ shared[t]); ``weights`` None means ones (scores already applied to the experts' inputs).
+    ``add_rmsnorm`` forms it on the fly; ``tensor()`` forms it with a kernel of its own.  Either
+    way the sum is rounded once to y's storage type."""
 
-    __slots__ = ("y", "inv_pos", "shared", "n_tokens", "k")
+    __slots__ = ("y", "inv_pos", "shared", "n_tokens", "k", "weights")
 
-    def __init__(self, y: torch.Tensor, inv_pos: torch.Tensor, shared: Optional[torch.Tensor], n_tokens: int, k: int):
+    def __init__(self, y: torch.Tensor, inv_pos: torch.Tensor, shared: Optional[torch.Tensor], n_tokens: int, k: int,
+                 weights: Optional[torch.Tensor] = None):
         _need(y.dim() == 2 and inv_pos.numel() == n_tokens * k, "ExpertSum: y [rows, H], inv_pos [T*k]")
         if shared is not None:
             _need(shared.shape == (n_tokens, y.shape[1]) and shared.dtype == y.dtype and shared.is_contiguous(),
                   "ExpertSum: shared must be contiguous [T, H] of y's dtype")
-        self.y, self.inv_pos, self.shared, self.n_tokens, self.k = y, inv_pos, shared, n_tokens, k
+        if weights is not None:
+            _need(weights.numel() == n_tokens * k and weights.dtype == torch.float32 and weights.is_contiguous(),
+                  "ExpertSum: weights must be contiguous float32 [T, k]")
+        self.y, self.inv_pos, self.shared, self.n_tokens, self.k, self.weights = y, inv_pos, shared, n_tokens, k, weights
 
     @property
     def shape(self):
@@ -97,7 +102,8 @@ class ExpertSum:
         return self.y.dtype
 
     def tensor(self) -> torch.Tensor:
-        return moe_combine(self.y[: self.n_tokens * self.k], self.inv_pos, self.shared, self.n_tokens, self.k)
+        return moe_combine(self.y[: self.n_tokens * self.k], self.inv_pos, self.shared, self.n_tokens, self.k,
+                           self.weights)
 
 
 def add_rmsnorm(h: torch.Tensor, delta, weight: Optional[torch.Tensor], eps: float,
@@ -109,7 +115,7 @@ def add_rmsnorm(h: torch.Tensor, delta, weight: Optional[torch.Tensor], eps: flo
     if lazy is not None and h.shape[1] % 8 != 0:
         delta, lazy = lazy.tensor(), None          # the kernel folds a sum in only at widths that are multiples of 8
     base = lazy.y if lazy is not None else delta
-    _dev(h, base, weight, rows, out)
+    _dev(h, base, weight, rows, out, lazy.weights if lazy is not None else None)
     _i32(rows, "rows")
     _need(h.dim() == 2 and h.dtype == torch.float32, "add_rmsnorm: h must be float32 [T, H]")
     T, H = h.shape
@@ -127,7 +133,7 @@ def add_rmsnorm(h: torch.Tensor, delta, weight: Optional[torch.Tensor], eps: flo
          _ptr(weight), _code(weight.dtype) if weight is not None else 0, _ptr(out), _code(out_dtype), _ptr(rows),
          n_out, H, float(eps), 1 if write_back else 0,
          _ptr(lazy.inv_pos) if lazy is not None else None, _ptr(lazy.shared) if lazy is not None else None,
-         lazy.k if lazy is not None else 0, _stream())
+         _ptr(lazy.weights) if lazy is not None else None, lazy.k if lazy is not None else 0, _stream())
     return out
 
 
@@ -144,18 +150,20 @@ def silu_mul(gate_up: torch.Tensor, scale: Optional[torch.Tensor] = None) -> tor
 
 
 def moe_combine(y: torch.Tensor, inv_pos: torch.Tensor, shared: Optional[torch.Tensor], n_tokens: int,
-                k: int) -> torch.Tensor:
-    """out[t] = sum_j y[inv_pos[t*k+j]] (+ shared[t])."""
-    _dev(y, inv_pos, shared)
+                k: int, weights: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[t] = sum_j w[t, j] * y[inv_pos[t*k+j]] (+ shared[t]); weights None: ones."""
+    _dev(y, inv_pos, shared, weights)
     _i32(inv_pos, "inv_pos")
     _need(y.dim() == 2 and y.shape[0] == n_tokens * k and inv_pos.numel() == n_tokens * k,
           "moe_combine: y must be [T*k, H] and inv_pos [T*k]")
     H = y.shape[1]
     if shared is not None:
         _need(shared.shape == (n_tokens, H) and shared.dtype == y.dtype, "moe_combine: shared must be [T, H]")
+    if weights is not None:
+        _need(weights.numel() == n_tokens * k and weights.dtype == torch.float32, "moe_combine: weights must be float32 [T, k]")
     out = torch.empty(n_tokens, H, dtype=y.dtype, device=y.device)
-    _run("sharpi_moe_combine", _ptr(y), _ptr(inv_pos), _ptr(shared), _ptr(out), _code(y.dtype), n_tokens, H, k,
-         _stream())
+    _run("sharpi_moe_combine", _ptr(y), _ptr(inv_pos), _ptr(shared), _ptr(weights), _ptr(out), _code(y.dtype), n_tokens,
+         H, k, _stream())
     return out
 
 
@@ -172,11 +180,17 @@ def _cache_shapes_ok(k_cache: torch.Tensor, v_cache: torch.Tensor, nkv: int, hd:
             and v_cache.shape == (k_cache.shape[0], nkv, hd, k_cache.shape[2]))
 
 
+PAIRS_INTERLEAVED, PAIRS_HALF_SPLIT = 0, 1
+
+
 def rope_kv(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, slot_mapping: torch.Tensor,
             positions: torch.Tensor, inv_freq: Optional[torch.Tensor], qk_norm: bool, eps: float,
-            temperature: Optional[Tuple[float, float]], nh: int, nkv: int, hd: int) -> torch.Tensor:
+            temperature: Optional[Tuple[float, float]], nh: int, nkv: int, hd: int,
+            pair_layout: int = PAIRS_INTERLEAVED) -> torch.Tensor:
     """Rotate / norm / scale the heads of qkv [T, (nh+2nkv)*hd]; K and V go into the layer's
-    cache [pages, nkv, page_size, hd] at slot_mapping; returns q [T, nh*hd]."""
+    cache [pages, nkv, page_size, hd] at slot_mapping; returns q [T, nh*hd].  inv_freq [r/2]
+    rotates the first r <= hd elements of every head, in pairs (2i, 2i+1) or (i, i + r/2)
+    (``pair_layout``); the rest of the head passes through."""
     _dev(qkv, k_cache, v_cache, slot_mapping, positions, inv_freq)
     _i32(slot_mapping, "slot_mapping")
     _i32(positions, "positions")
@@ -185,14 +199,19 @@ def rope_kv(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, slo
     _need(_cache_shapes_ok(k_cache, v_cache, nkv, hd), "rope_kv: caches must be K [pages, nkv, page_size, hd], V [pages, nkv, hd, page_size]")
     _need(k_cache.dtype == qkv.dtype and v_cache.dtype == qkv.dtype, "rope_kv: cache dtype differs from qkv's")
     _need(slot_mapping.shape == (T,) and positions.shape == (T,), "rope_kv: slot_mapping / positions must be [T]")
+    rotary_dim = 0
     if inv_freq is not None:
-        _need(inv_freq.dtype == torch.float32 and inv_freq.shape == (hd // 2,), "rope_kv: inv_freq must be float32 [hd/2]")
+        _need(inv_freq.dtype == torch.float32 and inv_freq.dim() == 1 and 1 <= inv_freq.shape[0] <= hd // 2,
+              "rope_kv: inv_freq must be float32 [rotary_dim / 2], rotary_dim <= hd")
+        rotary_dim = 2 * inv_freq.shape[0]
+    _need(pair_layout in (PAIRS_INTERLEAVED, PAIRS_HALF_SPLIT), "rope_kv: pair_layout must be interleaved (0) or half-split (1)")
     page_size = k_cache.shape[2]
     q_out = torch.empty(T, nh * hd, dtype=qkv.dtype, device=qkv.device)
     fs, asc = temperature if temperature is not None else (1.0, 0.0)
     _run("sharpi_rope_kv", _ptr(qkv), _ptr(q_out), _ptr(k_cache), _ptr(v_cache), _code(qkv.dtype),
          _ptr(slot_mapping), _ptr(positions), _ptr(inv_freq), 1 if qk_norm else 0, float(eps),
-         1 if temperature is not None else 0, float(fs), float(asc), T, nh, nkv, hd, page_size, _stream())
+         1 if temperature is not None else 0, float(fs), float(asc), T, nh, nkv, hd, page_size, int(pair_layout),
+         rotary_dim, _stream())
     return q_out
 
 
@@ -773,19 +792,20 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, gro
                              window, scale, nh, nkv, hd)
 
 
-def grouped_swiglu(x: torch.Tensor, w_gate_up, rt: Routing, out_dtype: torch.dtype) -> torch.Tensor:
+def grouped_swiglu(x: torch.Tensor, w_gate_up, rt: Routing, out_dtype: torch.dtype, scaled: bool = True) -> torch.Tensor:
     """The experts' gate|up products of the routed tokens and their activation,
-    silu(s g) * (s u) with s the pick's weight: [n_rows, I] in expert-sorted order.  On the
-    matrix cores the activation is the product's epilogue (the few-rows kernel or the many-rows
-    one); otherwise the product and the activation are two kernels."""
+    silu(s g) * (s u) with s the pick's weight (``scaled``; otherwise s = 1): [n_rows, I] in
+    expert-sorted order.  On the matrix cores the activation is the product's epilogue (the
+    few-rows kernel or the many-rows one); otherwise the product and the activation are two kernels."""
     N, K = w_gate_up.shape[1], w_gate_up.shape[2]
+    scale = rt.sorted_w if scaled else None
     if x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16 and out_dtype == torch.bfloat16 and K % 128 == 0:
         if rt.n_tokens <= SKINNY_MAX_ROWS and N % (32 if isinstance(w_gate_up, PackedWeight) else 8) == 0:
-            return gemm_skinny_swiglu(x, w_gate_up, rt.offsets, rt.sorted_token, rt.n_rows, rt.sorted_w,
+            return gemm_skinny_swiglu(x, w_gate_up, rt.offsets, rt.sorted_token, rt.n_rows, scale,
                                       group_rows=rt.n_tokens)
         if rt.n_tokens > SKINNY_MAX_ROWS and N % 32 == 0 and rt.n_groups == rt.n_experts:
-            return gemm_grouped_swiglu(x, w_gate_up, rt, rt.sorted_w)
-    return silu_mul(grouped_linear(x, w_gate_up, rt, True, out_dtype), rt.sorted_w)
+            return gemm_grouped_swiglu(x, w_gate_up, rt, scale)
+    return silu_mul(grouped_linear(x, w_gate_up, rt, True, out_dtype), scale)
 
 
 def grouped_linear(x: torch.Tensor, w, rt: Routing, gather: bool, out_dtype: torch.dtype) -> torch.Tensor:

@@ -18,11 +18,11 @@ F = c_float
 
 _SIGNATURES = {
     "sharpi_embed_gather": [P, P, I, P, I, I, P],
-    "sharpi_add_rmsnorm": [P, P, I, P, I, P, I, P, I, I, F, I, P, P, I, P],
+    "sharpi_add_rmsnorm": [P, P, I, P, I, P, I, P, I, I, F, I, P, P, P, I, P],
     "sharpi_silu_mul": [P, P, P, I, I, I, P],
-    "sharpi_moe_combine": [P, P, P, P, I, I, I, I, P],
+    "sharpi_moe_combine": [P, P, P, P, P, I, I, I, I, P],
     "sharpi_cast": [P, I, P, I, c_longlong, P],
-    "sharpi_rope_kv": [P, P, P, P, I, P, P, P, I, F, I, F, F, I, I, I, I, I, P],
+    "sharpi_rope_kv": [P, P, P, P, I, P, P, P, I, F, I, F, F, I, I, I, I, I, I, I, P],
     "sharpi_attention_generic": [P, P, P, I, P, P, P, P, I, I, F, I, I, I, I, I, I, I, P],
     "sharpi_attention_decode": [P, P, P, P, P, P, P, P, P, P, I, I, F, I, I, I, I, I, I, I, I, P],
     "sharpi_attention_prefill": [P, P, P, P, P, P, P, I, I, I, F, I, I, I, I, I, I, P],

@@ -9,7 +9,6 @@ import torch
 from .. import ops
 from ..cache.spec import KVSpec, WINDOW_CHUNK, WINDOW_NONE, WINDOW_SLIDING  # noqa: F401
 from .base import LayerCache, ParamSpec, Part, StepContext, TensorSource
-from .position import RotaryInterleaved
 
 
 class Attention(Part):
@@ -20,12 +19,13 @@ class Attention(Part):
     after the rotation, 1643-1648).
 
     Everything that differs between layers is an argument: ``rotary`` (None = no position
-    encoding), ``qk_norm_eps`` (None = no norm), ``q_temperature`` = (floor_scale, attn_scale)
+    encoding; otherwise any object with ``table(device)``, ``pair_layout``, ``rotary_dim`` and
+    ``head_dim``, see parts/position.py), ``qk_norm_eps`` (None = no norm), ``q_temperature`` = (floor_scale, attn_scale)
     multiplying queries by 1 + attn_scale * ln(floor((pos + 1) / floor_scale) + 1), and the
     window: all keys, the chunk [floor(pos/W)*W, pos], or the last W keys."""
 
     def __init__(self, hidden: int, num_heads: int, num_kv_heads: int, head_dim: int,
-                 rotary: Optional[RotaryInterleaved] = None, qk_norm_eps: Optional[float] = None,
+                 rotary=None, qk_norm_eps: Optional[float] = None,
                  q_temperature: Optional[Tuple[float, float]] = None, window_kind: int = WINDOW_NONE,
                  window: int = 0, scale: Optional[float] = None):
         if num_heads % num_kv_heads:
@@ -34,6 +34,8 @@ class Attention(Part):
             raise ValueError(f"head_dim {head_dim} is not taken: multiples of 16 from 16 to 256")
         if rotary is not None and rotary.head_dim != head_dim:
             raise ValueError("the rotary table's head_dim differs from the mixer's")
+        if rotary is not None and rotary.pair_layout not in ("interleaved", "half"):
+            raise ValueError(f"pair layout {rotary.pair_layout!r} is not taken by the rotation kernel")
         self.hidden, self.nh, self.nkv, self.hd = int(hidden), int(num_heads), int(num_kv_heads), int(head_dim)
         self.rotary, self.qk_norm_eps, self.q_temperature = rotary, qk_norm_eps, q_temperature
         self.window_kind, self.window = int(window_kind), int(window)
@@ -73,8 +75,9 @@ class Attention(Part):
         qkv = ops.linear(x, self.w_qkv, ctx.act_dtype)
         slots = g.slot_mapping if cache.write else ctx.no_store_slots
         inv_freq = self.rotary.table(x.device) if self.rotary is not None else None
+        layout = ops.PAIRS_HALF_SPLIT if self.rotary is not None and self.rotary.pair_layout == "half" else ops.PAIRS_INTERLEAVED
         q = ops.rope_kv(qkv, cache.k, cache.v, slots, ctx.positions, inv_freq, self.qk_norm_eps is not None,
-                        self.qk_norm_eps or 1e-6, self.q_temperature, self.nh, self.nkv, self.hd)
+                        self.qk_norm_eps or 1e-6, self.q_temperature, self.nh, self.nkv, self.hd, layout)
         o = ops.attention(q, cache.k, cache.v, g, ctx, self.window_kind, self.window, self.scale, self.nh, self.nkv,
                           self.hd)
         return ops.linear(o, self.w_o, ctx.act_dtype)

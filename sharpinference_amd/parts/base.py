@@ -46,7 +46,8 @@ class StepContext:
     positions: torch.Tensor            # int32 [tokens]
     entry_of_token: torch.Tensor       # int32 [tokens]
     cu_tokens: torch.Tensor            # int32 [entries + 1]
-    state_slots: torch.Tensor          # int32 [entries]: the state slot of each entry's request
+    state_slots: torch.Tensor          # int32 [entries]: the state slot of each entry's request (device: index
+                                       # state tensors with it; a replayed graph sees each step's slots here)
     groups: List[GroupView]
     act_dtype: torch.dtype
     no_store_slots: Optional[torch.Tensor] = None   # int32 [tokens] of -1: "store nothing" for cache readers

@@ -39,6 +39,13 @@ class PreNormBlock(Part):
         spec = getattr(self.mixer, "cache_spec", None)
         return spec() if spec else None
 
+    def decode_graph_safe(self) -> bool:
+        """Can a decode step through this block be captured into a graph?  Paged attention can; a
+        mixer with state of its own says so itself (``graph_safe``)."""
+        from ..cache.spec import StateSpec
+
+        return not isinstance(self.cache_spec(), StateSpec) or bool(getattr(self.mixer, "graph_safe", False))
+
     def forward(self, stream: ResidualStream, ctx: StepContext, cache: LayerCache) -> None:
         n = self.norm1.forward(stream, ctx.act_dtype)
         stream.pending = self.mixer.forward(n, ctx, cache)

@@ -61,8 +61,10 @@ class MoESwiGLU(Part):
 
     The router's logits, gate and picks are float and stay on the device.  With
     ``score_on_input`` the gate and up products of a chosen expert are multiplied by its score
-    before the SiLU (ForwardPass.cs:2083-2089); the shared expert sees the unscaled input
-    (2060-2066); the outputs are summed (2096-2097).  ``gate`` is "sigmoid" or "softmax"
+    before the SiLU (ForwardPass.cs:2083-2089); without it the expert runs on the unscaled input
+    and its output is multiplied by the score where the outputs are summed (the reference's other
+    order, src/SharpInference.Cuda/CudaKernels.cs:112-157 llm_moe_weighted_reduce).  The shared
+    expert sees the unscaled input (2060-2066); the outputs are summed (2096-2097).  ``gate`` is "sigmoid" or "softmax"
     (2031-2034); ``renormalise`` divides the k scores by their sum (2156-2162)."""
 
     MERGE_MAX_TOKENS = 16   # one row block of the few-rows kernel for the shared group (measured: up to 64 tokens
@@ -77,13 +79,12 @@ class MoESwiGLU(Part):
             raise ValueError(f"{num_experts} experts are not taken: the routing kernels hold scores for {ops.ROUTER_MAX_EXPERTS}")
         if gate not in ("sigmoid", "softmax"):
             raise ValueError(f"router gate {gate!r} is not known (sigmoid, softmax)")
-        if not score_on_input:
-            raise NotImplementedError("expert scores applied to the output are not built; only score_on_input=True")
         self.hidden, self.E, self.k = int(hidden), int(num_experts), int(top_k)
         self.inter = int(expert_intermediate)
         self.shared = DenseSwiGLU(hidden, shared_intermediate) if shared_intermediate else None
         self.gate = ops.GATE_SIGMOID if gate == "sigmoid" else ops.GATE_SOFTMAX
         self.renormalise = bool(renormalise)
+        self.score_on_input = bool(score_on_input)
         self.w_router: Optional[torch.Tensor] = None
         self.w_gate_up: Optional[torch.Tensor] = None     # [E, 2*I, H]
         self.w_down: Optional[torch.Tensor] = None        # [E, H, I]
@@ -159,9 +160,11 @@ class MoESwiGLU(Part):
             trace.append((ids, wts, x))
         along = self.merged and T <= self.MERGE_MAX_TOKENS
         shared = None if along or self.shared is None else self.shared.forward(x, ctx)
-        act = ops.gemm_skinny_picked(x, self.w_gate_up, ids, wts, along, True, True, ctx.act_dtype)
+        act = ops.gemm_skinny_picked(x, self.w_gate_up, ids, wts if self.score_on_input else None, along, True, True,
+                                     ctx.act_dtype)
         y = ops.gemm_skinny_picked(act, self.w_down, ids, None, along, False, False, ctx.act_dtype)
-        return ops.ExpertSum(y, ops.counting(T * self.k, x.device), y[T * self.k:] if along else shared, T, self.k)
+        return ops.ExpertSum(y, ops.counting(T * self.k, x.device), y[T * self.k:] if along else shared, T, self.k,
+                             None if self.score_on_input else wts)
 
     def forward_from_stream(self, stream: ResidualStream, norm: Part, ctx: StepContext):
         """The block's second half from the residual stream: normalise and feed forward.  With a
@@ -185,13 +188,14 @@ class MoESwiGLU(Part):
         ids, wts, rt = ops.route(x, self.w_router, self.k, self.gate, self.renormalise, shared_group=merge)
         if trace is not None:      # the picks of this step, layer by layer (reference: ForwardPass.cs:2042-2056)
             trace.append((ids, wts, x))
+        after = None if self.score_on_input else wts     # scores applied where the outputs are summed
         if merge:
             # few rows: the shared expert rides along as one more group of the same two launches
-            act = ops.grouped_swiglu(x, self.w_gate_up, rt, ctx.act_dtype)
+            act = ops.grouped_swiglu(x, self.w_gate_up, rt, ctx.act_dtype, scaled=self.score_on_input)
             y = ops.grouped_linear(act, self.w_down, rt, False, ctx.act_dtype)
             # left as a sum: the next norm forms it while it reads the residual stream
-            return ops.ExpertSum(y, rt.inv_pos, y[T * self.k:], T, self.k)
+            return ops.ExpertSum(y, rt.inv_pos, y[T * self.k:], T, self.k, after)
         shared = self.shared.forward(x, ctx) if self.shared is not None else None
-        act = ops.grouped_swiglu(x, self.w_gate_up, rt, ctx.act_dtype)
+        act = ops.grouped_swiglu(x, self.w_gate_up, rt, ctx.act_dtype, scaled=self.score_on_input)
         y = ops.grouped_linear(act, self.w_down, rt, False, ctx.act_dtype)
-        return ops.ExpertSum(y, rt.inv_pos, shared, T, self.k)   # formed by the next norm (or by whoever asks for a tensor)
+        return ops.ExpertSum(y, rt.inv_pos, shared, T, self.k, after)   # formed by the next norm (or by whoever asks for a tensor)

@@ -75,6 +75,9 @@ class DecoderModel(Part):
                 specs[r.cache] = self.blocks[r.layer].cache_spec()
         return specs
 
+    def decode_graph_safe(self) -> bool:
+        return all(getattr(b, "decode_graph_safe", lambda: True)() for b in self.blocks)
+
     # -- weights ------------------------------------------------------------------
     def param_specs(self, prefix: str = "") -> Dict[str, ParamSpec]:
         out = {self.embed_name: ParamSpec((self.vocab_size, self.hidden))}

@@ -76,7 +76,7 @@ def assert_picks_are_the_best(x: torch.Tensor, router_weight: torch.Tensor, ids:
 
 def assert_routes_are_the_best(model_dir: str, picks, inputs, what: str) -> None:
     """Every routed layer's picks against the rows its router saw (see assert_picks_are_the_best)."""
-    W = P.load_weights(model_dir)
+    W = _model(model_dir)[1]
     for layer, ids, x in zip(moe_layers_of(model_dir), picks, inputs):
         assert_picks_are_the_best(x, W[f"model.layers.{layer}.feed_forward.router.weight"], ids, f"{what} layer {layer}")
 
@@ -86,10 +86,16 @@ def random_tokens(n: int, vocab: int, seed: int) -> List[int]:
     return [rng.randrange(vocab) for _ in range(n)]
 
 
+@functools.lru_cache(maxsize=2)
+def _model(model_dir: str):
+    """(config, weights in float32) of a model folder, read once (a folder is written once by the tests)."""
+    W = {k: v.float() if v.is_floating_point() else v for k, v in P.load_weights(model_dir).items()}
+    return P.read_config(model_dir), W
+
+
 @functools.lru_cache(maxsize=128)
 def _plain_cached(model_dir: str, tokens: tuple, bf16_storage: bool) -> torch.Tensor:
-    c = P.read_config(model_dir)
-    W = P.load_weights(model_dir)
+    c, W = _model(model_dir)
     return P.forward(c, W, list(tokens), store=P.store_bf16 if bf16_storage else P._same)
 
 
@@ -106,8 +112,7 @@ def moe_layers_of(model_dir: str) -> List[int]:
 
 def plain_logits_routed(model_dir: str, tokens: Sequence[int], routes: Dict[int, torch.Tensor]) -> torch.Tensor:
     """The plain implementation with bfloat16 storage and the engine's own expert picks."""
-    c = P.read_config(model_dir)
-    W = P.load_weights(model_dir)
+    c, W = _model(model_dir)
     return P.forward(c, W, list(tokens), store=P.store_bf16, routes=routes)
 
 

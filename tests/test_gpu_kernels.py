@@ -674,6 +674,61 @@ def test_rope_kv_kernel(nh, nkv, hd, dtype, mode):
     assert float(kcc.permute(0, 2, 1, 3).reshape(pages * ps, -1)[~written].abs().max()) == 0.0
 
 
+def _rotate_plain(x, positions, inv_freq, layout):
+    """x [T, heads, hd]: the first 2 * len(inv_freq) elements of every head rotated by
+    pos * freq_i, on pairs (2i, 2i+1) ("interleaved") or (i, i + r/2) ("half"); the rest as it is."""
+    r = 2 * inv_freq.shape[0]
+    ang = positions.to(torch.float32)[:, None] * inv_freq[None, :]
+    cos, sin = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+    out = x.clone()
+    if layout == "interleaved":
+        a, b = x[..., 0:r:2], x[..., 1:r:2]
+        out[..., 0:r:2], out[..., 1:r:2] = a * cos - b * sin, a * sin + b * cos
+    else:
+        a, b = x[..., :r // 2], x[..., r // 2:r]
+        out[..., :r // 2], out[..., r // 2:r] = a * cos - b * sin, a * sin + b * cos
+    return out
+
+
+@pytest.mark.parametrize("hd,rotary_dim", [(16, 16), (32, 16), (48, 20), (64, 64), (128, 64), (128, 24)])
+@pytest.mark.parametrize("layout", ["interleaved", "half"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rope_kv_kernel_pair_layouts_and_partial_width(hd, rotary_dim, layout, dtype):
+    """The pairing and the rotated width are arguments of the kernel: half-split pairs, and heads
+    of which only the first elements rotate (the norm still runs over the whole head)."""
+    ops = _ops()
+    import plain_llama4 as P
+    from sharpinference_amd.parts.position import Rotary
+
+    nh, nkv, T, ps, pages = 3, 1, 9, 16, 4
+    rot = Rotary(hd, 10000.0, None, pair_layout=layout, rotary_dim=rotary_dim)
+    inv = rot.frequencies()
+    assert inv.shape == (rotary_dim // 2,)
+    assert torch.allclose(inv, P.rope_inv_freq(rotary_dim, 10000.0, None))
+    qkv = _rand(T, (nh + 2 * nkv) * hd, dtype=dtype, seed=hd + rotary_dim)
+    positions = torch.tensor([0, 1, 2, 17, 31, 100, 1000, 4095, 5], dtype=torch.int32)
+    slots = torch.arange(T, dtype=torch.int32) + 3
+    kc = torch.zeros(pages, nkv, ps, hd, dtype=dtype, device=DEV)
+    vc = torch.zeros(pages, nkv, hd, ps, dtype=dtype, device=DEV)
+    q = ops.rope_kv(qkv, kc, vc, slots.to(DEV), positions.to(DEV), inv.to(DEV), True, 1e-5, None, nh, nkv, hd,
+                    ops.PAIRS_HALF_SPLIT if layout == "half" else ops.PAIRS_INTERLEAVED)
+    x = qkv.float().cpu().view(T, nh + 2 * nkv, hd)
+    qr = P.l2_head_norm(_rotate_plain(x[:, :nh], positions, inv, layout), 1e-5)
+    kr = P.l2_head_norm(_rotate_plain(x[:, nh:nh + nkv], positions, inv, layout), 1e-5)
+    if layout == "interleaved" and rotary_dim == hd:      # the plain model's own rotation is this case
+        assert torch.allclose(_rotate_plain(x[:, :nh], positions, inv, layout), P.apply_rope_interleaved(x[:, :nh], positions, inv))
+    tol = 2e-5 if dtype == torch.float32 else 1e-2
+    assert float((q.float().cpu().view(T, nh, hd) - qr).abs().max()) <= tol * max(1.0, float(qr.abs().max()))
+    kcc = kc.float().cpu()
+    for t in range(T):
+        page, off = int(slots[t]) // ps, int(slots[t]) % ps
+        assert float((kcc[page, :, off, :] - kr[t]).abs().max()) <= tol * max(1.0, float(kr.abs().max())), t
+    # the two pairings differ (a kernel that ignored the argument would pass one of them only)
+    if rotary_dim > 2:
+        other = _rotate_plain(x[:, :nh], positions, inv, "half" if layout == "interleaved" else "interleaved")
+        assert float((other - _rotate_plain(x[:, :nh], positions, inv, layout)).abs().max()) > 0.1
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 5, 3), (70, 130, 50), (64, 64, 16), (129, 203, 96)])
 def test_gemm_tiled_is_a_true_float_product_and_batch_invariant(M, N, K):
     ops = _ops()

@@ -289,7 +289,7 @@ def test_toy_mixer_with_state_needs_no_change_to_the_framework():
     register_architecture("ToyRunningMean", ToyConfig, build, replace=True)
     try:
         eng = Engine(config=ToyConfig(), weight_seed=7, dtype="float32", kv_tokens=64, max_num_seqs=3, weight_std=0.3)
-        assert eng.cache.groups == [] and eng.cache.state[0].shape == (3, 33)
+        assert eng.cache.groups == [] and eng.cache.state[0].shape == (3 + 1, 33)      # a slot per request and the scratch slot
         a, b = H.random_tokens(40, 50, 1), H.random_tokens(25, 50, 2)
         whole_a = H.run_cut(eng, "a", a, [40])
         whole_b = H.run_cut(eng, "b", b, [25])
@@ -424,3 +424,178 @@ def test_toy_position_encoding_and_routed_feed_forward_need_no_change_to_the_fra
     finally:
         unregister_architecture("ToyLearnedPositions")
 
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_with_half_split_partial_rotary_and_scores_on_the_experts_outputs(dtype):
+    """An architecture defined here from the framework's own parts with other arguments than
+    Llama 4 gives them: rotary on half-split pairs over the first half of each head only, with its
+    own base per layer, and a softmax router with renormalised top-2 whose scores multiply the
+    experts' OUTPUTS.  No file of the framework knows of it."""
+    from sharpinference_amd.cache.spec import WINDOW_SLIDING
+    from sharpinference_amd.config.base import ModelConfig
+    from sharpinference_amd.engine import Engine
+    from sharpinference_amd.parts.attention import Attention
+    from sharpinference_amd.parts.block import PreNormBlock
+    from sharpinference_amd.parts.feedforward import MoESwiGLU
+    from sharpinference_amd.parts.model import DecoderModel
+    from sharpinference_amd.parts.norm import RMSNorm
+    from sharpinference_amd.parts.position import Rotary
+    from sharpinference_amd.registry import register_architecture, unregister_architecture
+
+    HID, NH, NKV, HD, RD, E, K, INTER, VOCAB, WIN = 128, 4, 2, 32, 16, 5, 2, 128, 70, 24
+    THETAS = (10000.0, 300.0)
+
+    @dataclass
+    class ToyConfig(ModelConfig):
+        architecture: str = "ToyHalfSplit"
+        vocab_size: int = VOCAB
+        max_position_embeddings: int = 256
+
+        @classmethod
+        def from_dict(cls, d):
+            return cls()
+
+        def to_dict(self):
+            return {"architectures": [self.architecture]}
+
+    def build(cfg):
+        blocks = []
+        for theta in THETAS:
+            att = Attention(HID, NH, NKV, HD, rotary=Rotary(HD, theta, None, pair_layout="half", rotary_dim=RD),
+                            window_kind=WINDOW_SLIDING, window=WIN)
+            ffn = MoESwiGLU(HID, E, K, INTER, shared_intermediate=None, gate="softmax", renormalise=True, score_on_input=False)
+            blocks.append(PreNormBlock(RMSNorm(HID, 1e-5), att, RMSNorm(HID, 1e-5), ffn))
+        return DecoderModel(VOCAB, HID, blocks, RMSNorm(HID, 1e-5), config=cfg)
+
+    register_architecture("ToyHalfSplit", ToyConfig, build, replace=True)
+    try:
+        eng = Engine(config=ToyConfig(), weight_seed=5, dtype=dtype, kv_tokens=256, max_num_seqs=3, weight_std=0.2)
+        a, b = H.random_tokens(60, VOCAB, 1), H.random_tokens(41, VOCAB, 2)
+        whole_a = H.run_cut(eng, "a", a, [60])
+        whole_b = H.run_cut(eng, "b", b, [41])
+        cut_tol = 1e-4 if dtype == "float32" else 0.15
+        assert float((H.run_cut(eng, "a2", a, H.last_decoded(60, 20)) - whole_a).abs().max()) <= cut_tol * float(whole_a.abs().max())
+        steps = H.mixed_trace({"a": a, "b": b, "c": H.random_tokens(9, VOCAB, 3)}, seed=3, max_live=3, tail=5)
+        got = H.replay(eng, steps)
+        assert float((got["a"] - whole_a).abs().max()) <= cut_tol * float(whole_a.abs().max())
+        assert float((got["b"] - whole_b).abs().max()) <= cut_tol * float(whole_b.abs().max())
+        if dtype != "float32":
+            return
+        # against the formulas, written out here
+        m = eng.model
+        n_tok = 60
+        pos = torch.arange(n_tok, device=DEV)
+        h = m.embed[torch.tensor(a, device=DEV)].float()
+        visible = (pos[None, :] <= pos[:, None]) & (pos[None, :] > pos[:, None] - WIN)
+        for blk, theta in zip(m.blocks, THETAS):
+            n = P.rms_norm(h, blk.norm1.weight, 1e-5)
+            att = blk.mixer
+            qkv = n @ att.w_qkv.T
+            q, k, v = (qkv[:, :NH * HD].view(n_tok, NH, HD).clone(), qkv[:, NH * HD:(NH + NKV) * HD].view(n_tok, NKV, HD).clone(),
+                       qkv[:, (NH + NKV) * HD:].view(n_tok, NKV, HD))
+            freq = torch.tensor([theta ** (-2.0 * i / RD) for i in range(RD // 2)], device=DEV, dtype=torch.float32)
+            ang = pos.float()[:, None] * freq[None, :]
+            cos, sin = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+            for t in (q, k):
+                x0, x1 = t[..., :RD // 2].clone(), t[..., RD // 2:RD].clone()
+                t[..., :RD // 2], t[..., RD // 2:RD] = x0 * cos - x1 * sin, x0 * sin + x1 * cos
+            outs = []
+            for hh in range(NH):
+                sc = (q[:, hh] @ k[:, hh // (NH // NKV)].T) / math.sqrt(HD)
+                outs.append(torch.softmax(sc.masked_fill(~visible, float("-inf")), -1) @ v[:, hh // (NH // NKV)])
+            h = h + torch.cat(outs, -1) @ att.w_o.T
+            n = P.rms_norm(h, blk.norm2.weight, 1e-5)
+            ffn = blk.ffn
+            gates = torch.softmax(n @ ffn.w_router.T.float(), -1)
+            top = gates.topk(K, dim=-1)
+            wts = top.values / top.values.sum(-1, keepdim=True)
+            y = torch.zeros_like(n)
+            for t in range(n_tok):
+                for j in range(K):
+                    e = int(top.indices[t, j])
+                    gu = ffn.w_gate_up[e] @ n[t]
+                    y[t] += wts[t, j] * (ffn.w_down[e] @ (P.silu(gu[:INTER]) * gu[INTER:]))
+            h = h + y
+        want = P.rms_norm(h, m.final_norm.weight, 1e-5) @ m.head.T
+        assert float((whole_a - want.cpu()).abs().max()) <= 1e-4 * max(1.0, float(want.abs().max()))
+    finally:
+        unregister_architecture("ToyHalfSplit")
+
+
+@pytest.mark.parametrize("graphs", [True, False])
+def test_a_stateful_mixer_that_can_be_captured_decodes_from_graphs(graphs):
+    """A mixer with state of its own that walks the entries through the context's device tensors
+    (no copy to the host) declares ``graph_safe``: its decode steps are then replayed from graphs.
+    The capture's trial run works on the scratch state slot, so no request's state moves; every
+    replay gives what the same step gives when launched part by part."""
+    from sharpinference_amd.cache.spec import StateSpec
+    from sharpinference_amd.config.base import ModelConfig
+    from sharpinference_amd.engine import Engine
+    from sharpinference_amd.parts.base import Part
+    from sharpinference_amd.parts.block import PreNormBlock
+    from sharpinference_amd.parts.feedforward import DenseSwiGLU
+    from sharpinference_amd.parts.model import DecoderModel
+    from sharpinference_amd.parts.norm import RMSNorm
+    from sharpinference_amd.registry import register_architecture, unregister_architecture
+
+    @dataclass
+    class ToyConfig(ModelConfig):
+        architecture: str = "ToyDecay"
+        vocab_size: int = 50
+        max_position_embeddings: int = 256
+
+        @classmethod
+        def from_dict(cls, d):
+            return cls()
+
+        def to_dict(self):
+            return {"architectures": [self.architecture]}
+
+    class Decay(Part):
+        """out[t] = s[t], s[t] = 0.5 * s[t-1] + x[t]: a state of fixed size per request."""
+        graph_safe = True
+
+        def cache_spec(self):
+            return StateSpec((32,), torch.float32)
+
+        def forward(self, x, ctx, cache):
+            slots = ctx.state_slots.long()                  # device tensor: no host copy
+            s = cache.state.index_select(0, slots)          # [entries, H]
+            out = torch.empty_like(x)
+            o, last = 0, []
+            for e, n in enumerate(ctx.entry_lens):          # lengths are the host's plan of the step
+                cur = s[e]
+                for t in range(n):
+                    cur = 0.5 * cur + x[o + t].float()
+                    out[o + t] = cur.to(x.dtype)
+                last.append(cur)
+                o += n
+            cache.state.index_copy_(0, slots, torch.stack(last))
+            return out
+
+    def build(cfg):
+        blocks = [PreNormBlock(RMSNorm(32, 1e-5), Decay(), RMSNorm(32, 1e-5), DenseSwiGLU(32, 48),
+                               names={"norm1": "n1.", "mixer": "mix.", "norm2": "n2.", "ffn": "ff."}) for _ in range(2)]
+        return DecoderModel(cfg.vocab_size, 32, blocks, RMSNorm(32, 1e-5), config=cfg)
+
+    register_architecture("ToyDecay", ToyConfig, build, replace=True)
+    try:
+        eng = Engine(config=ToyConfig(), weight_seed=3, dtype="float32", kv_tokens=64, max_num_seqs=3, weight_std=0.3,
+                     decode_graphs=graphs)
+        assert eng.runner.decode_graphs == graphs
+        a, b = H.random_tokens(30, 50, 1), H.random_tokens(22, 50, 2)
+        steps = [{"entries": [{"id": "a", "tokens": a[:20], "want": [19]}], "end": []},
+                 {"entries": [{"id": "b", "tokens": b[:12], "want": [11]}], "end": []}]
+        steps += [{"entries": [{"id": "a", "tokens": [a[20 + i]], "want": [0]}, {"id": "b", "tokens": [b[12 + i]], "want": [0]}],
+                   "end": []} for i in range(10)]
+        steps[-1]["end"] = ["a", "b"]
+        for i, st in enumerate(steps):
+            st["step"] = i
+        got = H.replay(eng, steps)
+        assert eng.runner.graph_replays == (10 if graphs else 0)
+        whole_a, whole_b = H.run_cut(eng, "wa", a, [30]), H.run_cut(eng, "wb", b, [22])
+        assert float((got["a"] - whole_a[19:]).abs().max()) <= 1e-5 and float((got["b"] - whole_b[11:]).abs().max()) <= 1e-5
+        assert float(eng.cache.state[0][:3].abs().max()) >= 0       # (the slots of requests; the scratch slot is the last)
+    finally:
+        unregister_architecture("ToyDecay")

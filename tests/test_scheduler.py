@@ -167,3 +167,29 @@ def test_the_penalty_window_is_the_tail_of_prompt_and_output():
         out = [rng.randrange(50) for _ in range(rng.randrange(0, 9))]
         whole = (prompt if p.penalty_seed_from_prompt else []) + out
         assert penalty_window(p, prompt, out) == (whole[-p.penalty_last_n:] if p.penalty_last_n > 0 else whole)
+
+
+def test_windowed_pools_are_bounded_by_the_window_and_admission_never_runs_dry():
+    """A windowed group's pool is made for what its windows can hold at once, (window + one step)
+    per request, however long the requests grow; admission reserves against exactly that, so a
+    running request never finds the pool empty."""
+    from sharpinference_amd.cache.manager import pool_sizes
+
+    page, window, step, n_req, length = 16, 32, 24, 5, 4000
+    specs = [KVSpec(1, 16, WINDOW_CHUNK, window), KVSpec(1, 16, WINDOW_NONE, 0)]
+    sizes = pool_sizes(specs, page, n_req, length, step)
+    assert sizes[("kv", 0, 0)] == n_req * (length // page)
+    assert sizes[("kv", 1, window)] * page <= (window + step + 2 * page) * n_req       # two pages of slack for the edges
+    assert sizes[("kv", 1, window)] < sizes[("kv", 0, 0)] // 20
+    cache = CacheManager(specs, page, sizes, n_req, allocate=False)
+    sched = Scheduler(cache, max_num_seqs=n_req, max_tokens_per_step=step, max_model_len=length)
+    reqs = [_req(i, 300 + 37 * i, 150) for i in range(n_req + 2)]
+    for r in reqs:
+        sched.add(r)
+    batches = _run(sched, lambda r: 1)            # _run asserts that no append of a running request fails
+    assert all(r.finish_reason == "length" and len(r.output) == 150 for r in reqs)
+    assert max(len(b) for b in batches) == n_req
+    assert all(g.pool.num_free == g.pool.num_pages for g in cache.groups)
+    # a budget in pages caps the unwindowed group only when it is the smaller
+    capped = pool_sizes(specs, page, n_req, length, step, budget_pages=100)
+    assert capped[("kv", 0, 0)] == 100 and capped[("kv", 1, window)] == sizes[("kv", 1, window)]
