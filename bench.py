@@ -5,7 +5,12 @@
 
 A step is one decode step of a batch of B requests, each with a 2,048-token prompt already in
 the cache.  Prints ONE JSON line: decoded tokens per second at the default batch, the prefill of
-one 2,048-token prompt, the decode step's HBM roofline, and decode at batch 1 and 64.
+one 2,048-token prompt, the decode step's HBM roofline, and decode at batch 1 and 64 (with the
+roofline fraction of each point), beside the peaks two measuring kernels of the library reach on
+this GPU.  ``--profile`` adds, on stderr, milliseconds / bytes / GB/s per kernel class of one
+prefill and one decode step, from event pairs.  ``--shape maverick8`` and ``--shape long16`` run
+two other workloads instead (128 experts alternating with dense layers at batch 64; 32,768-token
+prompts read in 4,096-token portions beside decoding requests) and print a JSON line of their own.
 """
 from __future__ import annotations
 
@@ -45,10 +50,11 @@ def log(msg: str) -> None:
 
 
 def build_engine(layers: int, max_batch: int, page_size: int, graphs: bool = True, gen_len: int = GEN_LEN,
-                 prompt_len: int = PROMPT_LEN):
+                 prompt_len: int = PROMPT_LEN, overrides: dict = None, max_tokens_per_step: int = 8192, **engine_kw):
     from sharpinference_amd.engine import Engine
 
     cfg = dict(SCOUT)
+    cfg.update(overrides or {})
     cfg["num_hidden_layers"] = layers
     cfg["no_rope_layers"] = [0 if (l + 1) % 4 == 0 else 1 for l in range(layers)]
     per_req = (prompt_len + gen_len + page_size - 1) // page_size * page_size
@@ -56,8 +62,8 @@ def build_engine(layers: int, max_batch: int, page_size: int, graphs: bool = Tru
     cfg["max_position_embeddings"] = context
     t0 = time.time()
     eng = Engine(config=cfg, weight_seed=2, dtype="bfloat16", device="cuda:0", max_model_len=context,
-                 max_num_seqs=max_batch, max_tokens_per_step=8192, kv_tokens=max_batch * per_req,
-                 page_size=page_size, decode_graphs=graphs)
+                 max_num_seqs=max_batch, max_tokens_per_step=max_tokens_per_step, kv_tokens=max_batch * per_req,
+                 page_size=page_size, decode_graphs=graphs, **engine_kw)
     log(f"engine with {layers} layers ready in {time.time() - t0:.1f}s")
     return eng
 
@@ -68,11 +74,24 @@ def layer_bytes(cfg) -> dict:
     q, kv = cfg.num_attention_heads * hd, cfg.num_key_value_heads * hd
     attn = 2 * ((q + 2 * kv) * H + H * q)
     expert = 2 * 3 * H * cfg.intermediate_size
+    dense = 2 * 3 * H * cfg.intermediate_size_mlp
     router = 2 * cfg.num_local_experts * H
     norms = 2 * 2 * H
     head = 2 * cfg.vocab_size * H
-    return {"attn": attn, "expert": expert, "router": router, "norms": norms, "head": head,
+    return {"attn": attn, "expert": expert, "dense": dense, "router": router, "norms": norms, "head": head,
             "kv_per_token": 2 * 2 * kv}
+
+
+def decode_step_bytes(cfg, layers: int, batch: int, context: int, distinct: float) -> float:
+    """Bytes one decode step has to read: every weight it uses once (the shared expert and
+    `distinct` routed experts on a routed layer, the dense feed-forward on the others) and the
+    cache of the live requests (what each layer's window lets the query at `context - 1` see)."""
+    b = layer_bytes(cfg)
+    total = b["head"]
+    for l in range(layers):
+        ffn = b["router"] + b["expert"] * (1 + distinct) if cfg.is_moe_layer(l) else b["dense"]
+        total += b["attn"] + b["norms"] + ffn + batch * b["kv_per_token"] * visible_keys(cfg, l, context - 1)
+    return total
 
 
 def visible_keys(cfg, layer: int, position: int) -> int:
@@ -85,13 +104,25 @@ def visible_keys(cfg, layer: int, position: int) -> int:
 def prefill_flops(cfg, T: int, layers: int) -> float:
     H, hd = cfg.hidden_size, cfg.head_dim
     q, kv = cfg.num_attention_heads * hd, cfg.num_key_value_heads * hd
-    lin = (q + 2 * kv) * H + H * q + cfg.num_local_experts * H + 2 * 3 * H * cfg.intermediate_size
+    attn_lin = (q + 2 * kv) * H + H * q
+    moe = cfg.num_local_experts * H + 2 * 3 * H * cfg.intermediate_size       # router, one routed expert, the shared one
+    dense = 3 * H * cfg.intermediate_size_mlp
+    lin = sum(attn_lin + (moe if cfg.is_moe_layer(l) else dense) for l in range(layers))
     C = cfg.attention_chunk_size
     whole, rest = divmod(T, C)
     pairs_chunked = whole * (C * (C + 1) / 2) + rest * (rest + 1) / 2       # (query, key) pairs, causal inside a chunk
     pairs = sum(T * (T + 1) / 2 if cfg.no_rope_layers[l] == 0 else pairs_chunked for l in range(layers))
     attn = 2 * 2 * cfg.num_attention_heads * hd * pairs                     # QK^T and PV
-    return layers * 2.0 * T * lin + attn + 2.0 * cfg.vocab_size * H        # one row through the head
+    return 2.0 * T * lin + attn + 2.0 * cfg.vocab_size * H                 # one row through the head
+
+
+def prefill_bytes(cfg, layers: int) -> float:
+    """Weights a prompt of thousands of tokens has to read once: every expert of every routed layer."""
+    b = layer_bytes(cfg)
+    total = b["head"]
+    for l in range(layers):
+        total += b["attn"] + b["norms"] + (b["router"] + b["expert"] * (1 + cfg.num_local_experts) if cfg.is_moe_layer(l) else b["dense"])
+    return total
 
 
 def run_prefill(eng, rid, prompt):
@@ -128,8 +159,9 @@ def decode_run(eng, batch: int, steps: int, warmup: int, rng: random.Random, cou
         log(f"  prefilled {min(i + per_step, batch)}/{batch}")
 
     def one_step(tokens, trace=None):
-        lg = eng.step([StepEntry(r, (t,), (0,)) for r, t in zip(ids, tokens)], router_trace=trace)
-        return ops.argmax_rows(lg).cpu().tolist()
+        # greedy decoding as the engine serves it: the choice is made on the device behind the head
+        return eng.step([StepEntry(r, (t,), (0,)) for r, t in zip(ids, tokens)], router_trace=trace,
+                        select="argmax").cpu().tolist()
 
     for _ in range(warmup):
         last = one_step(last)
@@ -150,6 +182,156 @@ def decode_run(eng, batch: int, steps: int, warmup: int, rng: random.Random, cou
     return dt, distinct, ctx
 
 
+def profile_report(eng, batch: int, prompt_len: int, rng: random.Random) -> None:
+    """ms / bytes / GB/s / TFLOP/s per kernel class of one prefill and one decode step (stderr)."""
+    from sharpinference_amd.engine import StepEntry
+    from sharpinference_amd.ops.profile import Profiler, format_table
+
+    vocab = eng.config.vocab_size
+    ids = [f"prof{i}" for i in range(batch)]
+    prof = Profiler()
+    for n, r in enumerate(ids):
+        eng.add_request(r)
+        entry = [StepEntry(r, [rng.randrange(vocab) for _ in range(prompt_len)], (prompt_len - 1,))]
+        if n == 0:
+            eng.profiled_step(entry, prof)
+        else:
+            eng.step(entry)
+    log("\n" + format_table(prof.table(), f"prefill of one prompt of {prompt_len} tokens, by kernel class (event pairs):"))
+    decode = [StepEntry(r, (rng.randrange(vocab),), (0,)) for r in ids]
+    eng.step(decode, select="argmax")                       # warm
+    prof = Profiler()
+    decode = [StepEntry(r, (rng.randrange(vocab),), (0,)) for r in ids]
+    eng.profiled_step(decode, prof, select="argmax", filler_ms=40.0)
+    log("\n" + format_table(prof.table(), f"one decode step at batch {batch}, contexts of {prompt_len + 2} tokens, launched part by "
+                                          "part behind filler work, by kernel class (event pairs):"))
+    for r in ids:
+        eng.free_request(r)
+
+
+def run_maverick8(args) -> int:
+    """Eight Maverick-shaped layers: dense feed-forward (16,384) alternating with 128 experts
+    top-1 + shared, no rotary scaling, no QK norm; router weights drawn so that router logits are
+    about N(0, 1) and the experts' load is uneven.  Batch 64 of 1,024-token prompts, 128 decode steps."""
+    import torch
+    from sharpinference_amd.engine import StepEntry
+
+    layers, batch, P, steps, warm = 8, 64, 1024, args.steps if args.steps != GEN_LEN - 8 else 120, 8
+    over = {"num_local_experts": 128, "interleave_moe_layer_step": 2, "rope_scaling": None, "use_qk_norm": False}
+    eng = build_engine(layers, batch, args.page_size, gen_len=steps + warm + 2, prompt_len=P, overrides=over,
+                       weight_std_by_suffix={"router.weight": 5120 ** -0.5})
+    cfg = eng.config
+    rng = random.Random(3)
+    prompt = [rng.randrange(cfg.vocab_size) for _ in range(P)]
+    run_prefill(eng, "warm", prompt)
+    eng.free_request("warm")
+    eng.add_request("load")
+    trace: list = []
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    eng.step([StepEntry("load", prompt, (P - 1,))], router_trace=trace)
+    torch.cuda.synchronize()
+    pre_s = time.perf_counter() - t0
+    eng.free_request("load")
+    hist = torch.bincount(trace[0][0].flatten().long().cpu(), minlength=cfg.num_local_experts).tolist()
+    log(f"prefill {P} tokens: {pre_s * 1e3:.1f} ms; tokens per expert in the first routed layer: min {min(hist)}, "
+        f"median {sorted(hist)[len(hist) // 2]}, max {max(hist)}, unused {hist.count(0)} of {len(hist)}")
+    dt, distinct, ctx = decode_run(eng, batch, steps, warm, rng, count_experts=True, prompt_len=P)
+    ms_step = dt / steps * 1e3
+    step_bytes = decode_step_bytes(cfg, layers, batch, ctx, distinct)
+    achieved = step_bytes / (ms_step * 1e-3) / 1e9
+    log(f"decode b{batch}: {ms_step:.2f} ms/step, {batch * steps / dt:.1f} tok/s, {achieved:.0f} GB/s ({distinct:.1f} experts per routed layer)")
+    out = {"metric": "decode tok/s at batch 64 (8 Maverick-shaped layers, 1,024-token prompts)", "value": batch * steps / dt,
+           "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warm, "ms_per_step": ms_step, "higher_is_better": True,
+           "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+           "config": {"model": "llama4-maverick-shaped-random", "global_batch": batch, "seq_len": eng.max_model_len,
+                      "parallelism": "single-gpu", "layers": layers, "layers_of_full_model": 48, "hidden_size": cfg.hidden_size,
+                      "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
+                      "experts": cfg.num_local_experts, "moe_every": cfg.interleave_moe_layer_step,
+                      "expert_ffn": cfg.intermediate_size, "dense_ffn": cfg.intermediate_size_mlp, "vocab": cfg.vocab_size,
+                      "prompt_len": P, "generated": steps + warm, "page_size": args.page_size},
+           "prefill": {"value": P / pre_s, "tokens": P, "ms": pre_s * 1e3,
+                       "frac": prefill_flops(cfg, P, layers) / pre_s / (PEAK_DENSE_TFLOPS["bf16"] * 1e12)},
+           "roofline": {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": achieved / PEAK_HBM_GBS},
+           "expert_load": {"min": min(hist), "median": sorted(hist)[len(hist) // 2], "max": max(hist), "unused": hist.count(0),
+                           "distinct_per_decode_step": distinct}}
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+def run_long16(args) -> int:
+    """Sixteen Scout-shaped layers, 8 prompts of 32,768 tokens read in portions of 4,096 beside the
+    decoded tokens of the requests that are already through (the scheduler mixes them), then
+    decoding alone; 512 generated tokens a request.  Four chunk edges of 8,192 are crossed, the
+    windowed layers give pages back behind them, and the query temperature works at long positions."""
+    import torch
+    from sharpinference_amd.engine import StepEntry
+    from sharpinference_amd.engine.scheduler import Request, Scheduler
+    from sharpinference_amd.sampling.params import SamplingParams
+
+    layers, batch, P, portion = 16, 8, 32768, 4096
+    gen = args.steps if args.steps != GEN_LEN - 8 else 512
+    eng = build_engine(layers, batch, args.page_size, gen_len=gen + 8, prompt_len=P, max_tokens_per_step=portion + batch)
+    cfg = eng.config
+    rng = random.Random(4)
+    sched = Scheduler(eng.cache, batch, portion + batch, eng.max_model_len)
+    reqs = [Request(("long", i), [rng.randrange(cfg.vocab_size) for _ in range(P)],
+                    SamplingParams(temperature=0.0, max_new_tokens=gen, stop_token_ids=())) for i in range(batch)]
+    for r in reqs:
+        sched.add(r)
+    phases = {"mixed": [0.0, 0, 0, 0], "decode": [0.0, 0, 0, 0]}        # seconds, steps, prompt tokens, decoded tokens
+    pools = {g.key: g.pool.num_pages for g in eng.cache.groups}
+    distinct = None
+    while sched.has_work():
+        b = sched.schedule()
+        if not b:
+            break
+        entries = [StepEntry(s.request.req_id, s.tokens, (len(s.tokens) - 1,) if s.samples else ()) for s in b]
+        n_prompt = sum(len(s.tokens) for s in b if s.request.in_prefill)
+        n_dec = sum(1 for s in b if not s.request.in_prefill)
+        trace = [] if (not n_prompt and distinct is None) else None   # the first step of decoding alone says how many experts a step uses
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        picked = eng.step(entries, select="argmax", router_trace=trace)
+        picked = picked.cpu().tolist() if picked is not None else []
+        dt = time.perf_counter() - t0
+        if trace:
+            distinct = sum(len(set(p.flatten().cpu().tolist())) for p, _, _ in trace) / len(trace)
+        it = iter(picked)
+        sched.update(b, [next(it) if s.samples else None for s in b])
+        ph = phases["mixed" if n_prompt else "decode"]
+        ph[0] += dt; ph[1] += 1; ph[2] += n_prompt; ph[3] += n_dec
+        if ph[1] % 64 == 0:
+            log(f"  {ph[1]} {'mixed' if n_prompt else 'decode'} steps")
+    mixed, dec = phases["mixed"], phases["decode"]
+    assert all(r.finish_reason == "length" and len(r.output) == gen for r in reqs)
+    ms_step = dec[0] / max(1, dec[1]) * 1e3
+    ctx = P + gen
+    # bytes of a decode step in the middle of the decoding phase
+    from_trace = distinct if distinct is not None else 0.0
+    step_bytes = decode_step_bytes(cfg, layers, dec[3] / max(1, dec[1]), ctx - gen // 2, from_trace)
+    achieved = step_bytes / (ms_step * 1e-3) / 1e9
+    log(f"mixed phase: {mixed[1]} steps, {mixed[2]} prompt tokens beside {mixed[3]} decoded tokens in {mixed[0]:.2f} s "
+        f"({mixed[2] / mixed[0]:.0f} prompt tok/s); decode alone: {dec[1]} steps, {dec[3] / dec[0]:.1f} tok/s, {ms_step:.2f} ms/step")
+    out = {"metric": "decode tok/s at batch 8 after 32,768-token prompts (16 Scout-shaped layers)", "value": dec[3] / dec[0],
+           "unit": "tok/s", "n_gpus": 1, "steps": dec[1], "warmup": 0, "ms_per_step": ms_step, "higher_is_better": True,
+           "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+           "config": {"model": "llama4-scout-shaped-random", "global_batch": batch, "seq_len": eng.max_model_len,
+                      "parallelism": "single-gpu", "layers": layers, "layers_of_full_model": FULL_LAYERS,
+                      "hidden_size": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
+                      "head_dim": cfg.head_dim, "experts": cfg.num_local_experts, "expert_ffn": cfg.intermediate_size,
+                      "vocab": cfg.vocab_size, "attention_chunk": cfg.attention_chunk_size, "prompt_len": P,
+                      "portion": portion, "generated": gen, "page_size": args.page_size},
+           "prefill": {"value": mixed[2] / mixed[0], "tokens": mixed[2], "ms": mixed[0] * 1e3,
+                       "frac": batch * prefill_flops(cfg, P, layers) / mixed[0] / (PEAK_DENSE_TFLOPS["bf16"] * 1e12),
+                       "steps": mixed[1], "decoded_beside": mixed[3]},
+           "roofline": {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": achieved / PEAK_HBM_GBS,
+                        "experts_per_step": from_trace},
+           "pools": {f"window_{k[1]}_{k[2]}": v for k, v in pools.items()}}
+    print(json.dumps(out), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -161,10 +343,18 @@ def main() -> int:
     ap.add_argument("--prompt-len", type=int, default=PROMPT_LEN, help="tokens of every prompt (the contract's run: 2,048)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 points")
     ap.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel instead of replaying a HIP graph")
+    ap.add_argument("--no-peaks", action="store_true", help="skip the two measuring kernels (pure read, matrix-core loop)")
+    ap.add_argument("--profile", action="store_true", help="also print ms / bytes / GB/s per kernel class of one prefill and one decode step")
+    ap.add_argument("--shape", default="scout", choices=["scout", "maverick8", "long16"],
+                    help="scout: the headline run; maverick8 / long16: two other workloads, each printing a JSON line of its own")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this engine has no multi-GPU path (N=1 only)")
         return 2
+    if args.shape == "maverick8":
+        return run_maverick8(args)
+    if args.shape == "long16":
+        return run_long16(args)
 
     import torch  # noqa: F401
 
@@ -174,6 +364,13 @@ def main() -> int:
     P = args.prompt_len
     eng = build_engine(args.layers, max_batch, args.page_size, graphs=not args.no_graphs, gen_len=gen_len, prompt_len=P)
     cfg = eng.config
+    measured = None
+    if not args.no_peaks:
+        from sharpinference_amd import ops
+
+        measured = ops.measured_peaks("cuda:0", read_bytes=2 << 30)
+        log(f"measured on this GPU: pure read {measured['hbm_gbs']:.0f} GB/s (published {PEAK_HBM_GBS:.0f}), "
+            f"matrix-core loop {measured['bf16_tflops']:.0f} TFLOP/s bf16 (published {PEAK_DENSE_TFLOPS['bf16']:.0f})")
 
     # prefill: one prompt (2,048 tokens) alone, once to warm up, then three times timed
     prompt = [rng.randrange(cfg.vocab_size) for _ in range(P)]
@@ -188,26 +385,29 @@ def main() -> int:
     log(f"prefill {P} tokens: {pre_s * 1e3:.1f} ms")
     flops = prefill_flops(cfg, P, args.layers)
     prefill = {"value": P / pre_s, "tokens": P, "ms": pre_s * 1e3,
-               "frac": flops / pre_s / (PEAK_DENSE_TFLOPS["bf16"] * 1e12)}
+               "frac": flops / pre_s / (PEAK_DENSE_TFLOPS["bf16"] * 1e12),
+               "hbm_frac": prefill_bytes(cfg, args.layers) / pre_s / 1e9 / PEAK_HBM_GBS}
 
     dt, distinct, ctx = decode_run(eng, args.batch, args.steps, args.warmup, rng, count_experts=True, prompt_len=P)
     ms_step = dt / args.steps * 1e3
     value = args.batch * args.steps / dt
-    b = layer_bytes(cfg)
-    shared_and_routed = b["expert"] * (1 + distinct)
-    step_bytes = args.layers * (b["attn"] + b["router"] + b["norms"] + shared_and_routed) + b["head"] \
-        + args.batch * b["kv_per_token"] * sum(visible_keys(cfg, l, ctx - 1) for l in range(args.layers))
+    step_bytes = decode_step_bytes(cfg, args.layers, args.batch, ctx, distinct)
     achieved = step_bytes / (ms_step * 1e-3) / 1e9
     log(f"decode b{args.batch}: {ms_step:.2f} ms/step, {value:.1f} tok/s, {achieved:.0f} GB/s "
         f"({distinct:.2f} experts per layer)")
 
-    points = {}
+    points, points_roofline = {}, {}
     if not args.no_points:
         for pb in (1, 64):
             k = max(8, args.steps // 2)
-            pdt, _, _ = decode_run(eng, pb, k, max(2, args.warmup // 2), rng, prompt_len=P)
+            pdt, pdist, pctx = decode_run(eng, pb, k, max(2, args.warmup // 2), rng, count_experts=True, prompt_len=P)
             points[f"decode_b{pb}"] = pb * k / pdt
-            log(f"decode b{pb}: {pdt / k * 1e3:.2f} ms/step, {points[f'decode_b{pb}']:.1f} tok/s")
+            gbs = decode_step_bytes(cfg, args.layers, pb, pctx, pdist) / (pdt / k) / 1e9
+            points_roofline[f"decode_b{pb}"] = gbs / PEAK_HBM_GBS
+            log(f"decode b{pb}: {pdt / k * 1e3:.2f} ms/step, {points[f'decode_b{pb}']:.1f} tok/s, {gbs:.0f} GB/s "
+                f"({gbs / PEAK_HBM_GBS:.3f} of the roofline; {pdist:.2f} experts per layer)")
+    if args.profile:
+        profile_report(eng, args.batch, P, rng)
 
     out = {
         "metric": f"decode tok/s at batch {args.batch} (Scout-shaped, {P:,}-token prompts)",
@@ -227,7 +427,11 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": achieved / PEAK_HBM_GBS},
         "points": points,
+        "points_roofline": points_roofline,
     }
+    if measured is not None:
+        out["measured_peaks"] = {"hbm_gbs": measured["hbm_gbs"], "bf16_tflops": measured["bf16_tflops"],
+                                 "roofline_frac_of_measured": achieved / measured["hbm_gbs"]}
     print(json.dumps(out), flush=True)
     return 0
 

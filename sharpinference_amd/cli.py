@@ -14,6 +14,15 @@ token ids, and ``--prompt-len N`` makes N random ids.  Generation stops at the c
 ``eos_token_id`` (``--ignore-eos`` switches that off; ``--stop-ids`` adds more).  ``-m`` names
 a model folder (config.json + model.safetensors); with ``--random-weights`` the folder needs
 only config.json.
+
+Text prompts are put into the Llama 4 chat form (RunCommand.cs:2588-2596) when the folder's
+tokenizer knows the form's marks, ``--system-prompt`` adds the system message of that form, and
+``--raw-prompt`` leaves the text as it is.  Without any prompt option the command reads prompts
+from standard input, one a line, until ``/exit``, ``/quit`` or the end of input (the reference's
+interactive mode, RunCommand.cs:2185-2226: every turn starts from an empty cache); ``--single-turn``
+ends after the first.  ``--profile`` launches every step part by part and prints milliseconds,
+bytes and GB/s per kernel class at the end (the reference's SHARPI_CUDA_PROFILE buckets,
+src/SharpInference.Engine/CudaForwardPass.cs:1523-1539).
 """
 from __future__ import annotations
 
@@ -33,13 +42,20 @@ def _ids(text: str) -> List[int]:
         raise SystemExit(f"token ids expected (comma or space separated numbers), got {text[:40]!r}") from None
 
 
-def prompt_ids(text: str, codec) -> List[int]:
+def prompt_ids(text: str, codec, system: Optional[str] = None, raw: bool = False) -> List[int]:
     """A prompt from the command line: numbers are token ids; anything else is text for the
-    folder's tokenizer."""
+    folder's tokenizer, in the chat form if the tokenizer knows its marks (and `raw` is not set)."""
     if re.fullmatch(r"[\d,\s]+", text) and re.search(r"\d", text):
+        if system is not None:
+            raise SystemExit("--system-prompt belongs to text prompts: token ids are taken as they are")
         return _ids(text)
     if codec is None:
         raise SystemExit("the model folder has no tokenizer.json: give the prompt as token ids, e.g. -p '1,2,3'")
+    if not raw and codec.knows_chat_marks():
+        return codec.encode_chat(text, system)
+    if system is not None:
+        raise SystemExit("--system-prompt needs the chat form, whose marks this folder's tokenizer does not know"
+                         if not raw else "--system-prompt and --raw-prompt contradict each other")
     return codec.encode(text)
 
 
@@ -79,6 +95,10 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--presence-penalty", type=float, default=0.0)
     ap.add_argument("--verbose-prompt", action="store_true", help="print the prompt's token ids")
     ap.add_argument("--no-display-prompt", action="store_true")
+    ap.add_argument("--single-turn", action="store_true", help="interactive mode: generate one response and exit")
+    ap.add_argument("--system-prompt", default=None, help="system message of the chat form (text prompts)")
+    ap.add_argument("--raw-prompt", action="store_true", help="text prompts as they are, without the chat form")
+    ap.add_argument("--profile", action="store_true", help="launch steps part by part and print ms / bytes / GB/s per kernel class")
     ap.add_argument("--stop-ids", default="", help="token ids that end generation, beside the model's eos_token_id")
     ap.add_argument("--ignore-eos", action="store_true", help="do not stop at the model's eos_token_id")
     ap.add_argument("-g", "--ngl", "--n-gpu-layers", "--gpu-layers", dest="n_gpu_layers", type=int, default=-1,
@@ -112,55 +132,103 @@ def main(argv: Optional[List[str]] = None) -> int:
     cfg = load_config(args.model)
     from .text import TextCodec
     codec = TextCodec.from_folder(args.model, cfg.bos_token_id)
+    def text_prompt(text):
+        return prompt_ids(text, codec, args.system_prompt, args.raw_prompt)
+
+    interactive = False
     if args.file:
         with open(args.file) as f:
-            prompt = prompt_ids(f.read(), codec)
+            prompt = text_prompt(f.read())
     elif args.prompt_ids:
         prompt = _ids(args.prompt_ids)
     elif args.prompt:
-        prompt = prompt_ids(args.prompt, codec)
+        prompt = text_prompt(args.prompt)
     elif args.prompt_len:
         rng = random.Random(args.weight_seed)
         prompt = [rng.randrange(cfg.vocab_size) for _ in range(args.prompt_len)]
     else:
-        raise SystemExit("no prompt: give -p / --prompt-ids / -f / --prompt-len (there is no interactive mode)")
+        interactive, prompt = True, None
     ctx = args.ctx_size or None
     common = dict(dtype=dtype, device=device, max_model_len=ctx, max_num_seqs=max(args.max_num_seqs, args.parallel),
-                  max_tokens_per_step=args.max_tokens_per_step, kv_tokens=args.kv_tokens, page_size=args.page_size)
+                  max_tokens_per_step=args.max_tokens_per_step, kv_tokens=args.kv_tokens, page_size=args.page_size,
+                  decode_graphs=not args.profile)
     if args.random_weights:
         eng = Engine(config=cfg, weight_seed=args.weight_seed, **common)
     else:
         eng = Engine(args.model, **common)
     seed = args.seed if args.seed >= 0 else int(time.time() * 1000) & 0x7FFFFFFF
-    params = [SamplingParams(temperature=args.temp, top_k=args.top_k, top_p=args.top_p, min_p=args.min_p,
-                             repetition_penalty=args.repeat_penalty, penalty_last_n=args.repeat_last_n,
-                             frequency_penalty=args.frequency_penalty, presence_penalty=args.presence_penalty,
-                             max_new_tokens=args.n_predict, stop_token_ids=() if args.ignore_eos else None,
-                             additional_stop_token_ids=tuple(_ids(args.stop_ids)) if args.stop_ids else (),
-                             seed=seed + i) for i in range(args.parallel)]
-    if args.verbose_prompt:
-        print(f"prompt tokens ({len(prompt)}): {prompt}")
-    elif not args.no_display_prompt:
-        print(codec.decode(prompt) if codec else " ".join(str(t) for t in prompt))
-    if args.parallel == 1:
-        # one request: its tokens are printed as they come (the reference streams its chunks the same way)
+
+    def sampling(turn: int):
+        return [SamplingParams(temperature=args.temp, top_k=args.top_k, top_p=args.top_p, min_p=args.min_p,
+                               repetition_penalty=args.repeat_penalty, penalty_last_n=args.repeat_last_n,
+                               frequency_penalty=args.frequency_penalty, presence_penalty=args.presence_penalty,
+                               max_new_tokens=args.n_predict, stop_token_ids=() if args.ignore_eos else None,
+                               additional_stop_token_ids=tuple(_ids(args.stop_ids)) if args.stop_ids else (),
+                               seed=seed + turn * args.parallel + i) for i in range(args.parallel)]
+
+    profiler = None
+    if args.profile:
+        from .ops.profile import Profiler
+
+        profiler = Profiler()
+        profiler.__enter__()
+
+    def stream_one(ids: List[int], params) -> None:
+        """One request: its tokens are printed as they come (the reference streams its chunks the same way)."""
         first = True
         stream = codec.streamer() if codec else None
-        for c in eng.generate_chunks([prompt], params):
+        for c in eng.generate_chunks([ids], params):
             if c.kind == "token":
                 piece = stream.push(c.token_id) if stream else ("" if first else " ") + str(c.token_id)
                 print(piece, end="", flush=True)
                 first = False
             elif c.kind == "stop":
                 print((stream.flush() if stream else "") + f"  ({c.finish_reason})", flush=True)
-    else:
-        for i, r in enumerate(eng.generate([prompt] * args.parallel, params)):
-            shown = codec.decode(r.token_ids) if codec else " ".join(str(t) for t in r.token_ids)
-            print(f"[{i}] {shown}  ({r.finish_reason})")
-    st = eng.last_stats
-    pre = st.prefill_tokens / st.prefill_seconds if st.prefill_seconds > 0 else 0.0
-    dec = st.decode_tokens / st.decode_seconds if st.decode_seconds > 0 else 0.0
-    print(f"Prefill: {st.prefill_tokens} tokens, {pre:.1f} t/s | Decode: {st.decode_tokens} tokens, {dec:.1f} t/s")
+
+    try:
+        if interactive:
+            # the reference's interactive chat (RunCommand.cs:2185-2226): a line a turn, every turn from an empty cache
+            print("Interactive mode: a prompt a line (text, or token ids); /exit to quit.", flush=True)
+            turn = 0
+            while True:
+                print("> ", end="", flush=True)
+                line = sys.stdin.readline()
+                if not line or line.strip() in ("/exit", "/quit"):
+                    break
+                if not line.strip():
+                    continue
+                ids = text_prompt(line.strip())
+                if args.verbose_prompt:
+                    print(f"prompt tokens ({len(ids)}): {ids}")
+                stream_one(ids, sampling(turn)[:1])
+                st = eng.last_stats
+                rate = st.decode_tokens / st.decode_seconds if st.decode_seconds > 0 else 0.0
+                print(f"{st.decode_tokens + 1} tokens, {rate:.1f} t/s\n", flush=True)
+                turn += 1
+                if args.single_turn:
+                    break
+        else:
+            if args.verbose_prompt:
+                print(f"prompt tokens ({len(prompt)}): {prompt}")
+            elif not args.no_display_prompt:
+                print(codec.decode(prompt) if codec else " ".join(str(t) for t in prompt))
+            if args.parallel == 1:
+                stream_one(prompt, sampling(0))
+            else:
+                for i, r in enumerate(eng.generate([prompt] * args.parallel, sampling(0))):
+                    shown = codec.decode(r.token_ids) if codec else " ".join(str(t) for t in r.token_ids)
+                    print(f"[{i}] {shown}  ({r.finish_reason})")
+            st = eng.last_stats
+            pre = st.prefill_tokens / st.prefill_seconds if st.prefill_seconds > 0 else 0.0
+            dec = st.decode_tokens / st.decode_seconds if st.decode_seconds > 0 else 0.0
+            print(f"Prefill: {st.prefill_tokens} tokens, {pre:.1f} t/s | Decode: {st.decode_tokens} tokens, {dec:.1f} t/s")
+    finally:
+        if profiler is not None:
+            from .ops.profile import format_table
+
+            profiler.__exit__(None, None, None)
+            print(format_table(profiler.table(), "all steps of this run, launched part by part, by kernel class (event pairs):"),
+                  file=sys.stderr, flush=True)
     return 0
 
 

@@ -143,8 +143,21 @@ class Engine:
     def free_request(self, req_id: Hashable) -> None:
         self.cache.free_request(req_id)
 
-    def step(self, entries: Sequence[StepEntry], router_trace: Optional[list] = None) -> Optional[torch.Tensor]:
-        return self.runner.step(entries, router_trace)
+    def step(self, entries: Sequence[StepEntry], router_trace: Optional[list] = None,
+             select: Optional[str] = None) -> Optional[torch.Tensor]:
+        return self.runner.step(entries, router_trace, select)
+
+    def profiled_step(self, entries: Sequence[StepEntry], profiler, select: Optional[str] = None,
+                      filler_ms: float = 0.0) -> Optional[torch.Tensor]:
+        """One step launched part by part with `profiler` (ops.profile.Profiler) active: its table
+        then holds milliseconds, bytes and flops per kernel class.  `filler_ms` of filler work is
+        queued first, so that the host's launch latency does not land inside the spans of short
+        kernels (wanted for decode steps)."""
+        graphs, self.runner.decode_graphs = self.runner.decode_graphs, False
+        try:
+            return profiler.run(lambda: self.runner.step(entries, select=select), filler_ms, self.device)
+        finally:
+            self.runner.decode_graphs = graphs
 
     # -- generation -------------------------------------------------------------
     def _sampling_params(self, n: int, params, max_new_tokens, temperature, seeds, stop_token_ids) -> List[SamplingParams]:
@@ -217,14 +230,21 @@ class Engine:
                     t0 = time.perf_counter()
                     entries = [StepEntry(s.request.req_id, s.tokens, (len(s.tokens) - 1,) if s.samples else ())
                                for s in batch]
-                    logits = self.runner.step(entries)
                     sampling = [s for s in batch if s.samples]
                     tokens: List[Optional[int]] = [None] * len(batch)
+                    if sampling and all(s.request.params.greedy for s in sampling):
+                        # every row greedy: the choice is made on the device behind the head, and only
+                        # the token ids come back (reference: ContinuousBatchingEngine.cs:332-347)
+                        picked = self.runner.step(entries, select="argmax").cpu().tolist()
+                    else:
+                        logits = self.runner.step(entries)
+                        picked = []
+                        if sampling:
+                            hist = [penalty_window(s.request.params, s.request.prompt, s.request.output)
+                                    if s.request.params.edits_logits else () for s in sampling]
+                            picked = self.sampler.sample(logits, [s.request.params for s in sampling],
+                                                         [s.request.draws for s in sampling], hist)
                     if sampling:
-                        hist = [penalty_window(s.request.params, s.request.prompt, s.request.output)
-                                if s.request.params.edits_logits else () for s in sampling]
-                        picked = self.sampler.sample(logits, [s.request.params for s in sampling],
-                                                     [s.request.draws for s in sampling], hist)
                         it = iter(picked)
                         tokens = [next(it) if s.samples else None for s in batch]
                     dt = time.perf_counter() - t0

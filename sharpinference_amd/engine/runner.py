@@ -175,7 +175,8 @@ class ModelRunner:
         return out
 
     # ------------------------------------------------------------------
-    def _decode_graph_step(self, entries: Sequence[StepEntry], router_trace: Optional[list] = None) -> Optional[torch.Tensor]:
+    def _decode_graph_step(self, entries: Sequence[StepEntry], router_trace: Optional[list] = None,
+                           select: Optional[str] = None) -> Optional[torch.Tensor]:
         """Replay the captured graph of this batch size if the step qualifies: every entry one
         token whose logits are wanted, all contexts within the captured bound.  None otherwise."""
         n = len(entries)
@@ -194,7 +195,7 @@ class ModelRunner:
         while bound < longest:
             bound *= 4
         bound = min(bound, self.max_context)
-        key = (n, bound)
+        key = (n, bound) if select is None else (n, bound, select)
         graph = self._graphs.get(key)
         if graph is False:
             return None
@@ -202,7 +203,7 @@ class ModelRunner:
         pieces, info = self._host_arrays(entries, static_blocks=static_blocks)
         if graph is None:
             try:
-                graph = _DecodeGraph(self, pieces, info, bound)
+                graph = _DecodeGraph(self, pieces, info, bound, select)
             except Exception as e:  # noqa: BLE001 - capture is an optimisation: report once, go on eagerly
                 print(f"[sharpi] decode graph for batch {n}, contexts to {bound} not captured ({type(e).__name__}: {e}); "
                       "running eagerly", file=sys.stderr, flush=True)
@@ -212,9 +213,12 @@ class ModelRunner:
         self.graph_replays += 1
         return graph.replay(pieces, router_trace)
 
-    def step(self, entries: Sequence[StepEntry], router_trace: Optional[list] = None) -> Optional[torch.Tensor]:
+    def step(self, entries: Sequence[StepEntry], router_trace: Optional[list] = None,
+             select: Optional[str] = None) -> Optional[torch.Tensor]:
         """Run one batch.  Returns float32 logits [wanted, vocab] in the order of the entries and
-        of their ``want`` lists, or None when nothing is wanted.  A list given as ``router_trace``
+        of their ``want`` lists, or None when nothing is wanted; with ``select="argmax"`` the index
+        of each wanted row's largest logit instead (int32 [wanted]), so that only token ids leave
+        the device.  A list given as ``router_trace``
         receives, per routed layer run, the (expert ids, weights, router input) of the step's tokens,
         as the reference can print its router picks (src/SharpInference.Engine/ForwardPass.cs:2042-2056)."""
         if not entries:
@@ -226,12 +230,13 @@ class ModelRunner:
                 if not self.cache.append(e.req_id, len(e.tokens)):
                     raise CacheExhausted(f"no pages left for request {e.req_id!r} ({len(e.tokens)} more tokens)")
                 appended.append(e.req_id)
-            logits = self._decode_graph_step(entries, router_trace)
+            logits = self._decode_graph_step(entries, router_trace, select)
             if logits is None:
                 ctx, rows = self.build_context(entries)
                 if router_trace is not None:
                     ctx.extras["router_trace"] = router_trace
-                logits = self.model.forward(ctx, self.layer_caches(ctx), rows)
+                logits = self.model.forward(ctx, self.layer_caches(ctx), rows, select) if select else \
+                    self.model.forward(ctx, self.layer_caches(ctx), rows)
         except BaseException:
             for r in appended:
                 self.cache.rollback(r)
@@ -250,7 +255,7 @@ class _DecodeGraph:
     step (block table width, context bound of the decode kernel) are fixed at ``max_context``.
     The logits tensor belongs to the graph: the caller gets a copy."""
 
-    def __init__(self, runner: ModelRunner, pieces, info: dict, max_context: int):
+    def __init__(self, runner: ModelRunner, pieces, info: dict, max_context: int, select: Optional[str] = None):
         self.sizes = [p.size for p in pieces]
         total = sum(self.sizes)
         self.host = torch.empty(total, dtype=torch.int32).pin_memory()
@@ -274,8 +279,9 @@ class _DecodeGraph:
         caches = runner.layer_caches(ctx)
         side = torch.cuda.Stream(device=runner.device)
         side.wait_stream(torch.cuda.current_stream())
+        args = (ctx, caches, rows, select) if select else (ctx, caches, rows)
         with torch.cuda.stream(side):                     # once eagerly: libraries initialise outside the capture
-            runner.model.forward(ctx, caches, rows)
+            runner.model.forward(*args)
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         # the captured run also notes where its router picks lie (tensors of the graph's own memory,
@@ -291,7 +297,7 @@ class _DecodeGraph:
         gc.disable()
         try:
             with torch.cuda.graph(self.graph):
-                self.logits = runner.model.forward(ctx, caches, rows)
+                self.logits = runner.model.forward(*args)
         finally:
             if collecting:
                 gc.enable()

@@ -11,6 +11,7 @@ from typing import Optional, Tuple
 import torch
 
 from . import lib as _lib
+from . import profile as _profile
 
 _DT = {torch.float32: 0, torch.bfloat16: 1}
 
@@ -54,6 +55,9 @@ def _i32(t: Optional[torch.Tensor], name: str) -> None:
 
 
 def _run(name: str, *args) -> None:
+    if _profile._active is not None and _profile._active.depth == 0:
+        with _profile.section(name[len("sharpi_"):]):       # a launch outside any section: a class of its own
+            return _run(name, *args)
     rc = getattr(_lib.load(), name)(*args)
     if rc != 0:
         what = {1001: "a size or option the kernel does not take", 1002: "launch failed"}.get(rc, f"HIP error {rc}")
@@ -171,6 +175,23 @@ def cast(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
     _dev(x)
     out = torch.empty(x.shape, dtype=dtype, device=x.device)
     _run("sharpi_cast", _ptr(x), _code(x.dtype), _ptr(out), _code(dtype), x.numel(), _stream())
+    return out
+
+
+def random_fill(out: torch.Tensor, key: int, kind: int, std: float = 0.02, lo: float = 0.9, hi: float = 1.1) -> torch.Tensor:
+    """Fill `out` (float32, bfloat16, or int32 for integers) with the seeded values of
+    weights/random_fill.py: element i is a function of (key, i) alone, the same bits as the host makes."""
+    from ..weights import random_fill as rf
+
+    _dev(out)
+    if kind == rf.FILL_INT:
+        _need(out.dtype == torch.int32, "random_fill: integers go into int32")
+        code = 0
+    else:
+        code = _code(out.dtype)
+    lo_f, span_f = rf.uniform_fixed(lo, hi)
+    _run("sharpi_random_fill", _ptr(out), code, out.numel(), int(key) & ((1 << 64) - 1), int(kind),
+         rf.normal_scale(std), lo_f, span_f, _stream())
     return out
 
 
@@ -823,3 +844,31 @@ def grouped_linear(x: torch.Tensor, w, rt: Routing, gather: bool, out_dtype: tor
         return gemm_grouped(x, w, rt, gather, out_dtype)
     y = grouped_gemm(x, w, rt.offsets, a_rows, rt.n_rows)
     return y if y.dtype == out_dtype else cast(y, out_dtype)
+
+
+# ---------------------------------------------------------------------------
+# what the GPU gives at best (measured beside the published peaks)
+# ---------------------------------------------------------------------------
+def measured_peaks(device="cuda:0", read_bytes: int = 4 << 30, repeats: int = 5) -> dict:
+    """{"hbm_gbs": GB/s of a pure read of `read_bytes`, "bf16_tflops": TFLOP/s of a resident loop of
+    matrix-core products}: the best of `repeats` runs of two measuring kernels of this library."""
+    dev = torch.device(device)
+    buf = torch.empty(read_bytes, dtype=torch.uint8, device=dev)
+    buf.fill_(1)
+    sink = torch.zeros(4, dtype=torch.float32, device=dev)
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    best_read = best_mfma = float("inf")
+    blocks, iters = 256 * 8, 4096
+    for _ in range(repeats + 1):
+        a.record()
+        _run("sharpi_peak_read", _ptr(buf), read_bytes, _ptr(sink), _stream())
+        b.record()
+        b.synchronize()
+        best_read = min(best_read, a.elapsed_time(b))
+        a.record()
+        _run("sharpi_peak_mfma", _ptr(sink), blocks, iters, _stream())
+        b.record()
+        b.synchronize()
+        best_mfma = min(best_mfma, a.elapsed_time(b))
+    flops = blocks * 4 * iters * 8 * (2.0 * 16 * 16 * 32)
+    return {"hbm_gbs": read_bytes / best_read / 1e6, "bf16_tflops": flops / best_mfma / 1e9}

@@ -6,7 +6,7 @@ raises, so a GPU run can never silently use something else.
 from __future__ import annotations
 
 import ctypes
-from ctypes import c_float, c_int, c_longlong, c_void_p
+from ctypes import c_float, c_int, c_longlong, c_ulonglong, c_void_p
 from typing import Optional
 
 _lib: Optional[ctypes.CDLL] = None
@@ -22,6 +22,9 @@ _SIGNATURES = {
     "sharpi_silu_mul": [P, P, P, I, I, I, P],
     "sharpi_moe_combine": [P, P, P, P, P, I, I, I, I, P],
     "sharpi_cast": [P, I, P, I, c_longlong, P],
+    "sharpi_peak_read": [P, c_longlong, P, P],
+    "sharpi_peak_mfma": [P, I, I, P],
+    "sharpi_random_fill": [P, I, c_longlong, c_ulonglong, I, F, I, I, P],
     "sharpi_rope_kv": [P, P, P, P, I, P, P, P, I, F, I, F, F, I, I, I, I, I, I, I, P],
     "sharpi_attention_generic": [P, P, P, I, P, P, P, P, I, I, F, I, I, I, I, I, I, I, P],
     "sharpi_attention_decode": [P, P, P, P, P, P, P, P, P, P, I, I, F, I, I, I, I, I, I, I, I, P],

@@ -7,6 +7,7 @@ from typing import Dict, Optional, Tuple
 import torch
 
 from .. import ops
+from ..ops.profile import section
 from ..cache.spec import KVSpec, WINDOW_CHUNK, WINDOW_NONE, WINDOW_SLIDING  # noqa: F401
 from .base import LayerCache, ParamSpec, Part, StepContext, TensorSource
 
@@ -72,12 +73,31 @@ class Attention(Part):
     # -- compute --------------------------------------------------------------
     def forward(self, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> torch.Tensor:
         g = cache.group
-        qkv = ops.linear(x, self.w_qkv, ctx.act_dtype)
+        T = x.shape[0]
+        width = 2 if ctx.act_dtype == torch.bfloat16 else 4
+        q_dim, kv_dim = self.nh * self.hd, self.nkv * self.hd
+        with section("qkv", nbytes=width * (q_dim + 2 * kv_dim) * (self.hidden + T) + width * T * self.hidden,
+                     flops=2.0 * T * self.hidden * (q_dim + 2 * kv_dim)):
+            qkv = ops.linear(x, self.w_qkv, ctx.act_dtype)
         slots = g.slot_mapping if cache.write else ctx.no_store_slots
         inv_freq = self.rotary.table(x.device) if self.rotary is not None else None
         layout = ops.PAIRS_HALF_SPLIT if self.rotary is not None and self.rotary.pair_layout == "half" else ops.PAIRS_INTERLEAVED
-        q = ops.rope_kv(qkv, cache.k, cache.v, slots, ctx.positions, inv_freq, self.qk_norm_eps is not None,
-                        self.qk_norm_eps or 1e-6, self.q_temperature, self.nh, self.nkv, self.hd, layout)
-        o = ops.attention(q, cache.k, cache.v, g, ctx, self.window_kind, self.window, self.scale, self.nh, self.nkv,
-                          self.hd)
-        return ops.linear(o, self.w_o, ctx.act_dtype)
+        with section("rope + cache write", nbytes=2 * width * T * (q_dim + 2 * kv_dim)):
+            q = ops.rope_kv(qkv, cache.k, cache.v, slots, ctx.positions, inv_freq, self.qk_norm_eps is not None,
+                            self.qk_norm_eps or 1e-6, self.q_temperature, self.nh, self.nkv, self.hd, layout)
+        with section("attention", nbytes=lambda: self._keys_held(ctx) * 2 * kv_dim * width + 2 * T * q_dim * width,
+                     flops=lambda: 4.0 * self._keys_read(ctx) * q_dim):
+            o = ops.attention(q, cache.k, cache.v, g, ctx, self.window_kind, self.window, self.scale, self.nh, self.nkv,
+                              self.hd)
+        with section("o", nbytes=width * self.hidden * (q_dim + T) + width * T * q_dim, flops=2.0 * T * self.hidden * q_dim):
+            return ops.linear(o, self.w_o, ctx.act_dtype)
+
+    def _keys_read(self, ctx: StepContext) -> int:
+        """(query, key) pairs of the step: what is computed."""
+        spec = self.cache_spec()
+        return sum(p - spec.first_visible(p) + 1 for s, n in zip(ctx.entry_starts, ctx.entry_lens) for p in range(s, s + n))
+
+    def _keys_held(self, ctx: StepContext) -> int:
+        """Keys that some query of the step sees, each counted once per entry: what has to be read."""
+        spec = self.cache_spec()
+        return sum(s + n - spec.first_visible(s) for s, n in zip(ctx.entry_starts, ctx.entry_lens))

@@ -6,6 +6,7 @@ from typing import Dict, Optional
 import torch
 
 from .. import ops
+from ..ops.profile import active as profiling, section
 from .base import ParamSpec, Part, ResidualStream, StepContext, TensorSource
 from .norm import RMSNorm
 
@@ -50,9 +51,13 @@ class DenseSwiGLU(Part):
         self.w_down = ops.pack_weight(source.get(prefix + "down_proj.weight"))
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
-        gu = ops.linear(x, self.w_gate_up, ctx.act_dtype)
-        act = ops.silu_mul(gu)
-        return ops.linear(act, self.w_down, ctx.act_dtype)
+        T = x.shape[0]
+        width = 2 if ctx.act_dtype == torch.bfloat16 else 4
+        with section("dense feed-forward", nbytes=width * 3 * self.inter * self.hidden + width * T * (2 * self.hidden + 3 * self.inter),
+                     flops=6.0 * T * self.inter * self.hidden):
+            gu = ops.linear(x, self.w_gate_up, ctx.act_dtype)
+            act = ops.silu_mul(gu)
+            return ops.linear(act, self.w_down, ctx.act_dtype)
 
 
 class MoESwiGLU(Part):
@@ -142,6 +147,18 @@ class MoESwiGLU(Part):
         self.w_gate_up = ops.PackedWeight(gu, None) if pack else gu
         self.w_down = ops.PackedWeight(dn, None) if pack else dn
 
+    def _experts_section(self, ids: torch.Tensor, T: int, with_shared: bool):
+        """The profiler's span of the experts' two products: every expert that a token picked is
+        read once (the count is taken from the picks, only while profiling)."""
+        if not profiling():
+            return section("experts")
+        width = 2 if self.w_gate_up.dtype == torch.bfloat16 else 4
+        used = int(ids.unique().numel()) + (1 if with_shared else 0)
+        rows = T * self.k + (T if with_shared else 0)
+        per_expert = 3 * self.inter * self.hidden
+        return section("experts" + (" + shared" if with_shared else ""), nbytes=width * (used * per_expert + rows * (2 * self.hidden + 3 * self.inter)),
+                       flops=2.0 * rows * per_expert)
+
     def _few_tokens(self, T: int, ctx: StepContext) -> bool:
         """A few decode tokens in bfloat16 (at most 64 picks): the experts' two products find their
         rows from the picks themselves."""
@@ -160,9 +177,10 @@ class MoESwiGLU(Part):
             trace.append((ids, wts, x))
         along = self.merged and T <= self.MERGE_MAX_TOKENS
         shared = None if along or self.shared is None else self.shared.forward(x, ctx)
-        act = ops.gemm_skinny_picked(x, self.w_gate_up, ids, wts if self.score_on_input else None, along, True, True,
-                                     ctx.act_dtype)
-        y = ops.gemm_skinny_picked(act, self.w_down, ids, None, along, False, False, ctx.act_dtype)
+        with self._experts_section(ids, T, along):
+            act = ops.gemm_skinny_picked(x, self.w_gate_up, ids, wts if self.score_on_input else None, along, True, True,
+                                         ctx.act_dtype)
+            y = ops.gemm_skinny_picked(act, self.w_down, ids, None, along, False, False, ctx.act_dtype)
         return ops.ExpertSum(y, ops.counting(T * self.k, x.device), y[T * self.k:] if along else shared, T, self.k,
                              None if self.score_on_input else wts)
 
@@ -172,8 +190,9 @@ class MoESwiGLU(Part):
         T = stream.h.shape[0]
         if (self._few_tokens(T, ctx) and isinstance(norm, RMSNorm)
                 and ops.norm_router_ok(stream.h, stream.pending, ctx.act_dtype)):
-            x, ids, wts = ops.add_rmsnorm_router(stream.h, stream.pending, norm.weight, norm.eps, self.w_router, self.k,
-                                                 self.gate, self.renormalise)
+            with section("norm + router", nbytes=T * self.hidden * 10 + 2 * self.E * self.hidden):
+                x, ids, wts = ops.add_rmsnorm_router(stream.h, stream.pending, norm.weight, norm.eps, self.w_router, self.k,
+                                                     self.gate, self.renormalise)
             stream.pending = None
             return self._picked(x, ids, wts, ctx)
         return self.forward(norm.forward(stream, ctx.act_dtype), ctx)
@@ -182,20 +201,24 @@ class MoESwiGLU(Part):
         T = x.shape[0]
         trace = ctx.extras.get("router_trace")
         if self._few_tokens(T, ctx):
-            ids, wts = ops.router_topk(x, self.w_router, self.k, self.gate, self.renormalise)
+            with section("router", nbytes=2 * T * self.hidden + 2 * self.E * self.hidden):
+                ids, wts = ops.router_topk(x, self.w_router, self.k, self.gate, self.renormalise)
             return self._picked(x, ids, wts, ctx)
         merge = self.merged and T <= self.MERGE_MAX_TOKENS and ctx.act_dtype == torch.bfloat16
-        ids, wts, rt = ops.route(x, self.w_router, self.k, self.gate, self.renormalise, shared_group=merge)
+        with section("router", nbytes=2 * T * self.hidden + 2 * self.E * self.hidden):
+            ids, wts, rt = ops.route(x, self.w_router, self.k, self.gate, self.renormalise, shared_group=merge)
         if trace is not None:      # the picks of this step, layer by layer (reference: ForwardPass.cs:2042-2056)
             trace.append((ids, wts, x))
         after = None if self.score_on_input else wts     # scores applied where the outputs are summed
         if merge:
             # few rows: the shared expert rides along as one more group of the same two launches
-            act = ops.grouped_swiglu(x, self.w_gate_up, rt, ctx.act_dtype, scaled=self.score_on_input)
-            y = ops.grouped_linear(act, self.w_down, rt, False, ctx.act_dtype)
+            with self._experts_section(ids, T, True):
+                act = ops.grouped_swiglu(x, self.w_gate_up, rt, ctx.act_dtype, scaled=self.score_on_input)
+                y = ops.grouped_linear(act, self.w_down, rt, False, ctx.act_dtype)
             # left as a sum: the next norm forms it while it reads the residual stream
             return ops.ExpertSum(y, rt.inv_pos, y[T * self.k:], T, self.k, after)
         shared = self.shared.forward(x, ctx) if self.shared is not None else None
-        act = ops.grouped_swiglu(x, self.w_gate_up, rt, ctx.act_dtype, scaled=self.score_on_input)
-        y = ops.grouped_linear(act, self.w_down, rt, False, ctx.act_dtype)
+        with self._experts_section(ids, T, False):
+            act = ops.grouped_swiglu(x, self.w_gate_up, rt, ctx.act_dtype, scaled=self.score_on_input)
+            y = ops.grouped_linear(act, self.w_down, rt, False, ctx.act_dtype)
         return ops.ExpertSum(y, rt.inv_pos, shared, T, self.k, after)   # formed by the next norm (or by whoever asks for a tensor)

@@ -7,6 +7,7 @@ from typing import Dict, List, Optional, Sequence
 import torch
 
 from .. import ops
+from ..ops.profile import section
 from .base import LayerCache, ParamSpec, Part, ResidualStream, StepContext, TensorSource
 from .norm import RMSNorm
 
@@ -98,10 +99,16 @@ class DecoderModel(Part):
         self.head = ops.pack_weight(self.embed if self.tie_embeddings else source.get(self.head_name))
 
     # -- compute ------------------------------------------------------------------
-    def forward(self, ctx: StepContext, caches: Sequence[LayerCache], logit_rows: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+    def forward(self, ctx: StepContext, caches: Sequence[LayerCache], logit_rows: Optional[torch.Tensor],
+                select: Optional[str] = None) -> Optional[torch.Tensor]:
         """Run the step's tokens through every entry of the schedule.  Returns float32 logits
-        [len(logit_rows), vocab], or None if no row is wanted."""
-        stream = ResidualStream(ops.embed_gather(ctx.token_ids, self.embed))
+        [len(logit_rows), vocab], or None if no row is wanted.  With ``select="argmax"`` the
+        largest logit's index per wanted row is returned instead (int32 [rows], the lowest index
+        on a tie), chosen on the device right behind the head: the logits then never leave it
+        (the reference keeps such a path for all-greedy batches,
+        src/SharpInference.Engine/CudaForwardPass.cs:1574-1583)."""
+        with section("embed", nbytes=ctx.n_tokens * self.hidden * 6):
+            stream = ResidualStream(ops.embed_gather(ctx.token_ids, self.embed))
         for r in self.schedule:
             c = caches[r.cache]
             if not r.write:
@@ -110,4 +117,12 @@ class DecoderModel(Part):
         if logit_rows is None or logit_rows.numel() == 0:
             return None
         n = self.final_norm.forward(stream, ctx.act_dtype, rows=logit_rows)
-        return ops.linear(n, self.head, torch.float32)
+        m = n.shape[0]
+        with section("head", nbytes=2 * self.vocab_size * self.hidden + 4 * m * self.vocab_size, flops=2.0 * m * self.vocab_size * self.hidden):
+            logits = ops.linear(n, self.head, torch.float32)
+        if select is None:
+            return logits
+        if select == "argmax":
+            with section("select", nbytes=4 * m * self.vocab_size):
+                return ops.argmax_rows(logits)
+        raise ValueError(f"select {select!r} is not known (None for logits, 'argmax')")

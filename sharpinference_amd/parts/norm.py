@@ -6,6 +6,7 @@ from typing import Dict, Optional
 import torch
 
 from .. import ops
+from ..ops.profile import section
 from .base import INIT_NORM_WEIGHT, ParamSpec, Part, ResidualStream, TensorSource
 
 
@@ -29,8 +30,10 @@ class RMSNorm(Part):
     def forward(self, stream: ResidualStream, out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Fold the pending branch output into the residual sum and normalise.  With ``rows``
         only those rows are produced and the stream is left as it is."""
-        out = ops.add_rmsnorm(stream.h, stream.pending, self.weight, self.eps, out_dtype, rows=rows,
-                              write_back=rows is None)
+        n = stream.h.shape[0] if rows is None else rows.shape[0]
+        with section("norm", nbytes=n * self.dim * 12):
+            out = ops.add_rmsnorm(stream.h, stream.pending, self.weight, self.eps, out_dtype, rows=rows,
+                                  write_back=rows is None)
         if rows is None:
             stream.pending = None
         return out

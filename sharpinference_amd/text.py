@@ -11,6 +11,18 @@ import os
 from typing import List, Optional, Sequence
 
 
+def format_llama4_chat(user: str, system: Optional[str] = None) -> str:
+    """One user turn in the Llama 4 chat form the reference falls back to when a model carries no
+    template of its own (reference: src/SharpInference.Cli/RunCommand.cs:2588-2596): begin of
+    text, then per message a header naming the role, a blank line, the text and an end-of-turn
+    mark; it ends with the assistant's header, which the model continues."""
+    out = "<|begin_of_text|>"
+    if system is not None:
+        out += f"<|header_start|>system<|header_end|>\n\n{system}<|eot|>"
+    out += f"<|header_start|>user<|header_end|>\n\n{user}<|eot|>"
+    return out + "<|header_start|>assistant<|header_end|>\n\n"
+
+
 class TextCodec:
     """Encodes a prompt and decodes generated ids as they come."""
 
@@ -35,6 +47,16 @@ class TextCodec:
         ids = list(self._tok.encode(text).ids)
         if self.bos_token_id is not None and (not ids or ids[0] != self.bos_token_id):
             ids.insert(0, self.bos_token_id)
+        return ids
+
+    def knows_chat_marks(self) -> bool:
+        """Does the vocabulary hold the marks of the Llama 4 chat form as single tokens?"""
+        return all(self._tok.token_to_id(t) is not None for t in ("<|header_start|>", "<|header_end|>", "<|eot|>"))
+
+    def encode_chat(self, user: str, system: Optional[str] = None) -> List[int]:
+        """Token ids of one user turn (and a system message) in the chat form; the form's own
+        begin-of-text mark is the only one."""
+        ids = list(self._tok.encode(format_llama4_chat(user, system), add_special_tokens=False).ids)
         return ids
 
     def decode(self, ids: Sequence[int]) -> str:

@@ -13,7 +13,6 @@ float32 (exact for bfloat16 values).
 """
 from __future__ import annotations
 
-import hashlib
 import os
 from dataclasses import dataclass
 from typing import Dict, Iterable, List, Optional, Tuple
@@ -224,18 +223,15 @@ class LayoutAdapter(TensorSource):
         return (t.transpose(-1, -2) if transpose else t).contiguous()
 
 
-def _name_seed(seed: int, name: str) -> int:
-    h = hashlib.sha256(f"{seed}:{name}".encode()).digest()
-    return int.from_bytes(h[:8], "little") & ((1 << 63) - 1)
-
-
 class RandomSource(TensorSource):
     """Seeded random tensors: matrices N(0, std), norm weights U(0.9, 1.1).
 
-    Each tensor's generator is keyed by (seed, name), so the values do not depend on the
-    order of the requests.  ``stored_dtype`` is what a file written from this source holds
-    (values are rounded to it first); ``float32_names`` keeps tensors whose name ends with one
-    of the given suffixes in float32."""
+    Every element is a function of (seed, tensor name, element index) alone (see
+    weights/random_fill.py), so the values depend neither on the order of the requests nor on
+    where they are made: with ``generate_on_device`` the tensors are filled straight into device
+    memory by a kernel, otherwise on the host, and both give the same bits.  ``stored_dtype`` is
+    what a file written from this source holds (values are rounded to it first);
+    ``float32_names`` keeps tensors whose name ends with one of the given suffixes in float32."""
 
     def __init__(self, specs: Dict[str, ParamSpec], seed: int, compute_dtype: torch.dtype, device,
                  stored_dtype: torch.dtype = torch.bfloat16, std: float = 0.02,
@@ -265,26 +261,17 @@ class RandomSource(TensorSource):
 
     def stored(self, name: str) -> torch.Tensor:
         """The tensor as a file would hold it (host unless generating on the device)."""
+        from . import random_fill as rf
+
         spec = self.specs[name]
-        dev = self.device if self.generate_on_device else torch.device("cpu")
-        g = torch.Generator(device=dev)
-        g.manual_seed(_name_seed(self.seed, name))
+        key = rf.name_key(self.seed, name)
         sd = self.stored_dtype_of(name)
-        if spec.kind == "int":
-            return torch.randint(0, 2 ** 15, spec.shape, generator=g, device=dev, dtype=torch.int32)
+        kind = rf.FILL_INT if spec.kind == "int" else rf.FILL_UNIFORM if spec.init == INIT_NORM_WEIGHT else rf.FILL_NORMAL
         if self.generate_on_device:
-            t = torch.empty(spec.shape, dtype=sd, device=dev)
-            if spec.init == INIT_NORM_WEIGHT:
-                t.uniform_(0.9, 1.1, generator=g)
-            else:
-                t.normal_(0.0, self._std_of(name), generator=g)
-            return t
-        t = torch.empty(spec.shape, dtype=torch.float32)
-        if spec.init == INIT_NORM_WEIGHT:
-            t.uniform_(0.9, 1.1, generator=g)
-        else:
-            t.normal_(0.0, self._std_of(name), generator=g)
-        return t.to(sd)
+            from .. import ops
+
+            return ops.random_fill(torch.empty(spec.shape, dtype=sd, device=self.device), key, kind, self._std_of(name))
+        return rf.host_tensor(spec.shape, key, kind, sd, self._std_of(name))
 
     def _std_of(self, name: str) -> float:
         for suffix, s in self.std_by_suffix.items():

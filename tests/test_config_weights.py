@@ -193,6 +193,38 @@ def test_random_source_is_order_independent():
     check_specs(specs, a.available())
 
 
+def test_random_values_are_a_function_of_seed_name_and_element():
+    """Any part of a seeded tensor can be made on its own, and the numbers are pinned (the device
+    kernel must give the same ones: tests/test_gpu_kernels.py compares them)."""
+    from sharpinference_amd.weights import random_fill as rf
+
+    key = rf.name_key(2, "model.layers.0.self_attn.q_proj.weight")
+    whole = rf.host_fill(5000, key, rf.FILL_NORMAL, 0.02)
+    assert (rf.host_fill(17, key, rf.FILL_NORMAL, 0.02, start=4000) == whole[4000:4017]).all()
+    assert (whole != rf.host_fill(5000, rf.name_key(3, "model.layers.0.self_attn.q_proj.weight"), rf.FILL_NORMAL, 0.02)).mean() > 0.99
+    assert (whole != rf.host_fill(5000, rf.name_key(2, "model.layers.1.self_attn.q_proj.weight"), rf.FILL_NORMAL, 0.02)).mean() > 0.99
+    # written out from the formula for one element: word(c) = mix(key + (c + 1) * golden), twelve 16-bit fields
+    M = (1 << 64) - 1
+
+    def mix(z):
+        z ^= z >> 30
+        z = (z * 0xBF58476D1CE4E5B9) & M
+        z ^= z >> 27
+        z = (z * 0x94D049BB133111EB) & M
+        return z ^ (z >> 31)
+
+    i = 1234
+    s = 0
+    for j in range(3):
+        w = mix((key + (3 * i + j + 1) * 0x9E3779B97F4A7C15) & M)
+        s += sum((w >> sh) & 0xFFFF for sh in (0, 16, 32, 48))
+    import numpy as np
+    assert whole[i] == np.float32(s - 393210) * np.float32(0.02 / 65536.0)
+    u = rf.host_fill(3, key, rf.FILL_UNIFORM)
+    w0 = mix((key + 0x9E3779B97F4A7C15) & M) >> 40
+    assert u[0] == np.float32(15099494 + ((w0 * 3355443) >> 24)) * np.float32(2.0 ** -24)
+
+
 def test_bench_refuses_more_than_one_gpu():
     """The benchmark measures one GPU: for N > 1 it says so in one line and exits with 2, before
     anything touches a device."""
@@ -384,3 +416,43 @@ def test_axis_order_is_decided_by_name_where_the_shape_cannot_tell(tmp_path, hid
     # the canonical folder (separate gate and up, down [E, out, in]) with the same sizes is left as it is
     same = LayoutAdapter(SafetensorsSource(d, torch.bfloat16, "cpu"), specs)
     assert all(torch.equal(same.get(n), plain.get(n)) for n in specs)
+
+
+def test_chat_form_system_prompt_and_raw_text(tmp_path):
+    """Text prompts take the Llama 4 chat form of the reference's fallback template
+    (src/SharpInference.Cli/RunCommand.cs:2588-2596) when the tokenizer knows its marks;
+    --system-prompt adds the system message; --raw-prompt leaves the text alone."""
+    from tokenizers import Tokenizer, models, pre_tokenizers
+    from tokenizers import AddedToken
+
+    from sharpinference_amd.cli import build_parser, prompt_ids
+    from sharpinference_amd.text import TextCodec, format_llama4_chat
+
+    assert format_llama4_chat("hi", None) == \
+        "<|begin_of_text|><|header_start|>user<|header_end|>\n\nhi<|eot|><|header_start|>assistant<|header_end|>\n\n"
+    assert format_llama4_chat("hi", "be brief").startswith(
+        "<|begin_of_text|><|header_start|>system<|header_end|>\n\nbe brief<|eot|><|header_start|>user<|header_end|>")
+    words = ["<unk>", "hi", "there", "be", "brief", "user", "system", "assistant"]
+    tok = Tokenizer(models.WordLevel({w: i for i, w in enumerate(words)}, unk_token="<unk>"))
+    tok.pre_tokenizer = pre_tokenizers.Whitespace()
+    plain_dir = tmp_path / "plain"
+    plain_dir.mkdir()
+    tok.save(str(plain_dir / "tokenizer.json"))
+    plain = TextCodec.from_folder(str(plain_dir), None)
+    assert not plain.knows_chat_marks() and prompt_ids("hi there", plain) == [1, 2]
+    with pytest.raises(SystemExit, match="chat form"):
+        prompt_ids("hi", plain, system="be brief")
+    marks = ["<|begin_of_text|>", "<|header_start|>", "<|header_end|>", "<|eot|>"]
+    tok.add_special_tokens([AddedToken(m, special=True) for m in marks])
+    chat_dir = tmp_path / "chat"
+    chat_dir.mkdir()
+    tok.save(str(chat_dir / "tokenizer.json"))
+    chat = TextCodec.from_folder(str(chat_dir), None)
+    b, hs, he, eot = (tok.token_to_id(m) for m in marks)
+    assert chat.knows_chat_marks()
+    assert prompt_ids("hi there", chat) == [b, hs, 5, he, 1, 2, eot, hs, 7, he]
+    assert prompt_ids("hi", chat, system="be brief") == [b, hs, 6, he, 3, 4, eot, hs, 5, he, 1, eot, hs, 7, he]
+    assert prompt_ids("hi there", chat, raw=True) == [1, 2]
+    assert prompt_ids("5, 6 7", chat) == [5, 6, 7]                      # numbers are token ids, whatever the tokenizer
+    a = build_parser().parse_args(["-m", "X", "--single-turn", "--system-prompt", "be brief", "--profile"])
+    assert a.single_turn and a.system_prompt == "be brief" and a.profile and a.prompt is None

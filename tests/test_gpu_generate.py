@@ -66,6 +66,33 @@ def test_greedy_generation_in_bfloat16_token_for_token(tmp_path, which, std):
     assert strict >= 3 * n_new - 3, f"only {strict} of {3 * n_new} tokens are the plain implementation's own choice"
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_tokens_chosen_on_the_device_are_the_argmax_of_the_logits(tmp_path, dtype):
+    """select="argmax": only token ids leave the device; they are the lowest index of the largest
+    logit, whether the step is launched part by part, replayed from a graph, or mixed."""
+    from sharpinference_amd.engine import StepEntry
+
+    d = make_model_dir(tmp_path, "D", std=0.06)
+    toks = {r: H.random_tokens(30, 500, 20 + i) for i, r in enumerate("abc")}
+    engs = [H.make_engine(d, dtype, kv_tokens=192, max_num_seqs=3) for _ in range(2)]
+    for e in engs:
+        for r in toks:
+            e.add_request(r)
+    plan = [[("a", 12), ("b", 20)], [("a", 1), ("b", 1), ("c", 9)], [("a", 1), ("b", 1), ("c", 1)], [("a", 1), ("b", 1), ("c", 1)],
+            [("c", 1)], [("c", 1)]]
+    at = {r: 0 for r in toks}
+    for step in plan:
+        entries = []
+        for r, n in step:
+            entries.append(StepEntry(r, toks[r][at[r]:at[r] + n], (n - 1,)))
+            at[r] += n
+        lg = engs[0].step(entries)
+        ids = engs[1].step(entries, select="argmax")
+        assert ids.dtype == torch.int32 and ids.shape == (len(entries),)
+        assert ids.cpu().tolist() == [P.greedy(row) for row in lg.float().cpu()]
+    assert engs[1].runner.graph_replays >= 4 and any(len(k) == 3 and k[2] == "argmax" for k in engs[1].runner._graphs)
+
+
 def test_temperature_generation_matches_plain(tmp_path):
     """Tiny B, 32-bit: prompts of 1 / 17 / 50 / 77 tokens, 24 steps at temperature 0.8 with
     fixed seeds: the same uniforms give the same tokens."""
@@ -271,6 +298,30 @@ def test_command_line(tmp_path):
     assert lines[0] == " ".join(map(str, prompt))
     assert lines[1].startswith(" ".join(map(str, want))) and lines[1].endswith("(length)")
     assert lines[-1].startswith("Prefill: 12 tokens, ") and "| Decode: 7 tokens, " in lines[-1] and lines[-1].endswith("t/s")
+
+
+def test_command_line_interactive_mode_and_profile(tmp_path):
+    """Without a prompt option the command reads prompts from standard input, a line a turn, every
+    turn from an empty cache (the reference's interactive mode); --single-turn ends after the
+    first; --profile prints a table of kernel classes."""
+    d = make_model_dir(tmp_path, "A", std=0.1)
+    c, W = P.read_config(d), P.load_weights(d)
+    p1, p2 = H.random_tokens(9, 256, 4), H.random_tokens(14, 256, 5)
+    base = [sys.executable, os.path.join(ROOT, "bin", "sharpi-cli"), "-m", d, "-n", "5", "--temp", "0", "--dtype", "fp32",
+            "--kv-tokens", "128"]
+    feed = " ".join(map(str, p1)) + "\n\n" + ",".join(map(str, p2)) + "\n/exit\nnever read\n"
+    out = subprocess.run(base, input=feed, capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stderr
+    body = out.stdout
+    assert " ".join(map(str, P.generate(c, W, p1, 5))) + "  (length)" in body
+    assert " ".join(map(str, P.generate(c, W, p2, 5))) + "  (length)" in body
+    assert body.count("t/s") == 2 and "never" not in body
+    out = subprocess.run(base + ["--single-turn", "--profile"], input=feed, capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stderr
+    assert out.stdout.count("(length)") == 1
+    table = out.stderr
+    for word in ("qkv", "attention", "experts", "head", "GB/s"):
+        assert word in table, table
 
 
 def test_command_line_with_text_and_the_model_s_end_token(tmp_path):

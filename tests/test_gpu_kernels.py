@@ -752,3 +752,42 @@ def test_the_library_says_which_head_sizes_its_attention_kernels_take():
     assert [hd for hd in range(16, 273, 16) if ops.decode_attention_ok(torch.bfloat16, hd)] == [32, 64, 96, 128, 160, 192, 224, 256]
     assert [hd for hd in range(16, 273, 16) if ops.prefill_attention_ok(torch.bfloat16, hd)] == [32, 64, 96, 128, 160, 192]
     assert not ops.decode_attention_ok(torch.float32, 128) and not ops.prefill_attention_ok(torch.float32, 128)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_random_fill_on_the_device_equals_the_host(dtype):
+    """Seeded random weights are a function of (seed, name, element): the device's fill kernel and
+    the host give the same bits, so a model made in device memory is the model a file written on
+    the host from the same seed holds."""
+    ops = _ops()
+    from sharpinference_amd.weights import random_fill as rf
+
+    for name, shape, kind, std in (("a.weight", (3, 1001), rf.FILL_NORMAL, 0.02), ("b", (70001,), rf.FILL_NORMAL, 1.0),
+                                   ("norm.weight", (5120,), rf.FILL_UNIFORM, 0.0)):
+        key = rf.name_key(7, name)
+        dev = ops.random_fill(torch.empty(shape, dtype=dtype, device=DEV), key, kind, std).cpu()
+        host = rf.host_tensor(shape, key, kind, dtype, std)
+        assert torch.equal(dev, host), name
+    ints = ops.random_fill(torch.empty(999, dtype=torch.int32, device=DEV), rf.name_key(7, "i"), rf.FILL_INT).cpu()
+    assert torch.equal(ints, rf.host_tensor((999,), rf.name_key(7, "i"), rf.FILL_INT, torch.int32))
+    x = rf.host_tensor((200000,), rf.name_key(1, "x"), rf.FILL_NORMAL, torch.float32, 0.5)
+    assert abs(float(x.mean())) < 0.01 and abs(float(x.std()) - 0.5) < 0.01
+    u = rf.host_tensor((50000,), rf.name_key(1, "u"), rf.FILL_UNIFORM, torch.float32)
+    assert 0.9 <= float(u.min()) and float(u.max()) < 1.1 and abs(float(u.mean()) - 1.0) < 0.005
+
+
+def test_a_model_made_on_the_device_is_the_model_written_on_the_host(tmp_path):
+    from sharpinference_amd import load_config
+    from sharpinference_amd.engine import Engine, StepEntry
+    from sharpinference_amd.weights.loader import write_random_model
+    from tiny_configs import CONFIGS
+
+    cfg = load_config(CONFIGS["D"])
+    d = write_random_model(cfg, str(tmp_path / "m"), 4, std=0.06)
+    toks = [5, 17, 3, 99, 200, 41, 8, 8]
+    out = []
+    for eng in (Engine(d, dtype="bfloat16", kv_tokens=64, max_num_seqs=1),
+                Engine(config=cfg, weight_seed=4, weight_std=0.06, dtype="bfloat16", kv_tokens=64, max_num_seqs=1)):
+        eng.add_request("r")
+        out.append(eng.step([StepEntry("r", toks, list(range(len(toks))))]))
+    assert torch.equal(out[0], out[1])
