@@ -24,6 +24,9 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 // the head sizes the kernel is compiled for
 #define SHARPI_DECODE_HEAD_SIZES(X) X(32) X(64) X(96) X(128) X(160) X(192) X(224) X(256)
 
+#ifndef SHARPI_DEC_PRE2_MAX_HD
+#define SHARPI_DEC_PRE2_MAX_HD 128   // head sizes up to this keep two chunks of a wave's keys in flight
+#endif
 constexpr int kDecWaves = 4;
 constexpr int kSplitBlocks = 16;  // 16-key blocks per run: 256 keys
 
@@ -84,7 +87,7 @@ __global__ __launch_bounds__(kDecWaves* kWave) void attn_decode_kernel(
   // round trip to memory, not one per chunk).  Every load is unconditional: a block beyond the
   // run's last is fetched as the last one again and masked, so that the compiler's count of
   // outstanding loads stays exact and the first chunk does not wait for the second.
-  constexpr int PRE = HD <= 128 ? 2 : 1;
+  constexpr int PRE = HD <= SHARPI_DEC_PRE2_MAX_HD ? 2 : 1;
   for (int b0 = b_first + 2 * w; b0 <= b_last; b0 += 2 * kDecWaves * PRE) {
     bf16x8 kf[PRE][2][NJ];
     bf16x4 vq[PRE][2][ND];

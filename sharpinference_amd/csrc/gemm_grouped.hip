@@ -4,11 +4,13 @@
 //
 // The product is bound by reading the experts' weights, so a block takes ALL rows of its expert
 // that fit one tile (192, about one and a half times the mean load of 2,048 tokens over 16
-// experts) against 256 weight rows: a typical expert's weights are then read once.  Tiles are
-// listed on the device by the routing kernel (tile_expert, tile_row0, n_tiles); the host never
-// learns the routing.  The tile's work is compiled three times, for 64, 128 and 192 rows, and a
-// block takes the smallest that holds its rows: no branch inside a K stage, nothing multiplied or
-// staged for 64-row quarters that hold no row.
+// experts) against 256 weight rows: a typical expert's weights are then read once.  An expert
+// with more rows is cut into sibling tiles of equal height, and the blocks that multiply the SAME
+// weight rows by sibling tiles are neighbours on one XCD, so that the weights cross the memory
+// interface about once all the same (grouped_plan.h says how the routing kernel lays that out;
+// the host never learns the routing).  The tile's work is compiled for every height in steps of 32 rows up to 192,
+// and a block takes the smallest that holds its rows: no branch inside a K stage, nothing
+// multiplied for 32-row pieces that hold no row (rows are staged in passes of 64).
 //  * Each of the 8 waves owns 32 weight rows (2 MFMA tiles) and reads them straight from global
 //    memory into registers, a ring of 64-wide K stages ahead: a weight element is used by one wave only.
 //  * The x rows (gathered through a_rows) are shared by the waves and staged through LDS, 64
@@ -28,6 +30,7 @@
 #include <type_traits>
 
 #include "common.h"
+#include "grouped_plan.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
@@ -45,7 +48,8 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 #ifndef SHARPI_GK
 #define SHARPI_GK 64
 #endif
-constexpr int GM = SHARPI_GM;  // rows per tile (the routing kernel lists tiles of this height)
+constexpr int GM = SHARPI_GM;  // rows per tile
+static_assert(GM == kPlanTileRows, "the routing kernel's plan is made for tiles of this height");
 constexpr int GMT = GM / 16;  // 16-row groups per tile
 #ifndef SHARPI_GW
 #define SHARPI_GW 8
@@ -60,10 +64,10 @@ constexpr int GK = SHARPI_GK;  // K per LDS stage
 constexpr int GPAD = GK;      // LDS row: no pad, the 16-byte chunks of a row are swizzled instead (xs_col)
 constexpr int GROWS = GW * 64 / (GK / 8);   // rows staged per pass: GK / 8 threads per row
 constexpr int GPASS = GM / GROWS;  // staging passes
-constexpr int kXcds = 8;           // accelerator dies, each with its own L2
+constexpr int kXcds = kPlanXcds;   // accelerator dies, each with its own L2
 constexpr int kAhead = SHARPI_GAHEAD;  // K stages of weights in flight per wave (2, 3 or 4)
 constexpr int GQ = SHARPI_GQ;       // 16-row groups whose LDS reads go out together (divides 4)
-constexpr int kHalves = 2;         // a tile's column blocks are split over this many XCDs
+constexpr int kHalves = kPlanHalves;   // an expert's column blocks are split into this many units
 
 // Where column `col` (a multiple of 8 elements = one 16-byte chunk) of LDS row `row` is kept: the
 // chunk index is XORed with bits 1..3 of the row.  The LDS serves a 16-byte read of a wave in four
@@ -75,16 +79,17 @@ constexpr int kHalves = 2;         // a tile's column blocks are split over this
 static_assert(GK == 64, "the swizzle assumes rows of eight 16-byte chunks");
 __device__ __forceinline__ int xs_col(int row, int col) { return col ^ (((row >> 1) & 7) << 3); }
 
-// The work of one tile of NQ * 64 rows (the block's rows, rounded up) against GN weight rows.
-template <typename TO, int NQ, bool PACKED, bool ACT>
+// The work of one tile of MT * 16 rows (the block's rows, rounded up) against GN weight rows.
+template <typename TO, int MT, bool PACKED, bool ACT>
 __device__ __forceinline__ void grouped_tile(const bf16_t* __restrict__ x, const bf16_t* __restrict__ We,
                                              TO* __restrict__ out, int N, int K, const int* __restrict__ a_rows,
                                              const float* __restrict__ act_scale, int row0, int row_end, int n_base,
                                              bf16_t (*xs)[GM][GPAD]) {
   static_assert(!ACT || NT == 2, "the SwiGLU form pairs one gate tile with one up tile");
   const int n_out = ACT ? N / 2 : N;            // output columns
-  constexpr int MT = NQ * 4;                    // 16-row groups
-  constexpr int PASS = NQ * 64 / GROWS;         // staging passes
+  constexpr int PASS = (MT * 16 + GROWS - 1) / GROWS;   // staging passes
+  constexpr int Q = MT % GQ == 0 ? GQ : 2;      // 16-row groups whose LDS reads go out together
+  static_assert(MT % Q == 0, "tile heights come in steps of 32 rows");
   const int lane = threadIdx.x & (kWave - 1);
   const int r = lane & 15, g = lane >> 4;
 
@@ -175,12 +180,12 @@ __device__ __forceinline__ void grouped_tile(const bf16_t* __restrict__ x, const
     for (int j = 0; j < GK / 32; ++j) {
       // 16-row groups GQ at a time: their LDS reads go out together, then their MFMAs
 #pragma unroll
-      for (int mq = 0; mq < MT; mq += GQ) {
-        bf16x8 xf[GQ];
+      for (int mq = 0; mq < MT; mq += Q) {
+        bf16x8 xf[Q];
 #pragma unroll
-        for (int i = 0; i < GQ; ++i) xf[i] = *reinterpret_cast<const bf16x8*>(&xs[par][(mq + i) * 16 + r][xs_col(r, j * 32 + g * 8)]);
+        for (int i = 0; i < Q; ++i) xf[i] = *reinterpret_cast<const bf16x8*>(&xs[par][(mq + i) * 16 + r][xs_col(r, j * 32 + g * 8)]);
 #pragma unroll
-        for (int i = 0; i < GQ; ++i)
+        for (int i = 0; i < Q; ++i)
 #pragma unroll
           for (int t = 0; t < NT; ++t)
             acc[t][mq + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[slot][j][t], xf[i], acc[t][mq + i], 0, 0, 0);
@@ -258,67 +263,74 @@ template <typename TO, bool PACKED, bool ACT>
 __global__ __launch_bounds__(GW* kWave, 2) void grouped_gemm_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ W, TO* __restrict__ out, int N, int K,
     const int* __restrict__ a_rows, const float* __restrict__ act_scale, const int* __restrict__ group_offsets,
-    const int* __restrict__ tile_expert, const int* __restrict__ tile_row0, const int* __restrict__ n_tiles,
-    int nb_per_unit) {
+    const int* __restrict__ plan, int n_experts, int nb_per_unit) {
   __shared__ __attribute__((aligned(16))) bf16_t xs[2][GM][GPAD];
   constexpr int kCols = ACT ? GN / 2 : GN;   // output columns of a block
   const int n_out = ACT ? N / 2 : N;
-  // Workgroups go to the 8 XCDs round-robin by their linear id, and each XCD has an L2 of its
-  // own.  All column blocks of one (tile, half of the columns) unit are therefore given ids that
-  // are equal modulo 8: the unit's x rows are fetched into one L2 and stay there.
+  // Workgroups go to the 8 XCDs round-robin by their linear id: this block is slot `slot` of XCD
+  // `xcd`, which walks its units one after the other, nb_per_unit column blocks times the unit's
+  // siblings each, the siblings of a column block side by side.
   const int xcd = blockIdx.x % kXcds;
   const int slot = blockIdx.x / kXcds;
-  const int unit = (slot / nb_per_unit) * kXcds + xcd;
-  const int tile = unit / kHalves;
-  const int nblock = (unit % kHalves) * nb_per_unit + slot % nb_per_unit;
-  if (tile >= n_tiles[0] || nblock * kCols >= n_out) return;
-  const int e = tile_expert[tile];
-  const int row0 = tile_row0[tile];
-  const int row_end = min(group_offsets[e + 1], row0 + GM);   // the tile's rows end here; later ones are another tile's
+  const int* px = plan + xcd * plan_stride(n_experts);
+  const int n_units = px[0];
+  const int* cum = px + 1;                     // cum[j] = siblings of the units before unit j
+  if (slot >= cum[n_units] * nb_per_unit) return;
+  int lo = 0, hi = n_units - 1;                // the unit whose slots hold this one
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (cum[mid] * nb_per_unit <= slot) lo = mid; else hi = mid - 1;
+  }
+  const int n_sib = cum[lo + 1] - cum[lo];
+  const int within = slot - cum[lo] * nb_per_unit;
+  const int sib = within % n_sib;
+  const int e = px[2 + plan_units_max(n_experts) + 2 * lo];
+  const int half = px[2 + plan_units_max(n_experts) + 2 * lo + 1];
+  const int nblock = half * nb_per_unit + within / n_sib;
+  if (nblock * kCols >= n_out) return;
+  const int first = group_offsets[e];
+  const int last = group_offsets[e + 1];
+  const int height = plan_height(last - first, n_sib);
+  const int row0 = first + sib * height;
+  const int row_end = min(last, row0 + height);
   const int n_rows = row_end - row0;
   if (n_rows <= 0) return;
   const int n_base = nblock * kCols + (threadIdx.x >> 6) * (ACT ? 16 : 16 * NT);
   const bf16_t* We = W + (size_t)e * N * K;
-  static_assert(GM % 64 == 0 && GM >= 128 && GM <= 256, "tile heights are compiled in steps of 64 rows, up to GM");
-  if (n_rows <= 64) {
-    grouped_tile<TO, 1, PACKED, ACT>(x, We, out, N, K, a_rows, act_scale, row0, row_end, n_base, xs);
-  } else if (n_rows <= 128) {
-    grouped_tile<TO, 2, PACKED, ACT>(x, We, out, N, K, a_rows, act_scale, row0, row_end, n_base, xs);
-  } else if constexpr (GM >= 192) {
-    if (GM == 192 || n_rows <= 192) {
-      grouped_tile<TO, 3, PACKED, ACT>(x, We, out, N, K, a_rows, act_scale, row0, row_end, n_base, xs);
-    } else if constexpr (GM >= 256) {
-      grouped_tile<TO, 4, PACKED, ACT>(x, We, out, N, K, a_rows, act_scale, row0, row_end, n_base, xs);
-    }
-  }
+  static_assert(GM == 192, "tile heights are compiled in steps of 32 rows up to 192");
+#define GT(MTV) grouped_tile<TO, MTV, PACKED, ACT>(x, We, out, N, K, a_rows, act_scale, row0, row_end, n_base, xs)
+  if (n_rows <= 32) GT(2);
+  else if (n_rows <= 64) GT(4);
+  else if (n_rows <= 96) GT(6);
+  else if (n_rows <= 128) GT(8);
+  else if (n_rows <= 160) GT(10);
+  else GT(12);
+#undef GT
 }
 
-static bool grouped_args_ok(int x_rows, int N, int K, int max_tiles, int packed, const int* group_offsets,
-                            const int* tile_expert, const int* tile_row0, const int* n_tiles) {
-  if (N <= 0 || (N & 3) || K <= 0 || K % GK != 0 || max_tiles <= 0) return false;
+static bool grouped_args_ok(int x_rows, int n_rows, int N, int K, int n_experts, int packed, const int* group_offsets,
+                            const int* plan) {
+  if (N <= 0 || (N & 3) || K <= 0 || K % GK != 0 || n_experts <= 0) return false;
   if (packed && ((N & 15) || (K & 127))) return false;
-  if (!group_offsets || !tile_expert || !tile_row0 || !n_tiles) return false;
+  if (!group_offsets || !plan) return false;
   // the kernel addresses x and one expert's weights with 32-bit element offsets
   return (long long)N * K <= 0x7fffffffLL && x_rows > 0 && (long long)x_rows * K <= 0x7fffffffLL;
 }
 
 // x [x_rows, K] bf16 (rows gathered through a_rows if given), W [E, N, K] bf16, out [n_rows, N];
-// group_offsets [E + 1]; tile_expert / tile_row0 [max_tiles], n_tiles [1] from the routing kernel
-// (tiles of sharpi_gemm_grouped_tile_rows() rows).  max_tiles bounds the grid.  packed: W is stored
-// tile by tile, [E][N/16][K/128][16 runs of 8 k][16 rows][8] (N % 16 == 0, K % 128 == 0).
+// group_offsets [n_experts + 1] and plan (grouped_plan.h) from the routing kernel.  packed: W is
+// stored tile by tile, [E][N/16][K/128][16 runs of 8 k][16 rows][8] (N % 16 == 0, K % 128 == 0).
 SHARPI_EXPORT int sharpi_gemm_grouped(const void* x, int x_rows, const void* W, void* out, int out_dtype, int n_rows,
-                                      int N, int K, const int* a_rows, const int* group_offsets, const int* tile_expert,
-                                      const int* tile_row0, const int* n_tiles, int max_tiles, int packed,
-                                      hipStream_t stream) {
+                                      int N, int K, const int* a_rows, const int* group_offsets, const int* plan,
+                                      int n_experts, int packed, hipStream_t stream) {
   if (n_rows <= 0) return SHARPI_OK;
-  if (!grouped_args_ok(x_rows, N, K, max_tiles, packed, group_offsets, tile_expert, tile_row0, n_tiles)) return SHARPI_ERR_ARG;
+  if (!grouped_args_ok(x_rows, n_rows, N, K, n_experts, packed, group_offsets, plan)) return SHARPI_ERR_ARG;
   const int nb_per_unit = ceil_div(ceil_div(N, GN), kHalves);
-  const int units = ceil_div(max_tiles * kHalves, kXcds) * kXcds;
-  dim3 grid(units * nb_per_unit), block(GW * kWave);
+  dim3 grid(kXcds * plan_sibling_slots_bound(n_rows, n_experts) * nb_per_unit), block(GW * kWave);
 #define GG_LAUNCH(TOV, PK)                                                                                          \
   grouped_gemm_kernel<TOV, PK, false><<<grid, block, 0, stream>>>((const bf16_t*)x, (const bf16_t*)W, (TOV*)out, N, \
-                                                                 K, a_rows, nullptr, group_offsets, tile_expert,    \
-                                                                 tile_row0, n_tiles, nb_per_unit)
+                                                                 K, a_rows, nullptr, group_offsets, plan, n_experts, \
+                                                                 nb_per_unit)
   if (out_dtype == DT_BF16) {
     if (packed) GG_LAUNCH(bf16_t, true); else GG_LAUNCH(bf16_t, false);
   } else if (out_dtype == DT_F32) {
@@ -335,23 +347,20 @@ SHARPI_EXPORT int sharpi_gemm_grouped(const void* x, int x_rows, const void* W, 
 // of every expert; out [n_rows, N/2] bf16 = silu(s g) * (s u) with g, u the two products rounded
 // to bfloat16 and s = act_scale[row] (null: 1).  N % 32 == 0; the rest as above.
 SHARPI_EXPORT int sharpi_gemm_grouped_swiglu(const void* x, int x_rows, const void* W, void* out, int n_rows, int N,
-                                             int K, const int* a_rows, const int* group_offsets,
-                                             const int* tile_expert, const int* tile_row0, const int* n_tiles,
-                                             int max_tiles, const float* act_scale, int packed, hipStream_t stream) {
+                                             int K, const int* a_rows, const int* group_offsets, const int* plan,
+                                             int n_experts, const float* act_scale, int packed, hipStream_t stream) {
   if (n_rows <= 0) return SHARPI_OK;
-  if ((N & 31) || !grouped_args_ok(x_rows, N, K, max_tiles, packed, group_offsets, tile_expert, tile_row0, n_tiles))
-    return SHARPI_ERR_ARG;
+  if ((N & 31) || !grouped_args_ok(x_rows, n_rows, N, K, n_experts, packed, group_offsets, plan)) return SHARPI_ERR_ARG;
   const int nb_per_unit = ceil_div(ceil_div(N / 2, GN / 2), kHalves);
-  const int units = ceil_div(max_tiles * kHalves, kXcds) * kXcds;
-  dim3 grid(units * nb_per_unit), block(GW * kWave);
+  dim3 grid(kXcds * plan_sibling_slots_bound(n_rows, n_experts) * nb_per_unit), block(GW * kWave);
   if (packed)
     grouped_gemm_kernel<bf16_t, true, true><<<grid, block, 0, stream>>>(
-        (const bf16_t*)x, (const bf16_t*)W, (bf16_t*)out, N, K, a_rows, act_scale, group_offsets, tile_expert,
-        tile_row0, n_tiles, nb_per_unit);
+        (const bf16_t*)x, (const bf16_t*)W, (bf16_t*)out, N, K, a_rows, act_scale, group_offsets, plan, n_experts,
+        nb_per_unit);
   else
     grouped_gemm_kernel<bf16_t, false, true><<<grid, block, 0, stream>>>(
-        (const bf16_t*)x, (const bf16_t*)W, (bf16_t*)out, N, K, a_rows, act_scale, group_offsets, tile_expert,
-        tile_row0, n_tiles, nb_per_unit);
+        (const bf16_t*)x, (const bf16_t*)W, (bf16_t*)out, N, K, a_rows, act_scale, group_offsets, plan, n_experts,
+        nb_per_unit);
   SHARPI_CHECK_LAUNCH();
   return SHARPI_OK;
 }

@@ -9,14 +9,14 @@
 //
 // moe_permute: one block. Counts rows per expert, prefix-sums them into offsets[E + 1] and
 // writes, in expert order, the token and weight of every (token, pick) pair plus the inverse
-// map inv_pos[t * k + j] = row in that order, and the list of (expert, first row) tiles of
-// tile_rows rows that the grouped product of many rows walks (tallest tiles first).  With shared_group the list gets one
+// map inv_pos[t * k + j] = row in that order, and the plan that the grouped product of many rows
+// walks (grouped_plan.h: units of sibling row tiles dealt to the XCDs).  With shared_group the list gets one
 // more group after the experts: every token once, weight 1 (an always-on expert that shares the
 // experts' weight tensor); offsets then has n_experts + 2 entries and the row arrays n_tokens more.
 #include "common.h"
+#include "grouped_plan.h"
 
 constexpr int kMaxExperts = 1024;
-constexpr int kSortTiles = 512;   // tile lists up to this long are ordered tallest first
 
 // One thread: gate the logits g[0 .. n_experts) in place, pick k of them (ascending scan with a
 // strict >, so the lowest index wins a tie) into ids / w.
@@ -261,15 +261,8 @@ SHARPI_EXPORT int sharpi_router_topk(const void* x, int x_dtype, const void* wr,
 // n_experts ints.  Every thread of the block calls it; the pairs must be visible to the block.
 __device__ void permute_block(const int* __restrict__ topk_ids, const float* __restrict__ topk_w,
                               int* __restrict__ offsets, int* __restrict__ sorted_token,
-                              float* __restrict__ sorted_w, int* __restrict__ inv_pos,
-                              int* __restrict__ tile_expert, int* __restrict__ tile_row0, int* __restrict__ n_tiles,
-                              int n_pairs, int k, int n_experts, int tile_rows, int max_tiles, int shared_group,
-                              int* count, int* cursor) {
-  // Tallest tiles first: a block's time grows with its tile's rows, and the blocks that start
-  // last should be the short ones.  (Only lists that fit the LDS arrays are put in order.)
-  __shared__ int s_expert[kSortTiles], s_row0[kSortTiles], s_rows[kSortTiles];
-  __shared__ int s_nt;
-  const bool sort_tiles = max_tiles <= kSortTiles;
+                              float* __restrict__ sorted_w, int* __restrict__ inv_pos, int* __restrict__ plan,
+                              int n_pairs, int k, int n_experts, int shared_group, int* count, int* cursor) {
   for (int e = threadIdx.x; e < n_experts; e += blockDim.x) count[e] = 0;
   __syncthreads();
   for (int i = threadIdx.x; i < n_pairs; i += blockDim.x) atomicAdd(&count[topk_ids[i]], 1);
@@ -282,28 +275,6 @@ __device__ void permute_block(const int* __restrict__ topk_ids, const float* __r
       run += count[e];
     }
     offsets[n_experts] = run;
-    // row tiles of the experts that have rows, for the grouped product of many rows; up to
-    // kSortTiles of them are listed in LDS first and put in order below
-    int nt = 0;
-    run = 0;
-    for (int e = 0; e < n_experts; ++e) {
-      for (int r0 = run; r0 < run + count[e]; r0 += tile_rows) {
-        if (nt < max_tiles) {
-          if (sort_tiles) {
-            s_expert[nt] = e;
-            s_row0[nt] = r0;
-            s_rows[nt] = min(tile_rows, run + count[e] - r0);
-          } else {
-            tile_expert[nt] = e;
-            tile_row0[nt] = r0;
-          }
-          ++nt;
-        }
-      }
-      run += count[e];
-    }
-    n_tiles[0] = nt;
-    s_nt = nt;
     // an always-on expert as one more group: every token once, in token order, with weight 1
     if (shared_group) offsets[n_experts + 1] = run + n_pairs / k;
   }
@@ -313,16 +284,52 @@ __device__ void permute_block(const int* __restrict__ topk_ids, const float* __r
       sorted_w[n_pairs + t] = 1.0f;
     }
   }
-  __syncthreads();
-  if (sort_tiles) {
-    // a tile's place = the number of tiles that are taller, or as tall and listed before it
-    for (int i = threadIdx.x; i < s_nt; i += blockDim.x) {
-      int place = 0;
-      for (int j = 0; j < s_nt; ++j) place += (s_rows[j] > s_rows[i] || (s_rows[j] == s_rows[i] && j < i)) ? 1 : 0;
-      tile_expert[place] = s_expert[i];
-      tile_row0[place] = s_row0[i];
+  if (plan) {
+    // The plan of the grouped product (grouped_plan.h).  Experts in the order of their sibling
+    // counts, then of their rows (most first: the blocks that start last should be the short
+    // ones); expert of rank r gives units 2r and 2r + 1, unit u goes to row u / 8 of the XCDs,
+    // rows alternating in direction so that the XCDs' loads stay level.
+    const int stride = plan_stride(n_experts);
+    const int U = plan_units_max(n_experts);
+    for (int e = threadIdx.x; e < n_experts; e += blockDim.x) {
+      if (count[e] == 0) continue;
+      const int se = plan_siblings(count[e]);
+      int rank = 0;
+      for (int j = 0; j < n_experts; ++j) {
+        if (count[j] == 0 || j == e) continue;
+        const int sj = plan_siblings(count[j]);
+        rank += (sj > se || (sj == se && (count[j] > count[e] || (count[j] == count[e] && j < e)))) ? 1 : 0;
+      }
+      for (int half = 0; half < kPlanHalves; ++half) {
+        const int u = kPlanHalves * rank + half;
+        const int pos = u / kPlanXcds;
+        const int xcd = (pos & 1) ? kPlanXcds - 1 - u % kPlanXcds : u % kPlanXcds;
+        int* px = plan + xcd * stride;
+        px[2 + U + 2 * pos] = e;
+        px[2 + U + 2 * pos + 1] = half;
+      }
+    }
+    __syncthreads();
+    if (threadIdx.x < kPlanXcds) {
+      int busy = 0;
+      for (int e = 0; e < n_experts; ++e) busy += count[e] > 0 ? 1 : 0;
+      const int units = kPlanHalves * busy;
+      const int x = threadIdx.x;
+      int* px = plan + x * stride;
+      // XCD x holds, of every full row of 8 units, one; of the last row, the units that exist
+      int n = 0, run = 0;
+      px[1] = 0;
+      for (int pos = 0; pos * kPlanXcds < units; ++pos) {
+        const int u = pos * kPlanXcds + ((pos & 1) ? kPlanXcds - 1 - x : x);
+        if (u >= units) continue;     // (only in the last row; the units of a row are dealt in order, so n == pos here)
+        run += plan_siblings(count[px[2 + U + 2 * pos]]);
+        px[2 + n] = run;
+        ++n;
+      }
+      px[0] = n;
     }
   }
+  __syncthreads();
   for (int i = threadIdx.x; i < n_pairs; i += blockDim.x) {
     const int e = topk_ids[i];
     const int r = atomicAdd(&cursor[e], 1);
@@ -337,32 +344,27 @@ __global__ __launch_bounds__(1024) void moe_permute_kernel(const int* __restrict
                                                            int* __restrict__ offsets,
                                                            int* __restrict__ sorted_token,
                                                            float* __restrict__ sorted_w,
-                                                           int* __restrict__ inv_pos,
-                                                           int* __restrict__ tile_expert,
-                                                           int* __restrict__ tile_row0,
-                                                           int* __restrict__ n_tiles, int n_pairs, int k,
-                                                           int n_experts, int tile_rows, int max_tiles,
-                                                           int shared_group) {
+                                                           int* __restrict__ inv_pos, int* __restrict__ plan,
+                                                           int n_pairs, int k, int n_experts, int shared_group) {
   __shared__ int count[kMaxExperts];
   __shared__ int cursor[kMaxExperts];
-  permute_block(topk_ids, topk_w, offsets, sorted_token, sorted_w, inv_pos, tile_expert, tile_row0, n_tiles,
-                n_pairs, k, n_experts, tile_rows, max_tiles, shared_group, count, cursor);
+  permute_block(topk_ids, topk_w, offsets, sorted_token, sorted_w, inv_pos, plan, n_pairs, k, n_experts,
+                shared_group, count, cursor);
 }
 
+// plan: plan_ints(n_experts) ints (grouped_plan.h) for the grouped product of many rows, or null.
 SHARPI_EXPORT int sharpi_moe_permute(const int* topk_ids, const float* topk_w, int* offsets, int* sorted_token,
-                                     float* sorted_w, int* inv_pos, int* tile_expert, int* tile_row0,
-                                     int* n_tiles, int n_tokens, int k, int n_experts, int tile_rows,
-                                     int max_tiles, int shared_group, hipStream_t stream) {
+                                     float* sorted_w, int* inv_pos, int* plan, int plan_len, int n_tokens, int k,
+                                     int n_experts, int shared_group, hipStream_t stream) {
   if (n_experts <= 0 || n_experts > kMaxExperts || k <= 0) return SHARPI_ERR_ARG;
-  if (n_tokens < 0 || tile_rows <= 0) return SHARPI_ERR_ARG;
-  if (max_tiles < (n_tokens * k + tile_rows - 1) / tile_rows + n_experts) return SHARPI_ERR_ARG;
-  moe_permute_kernel<<<1, 1024, 0, stream>>>(topk_ids, topk_w, offsets, sorted_token, sorted_w, inv_pos,
-                                             tile_expert, tile_row0, n_tiles, n_tokens * k, k, n_experts,
-                                             tile_rows, max_tiles, shared_group);
+  if (n_tokens < 0) return SHARPI_ERR_ARG;
+  if (plan && plan_len < plan_ints(n_experts)) return SHARPI_ERR_ARG;
+  moe_permute_kernel<<<1, 1024, 0, stream>>>(topk_ids, topk_w, offsets, sorted_token, sorted_w, inv_pos, plan,
+                                             n_tokens * k, k, n_experts, shared_group);
   SHARPI_CHECK_LAUNCH();
   return SHARPI_OK;
 }
 
-SHARPI_EXPORT int sharpi_router_sorted_tiles() { return kSortTiles; }
+SHARPI_EXPORT int sharpi_grouped_plan_ints(int n_experts) { return plan_ints(n_experts); }
 SHARPI_EXPORT int sharpi_router_max_experts() { return kMaxExperts; }
 SHARPI_EXPORT int sharpi_add_rmsnorm_router_max_hidden() { return kFusedMaxHidden; }

@@ -656,15 +656,12 @@ def add_rmsnorm_router(h: torch.Tensor, delta: Optional[torch.Tensor], weight: O
     return out, ids, wts
 
 
-GROUPED_TILE_ROWS = _lib.GROUPED_TILE_ROWS   # rows per tile of the grouped product (csrc/gemm_grouped.hip GM)
-SORTED_TILE_LISTS = _lib.SORTED_TILE_LISTS   # tile lists up to this long come tallest first (csrc/router.hip kSortTiles)
 
 
 class Routing:
     """The expert-sorted view of a step's (token, pick) pairs, all on the device."""
 
-    __slots__ = ("n_tokens", "k", "n_experts", "n_groups", "offsets", "sorted_token", "sorted_w", "inv_pos",
-                 "tile_expert", "tile_row0", "n_tiles", "max_tiles")
+    __slots__ = ("n_tokens", "k", "n_experts", "n_groups", "offsets", "sorted_token", "sorted_w", "inv_pos", "plan")
 
     @property
     def n_rows(self) -> int:
@@ -672,27 +669,32 @@ class Routing:
         return self.n_tokens * self.k + (self.n_tokens if self.n_groups > self.n_experts else 0)
 
 
+_PLAN_INTS: dict = {}
+
+
 def _new_routing(T: int, k: int, n_experts: int, shared_group: bool, dev) -> Routing:
     rt = Routing()
     rt.n_tokens, rt.k, rt.n_experts = T, k, n_experts
     rt.n_groups = n_experts + (1 if shared_group else 0)
     rows = T * k + (T if shared_group else 0)
-    rt.max_tiles = (T * k + GROUPED_TILE_ROWS - 1) // GROUPED_TILE_ROWS + n_experts
-    ints = torch.empty(rt.n_groups + 1 + rows + T * k + 2 * rt.max_tiles + 1, dtype=torch.int32, device=dev)
+    if n_experts not in _PLAN_INTS:
+        _PLAN_INTS[n_experts] = _lib.grouped_plan_ints(n_experts)
+    # (a shared group rides with the experts only in the few-rows product, which needs no plan)
+    n_plan = 0 if shared_group else _PLAN_INTS[n_experts]
+    ints = torch.empty(rt.n_groups + 1 + rows + T * k + n_plan, dtype=torch.int32, device=dev)
     o = 0
     rt.offsets = ints[o:o + rt.n_groups + 1]; o += rt.n_groups + 1
     rt.sorted_token = ints[o:o + rows]; o += rows
     rt.inv_pos = ints[o:o + T * k]; o += T * k
-    rt.tile_expert = ints[o:o + rt.max_tiles]; o += rt.max_tiles
-    rt.tile_row0 = ints[o:o + rt.max_tiles]; o += rt.max_tiles
-    rt.n_tiles = ints[o:o + 1]
+    rt.plan = ints[o:o + n_plan] if n_plan else None
     rt.sorted_w = torch.empty(rows, dtype=torch.float32, device=dev)
     return rt
 
 
 def moe_permute(ids: torch.Tensor, wts: torch.Tensor, n_experts: int, shared_group: bool = False) -> Routing:
     """(token, pick) pairs sorted by expert: offsets [E+1], sorted_token, sorted_w, inv_pos, and
-    the list of row tiles (GROUPED_TILE_ROWS high) of the experts that have rows.  With
+    the plan of the grouped product for many rows, which
+    says how the experts' row tiles are dealt to the blocks (csrc/grouped_plan.h).  With
     shared_group one more group follows the experts: every token once with weight 1."""
     _dev(ids, wts)
     _i32(ids, "ids")
@@ -700,8 +702,8 @@ def moe_permute(ids: torch.Tensor, wts: torch.Tensor, n_experts: int, shared_gro
     T, k = ids.shape
     rt = _new_routing(T, k, n_experts, shared_group, ids.device)
     _run("sharpi_moe_permute", _ptr(ids), _ptr(wts), _ptr(rt.offsets), _ptr(rt.sorted_token), _ptr(rt.sorted_w),
-         _ptr(rt.inv_pos), _ptr(rt.tile_expert), _ptr(rt.tile_row0), _ptr(rt.n_tiles), T, k, n_experts,
-         GROUPED_TILE_ROWS, rt.max_tiles, 1 if shared_group else 0, _stream())
+         _ptr(rt.inv_pos), _ptr(rt.plan), rt.plan.numel() if rt.plan is not None else 0, T, k, n_experts,
+         1 if shared_group else 0, _stream())
     return rt
 
 
@@ -724,9 +726,10 @@ def gemm_grouped(x: torch.Tensor, w, rt: Routing, gather: bool, out_dtype: torch
     _need(K % 64 == 0 and N % 4 == 0, "gemm_grouped: K % 64 == 0 and N % 4 == 0 wanted")
     _need(x.shape[0] == (rt.n_tokens if gather else rt.n_rows), "gemm_grouped: x has the wrong number of rows")
     out = torch.empty(rt.n_rows, N, dtype=out_dtype, device=x.device)
+    _need(rt.plan is not None, "gemm_grouped: this routing was made without a plan (a shared group)")
     _run("sharpi_gemm_grouped", _ptr(x), x.shape[0], _ptr(w), _ptr(out), _code(out_dtype), rt.n_rows, N, K,
-         _ptr(rt.sorted_token) if gather else None, _ptr(rt.offsets), _ptr(rt.tile_expert), _ptr(rt.tile_row0),
-         _ptr(rt.n_tiles), rt.max_tiles, 1 if packed else 0, _stream())
+         _ptr(rt.sorted_token) if gather else None, _ptr(rt.offsets), _ptr(rt.plan), rt.n_experts,
+         1 if packed else 0, _stream())
     return out
 
 
@@ -745,9 +748,9 @@ def gemm_grouped_swiglu(x: torch.Tensor, w, rt: Routing, scale: Optional[torch.T
     if scale is not None:
         _need(scale.dtype == torch.float32 and scale.shape == (rt.n_rows,), "gemm_grouped_swiglu: scale must be float32 [n_rows]")
     out = torch.empty(rt.n_rows, N // 2, dtype=torch.bfloat16, device=x.device)
+    _need(rt.plan is not None, "gemm_grouped_swiglu: this routing was made without a plan (a shared group)")
     _run("sharpi_gemm_grouped_swiglu", _ptr(x), x.shape[0], _ptr(w), _ptr(out), rt.n_rows, N, K, _ptr(rt.sorted_token),
-         _ptr(rt.offsets), _ptr(rt.tile_expert), _ptr(rt.tile_row0), _ptr(rt.n_tiles), rt.max_tiles, _ptr(scale),
-         1 if packed else 0, _stream())
+         _ptr(rt.offsets), _ptr(rt.plan), rt.n_experts, _ptr(scale), 1 if packed else 0, _stream())
     return out
 
 

@@ -35,9 +35,9 @@ _SIGNATURES = {
     "sharpi_gemm_skinny_picked": [P, P, P, I, I, I, P, P, I, I, I, I, I, I, I, I, I, P],
     "sharpi_add_rmsnorm_router": [P, P, P, I, P, I, I, F, P, I, P, P, I, I, I, I, P],
     "sharpi_router_topk": [P, I, P, I, P, P, P, I, I, I, I, I, I, P],
-    "sharpi_moe_permute": [P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, P],
-    "sharpi_gemm_grouped": [P, I, P, P, I, I, I, I, P, P, P, P, P, I, I, P],
-    "sharpi_gemm_grouped_swiglu": [P, I, P, P, I, I, I, P, P, P, P, P, I, P, I, P],
+    "sharpi_moe_permute": [P, P, P, P, P, P, P, I, I, I, I, I, P],
+    "sharpi_gemm_grouped": [P, I, P, P, I, I, I, I, P, P, P, I, I, P],
+    "sharpi_gemm_grouped_swiglu": [P, I, P, P, I, I, I, P, P, P, I, P, I, P],
     "sharpi_argmax_rows": [P, P, I, I, P],
     "sharpi_sample_rows": [P, P, P, P, P, P, P, P, I, I, P],
     "sharpi_edit_logits": [P, P, P, P, P, P, P, P, I, I, P],
@@ -50,16 +50,12 @@ _OPTIONAL_SIGNATURES: dict = {}
 # it was built with, and a build with other sizes is refused at load (it would compute wrong results).
 DECODE_RUN_KEYS = 256       # keys per block of the decode attention kernel
 PREFILL_TILE_TOKENS = 128   # tokens per block of the prefill attention kernel
-GROUPED_TILE_ROWS = 192     # rows per tile of the grouped product for many rows
-SORTED_TILE_LISTS = 512     # tile lists up to this long come tallest first
 PICKED_MAX_PAIRS = 64       # (token, pick) pairs the few-rows product takes straight from the router's picks
 FUSED_NORM_ROUTER_MAX_HIDDEN = 8192   # widest row of the norm + router kernel
 ROUTER_MAX_EXPERTS = 1024   # experts the routing kernels hold scores for
 _BUILT_WITH = {
     "sharpi_attention_decode_split_keys": DECODE_RUN_KEYS,
     "sharpi_attention_prefill_tile_tokens": PREFILL_TILE_TOKENS,
-    "sharpi_gemm_grouped_tile_rows": GROUPED_TILE_ROWS,
-    "sharpi_router_sorted_tiles": SORTED_TILE_LISTS,
     "sharpi_router_max_experts": ROUTER_MAX_EXPERTS,
     "sharpi_gemm_skinny_max_picked": PICKED_MAX_PAIRS,
     "sharpi_add_rmsnorm_router_max_hidden": FUSED_NORM_ROUTER_MAX_HIDDEN,
@@ -123,6 +119,23 @@ def attention_takes(kind: str, hd: int) -> bool:
         fn.argtypes, fn.restype = [c_int], c_int
         _takes[key] = bool(fn(int(hd)))
     return _takes[key]
+
+
+def grouped_tile_rows() -> int:
+    """Rows of the tallest tile of the grouped product for many rows (an expert with more rows is
+    cut into sibling tiles): the library says what it was built with."""
+    if "tile_rows" not in _takes:
+        fn = load().sharpi_gemm_grouped_tile_rows
+        fn.argtypes, fn.restype = [], c_int
+        _takes["tile_rows"] = int(fn())
+    return _takes["tile_rows"]
+
+
+def grouped_plan_ints(n_experts: int) -> int:
+    """Length of the plan that the routing kernel writes for the grouped product of many rows."""
+    fn = load().sharpi_grouped_plan_ints
+    fn.argtypes, fn.restype = [c_int], c_int
+    return int(fn(int(n_experts)))
 
 
 def register_signature(name: str, argtypes) -> None:

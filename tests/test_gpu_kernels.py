@@ -349,13 +349,48 @@ def test_router_and_permute(T, E, k, H, dtype):
         assert all(int(flat[i]) == e for i in (inv >= off[e]).logical_and(inv < off[e + 1]).nonzero().flatten().tolist())
     assert torch.equal(st[inv].long(), torch.arange(T * k) // k)
     assert torch.equal(sw[inv], wts.flatten().cpu())
-    nt = int(rt.n_tiles.cpu())
-    tiles = list(zip(rt.tile_expert.cpu().tolist()[:nt], rt.tile_row0.cpu().tolist()[:nt]))
-    want = [(e, r0) for e in range(E) for r0 in range(off[e], off[e + 1], ops.GROUPED_TILE_ROWS)]
-    # tallest tiles first (the blocks that start last should be the short ones), otherwise in expert order
-    if rt.max_tiles <= ops.SORTED_TILE_LISTS:       # (longer lists stay in expert order)
-        want.sort(key=lambda t: -min(ops.GROUPED_TILE_ROWS, off[t[0] + 1] - t[1]))
-    assert tiles == want
+    _check_plan(ops, rt, counts)
+
+
+def _check_plan(ops, rt, counts):
+    """The plan of the grouped product for many rows: every expert with rows gives two units (the
+    halves of its weight rows), each once, dealt to the 8 XCDs so that their sibling counts stay
+    level; an XCD's running sums are those of its units' siblings; the experts with most siblings
+    (then most rows) come first."""
+    E = len(counts)
+    tile = ops._lib.grouped_tile_rows()
+    plan = rt.plan.cpu().tolist()
+    U = 2 * E
+    stride = 2 + 3 * U
+    assert len(plan) == 8 * stride
+    seen, loads = [], []
+    for x in range(8):
+        px = plan[x * stride:(x + 1) * stride]
+        n = px[0]
+        cum = px[1:2 + n]
+        assert cum[0] == 0
+        units = [(px[2 + U + 2 * j], px[2 + U + 2 * j + 1]) for j in range(n)]
+        for j, (e, half) in enumerate(units):
+            assert counts[e] > 0 and half in (0, 1)
+            assert cum[j + 1] - cum[j] == -(-counts[e] // tile)
+        sibs = [-(-counts[e] // tile) for e, _ in units]
+        assert sibs == sorted(sibs, reverse=True)
+        seen += units
+        loads.append(cum[-1])
+    busy = [e for e in range(E) if counts[e] > 0]
+    assert sorted(seen) == sorted((e, h) for e in busy for h in (0, 1))
+    assert max(loads) - min(loads) <= max([-(-c // tile) for c in counts] + [0])
+
+
+@pytest.mark.parametrize("counts", [[500, 0, 193, 192, 1, 64, 0, 700], [128] * 16, [3], [0, 0, 5000]])
+def test_plan_of_the_grouped_product(counts):
+    ops = _ops()
+    E = len(counts)
+    ids = torch.cat([torch.full((c,), e, dtype=torch.int32) for e, c in enumerate(counts)])
+    ids = ids[torch.randperm(len(ids), generator=torch.Generator().manual_seed(1))].view(-1, 1).to(DEV)
+    rt = ops.moe_permute(ids, torch.ones(ids.shape, device=DEV), E)
+    assert [b - a for a, b in zip(rt.offsets.cpu().tolist(), rt.offsets.cpu().tolist()[1:])] == counts
+    _check_plan(ops, rt, counts)
 
 
 @pytest.mark.parametrize("T,H,E,k", [(1, 5120, 16, 1), (8, 5120, 16, 1), (16, 256, 5, 2), (3, 8192, 128, 4), (5, 136, 3, 3)])
@@ -444,7 +479,7 @@ def test_gemm_skinny_swiglu_equals_product_then_activation(M, E, I, K):
 # the last two are deep enough in K for the kernel's steady loop (and its tail of 4 and of 1 stages)
 @pytest.mark.parametrize("T,E,k,N,K", [(300, 4, 1, 264, 256), (700, 16, 2, 512, 128), (65, 3, 1, 20, 384),
                                        (500, 5, 1, 200, 640), (260, 2, 2, 136, 1216), (500, 5, 1, 208, 640),
-                                       (260, 2, 2, 144, 1280), (70, 3, 1, 16, 128)])
+                                       (260, 2, 2, 144, 1280), (70, 3, 1, 16, 128), (1700, 2, 1, 264, 256)])
 def test_gemm_grouped(T, E, k, N, K):
     ops = _ops()
     x = _rand(T, K, dtype=torch.bfloat16, seed=1)
