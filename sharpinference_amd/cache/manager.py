@@ -153,7 +153,7 @@ class CacheManager:
                     # [page, kv head, head_dim, position], the layout the matrix-core kernels read
                     self.k[i] = torch.zeros((n, spec.num_kv_heads, page_size, spec.head_dim), dtype=dtype,
                                             device=self.device)
-                    self.v[i] = torch.zeros((n, spec.num_kv_heads, spec.head_dim, page_size), dtype=dtype,
+                    self.v[i] = torch.zeros((n, spec.num_kv_heads, spec.value_dim, page_size), dtype=dtype,
                                             device=self.device)
                 elif isinstance(spec, StateSpec):
                     self.state[i] = torch.zeros((max_requests + 1, *spec.shape), dtype=spec.dtype, device=self.device)
@@ -167,7 +167,7 @@ class CacheManager:
             b = 0
             for s in g.slots:
                 spec = self.slot_specs[s]
-                b += 2 * spec.num_kv_heads * spec.head_dim * self.page_size * width
+                b += spec.num_kv_heads * (spec.head_dim + spec.value_dim) * self.page_size * width
             out.append(b)
         return out
 

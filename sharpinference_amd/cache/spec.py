@@ -19,10 +19,19 @@ WINDOW_NONE, WINDOW_CHUNK, WINDOW_SLIDING = 0, 1, 2
 
 @dataclass(frozen=True)
 class KVSpec:
+    """Paged keys and values of one layer.  ``head_dim`` is the width of a key; ``v_head_dim`` the
+    width of a value where it differs (0: the same).  Keys are kept [page, kv head, position,
+    head_dim], values transposed inside the page, [page, kv head, v_head_dim, position]."""
+
     num_kv_heads: int
     head_dim: int
     window_kind: int = WINDOW_NONE
     window: int = 0
+    v_head_dim: int = 0
+
+    @property
+    def value_dim(self) -> int:
+        return self.v_head_dim or self.head_dim
 
     def first_visible(self, pos: int) -> int:
         """The earliest key position a query at `pos` can see."""

@@ -29,7 +29,7 @@ HIPCC_FLAGS = [
     f"--offload-arch={ARCH}",
     "-fvisibility=hidden",
     "-Wno-unused-result",
-    # packed FP32 instructions are kept out of the generated code on this hardware pool
+    # packed FP32 instructions (v_pk_*_f32) are kept out of the generated code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
 

@@ -67,7 +67,6 @@ constexpr int GPASS = GM / GROWS;  // staging passes
 constexpr int kXcds = kPlanXcds;   // accelerator dies, each with its own L2
 constexpr int kAhead = SHARPI_GAHEAD;  // K stages of weights in flight per wave (2, 3 or 4)
 constexpr int GQ = SHARPI_GQ;       // 16-row groups whose LDS reads go out together (divides 4)
-constexpr int kHalves = kPlanHalves;   // an expert's column blocks are split into this many units
 
 // Where column `col` (a multiple of 8 elements = one 16-byte chunk) of LDS row `row` is kept: the
 // chunk index is XORed with bits 1..3 of the row.  The LDS serves a 16-byte read of a wave in four
@@ -263,36 +262,39 @@ template <typename TO, bool PACKED, bool ACT>
 __global__ __launch_bounds__(GW* kWave, 2) void grouped_gemm_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ W, TO* __restrict__ out, int N, int K,
     const int* __restrict__ a_rows, const float* __restrict__ act_scale, const int* __restrict__ group_offsets,
-    const int* __restrict__ plan, int n_experts, int nb_per_unit) {
+    const int* __restrict__ plan, int n_groups, int nb) {
   __shared__ __attribute__((aligned(16))) bf16_t xs[2][GM][GPAD];
   constexpr int kCols = ACT ? GN / 2 : GN;   // output columns of a block
   const int n_out = ACT ? N / 2 : N;
   // Workgroups go to the 8 XCDs round-robin by their linear id: this block is slot `slot` of XCD
-  // `xcd`, which walks its units one after the other, nb_per_unit column blocks times the unit's
-  // siblings each, the siblings of a column block side by side.
+  // `xcd`, which walks its units one after the other: a unit's column blocks times its siblings,
+  // the siblings of a column block side by side.
   const int xcd = blockIdx.x % kXcds;
-  const int slot = blockIdx.x / kXcds;
-  const int* px = plan + xcd * plan_stride(n_experts);
+  int slot = blockIdx.x / kXcds;
+  const int* px = plan + xcd * plan_stride(n_groups);
   const int n_units = px[0];
-  const int* cum = px + 1;                     // cum[j] = siblings of the units before unit j
-  if (slot >= cum[n_units] * nb_per_unit) return;
-  int lo = 0, hi = n_units - 1;                // the unit whose slots hold this one
-  while (lo < hi) {
-    const int mid = (lo + hi + 1) >> 1;
-    if (cum[mid] * nb_per_unit <= slot) lo = mid; else hi = mid - 1;
+  int e = -1, n_sib = 1, col0 = 0;
+  for (int j = 0; j < n_units; ++j) {          // (a handful of units per XCD)
+    const int* pu = px + 1 + 4 * j;
+    const int first = plan_part_first(pu[1], pu[2], nb);
+    const int slots = (plan_part_first(pu[1] + 1, pu[2], nb) - first) * pu[3];
+    if (slot < slots) {
+      e = pu[0];
+      n_sib = pu[3];
+      col0 = first;
+      break;
+    }
+    slot -= slots;
   }
-  const int n_sib = cum[lo + 1] - cum[lo];
-  const int within = slot - cum[lo] * nb_per_unit;
-  const int sib = within % n_sib;
-  const int e = px[2 + plan_units_max(n_experts) + 2 * lo];
-  const int half = px[2 + plan_units_max(n_experts) + 2 * lo + 1];
-  const int nblock = half * nb_per_unit + within / n_sib;
+  if (e < 0) return;                           // behind the XCD's last unit
+  const int sib = slot % n_sib;
+  const int nblock = col0 + slot / n_sib;
   if (nblock * kCols >= n_out) return;
-  const int first = group_offsets[e];
-  const int last = group_offsets[e + 1];
-  const int height = plan_height(last - first, n_sib);
-  const int row0 = first + sib * height;
-  const int row_end = min(last, row0 + height);
+  const int first_row = group_offsets[e];
+  const int last_row = group_offsets[e + 1];
+  const int height = plan_height(last_row - first_row, n_sib);
+  const int row0 = first_row + sib * height;
+  const int row_end = min(last_row, row0 + height);
   const int n_rows = row_end - row0;
   if (n_rows <= 0) return;
   const int n_base = nblock * kCols + (threadIdx.x >> 6) * (ACT ? 16 : 16 * NT);
@@ -308,29 +310,37 @@ __global__ __launch_bounds__(GW* kWave, 2) void grouped_gemm_kernel(
 #undef GT
 }
 
-static bool grouped_args_ok(int x_rows, int n_rows, int N, int K, int n_experts, int packed, const int* group_offsets,
+static bool grouped_args_ok(int x_rows, int n_rows, int N, int K, int n_groups, int packed, const int* group_offsets,
                             const int* plan) {
-  if (N <= 0 || (N & 3) || K <= 0 || K % GK != 0 || n_experts <= 0) return false;
+  if (N <= 0 || (N & 3) || K <= 0 || K % GK != 0 || n_groups <= 0) return false;
   if (packed && ((N & 15) || (K & 127))) return false;
   if (!group_offsets || !plan) return false;
-  // the kernel addresses x and one expert's weights with 32-bit element offsets
+  // the kernel addresses x and one group's weights with 32-bit element offsets
   return (long long)N * K <= 0x7fffffffLL && x_rows > 0 && (long long)x_rows * K <= 0x7fffffffLL;
 }
 
-// x [x_rows, K] bf16 (rows gathered through a_rows if given), W [E, N, K] bf16, out [n_rows, N];
-// group_offsets [n_experts + 1] and plan (grouped_plan.h) from the routing kernel.  packed: W is
-// stored tile by tile, [E][N/16][K/128][16 runs of 8 k][16 rows][8] (N % 16 == 0, K % 128 == 0).
+static bool grouped_grid(int n_rows, int n_groups, int nb, dim3* grid) {
+  const long long blocks = (long long)kXcds * plan_slots_bound(n_rows, n_groups, nb);
+  if (blocks > 0x7fffffffLL) return false;
+  *grid = dim3((unsigned)blocks);
+  return true;
+}
+
+// x [x_rows, K] bf16 (rows gathered through a_rows if given), W [>= n_groups, N, K] bf16, out
+// [n_rows, N]; group_offsets [n_groups + 1] and plan (grouped_plan.h) from the routing kernel.
+// packed: W is stored tile by tile, [E][N/16][K/128][16 runs of 8 k][16 rows][8] (N % 16 == 0,
+// K % 128 == 0).
 SHARPI_EXPORT int sharpi_gemm_grouped(const void* x, int x_rows, const void* W, void* out, int out_dtype, int n_rows,
                                       int N, int K, const int* a_rows, const int* group_offsets, const int* plan,
-                                      int n_experts, int packed, hipStream_t stream) {
+                                      int n_groups, int packed, hipStream_t stream) {
   if (n_rows <= 0) return SHARPI_OK;
-  if (!grouped_args_ok(x_rows, n_rows, N, K, n_experts, packed, group_offsets, plan)) return SHARPI_ERR_ARG;
-  const int nb_per_unit = ceil_div(ceil_div(N, GN), kHalves);
-  dim3 grid(kXcds * plan_sibling_slots_bound(n_rows, n_experts) * nb_per_unit), block(GW * kWave);
+  if (!grouped_args_ok(x_rows, n_rows, N, K, n_groups, packed, group_offsets, plan)) return SHARPI_ERR_ARG;
+  const int nb = ceil_div(N, GN);
+  dim3 grid, block(GW * kWave);
+  if (!grouped_grid(n_rows, n_groups, nb, &grid)) return SHARPI_ERR_ARG;
 #define GG_LAUNCH(TOV, PK)                                                                                          \
   grouped_gemm_kernel<TOV, PK, false><<<grid, block, 0, stream>>>((const bf16_t*)x, (const bf16_t*)W, (TOV*)out, N, \
-                                                                 K, a_rows, nullptr, group_offsets, plan, n_experts, \
-                                                                 nb_per_unit)
+                                                                 K, a_rows, nullptr, group_offsets, plan, n_groups, nb)
   if (out_dtype == DT_BF16) {
     if (packed) GG_LAUNCH(bf16_t, true); else GG_LAUNCH(bf16_t, false);
   } else if (out_dtype == DT_F32) {
@@ -343,24 +353,23 @@ SHARPI_EXPORT int sharpi_gemm_grouped(const void* x, int x_rows, const void* W, 
   return SHARPI_OK;
 }
 
-// The grouped product with SwiGLU in its epilogue: W [E, N, K] holds gate rows [0, N/2) then up rows
-// of every expert; out [n_rows, N/2] bf16 = silu(s g) * (s u) with g, u the two products rounded
-// to bfloat16 and s = act_scale[row] (null: 1).  N % 32 == 0; the rest as above.
+// The grouped product with SwiGLU in its epilogue: W [>= n_groups, N, K] holds gate rows [0, N/2)
+// then up rows of every group; out [n_rows, N/2] bf16 = silu(s g) * (s u) with g, u the two
+// products rounded to bfloat16 and s = act_scale[row] (null: 1).  N % 32 == 0; the rest as above.
 SHARPI_EXPORT int sharpi_gemm_grouped_swiglu(const void* x, int x_rows, const void* W, void* out, int n_rows, int N,
                                              int K, const int* a_rows, const int* group_offsets, const int* plan,
-                                             int n_experts, const float* act_scale, int packed, hipStream_t stream) {
+                                             int n_groups, const float* act_scale, int packed, hipStream_t stream) {
   if (n_rows <= 0) return SHARPI_OK;
-  if ((N & 31) || !grouped_args_ok(x_rows, n_rows, N, K, n_experts, packed, group_offsets, plan)) return SHARPI_ERR_ARG;
-  const int nb_per_unit = ceil_div(ceil_div(N / 2, GN / 2), kHalves);
-  dim3 grid(kXcds * plan_sibling_slots_bound(n_rows, n_experts) * nb_per_unit), block(GW * kWave);
+  if ((N & 31) || !grouped_args_ok(x_rows, n_rows, N, K, n_groups, packed, group_offsets, plan)) return SHARPI_ERR_ARG;
+  const int nb = ceil_div(N / 2, GN / 2);
+  dim3 grid, block(GW * kWave);
+  if (!grouped_grid(n_rows, n_groups, nb, &grid)) return SHARPI_ERR_ARG;
   if (packed)
     grouped_gemm_kernel<bf16_t, true, true><<<grid, block, 0, stream>>>(
-        (const bf16_t*)x, (const bf16_t*)W, (bf16_t*)out, N, K, a_rows, act_scale, group_offsets, plan, n_experts,
-        nb_per_unit);
+        (const bf16_t*)x, (const bf16_t*)W, (bf16_t*)out, N, K, a_rows, act_scale, group_offsets, plan, n_groups, nb);
   else
     grouped_gemm_kernel<bf16_t, false, true><<<grid, block, 0, stream>>>(
-        (const bf16_t*)x, (const bf16_t*)W, (bf16_t*)out, N, K, a_rows, act_scale, group_offsets, plan, n_experts,
-        nb_per_unit);
+        (const bf16_t*)x, (const bf16_t*)W, (bf16_t*)out, N, K, a_rows, act_scale, group_offsets, plan, n_groups, nb);
   SHARPI_CHECK_LAUNCH();
   return SHARPI_OK;
 }

@@ -60,11 +60,12 @@ SHARPI_EXPORT int sharpi_gemm_skinny_picked(const void* x, const void* W, void* 
   if (packed && (N & (act ? 31 : 15))) return SHARPI_ERR_ARG;
   if (out_dtype != DT_F32 && out_dtype != DT_BF16) return SHARPI_ERR_ARG;
   if (act && out_dtype != DT_BF16) return SHARPI_ERR_ARG;
-  const int groups = n_experts + (shared ? 1 : 0);
+  // a group for every expert that can have rows: no more distinct experts than pairs
+  const int groups = (n_experts < n_pairs ? n_experts : n_pairs) + (shared ? 1 : 0);
   if (groups > 65535) return SHARPI_ERR_ARG;
   const int M = n_pairs + (shared ? n_pairs / k : 0);
-  const Picks pk = {ids, w, n_pairs, k, n_experts, gather};
-  if (act) return skinny_picked_swiglu(x, W, out, M, N, K, pk, n_experts + (shared ? 1 : 0), R, NW, packed, stream);
+  const Picks pk = {ids, w, n_pairs, k, n_experts, gather, shared ? 1 : 0};
+  if (act) return skinny_picked_swiglu(x, W, out, M, N, K, pk, groups, R, NW, packed, stream);
   // an expert has at most n_pairs rows: one, two or four blocks of sixteen rows against one stream of its weights
   const int MB = n_pairs <= 16 ? 1 : n_pairs <= 32 ? 2 : 4;
   // group_offsets is not read in this form; the pointer only has to be non-null for the grid's sake

@@ -58,6 +58,7 @@ struct Picks {
   const float* w;      // [n_pairs] its score (the SwiGLU form scales by it), or null
   int n_pairs, k, n_experts;
   int gather;          // x rows are tokens (pair i reads row i / k); otherwise x is in the output's row order
+  int shared;          // the tensor holds one more expert (index n_experts) that every token goes through
 };
 
 template <int R, int MB, int NW, typename TO, bool ACT, bool PACKED>
@@ -71,6 +72,7 @@ __global__ __launch_bounds__(NW* kWave) void skinny_gemm_kernel(
   __shared__ f32x4 red[NW][RT][kWave];
   __shared__ int members[kMaxPicked];       // picked form: the output rows of this block's expert
   __shared__ int n_members;
+  __shared__ int block_expert;
   const int lane = threadIdx.x & (kWave - 1);
   const int w = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
@@ -79,17 +81,43 @@ __global__ __launch_bounds__(NW* kWave) void skinny_gemm_kernel(
   const bool picked = pk.ids != nullptr;
   int row_begin = 0, row_end = M;
   if (picked) {
+    // The grid has a group for every expert that CAN have rows, not for every expert there is
+    // (a block that finds no rows still costs a launch slot, and with one token fifteen of
+    // seventeen would): group y < groups - shared is the y-th DISTINCT expert among the picks, in
+    // the order of its first pick; the last group is the always-on expert, if there is one.
     if (w == 0) {
-      // expert e < n_experts: the pairs that picked it; e == n_experts: every token once
-      const bool routed = e < pk.n_experts;
-      const bool mine = routed ? (lane < pk.n_pairs && pk.ids[lane] == e) : lane < pk.n_pairs / pk.k;
+      const int n_groups = gridDim.y;
+      const bool always_on = pk.shared && (int)blockIdx.y == n_groups - 1;
+      const int mine_e = lane < pk.n_pairs ? pk.ids[lane] : -1;
+      int expert = -1;                            // the block's expert; -1: there are fewer distinct experts than groups
+      if (always_on) {
+        expert = pk.n_experts;
+      } else if (n_groups - pk.shared == pk.n_experts) {
+        expert = blockIdx.y;                      // as many groups as experts: group y is expert y
+      } else {
+        bool first = lane < pk.n_pairs;           // no earlier pair picked this lane's expert
+        for (int j = 0; j < pk.n_pairs; ++j) {
+          const int ej = __shfl(mine_e, j, kWave);
+          if (j < lane && ej == mine_e) first = false;
+        }
+        const unsigned long long firsts = __builtin_amdgcn_ballot_w64(first);
+        const int ordinal = __popcll(firsts & ((1ull << lane) - 1ull));
+        const unsigned long long chosen = __builtin_amdgcn_ballot_w64(first && ordinal == (int)blockIdx.y);
+        if (chosen) expert = __shfl(mine_e, __ffsll((long long)chosen) - 1, kWave);
+      }
+      const bool routed = !always_on;
+      const bool mine = expert < 0 ? false : routed ? (lane < pk.n_pairs && mine_e == expert) : lane < pk.n_pairs / pk.k;
       const unsigned long long mask = __builtin_amdgcn_ballot_w64(mine);
       if (mine) members[__popcll(mask & ((1ull << lane) - 1ull))] = routed ? lane : pk.n_pairs + lane;
-      if (lane == 0) n_members = __popcll(mask);
+      if (lane == 0) {
+        n_members = __popcll(mask);
+        block_expert = expert;
+      }
     }
     __syncthreads();
     row_end = n_members;
-    W += (size_t)e * N * K;
+    if (row_end <= 0) return;
+    W += (size_t)block_expert * N * K;
   } else if (group_offsets) {
     row_begin = group_offsets[e];
     row_end = group_offsets[e + 1];

@@ -8,30 +8,34 @@ typedef __attribute__((ext_vector_type(8))) __bf16 peak_bf16x8;
 typedef __attribute__((ext_vector_type(4))) float peak_f32x4;
 typedef __attribute__((ext_vector_type(4))) unsigned peak_u32x4;
 
-// Every thread walks the buffer in 16-byte loads, eight on their way at a time; what is read is
-// folded into one word per thread so that no load can be dropped.
-__global__ __launch_bounds__(256) void peak_read_kernel(const peak_u32x4* __restrict__ buf, size_t n16, unsigned* __restrict__ sink) {
-  const size_t stride = (size_t)gridDim.x * blockDim.x;
-  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+// The buffer is read in chunks of 32 KB: a block of eight waves takes chunk (step * blocks + block)
+// at every step, a wave 4 KB of it as four loads of 1 KB, all four on their way before any is
+// used.  (Measured on MI355X: 6.8 to 7.0 TB/s with 2,048 blocks, whether a block's chunks lie side
+// by side or a grid apart; more loads in flight per thread do not read faster.)  What is read
+// is folded into one word per thread so that no load can be dropped.
+constexpr int kReadBlocks = 2048;
+__global__ __launch_bounds__(512) void peak_read_kernel(const peak_u32x4* __restrict__ buf, int steps, unsigned* __restrict__ sink) {
+  const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
   unsigned acc = 0;
-  for (; i + 7 * stride < n16; i += 8 * stride) {
-    peak_u32x4 v[8];
+  for (int s = 0; s < steps; ++s) {
+    const peak_u32x4* p = buf + ((size_t)s * gridDim.x + blockIdx.x) * 2048 + w * 256 + lane;
+    peak_u32x4 v[4];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) v[j] = __builtin_nontemporal_load(buf + i + j * stride);
+    for (int j = 0; j < 4; ++j) v[j] = __builtin_nontemporal_load(p + j * 64);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc ^= v[j].x ^ v[j].y ^ v[j].z ^ v[j].w;
-  }
-  for (; i < n16; i += stride) {
-    const peak_u32x4 v = buf[i];
-    acc ^= v.x ^ v.y ^ v.z ^ v.w;
+    for (int j = 0; j < 4; ++j) acc ^= v[j].x ^ v[j].y ^ v[j].z ^ v[j].w;
   }
   if (acc == 0x9e3779b9u) sink[0] = acc;   // practically never: the store only keeps the loads alive
 }
 
-// nbytes of buf are read once.  sink: one word of device memory.
-SHARPI_EXPORT int sharpi_peak_read(const void* buf, long long nbytes, void* sink, hipStream_t stream) {
-  if (nbytes < 16) return SHARPI_ERR_ARG;
-  peak_read_kernel<<<dim3(256 * 16), dim3(256), 0, stream>>>((const peak_u32x4*)buf, (size_t)(nbytes / 16), (unsigned*)sink);
+// The first (nbytes rounded down to a multiple of 64 MiB) bytes of buf are read once; the number
+// of bytes read is returned through *read_bytes (host memory).  sink: one word of device memory.
+SHARPI_EXPORT int sharpi_peak_read(const void* buf, long long nbytes, void* sink, long long* read_bytes, hipStream_t stream) {
+  const long long per_step = (long long)kReadBlocks * 32768;
+  const int steps = (int)(nbytes / per_step);
+  if (steps <= 0 || !read_bytes) return SHARPI_ERR_ARG;
+  *read_bytes = steps * per_step;
+  peak_read_kernel<<<dim3(kReadBlocks), dim3(512), 0, stream>>>((const peak_u32x4*)buf, steps, (unsigned*)sink);
   SHARPI_CHECK_LAUNCH();
   return SHARPI_OK;
 }

@@ -262,7 +262,8 @@ SHARPI_EXPORT int sharpi_router_topk(const void* x, int x_dtype, const void* wr,
 __device__ void permute_block(const int* __restrict__ topk_ids, const float* __restrict__ topk_w,
                               int* __restrict__ offsets, int* __restrict__ sorted_token,
                               float* __restrict__ sorted_w, int* __restrict__ inv_pos, int* __restrict__ plan,
-                              int n_pairs, int k, int n_experts, int shared_group, int* count, int* cursor) {
+                              int n_pairs, int k, int n_experts, int shared_group, int* count, int* cursor,
+                              int* plan_scratch) {
   for (int e = threadIdx.x; e < n_experts; e += blockDim.x) count[e] = 0;
   __syncthreads();
   for (int i = threadIdx.x; i < n_pairs; i += blockDim.x) atomicAdd(&count[topk_ids[i]], 1);
@@ -285,48 +286,58 @@ __device__ void permute_block(const int* __restrict__ topk_ids, const float* __r
     }
   }
   if (plan) {
-    // The plan of the grouped product (grouped_plan.h).  Experts in the order of their sibling
-    // counts, then of their rows (most first: the blocks that start last should be the short
-    // ones); expert of rank r gives units 2r and 2r + 1, unit u goes to row u / 8 of the XCDs,
-    // rows alternating in direction so that the XCDs' loads stay level.
-    const int stride = plan_stride(n_experts);
-    const int U = plan_units_max(n_experts);
-    for (int e = threadIdx.x; e < n_experts; e += blockDim.x) {
-      if (count[e] == 0) continue;
-      const int se = plan_siblings(count[e]);
-      int rank = 0;
-      for (int j = 0; j < n_experts; ++j) {
-        if (count[j] == 0 || j == e) continue;
-        const int sj = plan_siblings(count[j]);
-        rank += (sj > se || (sj == se && (count[j] > count[e] || (count[j] == count[e] && j < e)))) ? 1 : 0;
+    // The plan of the grouped product (grouped_plan.h).  Groups: the experts, and the always-on
+    // group (every token once) if there is one.  Every group with rows gives plan_parts units;
+    // units in the order of their weight (then of group and part) are dealt to the XCDs row by
+    // row, rows alternating in direction so that the XCDs' loads stay level.
+    const int n_groups = n_experts + (shared_group ? 1 : 0);
+    const int stride = plan_stride(n_groups);
+    if (shared_group && threadIdx.x == 0) count[n_experts] = n_pairs / k;
+    __syncthreads();
+    // unit_base[g]: units of the groups before g (in cursor's place it would clash: a second array)
+    int* unit_base = plan_scratch;
+    if (threadIdx.x == 0) {
+      int run = 0;
+      for (int g = 0; g < n_groups; ++g) {
+        unit_base[g] = run;
+        if (count[g] > 0) run += plan_parts(plan_siblings(count[g]));
       }
-      for (int half = 0; half < kPlanHalves; ++half) {
-        const int u = kPlanHalves * rank + half;
-        const int pos = u / kPlanXcds;
-        const int xcd = (pos & 1) ? kPlanXcds - 1 - u % kPlanXcds : u % kPlanXcds;
-        int* px = plan + xcd * stride;
-        px[2 + U + 2 * pos] = e;
-        px[2 + U + 2 * pos + 1] = half;
-      }
+      unit_base[n_groups] = run;
     }
     __syncthreads();
+    const int units = unit_base[n_groups];
+    for (int g = threadIdx.x; g < n_groups; g += blockDim.x) {
+      if (count[g] == 0) continue;
+      const int sg = plan_siblings(count[g]);
+      const int wg = plan_weight(sg), pg = plan_parts(sg);
+      // units that come before this group's: of heavier groups all, of equally heavy ones those of lower index
+      int before = 0;
+      for (int j = 0; j < n_groups; ++j) {
+        if (count[j] == 0 || j == g) continue;
+        const int sj = plan_siblings(count[j]);
+        const int wj = plan_weight(sj);
+        if (wj > wg || (wj == wg && j < g)) before += plan_parts(sj);
+      }
+      for (int part = 0; part < pg; ++part) {
+        const int u = before + part;
+        const int pos = u / kPlanXcds;
+        const int xcd = (pos & 1) ? kPlanXcds - 1 - u % kPlanXcds : u % kPlanXcds;
+        int* pu = plan + xcd * stride + 1 + 4 * pos;
+        pu[0] = g;
+        pu[1] = part;
+        pu[2] = pg;
+        pu[3] = sg;
+      }
+    }
     if (threadIdx.x < kPlanXcds) {
-      int busy = 0;
-      for (int e = 0; e < n_experts; ++e) busy += count[e] > 0 ? 1 : 0;
-      const int units = kPlanHalves * busy;
+      // XCD x holds one unit of every full row of 8, and of the last row the units that exist
       const int x = threadIdx.x;
-      int* px = plan + x * stride;
-      // XCD x holds, of every full row of 8 units, one; of the last row, the units that exist
-      int n = 0, run = 0;
-      px[1] = 0;
+      int n = 0;
       for (int pos = 0; pos * kPlanXcds < units; ++pos) {
         const int u = pos * kPlanXcds + ((pos & 1) ? kPlanXcds - 1 - x : x);
-        if (u >= units) continue;     // (only in the last row; the units of a row are dealt in order, so n == pos here)
-        run += plan_siblings(count[px[2 + U + 2 * pos]]);
-        px[2 + n] = run;
-        ++n;
+        if (u < units) ++n;
       }
-      px[0] = n;
+      plan[x * stride] = n;
     }
   }
   __syncthreads();
@@ -346,25 +357,26 @@ __global__ __launch_bounds__(1024) void moe_permute_kernel(const int* __restrict
                                                            float* __restrict__ sorted_w,
                                                            int* __restrict__ inv_pos, int* __restrict__ plan,
                                                            int n_pairs, int k, int n_experts, int shared_group) {
-  __shared__ int count[kMaxExperts];
+  __shared__ int count[kMaxExperts + 1];
   __shared__ int cursor[kMaxExperts];
+  __shared__ int plan_scratch[kMaxExperts + 2];
   permute_block(topk_ids, topk_w, offsets, sorted_token, sorted_w, inv_pos, plan, n_pairs, k, n_experts,
-                shared_group, count, cursor);
+                shared_group, count, cursor, plan_scratch);
 }
 
-// plan: plan_ints(n_experts) ints (grouped_plan.h) for the grouped product of many rows, or null.
+// plan: plan_ints(n_experts + shared_group) ints (grouped_plan.h) for the grouped product of many rows, or null.
 SHARPI_EXPORT int sharpi_moe_permute(const int* topk_ids, const float* topk_w, int* offsets, int* sorted_token,
                                      float* sorted_w, int* inv_pos, int* plan, int plan_len, int n_tokens, int k,
                                      int n_experts, int shared_group, hipStream_t stream) {
   if (n_experts <= 0 || n_experts > kMaxExperts || k <= 0) return SHARPI_ERR_ARG;
   if (n_tokens < 0) return SHARPI_ERR_ARG;
-  if (plan && plan_len < plan_ints(n_experts)) return SHARPI_ERR_ARG;
+  if (plan && plan_len < plan_ints(n_experts + (shared_group ? 1 : 0))) return SHARPI_ERR_ARG;
   moe_permute_kernel<<<1, 1024, 0, stream>>>(topk_ids, topk_w, offsets, sorted_token, sorted_w, inv_pos, plan,
                                              n_tokens * k, k, n_experts, shared_group);
   SHARPI_CHECK_LAUNCH();
   return SHARPI_OK;
 }
 
-SHARPI_EXPORT int sharpi_grouped_plan_ints(int n_experts) { return plan_ints(n_experts); }
+SHARPI_EXPORT int sharpi_grouped_plan_ints(int n_groups) { return plan_ints(n_groups); }
 SHARPI_EXPORT int sharpi_router_max_experts() { return kMaxExperts; }
 SHARPI_EXPORT int sharpi_add_rmsnorm_router_max_hidden() { return kFusedMaxHidden; }

@@ -69,10 +69,13 @@ class Engine:
                  max_model_len: Optional[int] = None, max_num_seqs: int = 8, max_tokens_per_step: int = 2048,
                  kv_tokens: Optional[int] = None, page_size: int = 16, weight_std: float = 0.02,
                  weight_std_by_suffix: Optional[Dict[str, float]] = None, verbose: bool = False,
-                 decode_graphs: bool = True, past_position_limit: bool = False):
+                 decode_graphs: bool = True, past_position_limit: bool = False, row_major_copies: bool = True):
         """max_model_len: the longest sequence a request may reach (default: the configuration's
         max_position_embeddings, 4096 if it names none); beyond max_position_embeddings only with
-        past_position_limit (replaying given tokens needs no trained positions)."""
+        past_position_limit (replaying given tokens needs no trained positions).
+        row_major_copies=False keeps the attention, dense feed-forward and head matrices only in
+        the packed order of the decode kernels (about a tenth less weight memory; prompt-sized
+        products then run in this library's own kernels instead of the library product, slower)."""
         self.dtype = parse_dtype(dtype)
         self.device = torch.device(device)
         if self.device.type != "cuda":
@@ -102,7 +105,13 @@ class Engine:
                                   stored_dtype=torch.bfloat16, std=weight_std, std_by_suffix=weight_std_by_suffix,
                                   generate_on_device=True)
         t0 = time.time()
-        load_model_weights(self.model, source)
+        from .. import ops as _ops
+
+        _ops.keep_row_major_copies(row_major_copies)
+        try:
+            load_model_weights(self.model, source)
+        finally:
+            _ops.keep_row_major_copies(True)
         if verbose:
             print(f"[engine] weights ready in {time.time() - t0:.1f}s", file=sys.stderr, flush=True)
         limit = getattr(self.config, "max_position_embeddings", 0) or 0
@@ -124,7 +133,7 @@ class Engine:
                            None if kv_tokens is None else max(1, (int(kv_tokens) + page_size - 1) // page_size))
         if kv_tokens is None and kv_specs:
             def total_bytes(sz):
-                return sum(sz[s.group_key()] * 2 * s.num_kv_heads * s.head_dim * page_size * width for s in kv_specs)
+                return sum(sz[s.group_key()] * s.num_kv_heads * (s.head_dim + s.value_dim) * page_size * width for s in kv_specs)
             budget = int(torch.cuda.mem_get_info(self.device)[0] * 0.8)
             while total_bytes(sizes) > budget and max(sizes.values()) > 1:
                 big = max(sizes, key=lambda k: sizes[k])       # the largest pools give way first

@@ -380,8 +380,22 @@ def pack_into(dst: torch.Tensor, w: torch.Tensor) -> None:
     dst.view(*lead, N // 16, K // 128, 16, 16, 8).copy_(src.permute(*range(n), n, n + 2, n + 3, n + 1, n + 4))
 
 
-def pack_weight(w: torch.Tensor, keep_rows: bool = True):
+_KEEP_ROWS = True
+
+
+def keep_row_major_copies(keep: bool) -> None:
+    """Whether matrices that are packed for the decode kernels also keep their row-major copy for
+    the library's product at prompt size (faster prefill, about a tenth more weight memory), or
+    only the packed copy (every product then runs in this library's kernels).  Read when weights
+    are loaded."""
+    global _KEEP_ROWS
+    _KEEP_ROWS = bool(keep)
+
+
+def pack_weight(w: torch.Tensor, keep_rows: Optional[bool] = None):
     """w as a PackedWeight if its shape and type allow it, else w itself."""
+    if keep_rows is None:
+        keep_rows = _KEEP_ROWS
     if not can_pack(w):
         return w
     packed = torch.empty_like(w, memory_format=torch.contiguous_format)
@@ -409,8 +423,8 @@ def _unwrap(w):
 # the weight-streaming product for few rows (decode)
 # ---------------------------------------------------------------------------
 SKINNY_MAX_ROWS = 64          # rows the kernel multiplies against one stream of a weight tile (4 blocks of 16)
-SKINNY_MAX_ROWS_PLAIN = 16    # plain form: beyond one row block the library's product is faster,
-SKINNY_MAX_ROWS_TALL = 32     # except against a very tall matrix (the head: 430 against 490 us at 32 rows)
+SKINNY_MAX_ROWS_PLAIN = 32    # plain form: beyond two row blocks the library's product is faster (measured at the
+SKINNY_MAX_ROWS_TALL = 32     # model's projection shapes: 18 against 23 us at 32 rows, 28 against 23.5 at 64)
 SKINNY_TALL = 65536
 
 
@@ -556,14 +570,26 @@ def gemm_skinny_picked(x: torch.Tensor, w, ids: torch.Tensor, wts: Optional[torc
 
 def linear(x: torch.Tensor, w, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """y = x W^T.  float32 weights: the float FMA kernel (true 32-bit, whatever x was stored
-    as).  bfloat16 weights: the weight-streaming kernel for a few rows (over the packed form if w
-    is a PackedWeight), the library's matrix product with float accumulation otherwise."""
+    as).  bfloat16 weights stored tile by tile (a PackedWeight): the weight-streaming kernel for a
+    few rows; beyond, the library's matrix product with float accumulation over the row-major
+    copy, as the reference calls a library there (reference:
+    src/SharpInference.Cuda/CuBlasInterop.cs:55-68; measured, the library is at the matrix cores'
+    peak for plain shapes), or, where only the packed copy is kept, this library's own kernels
+    (the few-rows kernel up to 64 rows, the grouped kernel with the matrix as its one group
+    beyond)."""
     out_dtype = out_dtype or x.dtype
     if isinstance(w, PackedWeight):
         xb = x if x.dtype == torch.bfloat16 else cast(x, torch.bfloat16)
         _need(xb.dim() == 2 and xb.shape[1] == w.shape[1], f"linear: x {tuple(x.shape)} vs w {tuple(w.shape)}")
-        if skinny_ok(xb.shape[0], w.shape[0], w.shape[1]):
+        M, (N, K) = xb.shape[0], w.shape
+        if skinny_ok(M, N, K):
             return gemm_skinny(xb, w, out_dtype)
+        if w.rows is None:
+            # only the packed copy is kept (the engine was asked to save memory): this library's own kernels
+            if M <= SKINNY_MAX_ROWS:
+                return gemm_skinny(xb, w, out_dtype)
+            if dense_grouped_ok(M, N, K):
+                return linear_many_rows(xb, w, out_dtype)
         w = unpack_weight(w)
     if w.dtype == torch.float32:
         xf = x if x.dtype == torch.float32 else cast(x, torch.float32)
@@ -677,16 +703,15 @@ def _new_routing(T: int, k: int, n_experts: int, shared_group: bool, dev) -> Rou
     rt.n_tokens, rt.k, rt.n_experts = T, k, n_experts
     rt.n_groups = n_experts + (1 if shared_group else 0)
     rows = T * k + (T if shared_group else 0)
-    if n_experts not in _PLAN_INTS:
-        _PLAN_INTS[n_experts] = _lib.grouped_plan_ints(n_experts)
-    # (a shared group rides with the experts only in the few-rows product, which needs no plan)
-    n_plan = 0 if shared_group else _PLAN_INTS[n_experts]
+    if rt.n_groups not in _PLAN_INTS:
+        _PLAN_INTS[rt.n_groups] = _lib.grouped_plan_ints(rt.n_groups)
+    n_plan = _PLAN_INTS[rt.n_groups]
     ints = torch.empty(rt.n_groups + 1 + rows + T * k + n_plan, dtype=torch.int32, device=dev)
     o = 0
     rt.offsets = ints[o:o + rt.n_groups + 1]; o += rt.n_groups + 1
     rt.sorted_token = ints[o:o + rows]; o += rows
     rt.inv_pos = ints[o:o + T * k]; o += T * k
-    rt.plan = ints[o:o + n_plan] if n_plan else None
+    rt.plan = ints[o:o + n_plan]
     rt.sorted_w = torch.empty(rows, dtype=torch.float32, device=dev)
     return rt
 
@@ -702,7 +727,7 @@ def moe_permute(ids: torch.Tensor, wts: torch.Tensor, n_experts: int, shared_gro
     T, k = ids.shape
     rt = _new_routing(T, k, n_experts, shared_group, ids.device)
     _run("sharpi_moe_permute", _ptr(ids), _ptr(wts), _ptr(rt.offsets), _ptr(rt.sorted_token), _ptr(rt.sorted_w),
-         _ptr(rt.inv_pos), _ptr(rt.plan), rt.plan.numel() if rt.plan is not None else 0, T, k, n_experts,
+         _ptr(rt.inv_pos), _ptr(rt.plan), rt.plan.numel(), T, k, n_experts,
          1 if shared_group else 0, _stream())
     return rt
 
@@ -715,43 +740,81 @@ def route(x: torch.Tensor, wr: torch.Tensor, k: int, gate: int = GATE_SIGMOID, r
 
 
 def gemm_grouped(x: torch.Tensor, w, rt: Routing, gather: bool, out_dtype: torch.dtype) -> torch.Tensor:
-    """Per-expert products for many rows on the matrix cores (bfloat16).  gather: x rows are read
-    through the routing's token list; otherwise x is already in expert-sorted order."""
+    """Per-group products for many rows on the matrix cores (bfloat16): the experts, and the
+    always-on group if the routing has one (group E of w).  gather: x rows are read through the
+    routing's token list; otherwise x is already in expert-sorted order."""
     w, packed = _unwrap(w)
     _dev(x, w)
     _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_grouped: bfloat16 operands only")
-    _need(w.dim() == 3 and w.shape[0] >= rt.n_experts and rt.n_groups == rt.n_experts and x.dim() == 2
-          and x.shape[1] == w.shape[2], f"gemm_grouped: x {tuple(x.shape)} vs w {tuple(w.shape)}")
+    _need(w.dim() == 3 and w.shape[0] >= rt.n_groups and x.dim() == 2 and x.shape[1] == w.shape[2],
+          f"gemm_grouped: x {tuple(x.shape)} vs w {tuple(w.shape)}")
     E, N, K = w.shape
     _need(K % 64 == 0 and N % 4 == 0, "gemm_grouped: K % 64 == 0 and N % 4 == 0 wanted")
     _need(x.shape[0] == (rt.n_tokens if gather else rt.n_rows), "gemm_grouped: x has the wrong number of rows")
     out = torch.empty(rt.n_rows, N, dtype=out_dtype, device=x.device)
-    _need(rt.plan is not None, "gemm_grouped: this routing was made without a plan (a shared group)")
     _run("sharpi_gemm_grouped", _ptr(x), x.shape[0], _ptr(w), _ptr(out), _code(out_dtype), rt.n_rows, N, K,
-         _ptr(rt.sorted_token) if gather else None, _ptr(rt.offsets), _ptr(rt.plan), rt.n_experts,
+         _ptr(rt.sorted_token) if gather else None, _ptr(rt.offsets), _ptr(rt.plan), rt.n_groups,
          1 if packed else 0, _stream())
     return out
 
 
 def gemm_grouped_swiglu(x: torch.Tensor, w, rt: Routing, scale: Optional[torch.Tensor]) -> torch.Tensor:
-    """Per expert, silu(s g) * (s u) with (g | u) = x @ w[e]^T rounded to bfloat16, for many rows: the
+    """Per group, silu(s g) * (s u) with (g | u) = x @ w[e]^T rounded to bfloat16, for many rows: the
     grouped product with the activation in its epilogue.  x rows are read through the routing's
-    token list; w [E, 2I, K] holds gate rows then up rows.  Returns [n_rows, I] bfloat16."""
+    token list; w [E (+ 1), 2I, K] holds gate rows then up rows.  Returns [n_rows, I] bfloat16."""
     w, packed = _unwrap(w)
     _dev(x, w, scale)
     _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_grouped_swiglu: bfloat16 operands only")
-    _need(w.dim() == 3 and w.shape[0] >= rt.n_experts and rt.n_groups == rt.n_experts and x.dim() == 2
-          and x.shape[1] == w.shape[2], f"gemm_grouped_swiglu: x {tuple(x.shape)} vs w {tuple(w.shape)}")
+    _need(w.dim() == 3 and w.shape[0] >= rt.n_groups and x.dim() == 2 and x.shape[1] == w.shape[2],
+          f"gemm_grouped_swiglu: x {tuple(x.shape)} vs w {tuple(w.shape)}")
     E, N, K = w.shape
     _need(K % 64 == 0 and N % 32 == 0, "gemm_grouped_swiglu: K % 64 == 0 and N % 32 == 0 wanted")
     _need(x.shape[0] == rt.n_tokens, "gemm_grouped_swiglu: x has the wrong number of rows")
     if scale is not None:
         _need(scale.dtype == torch.float32 and scale.shape == (rt.n_rows,), "gemm_grouped_swiglu: scale must be float32 [n_rows]")
     out = torch.empty(rt.n_rows, N // 2, dtype=torch.bfloat16, device=x.device)
-    _need(rt.plan is not None, "gemm_grouped_swiglu: this routing was made without a plan (a shared group)")
     _run("sharpi_gemm_grouped_swiglu", _ptr(x), x.shape[0], _ptr(w), _ptr(out), rt.n_rows, N, K, _ptr(rt.sorted_token),
-         _ptr(rt.offsets), _ptr(rt.plan), rt.n_experts, _ptr(scale), 1 if packed else 0, _stream())
+         _ptr(rt.offsets), _ptr(rt.plan), rt.n_groups, _ptr(scale), 1 if packed else 0, _stream())
     return out
+
+
+# ---------------------------------------------------------------------------
+# plain products of many rows through the grouped kernel (one group: the whole matrix)
+# ---------------------------------------------------------------------------
+_DENSE_ROUTING: dict = {}
+
+
+def _dense_routing(T: int, dev: torch.device) -> Routing:
+    """The routing of T rows that all belong to one group, in their own order: offsets [0, T] and
+    the plan of the grouped product for it.  Made once per (T, device) by the routing kernel."""
+    key = (T, dev)
+    rt = _DENSE_ROUTING.get(key)
+    if rt is None:
+        _need(not torch.cuda.is_current_stream_capturing(), "a dense routing's first use must not be captured")
+        if len(_DENSE_ROUTING) > 64:
+            _DENSE_ROUTING.clear()
+        ids = torch.zeros(T, 1, dtype=torch.int32, device=dev)
+        rt = _DENSE_ROUTING[key] = moe_permute(ids, torch.ones(T, 1, dtype=torch.float32, device=dev), 1)
+    return rt
+
+
+def dense_grouped_ok(M: int, N: int, K: int) -> bool:
+    return M > 0 and K % 128 == 0 and N % 16 == 0 and N * K <= 0x7fffffff
+
+
+def linear_many_rows(x: torch.Tensor, w: PackedWeight, out_dtype: torch.dtype) -> torch.Tensor:
+    """x [M, K] @ w^T for many rows against a matrix stored tile by tile, on the matrix cores: the
+    grouped product with the whole matrix as its one group (row tiles of up to 192 rows whose
+    blocks share the weight stream through an XCD's L2)."""
+    rt = _dense_routing(x.shape[0], x.device)
+    return gemm_grouped(x, PackedWeight(w.packed.unsqueeze(0), None), rt, False, out_dtype)
+
+
+def swiglu_many_rows(x: torch.Tensor, w_gate_up: PackedWeight) -> torch.Tensor:
+    """silu(g) * u with (g | u) = x @ w_gate_up^T rounded to bfloat16, for many rows, the activation
+    in the product's epilogue: [M, I] bfloat16."""
+    rt = _dense_routing(x.shape[0], x.device)
+    return gemm_grouped_swiglu(x, PackedWeight(w_gate_up.packed.unsqueeze(0), None), rt, None)
 
 
 # ---------------------------------------------------------------------------
@@ -827,7 +890,7 @@ def grouped_swiglu(x: torch.Tensor, w_gate_up, rt: Routing, out_dtype: torch.dty
         if rt.n_tokens <= SKINNY_MAX_ROWS and N % (32 if isinstance(w_gate_up, PackedWeight) else 8) == 0:
             return gemm_skinny_swiglu(x, w_gate_up, rt.offsets, rt.sorted_token, rt.n_rows, scale,
                                       group_rows=rt.n_tokens)
-        if rt.n_tokens > SKINNY_MAX_ROWS and N % 32 == 0 and rt.n_groups == rt.n_experts:
+        if rt.n_tokens > SKINNY_MAX_ROWS and N % 32 == 0:
             return gemm_grouped_swiglu(x, w_gate_up, rt, scale)
     return silu_mul(grouped_linear(x, w_gate_up, rt, True, out_dtype), scale)
 
@@ -862,9 +925,12 @@ def measured_peaks(device="cuda:0", read_bytes: int = 4 << 30, repeats: int = 5)
     a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     best_read = best_mfma = float("inf")
     blocks, iters = 256 * 8, 4096
+    import ctypes
+
+    done = ctypes.c_longlong(0)
     for _ in range(repeats + 1):
         a.record()
-        _run("sharpi_peak_read", _ptr(buf), read_bytes, _ptr(sink), _stream())
+        _run("sharpi_peak_read", _ptr(buf), read_bytes, _ptr(sink), ctypes.addressof(done), _stream())
         b.record()
         b.synchronize()
         best_read = min(best_read, a.elapsed_time(b))
@@ -874,4 +940,4 @@ def measured_peaks(device="cuda:0", read_bytes: int = 4 << 30, repeats: int = 5)
         b.synchronize()
         best_mfma = min(best_mfma, a.elapsed_time(b))
     flops = blocks * 4 * iters * 8 * (2.0 * 16 * 16 * 32)
-    return {"hbm_gbs": read_bytes / best_read / 1e6, "bf16_tflops": flops / best_mfma / 1e9}
+    return {"hbm_gbs": done.value / best_read / 1e6, "bf16_tflops": flops / best_mfma / 1e9}

@@ -74,6 +74,9 @@ class MoESwiGLU(Part):
 
     MERGE_MAX_TOKENS = 16   # one row block of the few-rows kernel for the shared group (measured: up to 64 tokens
                             # the merged launches and the library's product for the shared expert are as fast)
+    MERGE_MIN_MANY_TOKENS = None   # tokens from which the shared expert is one more group of the many-rows grouped
+                                   # product; off: measured at 2,048 tokens, 1.48 ms a layer against 0.93 + 0.45 with
+                                   # the library's product for the shared expert (which runs at the matrix cores' peak)
 
     def __init__(self, hidden: int, num_experts: int, top_k: int, expert_intermediate: int,
                  shared_intermediate: Optional[int] = None, gate: str = "sigmoid", renormalise: bool = False,
@@ -204,7 +207,8 @@ class MoESwiGLU(Part):
             with section("router", nbytes=2 * T * self.hidden + 2 * self.E * self.hidden):
                 ids, wts = ops.router_topk(x, self.w_router, self.k, self.gate, self.renormalise)
             return self._picked(x, ids, wts, ctx)
-        merge = self.merged and T <= self.MERGE_MAX_TOKENS and ctx.act_dtype == torch.bfloat16
+        many = self.MERGE_MIN_MANY_TOKENS is not None and T >= self.MERGE_MIN_MANY_TOKENS
+        merge = self.merged and ctx.act_dtype == torch.bfloat16 and (T <= self.MERGE_MAX_TOKENS or many)
         with section("router", nbytes=2 * T * self.hidden + 2 * self.E * self.hidden):
             ids, wts, rt = ops.route(x, self.w_router, self.k, self.gate, self.renormalise, shared_group=merge)
         if trace is not None:      # the picks of this step, layer by layer (reference: ForwardPass.cs:2042-2056)

@@ -141,3 +141,16 @@ def test_random_orders_never_lose_a_page(seed):
     m.check_invariants()
     assert all(g.pool.num_free == g.pool.num_pages for g in m.groups)
     assert reuse >= 1 or m.groups[0].pool.num_pages >= 40
+
+
+def test_keys_and_values_of_different_widths():
+    """A mixer may ask for values of another width than its keys: the value tensor and the bytes of
+    a page follow."""
+    import torch
+
+    spec = KVSpec(2, 48, WINDOW_NONE, 0, v_head_dim=32)
+    m = CacheManager([spec, KVSpec(2, 16)], 16, 4, 2, dtype=torch.float32)
+    assert m.k[0].shape == (4, 2, 16, 48) and m.v[0].shape == (4, 2, 32, 16)
+    assert m.k[1].shape == (4, 2, 16, 16) and m.v[1].shape == (4, 2, 16, 16)
+    assert m.bytes_per_page() == [2 * (48 + 32) * 16 * 4 + 2 * (16 + 16) * 16 * 4]
+    assert spec.value_dim == 32 and KVSpec(2, 16).value_dim == 16

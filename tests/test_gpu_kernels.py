@@ -52,7 +52,7 @@ def test_linear_against_a_very_tall_matrix(M):
     x = _rand(M, K, dtype=torch.bfloat16, seed=M)
     w = _rand(N, K, dtype=torch.bfloat16, scale=0.1, seed=7)
     ref = x.float() @ w.float().T
-    assert ops.skinny_ok(M, N, K) == (M <= 32) and ops.skinny_ok(M, 4096, K) == (M <= 16)
+    assert ops.skinny_ok(M, N, K) == (M <= 32) and ops.skinny_ok(M, 4096, K) == (M <= 32)
     for form in (w, ops.pack_weight(w)):
         for out_dtype, tol in ((torch.float32, 1e-3), (torch.bfloat16, 2e-2)):
             got = ops.linear(x, form, out_dtype)
@@ -353,33 +353,35 @@ def test_router_and_permute(T, E, k, H, dtype):
 
 
 def _check_plan(ops, rt, counts):
-    """The plan of the grouped product for many rows: every expert with rows gives two units (the
-    halves of its weight rows), each once, dealt to the 8 XCDs so that their sibling counts stay
-    level; an XCD's running sums are those of its units' siblings; the experts with most siblings
-    (then most rows) come first."""
-    E = len(counts)
+    """The plan of the grouped product for many rows: every group with rows is cut into sibling
+    row tiles (as few of at most 192 rows as hold its rows) and its column blocks into parts (2,
+    4, 8 or 16: more the more siblings); every (group, part) unit appears once, on one of the 8
+    XCDs, the heaviest units dealt first so that the XCDs' loads stay level."""
+    G = len(counts)
     tile = ops._lib.grouped_tile_rows()
     plan = rt.plan.cpu().tolist()
-    U = 2 * E
-    stride = 2 + 3 * U
+    per_xcd = (16 * G + 7) // 8 + 1
+    stride = 1 + 4 * per_xcd
     assert len(plan) == 8 * stride
+
+    def parts_of(sibs):
+        return 2 if sibs <= 2 else 4 if sibs <= 4 else 8 if sibs <= 8 else 16
+
     seen, loads = [], []
     for x in range(8):
         px = plan[x * stride:(x + 1) * stride]
-        n = px[0]
-        cum = px[1:2 + n]
-        assert cum[0] == 0
-        units = [(px[2 + U + 2 * j], px[2 + U + 2 * j + 1]) for j in range(n)]
-        for j, (e, half) in enumerate(units):
-            assert counts[e] > 0 and half in (0, 1)
-            assert cum[j + 1] - cum[j] == -(-counts[e] // tile)
-        sibs = [-(-counts[e] // tile) for e, _ in units]
-        assert sibs == sorted(sibs, reverse=True)
-        seen += units
-        loads.append(cum[-1])
-    busy = [e for e in range(E) if counts[e] > 0]
-    assert sorted(seen) == sorted((e, h) for e in busy for h in (0, 1))
-    assert max(loads) - min(loads) <= max([-(-c // tile) for c in counts] + [0])
+        units = [tuple(px[1 + 4 * j:5 + 4 * j]) for j in range(px[0])]
+        weights = []
+        for g, part, parts, sibs in units:
+            assert counts[g] > 0 and sibs == -(-counts[g] // tile) and parts == parts_of(sibs) and 0 <= part < parts
+            weights.append(sibs * (16 // parts))
+        assert weights == sorted(weights, reverse=True)
+        seen += [(g, part) for g, part, _, _ in units]
+        loads.append(sum(weights))
+    want = [(g, part) for g in range(G) if counts[g] > 0 for part in range(parts_of(-(-counts[g] // tile)))]
+    assert sorted(seen) == sorted(want)
+    heaviest = max([-(-c // tile) * (16 // parts_of(-(-c // tile))) for c in counts if c > 0] + [0])
+    assert max(loads) - min(loads) <= heaviest
 
 
 @pytest.mark.parametrize("counts", [[500, 0, 193, 192, 1, 64, 0, 700], [128] * 16, [3], [0, 0, 5000]])
@@ -391,6 +393,9 @@ def test_plan_of_the_grouped_product(counts):
     rt = ops.moe_permute(ids, torch.ones(ids.shape, device=DEV), E)
     assert [b - a for a, b in zip(rt.offsets.cpu().tolist(), rt.offsets.cpu().tolist()[1:])] == counts
     _check_plan(ops, rt, counts)
+    # with an always-on group behind the experts: one more group, of as many rows as there are tokens
+    rt = ops.moe_permute(ids, torch.ones(ids.shape, device=DEV), E, shared_group=True)
+    _check_plan(ops, rt, counts + [len(ids)])
 
 
 @pytest.mark.parametrize("T,H,E,k", [(1, 5120, 16, 1), (8, 5120, 16, 1), (16, 256, 5, 2), (3, 8192, 128, 4), (5, 136, 3, 3)])
@@ -826,3 +831,42 @@ def test_a_model_made_on_the_device_is_the_model_written_on_the_host(tmp_path):
         eng.add_request("r")
         out.append(eng.step([StepEntry("r", toks, list(range(len(toks))))]))
     assert torch.equal(out[0], out[1])
+
+
+@pytest.mark.parametrize("M,N,K", [(70, 272, 256), (200, 528, 640), (500, 5120, 1280)])
+def test_plain_products_of_many_rows_through_the_grouped_kernel(M, N, K):
+    """A matrix kept only in the packed order is multiplied by many rows in the grouped kernel,
+    the whole matrix as its one group (rows in their own order); with SwiGLU in the epilogue it
+    gives the bits of the product followed by the activation kernel."""
+    ops = _ops()
+    x = _rand(M, K, dtype=torch.bfloat16, seed=M)
+    w = _rand(N, K, dtype=torch.bfloat16, scale=0.1, seed=N)
+    pw = ops.pack_weight(w, keep_rows=False)
+    assert pw.rows is None
+    ref = x.float() @ w.float().T
+    for out_dtype, tol in ((torch.float32, 1e-3), (torch.bfloat16, 2e-2)):
+        got = ops.linear(x, pw, out_dtype)          # no row-major copy: this library's kernels, whatever the row count
+        assert got.dtype == out_dtype and float((got.float() - ref).abs().max()) <= tol * float(ref.abs().max())
+    few = ops.linear(x[:40].contiguous(), pw, torch.float32)       # 17 to 64 rows: the few-rows kernel
+    assert float((few - ref[:40]).abs().max()) <= 1e-3 * float(ref.abs().max())
+    if N % 32 == 0:
+        act = ops.swiglu_many_rows(x, pw)
+        assert torch.equal(act, ops.silu_mul(ops.linear_many_rows(x, pw, torch.bfloat16)))
+
+
+def test_an_engine_that_keeps_only_packed_weights_gives_the_same_logits(tmp_path):
+    from sharpinference_amd.engine import Engine, StepEntry
+    from tiny_configs import make_model_dir
+
+    d = make_model_dir(tmp_path, "D", std=0.06)
+    toks = [int(t) for t in torch.randint(0, 500, (150,), generator=torch.Generator().manual_seed(3))]
+    out = []
+    for copies in (True, False):
+        eng = Engine(d, dtype="bfloat16", kv_tokens=256, max_num_seqs=1, row_major_copies=copies)
+        assert (eng.model.blocks[0].mixer.w_qkv.rows is not None) == copies
+        eng.add_request("r")
+        out.append(eng.step([StepEntry("r", toks[:120], list(range(120)))]).float().cpu())
+        out.append(eng.step([StepEntry("r", toks[120:121], [0])]).float().cpu())      # a decode step: the same kernel either way
+    rms = out[0].pow(2).mean().sqrt()
+    assert float((out[0] - out[2]).abs().max()) <= 0.1 * float(rms)        # other kernels at prompt size: roundings apart
+    assert float((out[1] - out[3]).abs().max()) <= 0.1 * float(rms)
