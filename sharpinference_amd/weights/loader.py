@@ -307,10 +307,13 @@ def write_random_model(config, out_dir: str, seed: int, stored_dtype: torch.dtyp
 
     model = build_model(config)
     specs = model.param_specs()
-    src = RandomSource(specs, seed, torch.float32, "cpu", stored_dtype=stored_dtype, std=std,
-                       float32_names=float32_names, std_by_suffix=std_by_suffix)
+    # the values are a function of (seed, name, element) wherever they are made: on a machine with a
+    # GPU the fill kernel makes them (a large model's file is then written in seconds, not minutes)
+    on_gpu = torch.cuda.is_available()
+    src = RandomSource(specs, seed, torch.float32, "cuda" if on_gpu else "cpu", stored_dtype=stored_dtype, std=std,
+                       float32_names=float32_names, std_by_suffix=std_by_suffix, generate_on_device=on_gpu)
     os.makedirs(out_dir, exist_ok=True)
     save_config(config, out_dir)
-    st.write_file(os.path.join(out_dir, "model.safetensors"), ((n, src.stored(n)) for n in sorted(specs)),
+    st.write_file(os.path.join(out_dir, "model.safetensors"), ((n, src.stored(n).cpu()) for n in sorted(specs)),
                   metadata={"format": "pt", "seed": str(seed)})
     return out_dir
