@@ -758,10 +758,12 @@ def gemm_grouped(x: torch.Tensor, w, rt: Routing, gather: bool, out_dtype: torch
     return out
 
 
-def gemm_grouped_swiglu(x: torch.Tensor, w, rt: Routing, scale: Optional[torch.Tensor]) -> torch.Tensor:
+def gemm_grouped_swiglu(x: torch.Tensor, w, rt: Routing, scale: Optional[torch.Tensor], gather: bool = True) -> torch.Tensor:
     """Per group, silu(s g) * (s u) with (g | u) = x @ w[e]^T rounded to bfloat16, for many rows: the
-    grouped product with the activation in its epilogue.  x rows are read through the routing's
-    token list; w [E (+ 1), 2I, K] holds gate rows then up rows.  Returns [n_rows, I] bfloat16."""
+    grouped product with the activation in its epilogue.  gather: x rows are read through the
+    routing's token list (the order inside a group is whatever the routing kernel made it);
+    otherwise x is already in the groups' order.  w [E (+ 1), 2I, K] holds gate rows then up
+    rows.  Returns [n_rows, I] bfloat16."""
     w, packed = _unwrap(w)
     _dev(x, w, scale)
     _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_grouped_swiglu: bfloat16 operands only")
@@ -769,12 +771,12 @@ def gemm_grouped_swiglu(x: torch.Tensor, w, rt: Routing, scale: Optional[torch.T
           f"gemm_grouped_swiglu: x {tuple(x.shape)} vs w {tuple(w.shape)}")
     E, N, K = w.shape
     _need(K % 64 == 0 and N % 32 == 0, "gemm_grouped_swiglu: K % 64 == 0 and N % 32 == 0 wanted")
-    _need(x.shape[0] == rt.n_tokens, "gemm_grouped_swiglu: x has the wrong number of rows")
+    _need(x.shape[0] == (rt.n_tokens if gather else rt.n_rows), "gemm_grouped_swiglu: x has the wrong number of rows")
     if scale is not None:
         _need(scale.dtype == torch.float32 and scale.shape == (rt.n_rows,), "gemm_grouped_swiglu: scale must be float32 [n_rows]")
     out = torch.empty(rt.n_rows, N // 2, dtype=torch.bfloat16, device=x.device)
-    _run("sharpi_gemm_grouped_swiglu", _ptr(x), x.shape[0], _ptr(w), _ptr(out), rt.n_rows, N, K, _ptr(rt.sorted_token),
-         _ptr(rt.offsets), _ptr(rt.plan), rt.n_groups, _ptr(scale), 1 if packed else 0, _stream())
+    _run("sharpi_gemm_grouped_swiglu", _ptr(x), x.shape[0], _ptr(w), _ptr(out), rt.n_rows, N, K,
+         _ptr(rt.sorted_token) if gather else None, _ptr(rt.offsets), _ptr(rt.plan), rt.n_groups, _ptr(scale), 1 if packed else 0, _stream())
     return out
 
 
@@ -785,8 +787,10 @@ _DENSE_ROUTING: dict = {}
 
 
 def _dense_routing(T: int, dev: torch.device) -> Routing:
-    """The routing of T rows that all belong to one group, in their own order: offsets [0, T] and
-    the plan of the grouped product for it.  Made once per (T, device) by the routing kernel."""
+    """The routing of T rows that all belong to one group: offsets [0, T] and the plan of the
+    grouped product for it, made once per (T, device) by the routing kernel.  Its token list is
+    not used (the routing kernel promises no order inside a group): the products read x row by
+    row (gather off)."""
     key = (T, dev)
     rt = _DENSE_ROUTING.get(key)
     if rt is None:
@@ -814,7 +818,7 @@ def swiglu_many_rows(x: torch.Tensor, w_gate_up: PackedWeight) -> torch.Tensor:
     """silu(g) * u with (g | u) = x @ w_gate_up^T rounded to bfloat16, for many rows, the activation
     in the product's epilogue: [M, I] bfloat16."""
     rt = _dense_routing(x.shape[0], x.device)
-    return gemm_grouped_swiglu(x, PackedWeight(w_gate_up.packed.unsqueeze(0), None), rt, None)
+    return gemm_grouped_swiglu(x, PackedWeight(w_gate_up.packed.unsqueeze(0), None), rt, None, gather=False)
 
 
 # ---------------------------------------------------------------------------

@@ -833,7 +833,7 @@ def test_a_model_made_on_the_device_is_the_model_written_on_the_host(tmp_path):
     assert torch.equal(out[0], out[1])
 
 
-@pytest.mark.parametrize("M,N,K", [(70, 272, 256), (200, 528, 640), (500, 5120, 1280)])
+@pytest.mark.parametrize("M,N,K", [(70, 272, 256), (200, 528, 640), (200, 512, 256), (384, 5120, 256), (500, 5120, 1280)])
 def test_plain_products_of_many_rows_through_the_grouped_kernel(M, N, K):
     """A matrix kept only in the packed order is multiplied by many rows in the grouped kernel,
     the whole matrix as its one group (rows in their own order); with SwiGLU in the epilogue it
@@ -859,14 +859,15 @@ def test_an_engine_that_keeps_only_packed_weights_gives_the_same_logits(tmp_path
     from tiny_configs import make_model_dir
 
     d = make_model_dir(tmp_path, "D", std=0.06)
-    toks = [int(t) for t in torch.randint(0, 500, (150,), generator=torch.Generator().manual_seed(3))]
+    toks = [int(t) for t in torch.randint(0, 500, (450,), generator=torch.Generator().manual_seed(3))]
     out = []
     for copies in (True, False):
-        eng = Engine(d, dtype="bfloat16", kv_tokens=256, max_num_seqs=1, row_major_copies=copies)
+        eng = Engine(d, dtype="bfloat16", kv_tokens=512, max_num_seqs=1, row_major_copies=copies)
         assert (eng.model.blocks[0].mixer.w_qkv.rows is not None) == copies
         eng.add_request("r")
-        out.append(eng.step([StepEntry("r", toks[:120], list(range(120)))]).float().cpu())
-        out.append(eng.step([StepEntry("r", toks[120:121], [0])]).float().cpu())      # a decode step: the same kernel either way
+        # 420 rows: three row tiles side by side in the grouped kernel
+        out.append(eng.step([StepEntry("r", toks[:420], list(range(420)))]).float().cpu())
+        out.append(eng.step([StepEntry("r", toks[420:421], [0])]).float().cpu())      # a decode step: the same kernel either way
     rms = out[0].pow(2).mean().sqrt()
     assert float((out[0] - out[2]).abs().max()) <= 0.1 * float(rms)        # other kernels at prompt size: roundings apart
     assert float((out[1] - out[3]).abs().max()) <= 0.1 * float(rms)
