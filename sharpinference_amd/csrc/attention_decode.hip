@@ -82,6 +82,7 @@ __global__ __launch_bounds__(kDecWaves* kWave) void attn_decode_kernel(
 #pragma unroll
   for (int d = 0; d < ND; ++d) acc[d] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+  // Keys and values are read once per step, so with the streaming hint (nontemporal).
   // A wave's chunks of the run are 2 * kDecWaves blocks apart; PRE of them are requested before
   // anything is computed (all of a 256-key run where the registers allow it: the run is then one
   // round trip to memory, not one per chunk).  Every load is unconditional: a block beyond the
@@ -103,10 +104,10 @@ __global__ __launch_bounds__(kDecWaves* kWave) void attn_decode_kernel(
         const long long vbase = ((long long)page * nkv + kvh) * HD * page_size + off;
 #pragma unroll
         for (int j = 0; j < NJ; ++j)
-          kf[it][u][j] = *reinterpret_cast<const bf16x8*>(k_cache + kbase + (size_t)r * HD + j * 32 + g * 8);
+          kf[it][u][j] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(k_cache + kbase + (size_t)r * HD + j * 32 + g * 8));
 #pragma unroll
         for (int d = 0; d < ND; ++d)   // V^T fragment: lane (d row r, group g) holds keys 4g..4g+3 of the block
-          vq[it][u][d] = *reinterpret_cast<const bf16x4*>(v_cache + vbase + (size_t)(d * 16 + r) * page_size + 4 * g);
+          vq[it][u][d] = __builtin_nontemporal_load(reinterpret_cast<const bf16x4*>(v_cache + vbase + (size_t)(d * 16 + r) * page_size + 4 * g));
       }
     }
 #pragma unroll

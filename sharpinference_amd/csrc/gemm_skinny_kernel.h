@@ -2,7 +2,10 @@
 // inputs, float accumulation on the matrix cores (v_mfma_f32_16x16x32_bf16); M <= 64, or any number
 // of rows in the grouped form as long as an expert has few.
 //
-// The weights are read from HBM exactly once; everything else is arranged around that.
+// The weights are read from HBM exactly once; everything else is arranged around that.  They are
+// read with the streaming hint (nontemporal: a line is not kept in the caches for a second use
+// that never comes), which alone is worth a tenth of the bandwidth: 6.3 against 5.7 TB/s for a
+// pure read in this kernel's access pattern.
 //  * A block owns R tiles of 16 weight rows; its NW waves split K into contiguous slices.  Per
 //    128-wide K unit a lane loads 64 contiguous bytes of each of its weight rows and of each of
 //    its x rows and feeds 4 MFMAs per (tile, row block): W is the A operand (rows = n), x the
@@ -187,7 +190,8 @@ __global__ __launch_bounds__(NW* kWave) void skinny_gemm_kernel(
       for (int t = 0; t < R; ++t)
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-          wf[t][j] = *reinterpret_cast<const bf16x8*>(wrow[t] + (PACKED ? (size_t)u * 2048 + j * 512 : (size_t)k0 + j * 8));
+          wf[t][j] = __builtin_nontemporal_load(
+              reinterpret_cast<const bf16x8*>(wrow[t] + (PACKED ? (size_t)u * 2048 + j * 512 : (size_t)k0 + j * 8)));
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
