@@ -433,14 +433,22 @@ def skinny_ok(M: int, N: int, K: int, grouped: bool = False) -> bool:
     return 0 < M <= limit and K % 128 == 0 and N % 4 == 0
 
 
-def skinny_plan(N: int, K: int, row_blocks: int = 1):
+def skinny_plan(N: int, K: int, row_blocks: int = 1, groups: int = 1, act: bool = False):
     """(R, NW): 16-row weight tiles per block and waves per block splitting K (measured on
     MI355X over the projection shapes of the model).  NW, which decides the order of a row's
     sums, depends on nothing (so a row's result does not change with the batch); R only says how
     many independent columns a block computes: two tiles where a block holds one block of 16
     rows (the kernel then keeps two K units in flight per wave), four for wide matrices with
-    more rows."""
-    return (4 if N >= 12288 and row_blocks > 1 else 2), 8
+    more rows; one where two would make between one and two blocks per compute unit (some
+    units would then stream twice what the others do: 30.7 against 33.3 us for the merged down
+    projection of one token)."""
+    if row_blocks > 1:
+        return (4 if N >= 12288 else 2), 8
+    blocks = groups * ((N + 31) // 32)
+    return (1 if not act and COMPUTE_UNITS < blocks < 2 * COMPUTE_UNITS else 2), 8
+
+
+COMPUTE_UNITS = 256     # of the GPU this library is written for
 
 
 def _row_blocks(group_rows: Optional[int]) -> int:
@@ -479,7 +487,7 @@ def gemm_skinny(x: torch.Tensor, w, out_dtype: torch.dtype, a_rows: Optional[tor
     _need(x.dim() == 2 and x.shape[1] == K, f"gemm_skinny: x {tuple(x.shape)} vs w {tuple(w.shape)}")
     _need(M > 0 and (grouped or M <= SKINNY_MAX_ROWS) and K % 128 == 0 and N % 4 == 0,
           f"gemm_skinny: shape M={M} N={N} K={K} is not taken (M <= 64 unless grouped, K % 128 == 0, N % 4 == 0)")
-    pr, pw = skinny_plan(N, K, _row_blocks(group_rows) if grouped else (M + 15) // 16)
+    pr, pw = skinny_plan(N, K, _row_blocks(group_rows) if grouped else (M + 15) // 16, max(E, 1))
     out = torch.empty(M, N, dtype=out_dtype, device=x.device)
     _run("sharpi_gemm_skinny", _ptr(x), _ptr(w), _ptr(out), _code(out_dtype), M, N, K, _ptr(a_rows), _ptr(offsets), E,
          R or pr, NW or pw, 1 if packed else 0, _row_blocks(group_rows) if grouped else 0, _stream())
@@ -511,7 +519,7 @@ def gemm_skinny_swiglu(x: torch.Tensor, w, offsets: torch.Tensor, a_rows: Option
     _need(not packed or N % 32 == 0, "gemm_skinny_swiglu: packed weights need gate and up rows in whole 16-row tiles")
     if scale is not None:
         _need(scale.dtype == torch.float32 and scale.shape == (M,), "gemm_skinny_swiglu: scale must be float32 [n_rows]")
-    pr, pw = skinny_plan(N, K, _row_blocks(group_rows))
+    pr, pw = skinny_plan(N, K, _row_blocks(group_rows), E, act=True)
     out = torch.empty(M, N // 2, dtype=torch.bfloat16, device=x.device)
     _run("sharpi_gemm_skinny_swiglu", _ptr(x), _ptr(w), _ptr(out), M, N, K, _ptr(a_rows), _ptr(offsets), E,
          _ptr(scale), R or pr, NW or pw, 1 if packed else 0, _row_blocks(group_rows), _stream())
@@ -564,7 +572,8 @@ def gemm_skinny_picked(x: torch.Tensor, w, ids: torch.Tensor, wts: Optional[torc
               "gemm_skinny_picked: weights are float32 [T, k] and belong to the activation form")
     if act:
         _need(out_dtype == torch.bfloat16, "gemm_skinny_picked: the activation form stores bfloat16")
-    pr, pw = skinny_plan(N, K, 1 if T * k <= 16 else 2 if T * k <= 32 else 4)   # (the kernel's own rule for its row blocks)
+    # (row blocks: the kernel's own rule; groups: what it launches)
+    pr, pw = skinny_plan(N, K, 1 if T * k <= 16 else 2 if T * k <= 32 else 4, min(E, T * k) + (1 if shared else 0), act)
     out = torch.empty(rows, N // 2 if act else N, dtype=out_dtype, device=x.device)
     _run("sharpi_gemm_skinny_picked", _ptr(x), _ptr(w), _ptr(out), _code(out_dtype), N, K, _ptr(ids), _ptr(wts), T * k, k, E,
          1 if shared else 0, 1 if gather else 0, 1 if act else 0, pr, pw, 1 if packed else 0, _stream())
