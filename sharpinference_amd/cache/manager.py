@@ -19,6 +19,7 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence, Union
 
+import numpy as np
 import torch
 
 from .spec import KVSpec, StateSpec
@@ -105,6 +106,9 @@ class RequestCache:
     state_slot: int = -1
     tables: List[List[int]] = field(default_factory=list)      # per group: block index -> page or -1
     reserved: List[int] = field(default_factory=list)          # per group: pages promised at admission
+    changed: List[int] = field(default_factory=list)           # per group: how often the table has changed
+    arrays: List[Optional[tuple]] = field(default_factory=list)   # per group: (changed then, the table as int32 array)
+    passed: List[int] = field(default_factory=list)            # per group: blocks below this one were given back
 
 
 class CacheManager:
@@ -206,6 +210,9 @@ class CacheManager:
         rc = RequestCache(req_id)
         rc.tables = [[] for _ in self.groups]
         rc.reserved = [0] * len(self.groups)
+        rc.changed = [0] * len(self.groups)
+        rc.arrays = [None] * len(self.groups)
+        rc.passed = [0] * len(self.groups)
         if reserve_tokens > 0:
             if not self.can_admit(reserve_tokens, max_step_tokens):
                 raise CacheError(f"request {req_id!r}: not enough pages to reserve {reserve_tokens} tokens")
@@ -242,6 +249,14 @@ class CacheManager:
         if n_tokens <= 0:
             raise CacheError("append needs at least one token")
         rc = self.requests[req_id]
+        if n_tokens == 1:      # a decoded token that lands in a page the request already holds: nothing to find
+            b = (rc.length + rc.pending) // self.page_size
+            for tbl in rc.tables:
+                if b >= len(tbl) or tbl[b] < 0:
+                    break
+            else:
+                rc.pending += 1
+                return True
         if not self.can_append(req_id, n_tokens):
             return False
         start = rc.length + rc.pending
@@ -250,13 +265,15 @@ class CacheManager:
             tbl = rc.tables[g]
             first = start // self.page_size
             last = self.blocks_for(end)
-            while len(tbl) < last:
-                tbl.append(-1)
+            if len(tbl) < last:
+                tbl.extend([-1] * (last - len(tbl)))
+                rc.changed[g] += 1
             for b in range(first, last):
                 if tbl[b] < 0:
                     page = grp.pool.alloc()
                     assert page is not None
                     tbl[b] = page
+                    rc.changed[g] += 1
         rc.pending += n_tokens
         return True
 
@@ -272,11 +289,14 @@ class CacheManager:
                 continue
             first_needed = grp.spec.first_visible(rc.length)   # the next query sits at position `length`
             tbl = rc.tables[g]
-            for b in range(min(first_needed // self.page_size, len(tbl))):
+            upto = min(first_needed // self.page_size, len(tbl))
+            for b in range(rc.passed[g], upto):                # (blocks below `passed` went back in earlier steps)
                 if tbl[b] >= 0:
                     grp.pool.release(tbl[b])
                     tbl[b] = -1
                     released += 1
+                    rc.changed[g] += 1
+            rc.passed[g] = max(rc.passed[g], upto)
         return released
 
     def rollback(self, req_id) -> None:
@@ -292,6 +312,7 @@ class CacheManager:
                     grp.pool.release(tbl[b])
                     tbl[b] = -1
             del tbl[keep_blocks:]
+            rc.changed[g] += 1
         rc.pending = 0
 
     def free_request(self, req_id) -> None:
@@ -311,6 +332,16 @@ class CacheManager:
 
     def block_table(self, req_id, group: int) -> List[int]:
         return self.requests[req_id].tables[group]
+
+    def block_table_array(self, req_id, group: int) -> np.ndarray:
+        """The block table as an int32 array (not to be written to), made anew only when the
+        table has changed since it was last asked for: a decoding request changes its table once
+        a page, not once a step."""
+        rc = self.requests[req_id]
+        held = rc.arrays[group]
+        if held is None or held[0] != rc.changed[group]:
+            held = rc.arrays[group] = (rc.changed[group], np.asarray(rc.tables[group], dtype=np.int32))
+        return held[1]
 
     def slots_for(self, req_id, group: int, start: int, n: int) -> List[int]:
         """Flat cache slots (page * page_size + offset) of positions start..start+n-1."""

@@ -51,13 +51,17 @@ __global__ __launch_bounds__(kDecWaves* kWave) void attn_decode_kernel(
   const int lane = threadIdx.x & (kWave - 1);
   const int w = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
-  const int sp = blockIdx.x;
+  // Blocks are handed out kv head first, then token, then run: the heads of a (token, run) read
+  // neighbouring pieces of the same pages at the same time, and the runs that lie beyond a
+  // token's keys (the launch is sized for the longest context it may meet) all come last, where
+  // they hold nobody up.
+  const int sp = blockIdx.z;
   const int li = blockIdx.y;
   const int t = token_list ? token_list[li] : li;
   const int G = nh / nkv;
   const int hgroups = (G + 15) / 16;
-  const int kvh = blockIdx.z / hgroups;
-  const int h0 = kvh * G + (blockIdx.z % hgroups) * 16;
+  const int kvh = blockIdx.x / hgroups;
+  const int h0 = kvh * G + (blockIdx.x % hgroups) * 16;
   const int hcount = min(16, kvh * G + G - h0);
 
   const int p = positions[t];
@@ -275,7 +279,7 @@ static int launch_decode(const void* q, const void* k_cache, const void* v_cache
                          float* part_ml, void* out, int window_kind, int window, float scale, int n_list, int nh,
                          int nkv, int page_size, int max_blocks, int num_pages, int max_splits, hipStream_t stream) {
   const int G = nh / nkv;
-  dim3 grid(max_splits, n_list, nkv * ((G + 15) / 16)), block(kDecWaves * kWave);
+  dim3 grid(nkv * ((G + 15) / 16), n_list, max_splits), block(kDecWaves * kWave);
   attn_decode_kernel<HD><<<grid, block, 0, stream>>>((const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache,
                                                     block_table, entry_of_token, positions, token_list, part_o,
                                                     part_ml, window_kind, window, scale, nh, nkv, page_size,
@@ -300,7 +304,7 @@ SHARPI_EXPORT int sharpi_attention_decode(const void* q, const void* k_cache, co
                                           hipStream_t stream) {
   if (n_list <= 0) return SHARPI_OK;
   if (nh <= 0 || nkv <= 0 || nh % nkv != 0 || nh > 65535 || n_list > 65535) return SHARPI_ERR_ARG;
-  if (page_size <= 0 || page_size % 16 != 0 || max_blocks <= 0 || num_pages <= 0 || max_splits <= 0) return SHARPI_ERR_ARG;
+  if (page_size <= 0 || page_size % 16 != 0 || max_blocks <= 0 || num_pages <= 0 || max_splits <= 0 || max_splits > 65535) return SHARPI_ERR_ARG;
   if (window_kind < 0 || window_kind > 2 || (window_kind != 0 && window <= 0)) return SHARPI_ERR_ARG;
   if (nkv * ((nh / nkv + 15) / 16) > 65535) return SHARPI_ERR_ARG;
 #define DEC(HDV)                                                                                                  \

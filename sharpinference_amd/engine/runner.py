@@ -23,7 +23,9 @@ from ..ops.lib import PREFILL_TILE_TOKENS
 from ..parts.base import GroupView, LayerCache, StepContext
 
 
-MAX_GRAPH_BATCH = 16   # decode steps of up to this many requests are replayed from a HIP graph (beyond, launches no longer bound the step and the fixed maxima cost more than they save)
+MAX_GRAPH_BATCH = 64   # decode steps of up to this many requests are replayed from a HIP graph (at 64 the host's part of an eager step is still a tenth of the step)
+GRAPH_AT_ONCE = 16     # up to this many requests a graph is captured when its shape is first met; wider ones once the
+GRAPH_AFTER_ASKS = 4   # shape has been met this often (a graph per width costs capture time and memory of its own)
 GRAPH_CONTEXT_MIN = 4096   # a graph is captured for a bound on the contexts of its requests: this, or 4, 16, 64 ... times it
 TILE = PREFILL_TILE_TOKENS   # tokens per attention tile of multi-token entries
 
@@ -57,6 +59,7 @@ class ModelRunner:
             all(t is None for t in cache.state) or bool(safe and safe()))
         self.max_context = int(max_context)
         self._graphs: dict = {}
+        self._graph_asks: dict = {}
         self.graph_replays = 0
 
     # ------------------------------------------------------------------
@@ -87,39 +90,46 @@ class ModelRunner:
         lens = [len(e.tokens) for e in entries]
         starts = [cache.length(e.req_id) for e in entries]
         T = sum(lens)
-        token_ids = np.empty(T, dtype=np.int32)
-        positions = np.empty(T, dtype=np.int32)
-        entry_of = np.empty(T, dtype=np.int32)
-        cu = np.zeros(n + 1, dtype=np.int32)
-        rows: List[int] = []
-        o = 0
-        for i, e in enumerate(entries):
-            L = lens[i]
-            token_ids[o:o + L] = np.asarray(e.tokens, dtype=np.int32)
-            positions[o:o + L] = np.arange(starts[i], starts[i] + L, dtype=np.int32)
-            entry_of[o:o + L] = i
-            rows.extend(o + int(w) for w in e.want)
-            o += L
-            cu[i + 1] = o
+        if T == n:
+            # single tokens only (a decode step): no loop over the entries' tokens
+            token_ids = np.fromiter((e.tokens[0] for e in entries), dtype=np.int32, count=n)
+            positions = np.asarray(starts, dtype=np.int32)
+            entry_of = np.arange(n, dtype=np.int32)
+            cu = np.arange(n + 1, dtype=np.int32)
+            rows = [i for i, e in enumerate(entries) for _ in e.want]
+        else:
+            token_ids = np.empty(T, dtype=np.int32)
+            positions = np.empty(T, dtype=np.int32)
+            entry_of = np.empty(T, dtype=np.int32)
+            cu = np.zeros(n + 1, dtype=np.int32)
+            rows = []
+            o = 0
+            for i, e in enumerate(entries):
+                L = lens[i]
+                token_ids[o:o + L] = np.asarray(e.tokens, dtype=np.int32)
+                positions[o:o + L] = np.arange(starts[i], starts[i] + L, dtype=np.int32)
+                entry_of[o:o + L] = i
+                rows.extend(o + int(w) for w in e.want)
+                o += L
+                cu[i + 1] = o
         state_slots = np.asarray([cache.requests[e.req_id].state_slot for e in entries], dtype=np.int32)
         group_tables, group_slots = [], []
+        block_of = positions // ps
         for g in range(len(cache.groups)):
-            tables = [cache.block_table(e.req_id, g) for e in entries]
+            tables = [cache.block_table_array(e.req_id, g) for e in entries]
             if static_blocks is not None:
                 maxb = static_blocks
             else:
-                maxb = max(1, max(len(t) for t in tables))
+                maxb = max(1, max(t.size for t in tables))
                 maxb = (maxb + 3) // 4 * 4
             bt = np.full((n, maxb), -1, dtype=np.int32)
             for i, t in enumerate(tables):
-                bt[i, :len(t)] = t
-            sm = np.empty(T, dtype=np.int32)
-            for i in range(n):
-                pos = positions[cu[i]:cu[i + 1]]
-                pages = bt[i, pos // ps]
-                if (pages < 0).any():
-                    raise CacheError(f"request {entries[i].req_id!r}: a new position has no page in group {g}")
-                sm[cu[i]:cu[i + 1]] = pages * ps + pos % ps
+                bt[i, :t.size] = t
+            pages = bt[entry_of, block_of]          # every token's page, at once
+            if T and int(pages.min()) < 0:
+                i = int(entry_of[int(np.argmin(pages))])
+                raise CacheError(f"request {entries[i].req_id!r}: a new position has no page in group {g}")
+            sm = (pages * ps + positions % ps).astype(np.int32, copy=False)
             group_tables.append(bt)
             group_slots.append(sm)
         rows_np = np.asarray(rows, dtype=np.int32)
@@ -199,6 +209,11 @@ class ModelRunner:
         graph = self._graphs.get(key)
         if graph is False:
             return None
+        if graph is None and n > GRAPH_AT_ONCE:
+            asks = self._graph_asks.get(key, 0) + 1
+            self._graph_asks[key] = asks
+            if asks < GRAPH_AFTER_ASKS:
+                return None
         static_blocks = (bound + self.cache.page_size - 1) // self.cache.page_size
         pieces, info = self._host_arrays(entries, static_blocks=static_blocks)
         if graph is None:

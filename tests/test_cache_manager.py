@@ -135,6 +135,11 @@ def test_random_orders_never_lose_a_page(seed):
                 first = grp.spec.first_visible(L)
                 tbl = m.block_table(rid, g)
                 assert all(tbl[b] >= 0 for b in range(first // m.page_size, (L + m.page_size - 1) // m.page_size))
+                # pages behind the window are all given back (none is kept by a step that skipped them), and
+                # the table as an array, which is made anew only when the table changed, is the table
+                if grp.spec.window_kind != 0:
+                    assert all(tbl[b] < 0 for b in range(min(first // m.page_size, len(tbl))))
+                assert m.block_table_array(rid, g).tolist() == list(tbl)
     reuse = sum(g.pool.total_allocs > g.pool.num_pages for g in m.groups)
     for rid in list(live):
         m.free_request(rid)

@@ -101,7 +101,7 @@ def wide_requests(n: int, vocab: int, seed: int, lo: int = 4, hi: int = 40):
 @pytest.mark.parametrize("width", WIDTHS)
 def test_wide_decode_batches(tmp_path_factory, width, dtype):
     """As many live requests as a serving step has: 5 to 65 single-token entries in one step
-    (graphs up to 16; the shared expert riding with the routed ones up to 16 tokens; the few-rows
+    (graphs at once up to 16; the shared expert riding with the routed ones up to 16 tokens; the few-rows
     products up to 16 rows and the library beyond; picks taken straight from the router up to 64
     pairs and sorted beyond), every logit against the plain implementation."""
     d = make_model_dir(tmp_path_factory.mktemp("wide"), "D", std=0.06)
@@ -126,19 +126,21 @@ def test_sixty_decoded_tokens_beside_a_portion(tmp_path, dtype):
     H.check_trace_against_plain(eng, d, dtype, reqs, steps, f"D {dtype} 60 decoded tokens beside a portion of 40")
 
 
-@pytest.mark.parametrize("width", [8, 16])
+@pytest.mark.parametrize("width", [8, 16, 40, 64])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_decode_graphs_of_wide_batches_equal_eager_steps(tmp_path, width, dtype):
-    """The graphs of batch 8 and 16 (what a served batch replays) against the same steps launched
-    kernel by kernel: the same bits, on the first replay and on later ones."""
+    """The graphs of batch 8 to 64 (what a served batch replays) against the same steps launched
+    kernel by kernel: the same bits, on the first replay and on later ones.  Up to 16 requests a
+    graph is captured at the first step of its shape, wider ones at the fourth."""
     d = make_model_dir(tmp_path, "D", std=0.06)
-    reqs = wide_requests(width, 500, 50 + width)
-    steps = H.wide_trace(reqs, tail=4)
+    tail = 4 if width <= 16 else 8
+    reqs = wide_requests(width, 500, 50 + width, lo=tail + 2)
+    steps = H.wide_trace(reqs, tail=tail)
     out = {}
     for graphs in (True, False):
         eng = H.make_engine(d, dtype, kv_tokens=H.tokens_held(steps), max_num_seqs=width, decode_graphs=graphs)
         out[graphs] = H.replay(eng, steps)
-        assert eng.runner.graph_replays == (4 if graphs else 0)
+        assert eng.runner.graph_replays == ((tail if width <= 16 else tail - 3) if graphs else 0)
     for r in reqs:
         assert torch.equal(out[True][r], out[False][r]), r
 
