@@ -74,12 +74,20 @@ __device__ __forceinline__ void store8(bf16_t* p, const float* v) {
   *reinterpret_cast<uint4*>(p) = o;
 }
 
-// SwiGLU of one element: silu(s g) * (s u), silu(x) = x / (1 + exp(-x)); one definition for the
-// activation kernel and for the product that applies it in its epilogue, so both give the same bits
-__device__ __forceinline__ float swiglu_f32(float g, float u, float s, bool scaled) {
+// The gated unit of a feed-forward, one element: act(s g) * (s u), with the activation a code that
+// the caller passes (shared with the Python side): SiLU x / (1 + exp(-x)), or GELU in its tanh form
+// 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))).  One definition for the activation kernel and
+// for the products that apply it in their epilogue, so both give the same bits.
+enum : int { ACT_SILU = 1, ACT_GELU_TANH = 2 };
+static inline __host__ __device__ bool act_known(int act) { return act == ACT_SILU || act == ACT_GELU_TANH; }
+__device__ __forceinline__ float gated_f32(int act, float g, float u, float s, bool scaled) {
   if (scaled) {
     g *= s;
     u *= s;
+  }
+  if (act == ACT_GELU_TANH) {
+    const float t = tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g));
+    return (0.5f * g * (1.0f + t)) * u;
   }
   return (g / (1.0f + expf(-g))) * u;
 }

@@ -259,24 +259,24 @@ SHARPI_EXPORT int sharpi_add_rmsnorm(float* h, const void* delta, int delta_dtyp
 }
 
 // ---------------------------------------------------------------------------
-// SwiGLU activation on a fused [M, 2*I] buffer (gate columns first, up columns second):
-//   out[m, i] = silu(s_m * g) * (s_m * u),  silu(x) = x / (1 + exp(-x)),  s_m = scale ? scale[m] : 1
+// The gated unit on a fused [M, 2*I] buffer (gate columns first, up columns second):
+//   out[m, i] = act(s_m * g) * (s_m * u),  s_m = scale ? scale[m] : 1,  act as common.h codes it
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ void silu_mul_kernel(const T* __restrict__ gu, const float* __restrict__ scale,
-                                T* __restrict__ out, int inter) {
+                                T* __restrict__ out, int inter, int act) {
   const int m = blockIdx.x;
   const int i = blockIdx.y * blockDim.x + threadIdx.x;
   if (i >= inter) return;
   const T* row = gu + (size_t)m * 2 * inter;
   const float g = to_f32<T>(row[i]);
   const float u = to_f32<T>(row[inter + i]);
-  out[(size_t)m * inter + i] = from_f32<T>(swiglu_f32(g, u, scale ? scale[m] : 1.0f, scale != nullptr));
+  out[(size_t)m * inter + i] = from_f32<T>(gated_f32(act, g, u, scale ? scale[m] : 1.0f, scale != nullptr));
 }
 
 template <typename T>
 __global__ void silu_mul_vec_kernel(const T* __restrict__ gu, const float* __restrict__ scale,
-                                    T* __restrict__ out, int inter) {
+                                    T* __restrict__ out, int inter, int act) {
   const int m = blockIdx.x;
   const int i = (blockIdx.y * blockDim.x + threadIdx.x) * 8;
   if (i >= inter) return;
@@ -286,26 +286,26 @@ __global__ void silu_mul_vec_kernel(const T* __restrict__ gu, const float* __res
   load8(row + inter + i, u);
   const float s = scale ? scale[m] : 1.0f;
 #pragma unroll
-  for (int j = 0; j < 8; ++j) o[j] = swiglu_f32(g[j], u[j], s, scale != nullptr);
+  for (int j = 0; j < 8; ++j) o[j] = gated_f32(act, g[j], u[j], s, scale != nullptr);
   store8(out + (size_t)m * inter + i, o);
 }
 
 SHARPI_EXPORT int sharpi_silu_mul(const void* gu, const float* scale, void* out, int dtype, int rows, int inter,
-                                  hipStream_t stream) {
+                                  int act, hipStream_t stream) {
   if (rows <= 0) return SHARPI_OK;
-  if (inter <= 0 || ceil_div(inter, 256) > 65535) return SHARPI_ERR_ARG;
+  if (inter <= 0 || ceil_div(inter, 256) > 65535 || !act_known(act)) return SHARPI_ERR_ARG;
   dim3 block(256), grid(rows, ceil_div(inter, 256));
   if (dtype != DT_F32 && dtype != DT_BF16) return SHARPI_ERR_ARG;
   if ((inter & 7) == 0) {
     dim3 vgrid(rows, ceil_div(inter, 256 * 8));
     if (dtype == DT_F32)
-      silu_mul_vec_kernel<float><<<vgrid, block, 0, stream>>>((const float*)gu, scale, (float*)out, inter);
+      silu_mul_vec_kernel<float><<<vgrid, block, 0, stream>>>((const float*)gu, scale, (float*)out, inter, act);
     else
-      silu_mul_vec_kernel<bf16_t><<<vgrid, block, 0, stream>>>((const bf16_t*)gu, scale, (bf16_t*)out, inter);
+      silu_mul_vec_kernel<bf16_t><<<vgrid, block, 0, stream>>>((const bf16_t*)gu, scale, (bf16_t*)out, inter, act);
   } else if (dtype == DT_F32)
-    silu_mul_kernel<float><<<grid, block, 0, stream>>>((const float*)gu, scale, (float*)out, inter);
+    silu_mul_kernel<float><<<grid, block, 0, stream>>>((const float*)gu, scale, (float*)out, inter, act);
   else
-    silu_mul_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)gu, scale, (bf16_t*)out, inter);
+    silu_mul_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)gu, scale, (bf16_t*)out, inter, act);
   SHARPI_CHECK_LAUNCH();
   return SHARPI_OK;
 }

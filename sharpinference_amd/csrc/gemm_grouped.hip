@@ -82,8 +82,8 @@ __device__ __forceinline__ int xs_col(int row, int col) { return col ^ (((row >>
 template <typename TO, int MT, bool PACKED, bool ACT>
 __device__ __forceinline__ void grouped_tile(const bf16_t* __restrict__ x, const bf16_t* __restrict__ We,
                                              TO* __restrict__ out, int N, int K, const int* __restrict__ a_rows,
-                                             const float* __restrict__ act_scale, int row0, int row_end, int n_base,
-                                             bf16_t (*xs)[GM][GPAD]) {
+                                             const float* __restrict__ act_scale, int act, int row0, int row_end,
+                                             int n_base, bf16_t (*xs)[GM][GPAD]) {
   static_assert(!ACT || NT == 2, "the SwiGLU form pairs one gate tile with one up tile");
   const int n_out = ACT ? N / 2 : N;            // output columns
   constexpr int PASS = (MT * 16 + GROWS - 1) / GROWS;   // staging passes
@@ -244,8 +244,8 @@ __device__ __forceinline__ void grouped_tile(const bf16_t* __restrict__ x, const
       f32x4 o;
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        o[i] = swiglu_f32(bf16_to_f32(f32_to_bf16(acc[0][mb][i])), bf16_to_f32(f32_to_bf16(acc[1][mb][i])), sc,
-                          act_scale != nullptr);
+        o[i] = gated_f32(act, bf16_to_f32(f32_to_bf16(acc[0][mb][i])), bf16_to_f32(f32_to_bf16(acc[1][mb][i])), sc,
+                         act_scale != nullptr);
       store(out + (size_t)row * n_out + n, o);
     } else {
 #pragma unroll
@@ -261,8 +261,8 @@ __device__ __forceinline__ void grouped_tile(const bf16_t* __restrict__ x, const
 template <typename TO, bool PACKED, bool ACT>
 __global__ __launch_bounds__(GW* kWave, 2) void grouped_gemm_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ W, TO* __restrict__ out, int N, int K,
-    const int* __restrict__ a_rows, const float* __restrict__ act_scale, const int* __restrict__ group_offsets,
-    const int* __restrict__ plan, int n_groups, int nb) {
+    const int* __restrict__ a_rows, const float* __restrict__ act_scale, int act,
+    const int* __restrict__ group_offsets, const int* __restrict__ plan, int n_groups, int nb) {
   __shared__ __attribute__((aligned(16))) bf16_t xs[2][GM][GPAD];
   constexpr int kCols = ACT ? GN / 2 : GN;   // output columns of a block
   const int n_out = ACT ? N / 2 : N;
@@ -300,7 +300,7 @@ __global__ __launch_bounds__(GW* kWave, 2) void grouped_gemm_kernel(
   const int n_base = nblock * kCols + (threadIdx.x >> 6) * (ACT ? 16 : 16 * NT);
   const bf16_t* We = W + (size_t)e * N * K;
   static_assert(GM == 192, "tile heights are compiled in steps of 32 rows up to 192");
-#define GT(MTV) grouped_tile<TO, MTV, PACKED, ACT>(x, We, out, N, K, a_rows, act_scale, row0, row_end, n_base, xs)
+#define GT(MTV) grouped_tile<TO, MTV, PACKED, ACT>(x, We, out, N, K, a_rows, act_scale, act, row0, row_end, n_base, xs)
   if (n_rows <= 32) GT(2);
   else if (n_rows <= 64) GT(4);
   else if (n_rows <= 96) GT(6);
@@ -340,7 +340,7 @@ SHARPI_EXPORT int sharpi_gemm_grouped(const void* x, int x_rows, const void* W, 
   if (!grouped_grid(n_rows, n_groups, nb, &grid)) return SHARPI_ERR_ARG;
 #define GG_LAUNCH(TOV, PK)                                                                                          \
   grouped_gemm_kernel<TOV, PK, false><<<grid, block, 0, stream>>>((const bf16_t*)x, (const bf16_t*)W, (TOV*)out, N, \
-                                                                 K, a_rows, nullptr, group_offsets, plan, n_groups, nb)
+                                                                 K, a_rows, nullptr, 0, group_offsets, plan, n_groups, nb)
   if (out_dtype == DT_BF16) {
     if (packed) GG_LAUNCH(bf16_t, true); else GG_LAUNCH(bf16_t, false);
   } else if (out_dtype == DT_F32) {
@@ -353,23 +353,26 @@ SHARPI_EXPORT int sharpi_gemm_grouped(const void* x, int x_rows, const void* W, 
   return SHARPI_OK;
 }
 
-// The grouped product with SwiGLU in its epilogue: W [>= n_groups, N, K] holds gate rows [0, N/2)
-// then up rows of every group; out [n_rows, N/2] bf16 = silu(s g) * (s u) with g, u the two
-// products rounded to bfloat16 and s = act_scale[row] (null: 1).  N % 32 == 0; the rest as above.
+// The grouped product with the gated unit in its epilogue: W [>= n_groups, N, K] holds gate rows
+// [0, N/2) then up rows of every group; out [n_rows, N/2] bf16 = act(s g) * (s u) with g, u the two
+// products rounded to bfloat16, s = act_scale[row] (null: 1) and act the activation's code
+// (common.h).  N % 32 == 0; the rest as above.
 SHARPI_EXPORT int sharpi_gemm_grouped_swiglu(const void* x, int x_rows, const void* W, void* out, int n_rows, int N,
                                              int K, const int* a_rows, const int* group_offsets, const int* plan,
-                                             int n_groups, const float* act_scale, int packed, hipStream_t stream) {
+                                             int n_groups, const float* act_scale, int packed, int act,
+                                             hipStream_t stream) {
   if (n_rows <= 0) return SHARPI_OK;
+  if (!act_known(act)) return SHARPI_ERR_ARG;
   if ((N & 31) || !grouped_args_ok(x_rows, n_rows, N, K, n_groups, packed, group_offsets, plan)) return SHARPI_ERR_ARG;
   const int nb = ceil_div(N / 2, GN / 2);
   dim3 grid, block(GW * kWave);
   if (!grouped_grid(n_rows, n_groups, nb, &grid)) return SHARPI_ERR_ARG;
   if (packed)
     grouped_gemm_kernel<bf16_t, true, true><<<grid, block, 0, stream>>>(
-        (const bf16_t*)x, (const bf16_t*)W, (bf16_t*)out, N, K, a_rows, act_scale, group_offsets, plan, n_groups, nb);
+        (const bf16_t*)x, (const bf16_t*)W, (bf16_t*)out, N, K, a_rows, act_scale, act, group_offsets, plan, n_groups, nb);
   else
     grouped_gemm_kernel<bf16_t, false, true><<<grid, block, 0, stream>>>(
-        (const bf16_t*)x, (const bf16_t*)W, (bf16_t*)out, N, K, a_rows, act_scale, group_offsets, plan, n_groups, nb);
+        (const bf16_t*)x, (const bf16_t*)W, (bf16_t*)out, N, K, a_rows, act_scale, act, group_offsets, plan, n_groups, nb);
   SHARPI_CHECK_LAUNCH();
   return SHARPI_OK;
 }

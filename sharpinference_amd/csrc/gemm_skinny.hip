@@ -4,7 +4,7 @@
 
 // defined beside the SwiGLU form's kernels
 int skinny_picked_swiglu(const void* x, const void* W, void* out, int M, int N, int K, const Picks& pk, int groups, int R,
-                         int NW, int packed, hipStream_t stream);
+                         int NW, int packed, int act, hipStream_t stream);
 
 template <int R, int NW, bool PACKED>
 static int dispatch_mb(int MB, const void* x, const void* W, void* out, int out_dtype, int M, int N, int K,
@@ -48,8 +48,8 @@ SHARPI_EXPORT int sharpi_gemm_skinny(const void* x, const void* W, void* out, in
 // ids [n_pairs] (pair i = token i / k, pick i % k), W [n_experts (+ 1 if shared), N, K]; out row i is
 // pair i, rows n_pairs .. n_pairs + n_pairs / k - 1 are the tokens through expert n_experts (shared != 0).
 // gather: x [tokens, K] is read by token; otherwise x rows are in the output's order.  With act != 0
-// W holds gate then up rows and out [rows, N/2] bf16 = silu(s g) * (s u), s = w[i] for pair i (w may
-// be null: no scaling) and 1 for the shared rows.  n_pairs and the tokens fit one wave's ballot (<= 64).
+// (an activation's code, common.h) W holds gate then up rows and out [rows, N/2] bf16 =
+// act(s g) * (s u), s = w[i] for pair i (w may be null: no scaling) and 1 for the shared rows.  n_pairs and the tokens fit one wave's ballot (<= 64).
 SHARPI_EXPORT int sharpi_gemm_skinny_picked(const void* x, const void* W, void* out, int out_dtype, int N, int K,
                                             const int* ids, const float* w, int n_pairs, int k, int n_experts,
                                             int shared, int gather, int act, int R, int NW, int packed,
@@ -59,13 +59,13 @@ SHARPI_EXPORT int sharpi_gemm_skinny_picked(const void* x, const void* W, void* 
   if (N <= 0 || (N & (act ? 7 : 3)) || K <= 0 || (K & 127)) return SHARPI_ERR_ARG;
   if (packed && (N & (act ? 31 : 15))) return SHARPI_ERR_ARG;
   if (out_dtype != DT_F32 && out_dtype != DT_BF16) return SHARPI_ERR_ARG;
-  if (act && out_dtype != DT_BF16) return SHARPI_ERR_ARG;
+  if (act && (out_dtype != DT_BF16 || !act_known(act))) return SHARPI_ERR_ARG;
   // a group for every expert that can have rows: no more distinct experts than pairs
   const int groups = (n_experts < n_pairs ? n_experts : n_pairs) + (shared ? 1 : 0);
   if (groups > 65535) return SHARPI_ERR_ARG;
   const int M = n_pairs + (shared ? n_pairs / k : 0);
   const Picks pk = {ids, w, n_pairs, k, n_experts, gather, shared ? 1 : 0};
-  if (act) return skinny_picked_swiglu(x, W, out, M, N, K, pk, groups, R, NW, packed, stream);
+  if (act) return skinny_picked_swiglu(x, W, out, M, N, K, pk, groups, R, NW, packed, act, stream);
   // an expert has at most n_pairs rows: one, two or four blocks of sixteen rows against one stream of its weights
   const int MB = n_pairs <= 16 ? 1 : n_pairs <= 32 ? 2 : 4;
   // group_offsets is not read in this form; the pointer only has to be non-null for the grid's sake

@@ -29,10 +29,11 @@
 //    of a (16-row tile, 128-wide K unit) contiguous and in the order the lanes want them, and
 //    the K units are dealt to the waves in turn: a block's reads are contiguous runs of NW * 4 KB
 //    rather than 256-byte pieces a row apart, worth about a tenth of the bandwidth.
-//  * SwiGLU form (ACT): W holds gate rows [0, N/2) and up rows [N/2, N); a block takes R/2 tiles
+//  * Gated form (ACT): W holds gate rows [0, N/2) and up rows [N/2, N); a block takes R/2 tiles
 //    of each at the same columns, and the wave that adds up a gate tile adds up its up tile too,
 //    rounds both to bfloat16 (what a separate activation kernel would have read) and stores
-//    silu(s g) * (s u), s the row's score: out is [M, N/2] and the gate|up rows never go to memory.
+//    act(s g) * (s u), s the row's score and act the activation the caller names (SiLU, GELU):
+//    out is [M, N/2] and the gate|up rows never go to memory.
 //
 // Limits (the caller falls back to other kernels otherwise): K % 128 == 0, N % 4 == 0, M <= 64 (plain form).
 #pragma once
@@ -71,7 +72,7 @@ template <int R, int MB, int NW, typename TO, bool ACT, bool PACKED>
 __global__ __launch_bounds__(NW* kWave) void skinny_gemm_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ W, TO* __restrict__ out, int M, int N, int K,
     const int* __restrict__ a_rows, const int* __restrict__ group_offsets, const float* __restrict__ act_scale,
-    Picks pk) {
+    int act, Picks pk) {
   static_assert(!ACT || R % 2 == 0, "the SwiGLU form pairs gate and up tiles");
   constexpr int RT = ACT ? R : kRedTiles;   // tiles that meet in LDS per round
   constexpr int TG = ACT ? R / 2 : R;       // tiles of distinct output columns per block
@@ -279,7 +280,7 @@ __global__ __launch_bounds__(NW* kWave) void skinny_gemm_kernel(
             f32x4 o;
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-              o[i] = swiglu_f32(bf16_to_f32(f32_to_bf16(gv[i])), bf16_to_f32(f32_to_bf16(uv[i])), sc, scaled);
+              o[i] = gated_f32(act, bf16_to_f32(f32_to_bf16(gv[i])), bf16_to_f32(f32_to_bf16(uv[i])), sc, scaled);
             store4<TO>(out + (size_t)orow * n_out + n, o);
           }
         }
@@ -317,15 +318,15 @@ __global__ __launch_bounds__(NW* kWave) void skinny_gemm_kernel(
 template <int R, int MB, int NW, bool ACT, bool PACKED>
 static inline int launch_skinny(const void* x, const void* W, void* out, int out_dtype, int M, int N, int K,
                          const int* a_rows, const int* group_offsets, int groups, const float* act_scale,
-                         hipStream_t stream, Picks pk = Picks{}) {
+                         hipStream_t stream, Picks pk = Picks{}, int act = ACT_SILU) {
   dim3 grid(ceil_div(ACT ? N / 2 : N, 16 * (ACT ? R / 2 : R)), groups > 0 ? groups : 1), block(NW * kWave);
   const int* go = groups > 0 ? group_offsets : nullptr;
   if (out_dtype == DT_F32)
     skinny_gemm_kernel<R, MB, NW, float, ACT, PACKED><<<grid, block, 0, stream>>>(
-        (const bf16_t*)x, (const bf16_t*)W, (float*)out, M, N, K, a_rows, go, act_scale, pk);
+        (const bf16_t*)x, (const bf16_t*)W, (float*)out, M, N, K, a_rows, go, act_scale, act, pk);
   else
     skinny_gemm_kernel<R, MB, NW, bf16_t, ACT, PACKED><<<grid, block, 0, stream>>>(
-        (const bf16_t*)x, (const bf16_t*)W, (bf16_t*)out, M, N, K, a_rows, go, act_scale, pk);
+        (const bf16_t*)x, (const bf16_t*)W, (bf16_t*)out, M, N, K, a_rows, go, act_scale, act, pk);
   SHARPI_CHECK_LAUNCH();
   return SHARPI_OK;
 }

@@ -16,6 +16,8 @@ from . import profile as _profile
 _DT = {torch.float32: 0, torch.bfloat16: 1}
 
 WINDOW_NONE, WINDOW_CHUNK, WINDOW_SLIDING = 0, 1, 2
+ACT_SILU, ACT_GELU_TANH = 1, 2      # the gated unit's activation, as the kernels code it
+ACTIVATIONS = {"silu": ACT_SILU, "gelu_tanh": ACT_GELU_TANH}
 
 
 class KernelError(RuntimeError):
@@ -141,16 +143,22 @@ def add_rmsnorm(h: torch.Tensor, delta, weight: Optional[torch.Tensor], eps: flo
     return out
 
 
-def silu_mul(gate_up: torch.Tensor, scale: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """[M, 2I] (gate columns, then up columns) -> silu(s*g) * (s*u) [M, I]."""
+def gated_act(gate_up: torch.Tensor, scale: Optional[torch.Tensor] = None, act: int = ACT_SILU) -> torch.Tensor:
+    """[M, 2I] (gate columns, then up columns) -> act(s*g) * (s*u) [M, I]; act: ACT_SILU or
+    ACT_GELU_TANH."""
     _dev(gate_up, scale)
-    _need(gate_up.dim() == 2 and gate_up.shape[1] % 2 == 0, "silu_mul: input must be [M, 2I]")
+    _need(gate_up.dim() == 2 and gate_up.shape[1] % 2 == 0, "gated_act: input must be [M, 2I]")
     M, I2 = gate_up.shape
     if scale is not None:
-        _need(scale.dtype == torch.float32 and scale.shape == (M,), "silu_mul: scale must be float32 [M]")
+        _need(scale.dtype == torch.float32 and scale.shape == (M,), "gated_act: scale must be float32 [M]")
     out = torch.empty(M, I2 // 2, dtype=gate_up.dtype, device=gate_up.device)
-    _run("sharpi_silu_mul", _ptr(gate_up), _ptr(scale), _ptr(out), _code(gate_up.dtype), M, I2 // 2, _stream())
+    _run("sharpi_silu_mul", _ptr(gate_up), _ptr(scale), _ptr(out), _code(gate_up.dtype), M, I2 // 2, int(act), _stream())
     return out
+
+
+def silu_mul(gate_up: torch.Tensor, scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """[M, 2I] (gate columns, then up columns) -> silu(s*g) * (s*u) [M, I]."""
+    return gated_act(gate_up, scale, ACT_SILU)
 
 
 def moe_combine(y: torch.Tensor, inv_pos: torch.Tensor, shared: Optional[torch.Tensor], n_tokens: int,
@@ -496,7 +504,7 @@ def gemm_skinny(x: torch.Tensor, w, out_dtype: torch.dtype, a_rows: Optional[tor
 
 def gemm_skinny_swiglu(x: torch.Tensor, w, offsets: torch.Tensor, a_rows: Optional[torch.Tensor],
                        n_rows: int, scale: Optional[torch.Tensor], R: Optional[int] = None,
-                       NW: Optional[int] = None, group_rows: Optional[int] = None) -> torch.Tensor:
+                       NW: Optional[int] = None, group_rows: Optional[int] = None, act: int = ACT_SILU) -> torch.Tensor:
     """Per expert, silu(s g) * (s u) with (g | u) = x @ w[e]^T rounded to bfloat16, w [E, 2I, K]
     holding gate rows then up rows: the product and the activation in one kernel, for at most
     64 rows.  Returns [n_rows, I] bfloat16."""
@@ -522,7 +530,7 @@ def gemm_skinny_swiglu(x: torch.Tensor, w, offsets: torch.Tensor, a_rows: Option
     pr, pw = skinny_plan(N, K, _row_blocks(group_rows), E, act=True)
     out = torch.empty(M, N // 2, dtype=torch.bfloat16, device=x.device)
     _run("sharpi_gemm_skinny_swiglu", _ptr(x), _ptr(w), _ptr(out), M, N, K, _ptr(a_rows), _ptr(offsets), E,
-         _ptr(scale), R or pr, NW or pw, 1 if packed else 0, _row_blocks(group_rows), _stream())
+         _ptr(scale), R or pr, NW or pw, 1 if packed else 0, _row_blocks(group_rows), int(act), _stream())
     return out
 
 
@@ -548,12 +556,14 @@ def picked_ok(n_tokens: int, k: int, N: int, K: int, act: bool, packed: bool) ->
 
 
 def gemm_skinny_picked(x: torch.Tensor, w, ids: torch.Tensor, wts: Optional[torch.Tensor], shared: bool, gather: bool,
-                       act: bool, out_dtype: torch.dtype) -> torch.Tensor:
+                       act, out_dtype: torch.dtype) -> torch.Tensor:
     """Per-expert products of a few decode tokens straight from the router's picks ids [T, k]:
     row i of the result is pair i = (token i // k, pick i % k), followed (shared) by one row per
     token through expert E of w [E + 1, N, K].  gather: x [T, K] is read by token, otherwise x is in
-    the result's row order.  act: w holds gate rows then up rows and the result is
-    silu(s g) * (s u) [rows, N/2] with s the pair's weight (wts; 1 for the shared rows)."""
+    the result's row order.  act (True: SiLU; or an activation's code; False: none): w holds gate
+    rows then up rows and the result is act(s g) * (s u) [rows, N/2] with s the pair's weight (wts;
+    1 for the shared rows)."""
+    act = ACT_SILU if act is True else int(act or 0)
     w, packed = _unwrap(w)
     _dev(x, w, ids, wts)
     _i32(ids, "ids")
@@ -573,10 +583,10 @@ def gemm_skinny_picked(x: torch.Tensor, w, ids: torch.Tensor, wts: Optional[torc
     if act:
         _need(out_dtype == torch.bfloat16, "gemm_skinny_picked: the activation form stores bfloat16")
     # (row blocks: the kernel's own rule; groups: what it launches)
-    pr, pw = skinny_plan(N, K, 1 if T * k <= 16 else 2 if T * k <= 32 else 4, min(E, T * k) + (1 if shared else 0), act)
+    pr, pw = skinny_plan(N, K, 1 if T * k <= 16 else 2 if T * k <= 32 else 4, min(E, T * k) + (1 if shared else 0), bool(act))
     out = torch.empty(rows, N // 2 if act else N, dtype=out_dtype, device=x.device)
     _run("sharpi_gemm_skinny_picked", _ptr(x), _ptr(w), _ptr(out), _code(out_dtype), N, K, _ptr(ids), _ptr(wts), T * k, k, E,
-         1 if shared else 0, 1 if gather else 0, 1 if act else 0, pr, pw, 1 if packed else 0, _stream())
+         1 if shared else 0, 1 if gather else 0, act, pr, pw, 1 if packed else 0, _stream())
     return out
 
 
@@ -770,9 +780,10 @@ def gemm_grouped(x: torch.Tensor, w, rt: Routing, gather: bool, out_dtype: torch
     return out
 
 
-def gemm_grouped_swiglu(x: torch.Tensor, w, rt: Routing, scale: Optional[torch.Tensor], gather: bool = True) -> torch.Tensor:
-    """Per group, silu(s g) * (s u) with (g | u) = x @ w[e]^T rounded to bfloat16, for many rows: the
-    grouped product with the activation in its epilogue.  gather: x rows are read through the
+def gemm_grouped_swiglu(x: torch.Tensor, w, rt: Routing, scale: Optional[torch.Tensor], gather: bool = True,
+                        act: int = ACT_SILU) -> torch.Tensor:
+    """Per group, act(s g) * (s u) with (g | u) = x @ w[e]^T rounded to bfloat16, for many rows: the
+    grouped product with the activation (ACT_SILU, ACT_GELU_TANH) in its epilogue.  gather: x rows are read through the
     routing's token list (the order inside a group is whatever the routing kernel made it);
     otherwise x is already in the groups' order.  w [E (+ 1), 2I, K] holds gate rows then up
     rows.  Returns [n_rows, I] bfloat16."""
@@ -788,7 +799,8 @@ def gemm_grouped_swiglu(x: torch.Tensor, w, rt: Routing, scale: Optional[torch.T
         _need(scale.dtype == torch.float32 and scale.shape == (rt.n_rows,), "gemm_grouped_swiglu: scale must be float32 [n_rows]")
     out = torch.empty(rt.n_rows, N // 2, dtype=torch.bfloat16, device=x.device)
     _run("sharpi_gemm_grouped_swiglu", _ptr(x), x.shape[0], _ptr(w), _ptr(out), rt.n_rows, N, K,
-         _ptr(rt.sorted_token) if gather else None, _ptr(rt.offsets), _ptr(rt.plan), rt.n_groups, _ptr(scale), 1 if packed else 0, _stream())
+         _ptr(rt.sorted_token) if gather else None, _ptr(rt.offsets), _ptr(rt.plan), rt.n_groups, _ptr(scale), 1 if packed else 0,
+         int(act), _stream())
     return out
 
 
@@ -826,11 +838,11 @@ def linear_many_rows(x: torch.Tensor, w: PackedWeight, out_dtype: torch.dtype) -
     return gemm_grouped(x, PackedWeight(w.packed.unsqueeze(0), None), rt, False, out_dtype)
 
 
-def swiglu_many_rows(x: torch.Tensor, w_gate_up: PackedWeight) -> torch.Tensor:
+def swiglu_many_rows(x: torch.Tensor, w_gate_up: PackedWeight, act: int = ACT_SILU) -> torch.Tensor:
     """silu(g) * u with (g | u) = x @ w_gate_up^T rounded to bfloat16, for many rows, the activation
     in the product's epilogue: [M, I] bfloat16."""
     rt = _dense_routing(x.shape[0], x.device)
-    return gemm_grouped_swiglu(x, PackedWeight(w_gate_up.packed.unsqueeze(0), None), rt, None, gather=False)
+    return gemm_grouped_swiglu(x, PackedWeight(w_gate_up.packed.unsqueeze(0), None), rt, None, gather=False, act=act)
 
 
 # ---------------------------------------------------------------------------
@@ -895,9 +907,10 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, gro
                              window, scale, nh, nkv, hd)
 
 
-def grouped_swiglu(x: torch.Tensor, w_gate_up, rt: Routing, out_dtype: torch.dtype, scaled: bool = True) -> torch.Tensor:
+def grouped_swiglu(x: torch.Tensor, w_gate_up, rt: Routing, out_dtype: torch.dtype, scaled: bool = True,
+                   act: int = ACT_SILU) -> torch.Tensor:
     """The experts' gate|up products of the routed tokens and their activation,
-    silu(s g) * (s u) with s the pick's weight (``scaled``; otherwise s = 1): [n_rows, I] in
+    act(s g) * (s u) with s the pick's weight (``scaled``; otherwise s = 1): [n_rows, I] in
     expert-sorted order.  On the matrix cores the activation is the product's epilogue (the
     few-rows kernel or the many-rows one); otherwise the product and the activation are two kernels."""
     N, K = w_gate_up.shape[1], w_gate_up.shape[2]
@@ -905,10 +918,10 @@ def grouped_swiglu(x: torch.Tensor, w_gate_up, rt: Routing, out_dtype: torch.dty
     if x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16 and out_dtype == torch.bfloat16 and K % 128 == 0:
         if rt.n_tokens <= SKINNY_MAX_ROWS and N % (32 if isinstance(w_gate_up, PackedWeight) else 8) == 0:
             return gemm_skinny_swiglu(x, w_gate_up, rt.offsets, rt.sorted_token, rt.n_rows, scale,
-                                      group_rows=rt.n_tokens)
+                                      group_rows=rt.n_tokens, act=act)
         if rt.n_tokens > SKINNY_MAX_ROWS and N % 32 == 0:
-            return gemm_grouped_swiglu(x, w_gate_up, rt, scale)
-    return silu_mul(grouped_linear(x, w_gate_up, rt, True, out_dtype), scale)
+            return gemm_grouped_swiglu(x, w_gate_up, rt, scale, act=act)
+    return gated_act(grouped_linear(x, w_gate_up, rt, True, out_dtype), scale, act)
 
 
 def grouped_linear(x: torch.Tensor, w, rt: Routing, gather: bool, out_dtype: torch.dtype) -> torch.Tensor:

@@ -19,7 +19,7 @@ F = c_float
 _SIGNATURES = {
     "sharpi_embed_gather": [P, P, I, P, I, I, P],
     "sharpi_add_rmsnorm": [P, P, I, P, I, P, I, P, I, I, F, I, P, P, P, I, P],
-    "sharpi_silu_mul": [P, P, P, I, I, I, P],
+    "sharpi_silu_mul": [P, P, P, I, I, I, I, P],
     "sharpi_moe_combine": [P, P, P, P, P, I, I, I, I, P],
     "sharpi_cast": [P, I, P, I, c_longlong, P],
     "sharpi_peak_read": [P, c_longlong, P, P, P],
@@ -31,13 +31,13 @@ _SIGNATURES = {
     "sharpi_attention_prefill": [P, P, P, P, P, P, P, I, I, I, F, I, I, I, I, I, I, P],
     "sharpi_gemm_tiled": [P, P, P, I, I, I, I, I, P, P, I, P],
     "sharpi_gemm_skinny": [P, P, P, I, I, I, I, P, P, I, I, I, I, I, P],
-    "sharpi_gemm_skinny_swiglu": [P, P, P, I, I, I, P, P, I, P, I, I, I, I, P],
+    "sharpi_gemm_skinny_swiglu": [P, P, P, I, I, I, P, P, I, P, I, I, I, I, I, P],
     "sharpi_gemm_skinny_picked": [P, P, P, I, I, I, P, P, I, I, I, I, I, I, I, I, I, P],
     "sharpi_add_rmsnorm_router": [P, P, P, I, P, I, I, F, P, I, P, P, I, I, I, I, P],
     "sharpi_router_topk": [P, I, P, I, P, P, P, I, I, I, I, I, I, P],
     "sharpi_moe_permute": [P, P, P, P, P, P, P, I, I, I, I, I, P],
     "sharpi_gemm_grouped": [P, I, P, P, I, I, I, I, P, P, P, I, I, P],
-    "sharpi_gemm_grouped_swiglu": [P, I, P, P, I, I, I, P, P, P, I, P, I, P],
+    "sharpi_gemm_grouped_swiglu": [P, I, P, P, I, I, I, P, P, P, I, P, I, I, P],
     "sharpi_argmax_rows": [P, P, I, I, P],
     "sharpi_sample_rows": [P, P, P, P, P, P, P, P, I, I, P],
     "sharpi_edit_logits": [P, P, P, P, P, P, P, P, I, I, P],

@@ -26,12 +26,21 @@ def _rows(w) -> torch.Tensor:
     return ops.unpack_weight(w) if isinstance(w, ops.PackedWeight) else w
 
 
-class DenseSwiGLU(Part):
-    """down( silu(gate x) * (up x) ) (reference: src/SharpInference.Engine/ForwardPass.cs:2006-2015;
-    silu(g) = g / (1 + exp(-g)), src/SharpInference.Cpu/SimdKernels.cs:4377-4408)."""
+def _activation_code(name: str) -> int:
+    try:
+        return ops.ACTIVATIONS[name]
+    except KeyError:
+        raise ValueError(f"activation {name!r} is not known ({', '.join(sorted(ops.ACTIVATIONS))})") from None
 
-    def __init__(self, hidden: int, intermediate: int):
+
+class DenseSwiGLU(Part):
+    """down( act(gate x) * (up x) ) (reference: src/SharpInference.Engine/ForwardPass.cs:2006-2015;
+    silu(g) = g / (1 + exp(-g)), src/SharpInference.Cpu/SimdKernels.cs:4377-4408).  ``activation``
+    names the gate's function: "silu" (the reference's) or "gelu_tanh"."""
+
+    def __init__(self, hidden: int, intermediate: int, activation: str = "silu"):
         self.hidden, self.inter = int(hidden), int(intermediate)
+        self.act = _activation_code(activation)
         self.w_gate_up: Optional[torch.Tensor] = None
         self.w_down: Optional[torch.Tensor] = None
 
@@ -56,7 +65,7 @@ class DenseSwiGLU(Part):
         with section("dense feed-forward", nbytes=width * 3 * self.inter * self.hidden + width * T * (2 * self.hidden + 3 * self.inter),
                      flops=6.0 * T * self.inter * self.hidden):
             gu = ops.linear(x, self.w_gate_up, ctx.act_dtype)
-            act = ops.silu_mul(gu)
+            act = ops.gated_act(gu, None, self.act)
             return ops.linear(act, self.w_down, ctx.act_dtype)
 
 
@@ -70,7 +79,8 @@ class MoESwiGLU(Part):
     and its output is multiplied by the score where the outputs are summed (the reference's other
     order, src/SharpInference.Cuda/CudaKernels.cs:112-157 llm_moe_weighted_reduce).  The shared
     expert sees the unscaled input (2060-2066); the outputs are summed (2096-2097).  ``gate`` is "sigmoid" or "softmax"
-    (2031-2034); ``renormalise`` divides the k scores by their sum (2156-2162)."""
+    (2031-2034); ``renormalise`` divides the k scores by their sum (2156-2162); ``activation`` names the
+    experts' gate function ("silu", the reference's, or "gelu_tanh")."""
 
     MERGE_MAX_TOKENS = 16   # one row block of the few-rows kernel for the shared group (measured: up to 64 tokens
                             # the merged launches and the library's product for the shared expert are as fast)
@@ -80,7 +90,7 @@ class MoESwiGLU(Part):
 
     def __init__(self, hidden: int, num_experts: int, top_k: int, expert_intermediate: int,
                  shared_intermediate: Optional[int] = None, gate: str = "sigmoid", renormalise: bool = False,
-                 score_on_input: bool = True):
+                 score_on_input: bool = True, activation: str = "silu"):
         if not 1 <= top_k <= num_experts:
             raise ValueError(f"top_k {top_k} must lie in 1..{num_experts}")
         if num_experts > ops.ROUTER_MAX_EXPERTS:
@@ -89,7 +99,8 @@ class MoESwiGLU(Part):
             raise ValueError(f"router gate {gate!r} is not known (sigmoid, softmax)")
         self.hidden, self.E, self.k = int(hidden), int(num_experts), int(top_k)
         self.inter = int(expert_intermediate)
-        self.shared = DenseSwiGLU(hidden, shared_intermediate) if shared_intermediate else None
+        self.act = _activation_code(activation)
+        self.shared = DenseSwiGLU(hidden, shared_intermediate, activation) if shared_intermediate else None
         self.gate = ops.GATE_SIGMOID if gate == "sigmoid" else ops.GATE_SOFTMAX
         self.renormalise = bool(renormalise)
         self.score_on_input = bool(score_on_input)
@@ -181,8 +192,8 @@ class MoESwiGLU(Part):
         along = self.merged and T <= self.MERGE_MAX_TOKENS
         shared = None if along or self.shared is None else self.shared.forward(x, ctx)
         with self._experts_section(ids, T, along):
-            act = ops.gemm_skinny_picked(x, self.w_gate_up, ids, wts if self.score_on_input else None, along, True, True,
-                                         ctx.act_dtype)
+            act = ops.gemm_skinny_picked(x, self.w_gate_up, ids, wts if self.score_on_input else None, along, True,
+                                         self.act, ctx.act_dtype)
             y = ops.gemm_skinny_picked(act, self.w_down, ids, None, along, False, False, ctx.act_dtype)
         return ops.ExpertSum(y, ops.counting(T * self.k, x.device), y[T * self.k:] if along else shared, T, self.k,
                              None if self.score_on_input else wts)
@@ -217,12 +228,12 @@ class MoESwiGLU(Part):
         if merge:
             # few rows: the shared expert rides along as one more group of the same two launches
             with self._experts_section(ids, T, True):
-                act = ops.grouped_swiglu(x, self.w_gate_up, rt, ctx.act_dtype, scaled=self.score_on_input)
+                act = ops.grouped_swiglu(x, self.w_gate_up, rt, ctx.act_dtype, scaled=self.score_on_input, act=self.act)
                 y = ops.grouped_linear(act, self.w_down, rt, False, ctx.act_dtype)
             # left as a sum: the next norm forms it while it reads the residual stream
             return ops.ExpertSum(y, rt.inv_pos, y[T * self.k:], T, self.k, after)
         shared = self.shared.forward(x, ctx) if self.shared is not None else None
         with self._experts_section(ids, T, False):
-            act = ops.grouped_swiglu(x, self.w_gate_up, rt, ctx.act_dtype, scaled=self.score_on_input)
+            act = ops.grouped_swiglu(x, self.w_gate_up, rt, ctx.act_dtype, scaled=self.score_on_input, act=self.act)
             y = ops.grouped_linear(act, self.w_down, rt, False, ctx.act_dtype)
         return ops.ExpertSum(y, rt.inv_pos, shared, T, self.k, after)   # formed by the next norm (or by whoever asks for a tensor)

@@ -185,6 +185,63 @@ def test_feed_forward_parts_alone(tmp_path, dtype):
             assert torch.equal(a.pending_tensor(), b.pending) if r is not None else a.pending is None
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gated_feed_forwards_take_another_activation(dtype):
+    """The gate's function is an argument of the feed-forward parts (a code the kernels take: in
+    the activation kernel and in the epilogues of the few-rows and many-rows products alike): GELU
+    in its tanh form, dense and routed, with few rows and with many, against the formula."""
+    from sharpinference_amd import ops
+    from sharpinference_amd.parts.feedforward import DenseSwiGLU, MoESwiGLU
+
+    HID, INTER, E = 128, 128, 4
+    g = torch.Generator().manual_seed(11)
+    rnd = lambda *shape: (torch.randn(*shape, generator=g) * 0.1).to(torch.bfloat16).float()  # noqa: E731
+    W = {"d.gate_proj.weight": rnd(INTER, HID), "d.up_proj.weight": rnd(INTER, HID), "d.down_proj.weight": rnd(HID, INTER),
+         "m.router.weight": rnd(E, HID) * 10, "m.experts.gate_proj": rnd(E, INTER, HID), "m.experts.up_proj": rnd(E, INTER, HID),
+         "m.experts.down_proj": rnd(E, HID, INTER), "m.shared_expert.gate_proj.weight": rnd(INTER, HID),
+         "m.shared_expert.up_proj.weight": rnd(INTER, HID), "m.shared_expert.down_proj.weight": rnd(HID, INTER)}
+    src = _Dict(W, dtype)
+    with pytest.raises(ValueError, match="not known"):
+        DenseSwiGLU(HID, INTER, activation="relu6")
+    dense = DenseSwiGLU(HID, INTER, activation="gelu_tanh")
+    dense.load("d.", src)
+    moe = MoESwiGLU(HID, E, 1, INTER, shared_intermediate=INTER, activation="gelu_tanh")
+    moe.load("m.", src)
+    store = P.store_bf16 if dtype == torch.bfloat16 else P._same
+    gelu = lambda v: torch.nn.functional.gelu(v, approximate="tanh")  # noqa: E731
+
+    def unit(x, wg, wu, wd, s=None):
+        gg, uu = store(x @ wg.T), store(x @ wu.T)
+        if s is not None:
+            gg, uu = gg * s[:, None], uu * s[:, None]
+        return store(store(gelu(gg) * uu) @ wd.T)
+
+    tol = 1e-4 if dtype == torch.float32 else 3e-2
+    x_all = torch.randn(200, HID, generator=g).to(torch.bfloat16).float()
+    for n_rows in (200, 70, 5):       # many rows, some, a few (the picked form in bfloat16)
+        x = x_all[:n_rows]
+        ctx, _ = _ctx([(0, n_rows)], dtype=dtype)
+        got = dense.forward(x.to(dtype).to(DEV), ctx).float().cpu()
+        want = unit(x, W["d.gate_proj.weight"], W["d.up_proj.weight"], W["d.down_proj.weight"])
+        assert float((got - want).abs().max()) <= tol * float(want.abs().max()), (n_rows, "dense")
+        trace = []
+        ctx.extras["router_trace"] = trace
+        got = moe.forward(x.to(dtype).to(DEV), ctx).tensor().float().cpu()
+        ids = trace[0][0].cpu().long()[:, 0]                 # the experts the router took (its own choice in both dtypes)
+        score = torch.sigmoid((x @ W["m.router.weight"].T).gather(1, ids[:, None]))[:, 0]
+        want = unit(x, W["m.shared_expert.gate_proj.weight"], W["m.shared_expert.up_proj.weight"], W["m.shared_expert.down_proj.weight"])
+        for e in range(E):
+            rows = (ids == e).nonzero().flatten()
+            if rows.numel():
+                want[rows] = store(want[rows] + unit(x[rows], W["m.experts.gate_proj"][e], W["m.experts.up_proj"][e],
+                                                     W["m.experts.down_proj"][e], score[rows]))
+        assert float((got - want).abs().max()) <= tol * float(want.abs().max()), (n_rows, "routed")
+    # the activation kernel alone, both codes
+    gu = torch.randn(9, 2 * 40, generator=g).to(DEV)
+    assert torch.allclose(ops.gated_act(gu, None, ops.ACT_GELU_TANH).cpu(), gelu(gu[:, :40].cpu()) * gu[:, 40:].cpu(), atol=1e-6)
+    assert torch.equal(ops.gated_act(gu, None, ops.ACT_SILU), ops.silu_mul(gu))
+
+
 def test_schedule_runs_a_layer_twice_and_shares_a_cache(tmp_path):
     """The order of execution is data: layer 0 runs twice (two cache slots), and the second run of
     layer 1 reads the keys and values that its first run stored."""
