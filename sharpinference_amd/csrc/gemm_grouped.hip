@@ -36,9 +36,6 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
-#ifndef SHARPI_GM
-#define SHARPI_GM 192
-#endif
 #ifndef SHARPI_GAHEAD
 #define SHARPI_GAHEAD 2
 #endif
@@ -48,7 +45,7 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 #ifndef SHARPI_GK
 #define SHARPI_GK 64
 #endif
-constexpr int GM = SHARPI_GM;  // rows per tile
+constexpr int GM = kPlanTileRows;  // rows per tile
 static_assert(GM == kPlanTileRows, "the routing kernel's plan is made for tiles of this height");
 constexpr int GMT = GM / 16;  // 16-row groups per tile
 #ifndef SHARPI_GW
@@ -58,8 +55,11 @@ constexpr int GMT = GM / 16;  // 16-row groups per tile
 #define SHARPI_GNT 2
 #endif
 constexpr int GW = SHARPI_GW;   // waves per block
-constexpr int NT = SHARPI_GNT;  // 16-row weight tiles per wave
-constexpr int GN = 16 * NT * GW;   // columns per tile
+#ifndef SHARPI_GNARROW_BELOW
+#define SHARPI_GNARROW_BELOW 512   // blocks (two per compute unit) below which the plain form halves its column tiles
+#endif
+constexpr int kMaxNT = SHARPI_GNT;  // 16-row weight tiles per wave: this many, or one (narrow form)
+constexpr int columns_of(int nt) { return 16 * nt * GW; }   // weight rows (output columns) of a block
 constexpr int GK = SHARPI_GK;  // K per LDS stage
 constexpr int GPAD = GK;      // LDS row: no pad, the 16-byte chunks of a row are swizzled instead (xs_col)
 constexpr int GROWS = GW * 64 / (GK / 8);   // rows staged per pass: GK / 8 threads per row
@@ -78,8 +78,8 @@ constexpr int GQ = SHARPI_GQ;       // 16-row groups whose LDS reads go out toge
 static_assert(GK == 64, "the swizzle assumes rows of eight 16-byte chunks");
 __device__ __forceinline__ int xs_col(int row, int col) { return col ^ (((row >> 1) & 7) << 3); }
 
-// The work of one tile of MT * 16 rows (the block's rows, rounded up) against GN weight rows.
-template <typename TO, int MT, bool PACKED, bool ACT>
+// The work of one tile of MT * 16 rows (the block's rows, rounded up) against 16 * NT * GW weight rows.
+template <typename TO, int MT, int NT, bool PACKED, bool ACT>
 __device__ __forceinline__ void grouped_tile(const bf16_t* __restrict__ x, const bf16_t* __restrict__ We,
                                              TO* __restrict__ out, int N, int K, const int* __restrict__ a_rows,
                                              const float* __restrict__ act_scale, int act, int row0, int row_end,
@@ -258,12 +258,13 @@ __device__ __forceinline__ void grouped_tile(const bf16_t* __restrict__ x, const
   }
 }
 
-template <typename TO, bool PACKED, bool ACT>
-__global__ __launch_bounds__(GW* kWave, 2) void grouped_gemm_kernel(
+template <typename TO, int NT, bool PACKED, bool ACT>
+__global__ __launch_bounds__(GW* kWave, (NT == 1 ? 4 : 2)) void grouped_gemm_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ W, TO* __restrict__ out, int N, int K,
     const int* __restrict__ a_rows, const float* __restrict__ act_scale, int act,
     const int* __restrict__ group_offsets, const int* __restrict__ plan, int n_groups, int nb) {
   __shared__ __attribute__((aligned(16))) bf16_t xs[2][GM][GPAD];
+  constexpr int GN = columns_of(NT);
   constexpr int kCols = ACT ? GN / 2 : GN;   // output columns of a block
   const int n_out = ACT ? N / 2 : N;
   // Workgroups go to the 8 XCDs round-robin by their linear id: this block is slot `slot` of XCD
@@ -300,7 +301,7 @@ __global__ __launch_bounds__(GW* kWave, 2) void grouped_gemm_kernel(
   const int n_base = nblock * kCols + (threadIdx.x >> 6) * (ACT ? 16 : 16 * NT);
   const bf16_t* We = W + (size_t)e * N * K;
   static_assert(GM == 192, "tile heights are compiled in steps of 32 rows up to 192");
-#define GT(MTV) grouped_tile<TO, MTV, PACKED, ACT>(x, We, out, N, K, a_rows, act_scale, act, row0, row_end, n_base, xs)
+#define GT(MTV) grouped_tile<TO, MTV, NT, PACKED, ACT>(x, We, out, N, K, a_rows, act_scale, act, row0, row_end, n_base, xs)
   if (n_rows <= 32) GT(2);
   else if (n_rows <= 64) GT(4);
   else if (n_rows <= 96) GT(6);
@@ -335,12 +336,25 @@ SHARPI_EXPORT int sharpi_gemm_grouped(const void* x, int x_rows, const void* W, 
                                       int n_groups, int packed, hipStream_t stream) {
   if (n_rows <= 0) return SHARPI_OK;
   if (!grouped_args_ok(x_rows, n_rows, N, K, n_groups, packed, group_offsets, plan)) return SHARPI_ERR_ARG;
-  const int nb = ceil_div(N, GN);
+  // Narrow form (one 16-row weight tile per wave: blocks of half the columns, two of them to a
+  // compute unit) where the wide one would make too few blocks to fill the compute units, as a
+  // 5,120-column projection of 16 experts with few rows each does (320 blocks of 256 columns for
+  // 256 units that hold one such block each: 236 against 269 us at 256 tokens, 262 against 288
+  // at 1,024; with more rows the wide form's larger share of weights per staged x row wins).
+  const long long wide_blocks = (long long)(n_groups + ceil_div(n_rows, GM)) * ceil_div(N, columns_of(kMaxNT));
+  const bool narrow = kMaxNT > 1 && wide_blocks < SHARPI_GNARROW_BELOW;
+  const int nb = ceil_div(N, columns_of(narrow ? 1 : kMaxNT));
   dim3 grid, block(GW * kWave);
   if (!grouped_grid(n_rows, n_groups, nb, &grid)) return SHARPI_ERR_ARG;
-#define GG_LAUNCH(TOV, PK)                                                                                          \
-  grouped_gemm_kernel<TOV, PK, false><<<grid, block, 0, stream>>>((const bf16_t*)x, (const bf16_t*)W, (TOV*)out, N, \
-                                                                 K, a_rows, nullptr, 0, group_offsets, plan, n_groups, nb)
+#define GG_LAUNCH1(TOV, NTV, PK)                                                                                     \
+  grouped_gemm_kernel<TOV, NTV, PK, false><<<grid, block, 0, stream>>>((const bf16_t*)x, (const bf16_t*)W, (TOV*)out, \
+                                                                      N, K, a_rows, nullptr, 0, group_offsets, plan,  \
+                                                                      n_groups, nb)
+#define GG_LAUNCH(TOV, PK)                   \
+  do {                                       \
+    if (narrow) GG_LAUNCH1(TOV, 1, PK);      \
+    else GG_LAUNCH1(TOV, kMaxNT, PK);        \
+  } while (0)
   if (out_dtype == DT_BF16) {
     if (packed) GG_LAUNCH(bf16_t, true); else GG_LAUNCH(bf16_t, false);
   } else if (out_dtype == DT_F32) {
@@ -348,6 +362,7 @@ SHARPI_EXPORT int sharpi_gemm_grouped(const void* x, int x_rows, const void* W, 
   } else {
     return SHARPI_ERR_ARG;
   }
+#undef GG_LAUNCH1
 #undef GG_LAUNCH
   SHARPI_CHECK_LAUNCH();
   return SHARPI_OK;
@@ -364,14 +379,15 @@ SHARPI_EXPORT int sharpi_gemm_grouped_swiglu(const void* x, int x_rows, const vo
   if (n_rows <= 0) return SHARPI_OK;
   if (!act_known(act)) return SHARPI_ERR_ARG;
   if ((N & 31) || !grouped_args_ok(x_rows, n_rows, N, K, n_groups, packed, group_offsets, plan)) return SHARPI_ERR_ARG;
+  constexpr int GN = columns_of(2);   // the gated form pairs a gate tile with an up tile
   const int nb = ceil_div(N / 2, GN / 2);
   dim3 grid, block(GW * kWave);
   if (!grouped_grid(n_rows, n_groups, nb, &grid)) return SHARPI_ERR_ARG;
   if (packed)
-    grouped_gemm_kernel<bf16_t, true, true><<<grid, block, 0, stream>>>(
+    grouped_gemm_kernel<bf16_t, 2, true, true><<<grid, block, 0, stream>>>(
         (const bf16_t*)x, (const bf16_t*)W, (bf16_t*)out, N, K, a_rows, act_scale, act, group_offsets, plan, n_groups, nb);
   else
-    grouped_gemm_kernel<bf16_t, false, true><<<grid, block, 0, stream>>>(
+    grouped_gemm_kernel<bf16_t, 2, false, true><<<grid, block, 0, stream>>>(
         (const bf16_t*)x, (const bf16_t*)W, (bf16_t*)out, N, K, a_rows, act_scale, act, group_offsets, plan, n_groups, nb);
   SHARPI_CHECK_LAUNCH();
   return SHARPI_OK;

@@ -481,10 +481,12 @@ def test_gemm_skinny_swiglu_equals_product_then_activation(M, E, I, K):
             assert float((got.float().cpu() - ref).abs().max()) <= 2e-2 * float(ref.abs().max())
 
 
-# the last two are deep enough in K for the kernel's steady loop (and its tail of 4 and of 1 stages)
+# (260, ...) are deep enough in K for the kernel's steady loop (and its tail of 4 and of 1 stages); the last two
+# make 512 blocks and more, from which on a block takes 256 columns instead of 128 (the others run the narrow form)
 @pytest.mark.parametrize("T,E,k,N,K", [(300, 4, 1, 264, 256), (700, 16, 2, 512, 128), (65, 3, 1, 20, 384),
                                        (500, 5, 1, 200, 640), (260, 2, 2, 136, 1216), (500, 5, 1, 208, 640),
-                                       (260, 2, 2, 144, 1280), (70, 3, 1, 16, 128), (1700, 2, 1, 264, 256)])
+                                       (260, 2, 2, 144, 1280), (70, 3, 1, 16, 128), (1700, 2, 1, 264, 256),
+                                       (600, 40, 1, 3344, 256), (2500, 16, 2, 3088, 128)])
 def test_gemm_grouped(T, E, k, N, K):
     ops = _ops()
     x = _rand(T, K, dtype=torch.bfloat16, seed=1)
