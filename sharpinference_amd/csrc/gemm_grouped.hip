@@ -78,8 +78,17 @@ constexpr int GQ = SHARPI_GQ;       // 16-row groups whose LDS reads go out toge
 static_assert(GK == 64, "the swizzle assumes rows of eight 16-byte chunks");
 __device__ __forceinline__ int xs_col(int row, int col) { return col ^ (((row >> 1) & 7) << 3); }
 
+// A weight fragment.  STREAM: with the streaming hint (nontemporal), for a group whose weights no
+// other row tile reads: a pure read in this kernel's pattern reaches 6.9 TB/s with the hint and
+// 6.2 without.  A group cut into sibling tiles reads them without the hint: what the first
+// sibling fetches the others are to find in the L2.
+template <bool STREAM> __device__ __forceinline__ bf16x8 load_weights(const bf16_t* p) {
+  if constexpr (STREAM) return __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(p));
+  else return *reinterpret_cast<const bf16x8*>(p);
+}
+
 // The work of one tile of MT * 16 rows (the block's rows, rounded up) against 16 * NT * GW weight rows.
-template <typename TO, int MT, int NT, bool PACKED, bool ACT>
+template <typename TO, int MT, int NT, bool PACKED, bool ACT, bool STREAM>
 __device__ __forceinline__ void grouped_tile(const bf16_t* __restrict__ x, const bf16_t* __restrict__ We,
                                              TO* __restrict__ out, int N, int K, const int* __restrict__ a_rows,
                                              const float* __restrict__ act_scale, int act, int row0, int row_end,
@@ -152,7 +161,7 @@ __device__ __forceinline__ void grouped_tile(const bf16_t* __restrict__ x, const
 #pragma unroll
         for (int j = 0; j < GK / 32; ++j)
 #pragma unroll
-          for (int t = 0; t < NT; ++t) wf[a][j][t] = *reinterpret_cast<const bf16x8*>(We + woff[t] + a * kStageStep + j * kSubStep);
+          for (int t = 0; t < NT; ++t) wf[a][j][t] = load_weights<STREAM>(We + woff[t] + a * kStageStep + j * kSubStep);
       }
   };
   if (chunks >= kAhead) fill_ring(std::true_type{}); else fill_ring(std::false_type{});
@@ -196,7 +205,7 @@ __device__ __forceinline__ void grouped_tile(const bf16_t* __restrict__ x, const
       for (int j = 0; j < GK / 32; ++j)
 #pragma unroll
         for (int t = 0; t < NT; ++t)
-          wf[slot][j][t] = *reinterpret_cast<const bf16x8*>(We + woff[t] + (c + kAhead) * kStageStep + j * kSubStep);
+          wf[slot][j][t] = load_weights<STREAM>(We + woff[t] + (c + kAhead) * kStageStep + j * kSubStep);
     }
     if (steady || c + 1 < chunks) {   // the next stage's x rows, fetched a stage ago
 #pragma unroll
@@ -301,7 +310,13 @@ __global__ __launch_bounds__(GW* kWave, (NT == 1 ? 4 : 2)) void grouped_gemm_ker
   const int n_base = nblock * kCols + (threadIdx.x >> 6) * (ACT ? 16 : 16 * NT);
   const bf16_t* We = W + (size_t)e * N * K;
   static_assert(GM == 192, "tile heights are compiled in steps of 32 rows up to 192");
-#define GT(MTV) grouped_tile<TO, MTV, NT, PACKED, ACT>(x, We, out, N, K, a_rows, act_scale, act, row0, row_end, n_base, xs)
+#define GT1(MTV, ST) grouped_tile<TO, MTV, NT, PACKED, ACT, ST>(x, We, out, N, K, a_rows, act_scale, act, row0, row_end, n_base, xs)
+  // (the hint only for weights stored tile by tile, the order the served model keeps them in)
+#define GT(MTV)                                \
+  do {                                         \
+    if (PACKED && n_sib == 1) GT1(MTV, PACKED); \
+    else GT1(MTV, false);                      \
+  } while (0)
   if (n_rows <= 32) GT(2);
   else if (n_rows <= 64) GT(4);
   else if (n_rows <= 96) GT(6);
@@ -309,6 +324,7 @@ __global__ __launch_bounds__(GW* kWave, (NT == 1 ? 4 : 2)) void grouped_gemm_ker
   else if (n_rows <= 160) GT(10);
   else GT(12);
 #undef GT
+#undef GT1
 }
 
 static bool grouped_args_ok(int x_rows, int n_rows, int N, int K, int n_groups, int packed, const int* group_offsets,
