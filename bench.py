@@ -140,7 +140,8 @@ def run_prefill(eng, rid, prompt):
 def decode_run(eng, batch: int, steps: int, warmup: int, rng: random.Random, count_experts: bool = False,
                prompt_len: int = PROMPT_LEN):
     """Prefill `batch` prompts, then time `steps` decode steps.  Returns seconds, the mean
-    number of distinct experts a step used per layer (if asked) and the length the requests reached."""
+    number of distinct experts a step used per layer (if asked), the length the requests reached and
+    the host's milliseconds per step."""
     import torch
     from sharpinference_amd import ops
     from sharpinference_amd.engine import StepEntry
@@ -158,19 +159,27 @@ def decode_run(eng, batch: int, steps: int, warmup: int, rng: random.Random, cou
         last += ops.argmax_rows(lg).cpu().tolist()
         log(f"  prefilled {min(i + per_step, batch)}/{batch}")
 
+    host = [0.0]
+
     def one_step(tokens, trace=None):
-        # greedy decoding as the engine serves it: the choice is made on the device behind the head
-        return eng.step([StepEntry(r, (t,), (0,)) for r, t in zip(ids, tokens)], router_trace=trace,
-                        select="argmax").cpu().tolist()
+        # greedy decoding as the engine serves it: the choice is made on the device behind the head.
+        # The host's share of a step is what passes inside `step` (bookkeeping, the index arrays, the
+        # launch); the wait for the chosen tokens after it is the GPU's.
+        h0 = time.perf_counter()
+        chosen = eng.step([StepEntry(r, (t,), (0,)) for r, t in zip(ids, tokens)], router_trace=trace, select="argmax")
+        host[0] += time.perf_counter() - h0
+        return chosen.cpu().tolist()
 
     for _ in range(warmup):
         last = one_step(last)
     torch.cuda.synchronize()
+    host[0] = 0.0
     t0 = time.perf_counter()
     for _ in range(steps):
         last = one_step(last)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
+    host_ms = host[0] / steps * 1e3
     distinct = None
     if count_experts:
         trace: list = []
@@ -179,7 +188,7 @@ def decode_run(eng, batch: int, steps: int, warmup: int, rng: random.Random, cou
     ctx = eng.cache.length(ids[0])
     for r in ids:
         eng.free_request(r)
-    return dt, distinct, ctx
+    return dt, distinct, ctx, host_ms
 
 
 def profile_report(eng, batch: int, prompt_len: int, rng: random.Random) -> None:
@@ -236,7 +245,7 @@ def run_maverick8(args) -> int:
     hist = torch.bincount(trace[0][0].flatten().long().cpu(), minlength=cfg.num_local_experts).tolist()
     log(f"prefill {P} tokens: {pre_s * 1e3:.1f} ms; tokens per expert in the first routed layer: min {min(hist)}, "
         f"median {sorted(hist)[len(hist) // 2]}, max {max(hist)}, unused {hist.count(0)} of {len(hist)}")
-    dt, distinct, ctx = decode_run(eng, batch, steps, warm, rng, count_experts=True, prompt_len=P)
+    dt, distinct, ctx, _ = decode_run(eng, batch, steps, warm, rng, count_experts=True, prompt_len=P)
     ms_step = dt / steps * 1e3
     step_bytes = decode_step_bytes(cfg, layers, batch, ctx, distinct)
     achieved = step_bytes / (ms_step * 1e-3) / 1e9
@@ -388,23 +397,25 @@ def main() -> int:
                "frac": flops / pre_s / (PEAK_DENSE_TFLOPS["bf16"] * 1e12),
                "hbm_frac": prefill_bytes(cfg, args.layers) / pre_s / 1e9 / PEAK_HBM_GBS}
 
-    dt, distinct, ctx = decode_run(eng, args.batch, args.steps, args.warmup, rng, count_experts=True, prompt_len=P)
+    dt, distinct, ctx, host_ms = decode_run(eng, args.batch, args.steps, args.warmup, rng, count_experts=True, prompt_len=P)
     ms_step = dt / args.steps * 1e3
     value = args.batch * args.steps / dt
     step_bytes = decode_step_bytes(cfg, args.layers, args.batch, ctx, distinct)
     achieved = step_bytes / (ms_step * 1e-3) / 1e9
-    log(f"decode b{args.batch}: {ms_step:.2f} ms/step, {value:.1f} tok/s, {achieved:.0f} GB/s "
+    log(f"decode b{args.batch}: {ms_step:.2f} ms/step ({host_ms:.2f} ms of it on the host), {value:.1f} tok/s, {achieved:.0f} GB/s "
         f"({distinct:.2f} experts per layer)")
 
-    points, points_roofline = {}, {}
+    points, points_roofline, points_host = {}, {}, {}
     if not args.no_points:
         for pb in (1, 64):
             k = max(8, args.steps // 2)
-            pdt, pdist, pctx = decode_run(eng, pb, k, max(2, args.warmup // 2), rng, count_experts=True, prompt_len=P)
+            pdt, pdist, pctx, phost = decode_run(eng, pb, k, max(2, args.warmup // 2), rng, count_experts=True, prompt_len=P)
             points[f"decode_b{pb}"] = pb * k / pdt
             gbs = decode_step_bytes(cfg, args.layers, pb, pctx, pdist) / (pdt / k) / 1e9
             points_roofline[f"decode_b{pb}"] = gbs / PEAK_HBM_GBS
-            log(f"decode b{pb}: {pdt / k * 1e3:.2f} ms/step, {points[f'decode_b{pb}']:.1f} tok/s, {gbs:.0f} GB/s "
+            points_host[f"decode_b{pb}"] = phost
+            log(f"decode b{pb}: {pdt / k * 1e3:.2f} ms/step ({phost:.2f} ms on the host), "
+                f"{points[f'decode_b{pb}']:.1f} tok/s, {gbs:.0f} GB/s "
                 f"({gbs / PEAK_HBM_GBS:.3f} of the roofline; {pdist:.2f} experts per layer)")
     if args.profile:
         profile_report(eng, args.batch, P, rng)
@@ -428,6 +439,8 @@ def main() -> int:
                      "frac": achieved / PEAK_HBM_GBS},
         "points": points,
         "points_roofline": points_roofline,
+        "host_ms_per_step": host_ms,
+        "points_host_ms_per_step": points_host,
     }
     if measured is not None:
         out["measured_peaks"] = {"hbm_gbs": measured["hbm_gbs"], "bf16_tflops": measured["bf16_tflops"],
