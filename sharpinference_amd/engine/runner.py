@@ -26,6 +26,7 @@ from ..parts.base import GroupView, LayerCache, StepContext
 MAX_GRAPH_BATCH = 64   # decode steps of up to this many requests are replayed from a HIP graph (at 64 the host's part of an eager step is still a tenth of the step)
 GRAPH_AT_ONCE = 16     # up to this many requests a graph is captured when its shape is first met; wider ones once the
 GRAPH_AFTER_ASKS = 4   # shape has been met this often (a graph per width costs capture time and memory of its own)
+MAX_GRAPHS = 48        # graphs kept at a time; beyond, the one replayed longest ago is dropped (and captured again if its shape returns)
 GRAPH_CONTEXT_MIN = 4096   # a graph is captured for a bound on the contexts of its requests: this, or 4, 16, 64 ... times it
 TILE = PREFILL_TILE_TOKENS   # tokens per attention tile of multi-token entries
 
@@ -225,6 +226,12 @@ class ModelRunner:
                 self._graphs[key] = False
                 return None
             self._graphs[key] = graph
+            live = [k for k, g in self._graphs.items() if g is not False]
+            if len(live) > MAX_GRAPHS:          # (the dict keeps the order of last use: see below)
+                del self._graphs[live[0]]
+                self._graph_asks.pop(live[0], None)
+        else:
+            self._graphs[key] = self._graphs.pop(key)     # moved to the end: the most recently used
         self.graph_replays += 1
         return graph.replay(pieces, router_trace)
 

@@ -221,6 +221,19 @@ def test_decode_graph_replays_equal_eager_steps(model_dir, dtype):
             assert eng.runner.graph_replays == 12
     for r in toks:
         assert torch.equal(out[True][r], out[False][r]), r
+    # no more graphs are kept than the limit says: the one used longest ago goes, and is captured
+    # again when its shape comes back (batch 1 here, after batches 2 and 3)
+    from sharpinference_amd.engine import runner as R
+    limit = R.MAX_GRAPHS
+    R.MAX_GRAPHS = 2
+    try:
+        eng = H.make_engine(d, dtype, kv_tokens=256, max_num_seqs=4, decode_graphs=True)
+        capped = H.replay(eng, steps)
+        assert len(eng.runner._graphs) == 2 and eng.runner.graph_replays == 12
+    finally:
+        R.MAX_GRAPHS = limit
+    for r in toks:
+        assert torch.equal(capped[r], out[False][r]), r
 
 
 def test_decode_graphs_follow_the_context(tmp_path):
