@@ -90,17 +90,20 @@ __global__ __launch_bounds__(NW* kWave) void skinny_gemm_kernel(
   if (picked) {
     // The grid has a group for every expert that CAN have rows, not for every expert there is
     // (a block that finds no rows still costs a launch slot, and with one token fifteen of
-    // seventeen would): group y < groups - shared is the y-th DISTINCT expert among the picks, in
-    // the order of its first pick; the last group is the always-on expert, if there is one.
+    // seventeen would): the first group is the always-on expert, if there is one; group y after it
+    // is the y-th DISTINCT expert among the picks, in the order of its first pick.  The groups
+    // that find no expert (fewer distinct experts than pairs) are then the grid's last blocks,
+    // where they hold nobody up.
     if (w == 0) {
       const int n_groups = gridDim.y;
-      const bool always_on = pk.shared && (int)blockIdx.y == n_groups - 1;
+      const bool always_on = pk.shared && blockIdx.y == 0;
+      const int ordinal_wanted = (int)blockIdx.y - pk.shared;
       const int mine_e = lane < pk.n_pairs ? pk.ids[lane] : -1;
       int expert = -1;                            // the block's expert; -1: there are fewer distinct experts than groups
       if (always_on) {
         expert = pk.n_experts;
       } else if (n_groups - pk.shared == pk.n_experts) {
-        expert = blockIdx.y;                      // as many groups as experts: group y is expert y
+        expert = ordinal_wanted;                  // as many groups as experts: group y is expert y
       } else {
         bool first = lane < pk.n_pairs;           // no earlier pair picked this lane's expert
         for (int j = 0; j < pk.n_pairs; ++j) {
@@ -109,7 +112,7 @@ __global__ __launch_bounds__(NW* kWave) void skinny_gemm_kernel(
         }
         const unsigned long long firsts = __builtin_amdgcn_ballot_w64(first);
         const int ordinal = __popcll(firsts & ((1ull << lane) - 1ull));
-        const unsigned long long chosen = __builtin_amdgcn_ballot_w64(first && ordinal == (int)blockIdx.y);
+        const unsigned long long chosen = __builtin_amdgcn_ballot_w64(first && ordinal == ordinal_wanted);
         if (chosen) expert = __shfl(mine_e, __ffsll((long long)chosen) - 1, kWave);
       }
       const bool routed = !always_on;
