@@ -69,13 +69,19 @@ class Engine:
                  max_model_len: Optional[int] = None, max_num_seqs: int = 8, max_tokens_per_step: int = 2048,
                  kv_tokens: Optional[int] = None, page_size: int = 16, weight_std: float = 0.02,
                  weight_std_by_suffix: Optional[Dict[str, float]] = None, verbose: bool = False,
-                 decode_graphs: bool = True, past_position_limit: bool = False, row_major_copies: bool = True):
+                 decode_graphs: bool = True, past_position_limit: bool = False, row_major_copies: bool = True,
+                 decode_run_ahead: int = 4):
         """max_model_len: the longest sequence a request may reach (default: the configuration's
         max_position_embeddings, 4096 if it names none); beyond max_position_embeddings only with
         past_position_limit (replaying given tokens needs no trained positions).
         row_major_copies=False keeps the attention, dense feed-forward and head matrices only in
         the packed order of the decode kernels (about a tenth less weight memory; prompt-sized
-        products then run in this library's own kernels instead of the library product, slower)."""
+        products then run in this library's own kernels instead of the library product, slower).
+        decode_run_ahead: while every running request decodes greedily and none waits, generation
+        launches this many steps on end, each on what the step before chose (on the device), and
+        reads the tokens back together: the host's part of a step then passes while the GPU works
+        (1: every step waits for its tokens)."""
+        self.decode_run_ahead = max(1, int(decode_run_ahead))
         self.dtype = parse_dtype(dtype)
         self.device = torch.device(device)
         if self.device.type != "cuda":
@@ -153,8 +159,13 @@ class Engine:
         self.cache.free_request(req_id)
 
     def step(self, entries: Sequence[StepEntry], router_trace: Optional[list] = None,
-             select: Optional[str] = None) -> Optional[torch.Tensor]:
-        return self.runner.step(entries, router_trace, select)
+             select: Optional[str] = None, device_tokens: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+        return self.runner.step(entries, router_trace, select, device_tokens)
+
+    def decode_steps(self, entries: Sequence[StepEntry], steps: int) -> torch.Tensor:
+        """Greedy decode steps run ahead of the host (see ModelRunner.decode_steps): int32
+        [steps run, entries] on the device."""
+        return self.runner.decode_steps(entries, steps)
 
     def profiled_step(self, entries: Sequence[StepEntry], profiler, select: Optional[str] = None,
                       filler_ms: float = 0.0) -> Optional[torch.Tensor]:
@@ -241,6 +252,32 @@ class Engine:
                                for s in batch]
                     sampling = [s for s in batch if s.samples]
                     tokens: List[Optional[int]] = [None] * len(batch)
+                    ahead = self._steps_ahead(sched, batch, should_cancel)
+                    if ahead > 1:
+                        # Every request decodes greedily and nobody waits: several steps on end, each
+                        # launched on what the one before chose; the scheduler is then told of them
+                        # step by step, exactly as if each had been waited for.
+                        rows = self.runner.decode_steps(entries, ahead).cpu().tolist()
+                        col = {s.request.req_id: j for j, s in enumerate(batch)}
+                        dt = (time.perf_counter() - t0) / len(rows)
+                        for i, row in enumerate(rows):
+                            if i > 0:
+                                batch = sched.schedule()       # the requests that are still running, in their order
+                                if not batch:
+                                    break
+                            stats.decode_tokens += len(batch)
+                            stats.decode_seconds += dt
+                            stats.steps += 1
+                            had = [len(s.request.output) for s in batch]
+                            sched.update(batch, [row[col[s.request.req_id]] for s in batch])
+                            for s, n0 in zip(batch, had):
+                                if len(s.request.output) > n0:
+                                    yield GenerateChunk("token", s.request.req_id[1], token_id=s.request.output[-1])
+                            for r in sched.finished[reported:]:
+                                yield GenerateChunk("stop", r.req_id[1], finish_reason=r.finish_reason,
+                                                    truncated_by_max_tokens=r.finish_reason == "length")
+                            reported = len(sched.finished)
+                        continue
                     if sampling and all(s.request.params.greedy for s in sampling):
                         # every row greedy: the choice is made on the device behind the head, and only
                         # the token ids come back (reference: ContinuousBatchingEngine.cs:332-347)
@@ -285,6 +322,22 @@ class Engine:
             for r in list(sched.running):                  # an error or an early close: give everything back
                 if self.cache.has_request(r.req_id):
                     self.cache.free_request(r.req_id)
+
+    def _steps_ahead(self, sched: Scheduler, batch, should_cancel) -> int:
+        """How many decode steps may be launched on end for this batch: more than one only while
+        every request of it decodes greedily, nobody waits to be admitted or can be cancelled in
+        between, and no request would pass its own limit (a request that meets a stop token on
+        the way is ended there; the steps run past it are dropped with its pages)."""
+        if self.decode_run_ahead <= 1 or should_cancel is not None or sched.waiting or not batch:
+            return 1
+        steps = self.decode_run_ahead
+        for s in batch:
+            r = s.request
+            if r.in_prefill or not s.samples or len(s.tokens) != 1 or not r.params.greedy:
+                return 1
+            steps = min(steps, r.params.max_new_tokens - len(r.output),
+                        self.max_model_len - (len(r.prompt) + len(r.output)))
+        return max(1, steps)
 
     def generate(self, prompts: Sequence[Sequence[int]], params: Union[SamplingParams, Sequence[SamplingParams], None] = None,
                  *, max_new_tokens: Optional[int] = None, temperature: Optional[float] = None,

@@ -187,7 +187,7 @@ class ModelRunner:
 
     # ------------------------------------------------------------------
     def _decode_graph_step(self, entries: Sequence[StepEntry], router_trace: Optional[list] = None,
-                           select: Optional[str] = None) -> Optional[torch.Tensor]:
+                           select: Optional[str] = None, device_tokens: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """Replay the captured graph of this batch size if the step qualifies: every entry one
         token whose logits are wanted, all contexts within the captured bound.  None otherwise."""
         n = len(entries)
@@ -233,14 +233,17 @@ class ModelRunner:
         else:
             self._graphs[key] = self._graphs.pop(key)     # moved to the end: the most recently used
         self.graph_replays += 1
-        return graph.replay(pieces, router_trace)
+        return graph.replay(pieces, router_trace, device_tokens)
 
     def step(self, entries: Sequence[StepEntry], router_trace: Optional[list] = None,
-             select: Optional[str] = None) -> Optional[torch.Tensor]:
+             select: Optional[str] = None, device_tokens: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """Run one batch.  Returns float32 logits [wanted, vocab] in the order of the entries and
         of their ``want`` lists, or None when nothing is wanted; with ``select="argmax"`` the index
         of each wanted row's largest logit instead (int32 [wanted]), so that only token ids leave
-        the device.  A list given as ``router_trace``
+        the device.  ``device_tokens`` (int32 [entries], on the device; every entry one token):
+        the token ids are taken from there instead of from the entries, whose own are then only
+        placeholders: a step can be launched on what the step before chose before the host has
+        seen it.  A list given as ``router_trace``
         receives, per routed layer run, the (expert ids, weights, router input) of the step's tokens,
         as the reference can print its router picks (src/SharpInference.Engine/ForwardPass.cs:2042-2056)."""
         if not entries:
@@ -252,9 +255,15 @@ class ModelRunner:
                 if not self.cache.append(e.req_id, len(e.tokens)):
                     raise CacheExhausted(f"no pages left for request {e.req_id!r} ({len(e.tokens)} more tokens)")
                 appended.append(e.req_id)
-            logits = self._decode_graph_step(entries, router_trace, select)
+            if device_tokens is not None:
+                if any(len(e.tokens) != 1 for e in entries) or device_tokens.shape != (len(entries),) \
+                        or device_tokens.dtype != torch.int32 or not device_tokens.is_cuda:
+                    raise ValueError("device_tokens: one int32 token per single-token entry, on the engine's device")
+            logits = self._decode_graph_step(entries, router_trace, select, device_tokens)
             if logits is None:
                 ctx, rows = self.build_context(entries)
+                if device_tokens is not None:
+                    ctx.token_ids.copy_(device_tokens)
                 if router_trace is not None:
                     ctx.extras["router_trace"] = router_trace
                 logits = self.model.forward(ctx, self.layer_caches(ctx), rows, select) if select else \
@@ -267,6 +276,31 @@ class ModelRunner:
             self.cache.commit(e.req_id)
         self.steps_run += 1
         return logits
+
+
+    def decode_steps(self, entries: Sequence[StepEntry], steps: int) -> torch.Tensor:
+        """`steps` greedy decode steps of the same requests, run ahead of the host: the first takes
+        the entries' own tokens, every later one what the step before chose, on the device, so
+        that the host prepares and launches a step while the one before it still runs and reads
+        nothing back in between.  Returns the chosen tokens, int32 [steps, entries], on the
+        device.  Fewer steps are run if the pages do not reach (at least one, or CacheExhausted
+        as in ``step``)."""
+        if not entries or steps <= 0:
+            raise ValueError("decode_steps needs entries and at least one step")
+        if any(len(e.tokens) != 1 for e in entries):
+            raise ValueError("decode_steps: every entry brings one token")
+        chosen: List[torch.Tensor] = []
+        ahead = [StepEntry(e.req_id, (0,), (0,)) for e in entries]
+        for i in range(steps):
+            try:
+                out = self.step(entries if i == 0 else ahead, select="argmax",
+                                device_tokens=None if i == 0 else chosen[-1])
+            except CacheExhausted:
+                if i == 0:
+                    raise
+                break
+            chosen.append(out)
+        return torch.stack(chosen)
 
 
 class _DecodeGraph:
@@ -334,8 +368,11 @@ class _DecodeGraph:
         self.dev.copy_(self.host, non_blocking=True)
         self.copied.record()
 
-    def replay(self, pieces, router_trace: Optional[list] = None) -> torch.Tensor:
+    def replay(self, pieces, router_trace: Optional[list] = None,
+               device_tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
         self._upload(pieces)
+        if device_tokens is not None:                    # the token ids lie first in the buffer
+            self.dev[:self.sizes[0]].copy_(device_tokens)
         self.graph.replay()
         if router_trace is not None:
             router_trace.extend(tuple(t.clone() for t in item) for item in self.trace)

@@ -123,6 +123,53 @@ def test_stop_tokens_and_tiny_pool(tmp_path):
     assert all(g.pool.total_allocs > g.pool.num_pages for g in eng.cache.groups)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("graphs", [True, False])
+def test_steps_launched_on_end_give_the_same_generation(tmp_path, dtype, graphs):
+    """While every request decodes greedily the engine launches several steps on end, each on
+    what the step before chose (on the device), and reads the tokens back together.  The tokens,
+    the reasons to stop and the pages are those of an engine that waits for every step, whatever
+    the number of steps on end, also when a request meets its stop token in the middle of a run
+    or the requests end at different lengths."""
+    from sharpinference_amd import SamplingParams
+    from sharpinference_amd.engine import StepEntry
+
+    d = make_model_dir(tmp_path, "D", std=0.06)
+    prompts = [H.random_tokens(n, 500, 70 + n) for n in (9, 30, 12, 25, 18)]
+    one = H.make_engine(d, dtype, kv_tokens=512, max_num_seqs=5, decode_graphs=graphs, decode_run_ahead=1)
+    free = one.generate(prompts, max_new_tokens=23)
+    stop = free[1].token_ids[9]
+    params = [SamplingParams(temperature=0.0, max_new_tokens=m, stop_token_ids=(stop,)) for m in (23, 23, 14, 20, 6)]
+    want = one.generate(prompts, params)
+    assert any(r.finish_reason == "stop" for r in want) and any(r.finish_reason == "length" for r in want)
+    for ahead in (2, 4, 7):
+        eng = H.make_engine(d, dtype, kv_tokens=512, max_num_seqs=5, decode_graphs=graphs, decode_run_ahead=ahead)
+        got = eng.generate(prompts, params)
+        assert [r.token_ids for r in got] == [r.token_ids for r in want], ahead
+        assert [r.finish_reason for r in got] == [r.finish_reason for r in want]
+        assert eng.last_stats.decode_tokens == one.last_stats.decode_tokens and eng.last_stats.steps == one.last_stats.steps
+        eng.cache.check_invariants()
+        assert all(g.pool.num_free == g.pool.num_pages for g in eng.cache.groups)
+    # the runner's own entry: steps on end against the same steps one by one
+    ids = ["x", "y", "z"]
+    runs = []
+    for on_end in (True, False):
+        eng = H.make_engine(d, dtype, kv_tokens=512, max_num_seqs=3, decode_graphs=graphs)
+        first = []
+        for r, p in zip(ids, prompts):
+            eng.add_request(r)
+            first.append(int(eng.step([StepEntry(r, p, (len(p) - 1,))], select="argmax").cpu()[0]))
+        if on_end:
+            runs.append(eng.decode_steps([StepEntry(r, (t,), (0,)) for r, t in zip(ids, first)], 6).cpu().tolist())
+        else:
+            rows, cur = [], first
+            for _ in range(6):
+                cur = eng.step([StepEntry(r, (t,), (0,)) for r, t in zip(ids, cur)], select="argmax").cpu().tolist()
+                rows.append(cur)
+            runs.append(rows)
+    assert runs[0] == runs[1]
+
+
 def test_chunks_stream_in_order_and_cancelling_gives_pages_back(tmp_path):
     """The typed chunks of a generation: per prompt one usage chunk first, its tokens in order,
     one stop chunk last; the tokens are those of generate().  A prompt cancelled half-way ends
