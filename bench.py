@@ -449,7 +449,10 @@ def main() -> int:
             "hidden_size": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
             "head_dim": cfg.head_dim, "experts": cfg.num_local_experts, "experts_per_tok": cfg.num_experts_per_tok,
             "expert_ffn": cfg.intermediate_size, "shared_ffn": cfg.intermediate_size, "vocab": cfg.vocab_size,
-            "attention_chunk": cfg.attention_chunk_size, "prompt_len": P, "generated": args.warmup + args.steps,
+            "attention_chunk": cfg.attention_chunk_size, "prompt_len": P,
+            # decoded tokens a request: warm-up, the two steps that time the host, the run-ahead's own warm-up, the
+            # timed steps and the traced one
+            "generated": args.warmup + 2 + (eng.decode_run_ahead if eng.decode_run_ahead > 1 else 0) + args.steps + 1,
             "page_size": args.page_size,
         },
         "prefill": prefill,
