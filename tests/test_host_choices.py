@@ -1,0 +1,49 @@
+"""Choices the host makes without a GPU: the shapes of the few-rows product's launches, the
+benchmark's refusal of more than one GPU, the byte counts its roofline is priced with."""
+import json
+import os
+import subprocess
+import sys
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_few_rows_launch_shapes_follow_the_rows_and_the_compute_units():
+    from sharpinference_amd import ops
+
+    # the waves that split K are the same whatever the rows: a row's sums do not change with the batch
+    assert {ops.skinny_plan(N, K, rb, g)[1] for N in (5120, 7168, 16384, 202048) for K in (5120, 8192)
+            for rb in (1, 2, 4) for g in (1, 2, 9, 17)} == {8}
+    # one block of rows: two tiles a block (two K units in flight), wide or not
+    assert ops.skinny_plan(7168, 5120, 1)[0] == 2 and ops.skinny_plan(202048, 5120, 1)[0] == 2
+    assert ops.skinny_plan(16384, 5120, 1, 9, act=True)[0] == 2
+    # ... unless that makes between one and two blocks per compute unit: the merged down projection of one token
+    assert ops.skinny_plan(5120, 8192, 1, 2)[0] == 1 and ops.skinny_plan(5120, 8192, 1, 9)[0] == 2
+    assert ops.skinny_plan(5120, 5120, 1, 1)[0] == 2            # 160 blocks: every unit has at most one
+    assert ops.skinny_plan(16384, 5120, 1, 1, act=True)[0] == 2  # the gated form pairs tiles: never one
+    # more rows: four tiles for wide matrices
+    assert ops.skinny_plan(16384, 5120, 4, 17)[0] == 4 and ops.skinny_plan(5120, 8192, 4, 17)[0] == 2
+
+
+def test_benchmark_refuses_more_than_one_gpu():
+    out = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 2
+    assert len(out.stdout.strip().splitlines()) == 1 and "one GPU" in out.stdout
+
+
+def test_roofline_bytes_count_every_weight_once_and_the_live_cache():
+    sys.path.insert(0, ROOT)
+    import bench
+    from sharpinference_amd import load_config
+
+    cfg = load_config(dict(bench.SCOUT, num_hidden_layers=48, no_rope_layers=[0 if (l + 1) % 4 == 0 else 1 for l in range(48)]))
+    H, I, V = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
+    attn = H * (cfg.num_attention_heads + 2 * cfg.num_key_value_heads) * cfg.head_dim + cfg.num_attention_heads * cfg.head_dim * H
+    expert = 3 * H * I
+    router = cfg.num_local_experts * H
+    ctx, batch, distinct = 2100, 8, 6.5
+    kv = 2 * cfg.num_key_value_heads * cfg.head_dim * ctx * batch
+    want = 2 * (48 * (attn + router + (distinct + 1) * expert + kv) + V * H)
+    got = bench.decode_step_bytes(cfg, 48, batch, ctx, distinct)
+    assert abs(got - want) / want < 0.01, (got, want)
+    json.dumps({"bytes": got})
