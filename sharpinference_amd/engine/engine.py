@@ -325,10 +325,14 @@ class Engine:
 
     def _steps_ahead(self, sched: Scheduler, batch, should_cancel) -> int:
         """How many decode steps may be launched on end for this batch: more than one only while
-        every request of it decodes greedily, nobody waits to be admitted or can be cancelled in
-        between, and no request would pass its own limit (a request that meets a stop token on
-        the way is ended there; the steps run past it are dropped with its pages)."""
+        the batch holds every running request and each of them decodes greedily, nobody waits to
+        be admitted or can be cancelled in between, and no request would pass its own limit (a
+        request that meets a stop token on the way is ended there; the steps run past it are
+        dropped with its pages).  With a token budget below the number of running requests the
+        batch changes from step to step, so every step is scheduled on its own."""
         if self.decode_run_ahead <= 1 or should_cancel is not None or sched.waiting or not batch:
+            return 1
+        if len(batch) != len(sched.running):
             return 1
         steps = self.decode_run_ahead
         for s in batch:

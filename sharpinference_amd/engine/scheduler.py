@@ -11,7 +11,10 @@ and its cache goes back at once (394-407, 697-714).
 
 Unlike the reference, one step carries decode tokens and prompt portions together: every
 decoding request first gets its one token, what is left of the budget goes to prompts in
-arrival order.
+arrival order.  The reference decodes every active sequence in every iteration (314-347);
+where the token budget is smaller than the number of requests that want a token, the ones
+that have waited longest go first with one token each, so that all of them advance within
+one step of each other.
 
 When pages run out: they cannot for a running request, because admission reserved the pages it
 can ever hold.  A waiting request waits until enough reservations are returned.  A request
@@ -44,6 +47,7 @@ class Request:
     cancelled: bool = False
     draws: int = 0                    # uniforms used so far
     stops: frozenset = frozenset()    # tokens that end it (its own and the model's), set on admission to the queue
+    last_step: int = -1               # ticket of the scheduling pass that last gave it tokens
 
     @property
     def finished(self) -> bool:
@@ -76,6 +80,7 @@ class Scheduler:
         self.waiting: Deque[Request] = deque()
         self.running: List[Request] = []
         self.finished: List[Request] = []
+        self._tickets = 0                                # one per request and scheduling pass, in the order served
 
     # ------------------------------------------------------------------
     def add(self, request: Request) -> None:
@@ -126,16 +131,31 @@ class Scheduler:
         self._admit()
         budget = self.max_tokens_per_step
         batch: List[Scheduled] = []
-        for r in self.running:                           # decoding requests first: one token each
-            if not r.in_prefill and budget > 0:
-                batch.append(Scheduled(r, [r.output[-1]], True))
-                budget -= 1
-        for r in self.running:                           # then prompts, in arrival order
-            if r.in_prefill and budget > 0:
-                take = min(len(r.prompt) - r.num_computed, budget)
+        decoders = [r for r in self.running if not r.in_prefill]
+        prompts = [r for r in self.running if r.in_prefill]
+        if len(decoders) > budget or (prompts and len(decoders) == budget):
+            # fewer tokens than requests that want one: one token each to those left out longest
+            # (the sort is stable, so equals keep their arrival order); the batch keeps the running
+            # order, and a prompt advances by a one-token portion
+            turn = sorted(self.running, key=lambda r: r.last_step)[:budget]
+            chosen = set(id(r) for r in turn)
+            decoders = [r for r in decoders if id(r) in chosen]
+            prompts = [r for r in prompts if id(r) in chosen]
+            share = 1
+        else:
+            share, turn = None, None
+        for r in decoders:                               # decoding requests first: one token each
+            batch.append(Scheduled(r, [r.output[-1]], True))
+            budget -= 1
+        for r in prompts:                                # then prompts, in arrival order
+            if budget > 0:
+                take = min(len(r.prompt) - r.num_computed, share or budget)
                 toks = r.prompt[r.num_computed:r.num_computed + take]
                 batch.append(Scheduled(r, toks, r.num_computed + take == len(r.prompt)))
                 budget -= take
+        for r in turn if turn is not None else [s.request for s in batch]:
+            r.last_step = self._tickets                  # strictly increasing: a round robin, no ties
+            self._tickets += 1
         return batch
 
     def update(self, batch: Sequence[Scheduled], sampled: Sequence[Optional[int]]) -> List[Request]:

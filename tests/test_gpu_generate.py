@@ -170,6 +170,40 @@ def test_steps_launched_on_end_give_the_same_generation(tmp_path, dtype, graphs)
     assert runs[0] == runs[1]
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_token_budget_below_the_live_requests_generates_the_same(tmp_path, dtype):
+    """Two tokens a step for three requests: the batch is then a changing part of the running
+    requests.  Steps are never launched on end for a batch that leaves a running request out (its
+    cache would not have been stepped), a stop token met on the way ends its request where the
+    waiting engine ends it, nobody starves, and in 32-bit the tokens are the plain
+    implementation's, which knows nothing of steps."""
+    from sharpinference_amd import SamplingParams
+
+    d = make_model_dir(tmp_path, "A", std=0.1)
+    prompts = [H.random_tokens(n, 256, 40 + n) for n in (7, 12, 5)]
+    one = H.make_engine(d, dtype, kv_tokens=512, max_num_seqs=3, max_tokens_per_step=2, decode_run_ahead=1)
+    free = one.generate(prompts, max_new_tokens=14)
+    stop = free[0].token_ids[6]
+    params = [SamplingParams(temperature=0.0, max_new_tokens=m, stop_token_ids=(stop,)) for m in (14, 14, 9)]
+    want = one.generate(prompts, params)
+    assert want[0].finish_reason == "stop" and len(want[0].token_ids) <= 6
+    if dtype == "float32":
+        c, W = P.read_config(d), P.load_weights(d)
+        plain = [P.generate(c, W, p, q.max_new_tokens, stop=(stop,)) for p, q in zip(prompts, params)]
+        assert [r.token_ids for r in want] == plain
+    for ahead in (4, 7):
+        eng = H.make_engine(d, dtype, kv_tokens=512, max_num_seqs=3, max_tokens_per_step=2, decode_run_ahead=ahead)
+        got = eng.generate(prompts, params)
+        assert [r.token_ids for r in got] == [r.token_ids for r in want], ahead
+        assert [r.finish_reason for r in got] == [r.finish_reason for r in want]
+        eng.cache.check_invariants()
+        assert all(g.pool.num_free == g.pool.num_pages for g in eng.cache.groups)
+    # the same prompts with room for everybody: the budget changes the steps, not the tokens
+    wide = H.make_engine(d, dtype, kv_tokens=512, max_num_seqs=3, max_tokens_per_step=64)
+    if dtype == "float32":
+        assert [r.token_ids for r in wide.generate(prompts, params)] == [r.token_ids for r in want]
+
+
 def test_chunks_stream_in_order_and_cancelling_gives_pages_back(tmp_path):
     """The typed chunks of a generation: per prompt one usage chunk first, its tokens in order,
     one stop chunk last; the tokens are those of generate().  A prompt cancelled half-way ends

@@ -56,6 +56,36 @@ def test_portions_respect_the_budget_and_decodes_come_first():
     assert all(g.pool.num_free == g.pool.num_pages for g in sched.cache.groups)
 
 
+def test_a_budget_below_the_number_of_decoders_starves_nobody():
+    """Two tokens a step for three decoding requests: the reference decodes every active sequence
+    in every iteration (reference: src/SharpInference.Engine/ContinuousBatchingEngine.cs:314-347);
+    with less budget than that, whoever was left out goes first next time, so no request is ever
+    more than one token behind another that was admitted with it."""
+    sched = Scheduler(_cache(64), max_num_seqs=4, max_tokens_per_step=2, max_model_len=256)
+    reqs = [_req(i, 2, 30) for i in range(3)]
+    for r in reqs:
+        sched.add(r)
+    spread, base = [], None
+    script = lambda r: 100 + len(r.output)
+    for _ in range(200):
+        if not sched.has_work():
+            break
+        batch = sched.schedule()
+        assert 0 < sum(len(s.tokens) for s in batch) <= 2
+        assert len(set(s.request.req_id for s in batch)) == len(batch)
+        for s in batch:
+            assert sched.cache.append(s.request.req_id, len(s.tokens))
+            sched.cache.commit(s.request.req_id)
+        sched.update(batch, [script(s.request) if s.samples else None for s in batch])
+        if all(not r.finished and not r.in_prefill for r in reqs):
+            base = base or [len(r.output) for r in reqs]
+            gains = [len(r.output) - b for r, b in zip(reqs, base)]
+            spread.append(max(gains) - min(gains))
+    assert len(spread) >= 6 and max(spread) <= 1, spread
+    assert [len(r.output) for r in reqs] == [30, 30, 30]
+    assert all(g.pool.num_free == g.pool.num_pages for g in sched.cache.groups)
+
+
 def test_stop_token_ends_without_being_emitted_even_as_first_token():
     sched = Scheduler(_cache(64), 4, 64, 256)
     a, b = _req("a", 4, 10, stop=(7,)), _req("b", 4, 10, stop=(7,))
