@@ -62,7 +62,7 @@ _REQUIRED = (
 # Every key of the text decoder's config.json falls in one of three classes: read into a field
 # (_READ), known to leave the forward pass of an inference engine as it is (_INERT: training
 # options, bookkeeping of the tool that wrote the file, hints for other runtimes), or checked
-# against the one value this engine computes with (hidden_act, attention_bias, layer_types).
+# against what the fields read elsewhere imply (layer_types).
 # A key outside the three whose value is a number, a list or an object may change the
 # computation: it is refused.  Text and null values of unknown keys are kept in ``unread_keys``.
 _READ = frozenset({
@@ -83,6 +83,8 @@ _INERT = frozenset({
     "_attn_implementation", "attn_implementation", "_attn_implementation_autoset", "quantization_config",
 })
 _LAYER_KIND_OF_ROPE = {True: "chunked_attention", False: "full_attention"}
+# config.json's names of the gated unit's activation -> the names the feed-forward parts take
+_ACTIVATIONS = {"silu": "silu", "swish": "silu", "gelu_pytorch_tanh": "gelu_tanh", "gelu_tanh": "gelu_tanh"}
 
 
 def _number(src: Dict[str, Any], key: str, kind, default=None):
@@ -163,6 +165,8 @@ class Llama4TextConfig(ModelConfig):
     rms_norm_eps: float = 1e-5
     rope_theta: float = 500000.0
     rope_scaling: Optional[RopeScaling] = None
+    hidden_act: str = "silu"              # the gated unit's activation, as config.json names it
+    attention_bias: bool = False          # q, k, v and o projections carry biases
     # head
     tie_word_embeddings: bool = False
     max_position_embeddings: int = 0
@@ -194,10 +198,12 @@ class Llama4TextConfig(ModelConfig):
             raise ConfigError("config.json holds key(s) that this reader does not understand and that may change "
                               "the computation: " + ", ".join(f"{k}={src[k]!r}" for k in refused))
         act = src.get("hidden_act", "silu")
-        if act != "silu":
-            raise ConfigError(f"hidden_act {act!r} is not supported: the feed-forward kernels apply silu")
-        if src.get("attention_bias"):
-            raise ConfigError("attention_bias true is not supported: the attention projections carry no bias")
+        if act not in _ACTIVATIONS:
+            raise ConfigError(f"hidden_act {act!r} is not supported: the feed-forward kernels apply "
+                              + ", ".join(sorted(_ACTIVATIONS)))
+        bias = src.get("attention_bias", False)
+        if not isinstance(bias, bool):
+            raise ConfigError(f"attention_bias must be true or false (got {bias!r})")
         nh = _number(src, "num_attention_heads", int)
         hidden = _number(src, "hidden_size", int)
         layers = _number(src, "num_hidden_layers", int)
@@ -252,6 +258,8 @@ class Llama4TextConfig(ModelConfig):
             rms_norm_eps=_number(src, "rms_norm_eps", float, 1e-5),
             rope_theta=theta,
             rope_scaling=scaling,
+            hidden_act=str(act),
+            attention_bias=bias,
             tie_word_embeddings=bool(src.get("tie_word_embeddings", False)),
             max_position_embeddings=_number(src, "max_position_embeddings", int) or 0,
             torch_dtype=str(src.get("torch_dtype") or src.get("dtype") or "bfloat16"),
@@ -283,6 +291,8 @@ class Llama4TextConfig(ModelConfig):
             "rms_norm_eps": self.rms_norm_eps,
             "rope_theta": self.rope_theta,
             "rope_scaling": self.rope_scaling.to_dict() if self.rope_scaling else None,
+            "hidden_act": self.hidden_act,
+            "attention_bias": self.attention_bias,
             "tie_word_embeddings": self.tie_word_embeddings,
             "max_position_embeddings": self.max_position_embeddings,
             "torch_dtype": self.torch_dtype,
@@ -312,6 +322,7 @@ class Llama4TextConfig(ModelConfig):
         need(self.rms_norm_eps > 0, "rms_norm_eps must be positive")
         need(self.rope_theta > 0, "rope_theta must be positive")
         need(self.floor_scale > 0, "floor_scale must be positive")
+        need(self.hidden_act in _ACTIVATIONS, f"hidden_act {self.hidden_act!r} is not known ({', '.join(sorted(_ACTIVATIONS))})")
         if self.moe_layers is not None:
             bad = [l for l in self.moe_layers if not 0 <= l < self.num_hidden_layers]
             need(not bad, f"moe_layers names layers out of range: {bad}")
@@ -340,6 +351,11 @@ class Llama4TextConfig(ModelConfig):
             return layer in self.moe_layers
         step = self.interleave_moe_layer_step
         return step > 0 and (layer + 1) % step == 0
+
+    @property
+    def activation(self) -> str:
+        """The gated unit's activation under the name the feed-forward parts take."""
+        return _ACTIVATIONS[self.hidden_act]
 
     def uses_rope(self, layer: int) -> bool:
         return self.no_rope_layers[layer] != 0

@@ -406,3 +406,26 @@ SHARPI_EXPORT int sharpi_cast(const void* in, int in_dtype, void* out, int out_d
   SHARPI_CHECK_LAUNCH();
   return SHARPI_OK;
 }
+
+// ---------------------------------------------------------------------------
+// x [T, N] += bias [N] (float), in place; the sum in float, rounded to x's storage.  For the
+// projections of architectures that carry biases (the products themselves have no bias term).
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ void add_bias_kernel(T* __restrict__ x, const float* __restrict__ bias, int n_rows, int N) {
+  const size_t total = (size_t)n_rows * N;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x)
+    x[i] = from_f32<T>(to_f32<T>(x[i]) + bias[i % N]);
+}
+
+SHARPI_EXPORT int sharpi_add_bias(void* x, int dtype, const float* bias, int n_rows, int N, hipStream_t stream) {
+  if (n_rows <= 0) return SHARPI_OK;
+  if (N <= 0 || !bias) return SHARPI_ERR_ARG;
+  const size_t total = (size_t)n_rows * N;
+  const dim3 block(256), grid((unsigned)min((size_t)4096, (total + 255) / 256));
+  if (dtype == DT_F32) add_bias_kernel<float><<<grid, block, 0, stream>>>((float*)x, bias, n_rows, N);
+  else if (dtype == DT_BF16) add_bias_kernel<bf16_t><<<grid, block, 0, stream>>>((bf16_t*)x, bias, n_rows, N);
+  else return SHARPI_ERR_ARG;
+  SHARPI_CHECK_LAUNCH();
+  return SHARPI_OK;
+}

@@ -1,6 +1,7 @@
 // Position encoding, weightless per-head norm, query temperature and the cache write, one kernel.
 //
-// Input  qkv [T, (nh + 2*nkv) * hd]: q heads, then k heads, then v heads of each token.
+// Input  qkv [T, (nh + 2*nkv) * hd]: q heads, then k heads, then v heads of each token; an optional
+// bias [(nh + 2*nkv) * hd] (float) is added to every token's row first, in float.
 // q head : rotate (if inv_freq) -> norm (if qk_norm) -> * temperature (if temp_tuning) -> q_out
 // k head : rotate (if inv_freq) -> norm (if qk_norm) -> cache K at slot_mapping[t]
 // v head : cache V at slot_mapping[t]
@@ -17,6 +18,7 @@ template <typename T>
 __global__ void rope_kv_kernel(const T* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_cache,
                                T* __restrict__ v_cache, const int* __restrict__ slot_mapping,
                                const int* __restrict__ positions, const float* __restrict__ inv_freq,
+                               const float* __restrict__ bias,
                                int qk_norm, float eps, int temp_tuning, float floor_scale, float attn_scale,
                                int nh, int nkv, int hd, int page_size, int half_split, int rotary_dim) {
   const int t = blockIdx.x;
@@ -24,6 +26,7 @@ __global__ void rope_kv_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
   const int lane = threadIdx.x;           // one wave
   const int half = hd >> 1;
   const T* src = qkv + ((size_t)t * (nh + 2 * nkv) + head) * hd;
+  const float* hb = bias ? bias + (size_t)head * hd : nullptr;
   const int pos = positions[t];
   const bool is_q = head < nh;
   const bool is_k = !is_q && head < nh + nkv;
@@ -33,7 +36,8 @@ __global__ void rope_kv_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
     if (slot < 0) return;
     const int kvh = head - nh - nkv;
     T* dst = v_cache + ((size_t)(slot / page_size) * nkv + kvh) * hd * page_size + (slot % page_size);
-    for (int d = lane; d < hd; d += kWave) dst[(size_t)d * page_size] = src[d];
+    for (int d = lane; d < hd; d += kWave)
+      dst[(size_t)d * page_size] = hb ? from_f32<T>(to_f32<T>(src[d]) + hb[d]) : src[d];
     return;
   }
   if (is_k && slot < 0) return;
@@ -64,6 +68,10 @@ __global__ void rope_kv_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
       }
       float a = to_f32<T>(src[e0[j]]);
       float b = to_f32<T>(src[e1[j]]);
+      if (hb) {
+        a += hb[e0[j]];
+        b += hb[e1[j]];
+      }
       if (inv_freq && i < rot_pairs) {
         const float ang = (float)pos * inv_freq[i];
         const float c = cosf(ang);
@@ -122,8 +130,8 @@ template <typename T>
 __global__ __launch_bounds__(256) void rope_kv_vec_kernel(
     const T* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
     const int* __restrict__ slot_mapping, const int* __restrict__ positions, const float* __restrict__ inv_freq,
-    int qk_norm, float eps, int temp_tuning, float floor_scale, float attn_scale, int nh, int nkv, int hd,
-    int page_size, int rotary_dim) {
+    const float* __restrict__ bias, int qk_norm, float eps, int temp_tuning, float floor_scale, float attn_scale,
+    int nh, int nkv, int hd, int page_size, int rotary_dim) {
   const int t = blockIdx.x;
   const int per_head = hd >> 3;                    // lanes per head: 4, 8, 16 or 32
   const int chunks = (nh + 2 * nkv) * per_head;
@@ -152,7 +160,15 @@ __global__ __launch_bounds__(256) void rope_kv_vec_kernel(
     const bool is_q = head < nh;
     const bool is_k = !is_q && head < nh + nkv;
     float x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    if (valid) load8(src + (size_t)head * hd + run * 8, x);
+    if (valid) {
+      load8(src + (size_t)head * hd + run * 8, x);
+      if (bias) {
+        float b8[8];
+        load8(bias + (size_t)head * hd + run * 8, b8);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) x[j] += b8[j];
+      }
+    }
     float ss = 0.f;
     if (valid && (is_q || is_k)) {
       if (rotates) {
@@ -197,7 +213,7 @@ __global__ __launch_bounds__(256) void rope_kv_vec_kernel(
 
 SHARPI_EXPORT int sharpi_rope_kv(const void* qkv, void* q_out, void* k_cache, void* v_cache, int dtype,
                                  const int* slot_mapping, const int* positions, const float* inv_freq,
-                                 int qk_norm, float eps, int temp_tuning, float floor_scale, float attn_scale,
+                                 const float* bias, int qk_norm, float eps, int temp_tuning, float floor_scale, float attn_scale,
                                  int n_tokens, int nh, int nkv, int hd, int page_size, int pair_layout,
                                  int rotary_dim, hipStream_t stream) {
   if (n_tokens <= 0) return SHARPI_OK;
@@ -217,24 +233,24 @@ SHARPI_EXPORT int sharpi_rope_kv(const void* qkv, void* q_out, void* k_cache, vo
     if (dtype == DT_F32)
       rope_kv_vec_kernel<float><<<vgrid, 256, 0, stream>>>((const float*)qkv, (float*)q_out, (float*)k_cache,
                                                              (float*)v_cache, slot_mapping, positions, inv_freq,
-                                                             qk_norm, eps, temp_tuning, floor_scale, attn_scale,
+                                                             bias, qk_norm, eps, temp_tuning, floor_scale, attn_scale,
                                                              nh, nkv, hd, page_size, rotary_dim);
     else
       rope_kv_vec_kernel<bf16_t><<<vgrid, 256, 0, stream>>>((const bf16_t*)qkv, (bf16_t*)q_out,
                                                               (bf16_t*)k_cache, (bf16_t*)v_cache, slot_mapping,
-                                                              positions, inv_freq, qk_norm, eps, temp_tuning,
+                                                              positions, inv_freq, bias, qk_norm, eps, temp_tuning,
                                                               floor_scale, attn_scale, nh, nkv, hd, page_size, rotary_dim);
     SHARPI_CHECK_LAUNCH();
     return SHARPI_OK;
   }
   if (dtype == DT_F32)
     rope_kv_kernel<float><<<grid, block, 0, stream>>>((const float*)qkv, (float*)q_out, (float*)k_cache,
-                                                     (float*)v_cache, slot_mapping, positions, inv_freq, qk_norm,
+                                                     (float*)v_cache, slot_mapping, positions, inv_freq, bias, qk_norm,
                                                      eps, temp_tuning, floor_scale, attn_scale, nh, nkv, hd,
                                                      page_size, pair_layout, rotary_dim);
   else if (dtype == DT_BF16)
     rope_kv_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)qkv, (bf16_t*)q_out, (bf16_t*)k_cache,
-                                                      (bf16_t*)v_cache, slot_mapping, positions, inv_freq,
+                                                      (bf16_t*)v_cache, slot_mapping, positions, inv_freq, bias,
                                                       qk_norm, eps, temp_tuning, floor_scale, attn_scale, nh, nkv,
                                                       hd, page_size, pair_layout, rotary_dim);
   else

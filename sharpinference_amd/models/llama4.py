@@ -10,6 +10,8 @@ layer from config.json:
   if ``use_qk_norm``, attention confined to the chunk of ``attention_chunk_size``;
 * layers without rotary: all keys, queries scaled by the position-dependent temperature if
   ``attn_temperature_tuning``;
+* ``hidden_act`` names the gated unit's activation of every feed-forward, ``attention_bias``
+  gives the four attention projections biases;
 * layer L carries experts iff (L + 1) % interleave_moe_layer_step == 0 (top-k sigmoid router
   scaling the expert input, plus the shared expert), otherwise the dense feed-forward of
   width ``intermediate_size_mlp``.
@@ -35,17 +37,19 @@ def build_llama4(cfg: Llama4TextConfig) -> DecoderModel:
         if cfg.uses_rope(layer):
             mixer = Attention(cfg.hidden_size, cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim,
                               rotary=rotary, qk_norm_eps=cfg.rms_norm_eps if cfg.use_qk_norm else None,
-                              q_temperature=None, window_kind=WINDOW_CHUNK, window=cfg.attention_chunk_size)
+                              q_temperature=None, window_kind=WINDOW_CHUNK, window=cfg.attention_chunk_size,
+                              bias=cfg.attention_bias)
         else:
             temp = (cfg.floor_scale, cfg.attn_scale) if cfg.attn_temperature_tuning else None
             mixer = Attention(cfg.hidden_size, cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim,
-                              rotary=None, qk_norm_eps=None, q_temperature=temp, window_kind=WINDOW_NONE)
+                              rotary=None, qk_norm_eps=None, q_temperature=temp, window_kind=WINDOW_NONE,
+                              bias=cfg.attention_bias)
         if cfg.is_moe_layer(layer):
             ffn = MoESwiGLU(cfg.hidden_size, cfg.num_local_experts, cfg.num_experts_per_tok, cfg.intermediate_size,
                             shared_intermediate=cfg.intermediate_size, gate="sigmoid", renormalise=False,
-                            score_on_input=True)
+                            score_on_input=True, activation=cfg.activation)
         else:
-            ffn = DenseSwiGLU(cfg.hidden_size, cfg.intermediate_size_mlp)
+            ffn = DenseSwiGLU(cfg.hidden_size, cfg.intermediate_size_mlp, activation=cfg.activation)
         blocks.append(PreNormBlock(RMSNorm(cfg.hidden_size, cfg.rms_norm_eps), mixer,
                                    RMSNorm(cfg.hidden_size, cfg.rms_norm_eps), ffn))
     return DecoderModel(cfg.vocab_size, cfg.hidden_size, blocks, RMSNorm(cfg.hidden_size, cfg.rms_norm_eps),

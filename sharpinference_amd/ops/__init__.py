@@ -179,6 +179,15 @@ def moe_combine(y: torch.Tensor, inv_pos: torch.Tensor, shared: Optional[torch.T
     return out
 
 
+def add_bias(x: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
+    """x [T, N] += bias [N] (float32), in place: the sum in float, rounded to x's storage."""
+    _dev(x, bias)
+    _need(x.dim() == 2 and x.is_contiguous() and bias.dtype == torch.float32 and bias.shape == (x.shape[1],)
+          and bias.is_contiguous(), "add_bias: x [T, N] contiguous and bias float32 [N] wanted")
+    _run("sharpi_add_bias", _ptr(x), _code(x.dtype), _ptr(bias), x.shape[0], x.shape[1], _stream())
+    return x
+
+
 def cast(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
     _dev(x)
     out = torch.empty(x.shape, dtype=dtype, device=x.device)
@@ -215,12 +224,16 @@ PAIRS_INTERLEAVED, PAIRS_HALF_SPLIT = 0, 1
 def rope_kv(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, slot_mapping: torch.Tensor,
             positions: torch.Tensor, inv_freq: Optional[torch.Tensor], qk_norm: bool, eps: float,
             temperature: Optional[Tuple[float, float]], nh: int, nkv: int, hd: int,
-            pair_layout: int = PAIRS_INTERLEAVED) -> torch.Tensor:
+            pair_layout: int = PAIRS_INTERLEAVED, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Rotate / norm / scale the heads of qkv [T, (nh+2nkv)*hd]; K and V go into the layer's
     cache [pages, nkv, page_size, hd] at slot_mapping; returns q [T, nh*hd].  inv_freq [r/2]
     rotates the first r <= hd elements of every head, in pairs (2i, 2i+1) or (i, i + r/2)
-    (``pair_layout``); the rest of the head passes through."""
-    _dev(qkv, k_cache, v_cache, slot_mapping, positions, inv_freq)
+    (``pair_layout``); the rest of the head passes through.  ``bias`` (float32, one value per
+    column of qkv) is added to every row first, in float."""
+    _dev(qkv, k_cache, v_cache, slot_mapping, positions, inv_freq, bias)
+    if bias is not None:
+        _need(bias.dtype == torch.float32 and bias.shape == (qkv.shape[1],) and bias.is_contiguous(),
+              "rope_kv: bias must be float32 [(nh+2nkv)*hd]")
     _i32(slot_mapping, "slot_mapping")
     _i32(positions, "positions")
     T = qkv.shape[0]
@@ -238,7 +251,7 @@ def rope_kv(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, slo
     q_out = torch.empty(T, nh * hd, dtype=qkv.dtype, device=qkv.device)
     fs, asc = temperature if temperature is not None else (1.0, 0.0)
     _run("sharpi_rope_kv", _ptr(qkv), _ptr(q_out), _ptr(k_cache), _ptr(v_cache), _code(qkv.dtype),
-         _ptr(slot_mapping), _ptr(positions), _ptr(inv_freq), 1 if qk_norm else 0, float(eps),
+         _ptr(slot_mapping), _ptr(positions), _ptr(inv_freq), _ptr(bias), 1 if qk_norm else 0, float(eps),
          1 if temperature is not None else 0, float(fs), float(asc), T, nh, nkv, hd, page_size, int(pair_layout),
          rotary_dim, _stream())
     return q_out

@@ -22,10 +22,11 @@ _SIGNATURES = {
     "sharpi_silu_mul": [P, P, P, I, I, I, I, P],
     "sharpi_moe_combine": [P, P, P, P, P, I, I, I, I, P],
     "sharpi_cast": [P, I, P, I, c_longlong, P],
+    "sharpi_add_bias": [P, I, P, I, I, P],
     "sharpi_peak_read": [P, c_longlong, P, P, P],
     "sharpi_peak_mfma": [P, I, I, P],
     "sharpi_random_fill": [P, I, c_longlong, c_ulonglong, I, F, I, I, P],
-    "sharpi_rope_kv": [P, P, P, P, I, P, P, P, I, F, I, F, F, I, I, I, I, I, I, I, P],
+    "sharpi_rope_kv": [P, P, P, P, I, P, P, P, P, I, F, I, F, F, I, I, I, I, I, I, I, P],
     "sharpi_attention_generic": [P, P, P, I, P, P, P, P, I, I, F, I, I, I, I, I, I, I, P],
     "sharpi_attention_decode": [P, P, P, P, P, P, P, P, P, P, I, I, F, I, I, I, I, I, I, I, I, P],
     "sharpi_attention_prefill": [P, P, P, P, P, P, P, I, I, I, F, I, I, I, I, I, I, P],

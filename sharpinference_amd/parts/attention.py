@@ -13,11 +13,12 @@ from .base import LayerCache, ParamSpec, Part, StepContext, TensorSource
 
 
 class Attention(Part):
-    """q/k/v projections without bias -> position encoding -> optional weightless per-head norm
+    """q/k/v projections (with biases if ``bias``) -> position encoding -> optional weightless per-head norm
     -> optional query temperature -> keys and values into the cache -> softmax(q k^T * scale) v
     over the keys the window admits -> output projection
     (reference: src/SharpInference.Engine/ForwardPass.cs:1576-1690, 1838-1912; the norm comes
-    after the rotation, 1643-1648).
+    after the rotation, 1643-1648; optional biases are added right after their products,
+    1605-1613, the output projection's may be absent on its own, 381-383).
 
     Everything that differs between layers is an argument: ``rotary`` (None = no position
     encoding; otherwise any object with ``table(device)``, ``pair_layout``, ``rotary_dim`` and
@@ -28,7 +29,7 @@ class Attention(Part):
     def __init__(self, hidden: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  rotary=None, qk_norm_eps: Optional[float] = None,
                  q_temperature: Optional[Tuple[float, float]] = None, window_kind: int = WINDOW_NONE,
-                 window: int = 0, scale: Optional[float] = None):
+                 window: int = 0, scale: Optional[float] = None, bias: bool = False, o_bias: Optional[bool] = None):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} heads cannot share {num_kv_heads} kv heads")
         if head_dim % 16 or not 16 <= head_dim <= 256:
@@ -41,8 +42,12 @@ class Attention(Part):
         self.rotary, self.qk_norm_eps, self.q_temperature = rotary, qk_norm_eps, q_temperature
         self.window_kind, self.window = int(window_kind), int(window)
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
+        self.bias = bool(bias)                                   # q, k and v carry biases
+        self.o_bias = self.bias if o_bias is None else bool(o_bias)   # the output projection carries one
         self.w_qkv: Optional[torch.Tensor] = None
         self.w_o: Optional[torch.Tensor] = None
+        self.b_qkv: Optional[torch.Tensor] = None                # float32 [q + 2 kv]: added by the rotation kernel
+        self.b_o: Optional[torch.Tensor] = None                  # float32 [hidden]
 
     # -- what it needs --------------------------------------------------------
     def cache_spec(self) -> KVSpec:
@@ -50,12 +55,18 @@ class Attention(Part):
 
     def param_specs(self, prefix: str) -> Dict[str, ParamSpec]:
         q, kv = self.nh * self.hd, self.nkv * self.hd
-        return {
+        specs = {
             prefix + "q_proj.weight": ParamSpec((q, self.hidden)),
             prefix + "k_proj.weight": ParamSpec((kv, self.hidden)),
             prefix + "v_proj.weight": ParamSpec((kv, self.hidden)),
             prefix + "o_proj.weight": ParamSpec((self.hidden, q)),
         }
+        if self.bias:
+            specs.update({prefix + "q_proj.bias": ParamSpec((q,)), prefix + "k_proj.bias": ParamSpec((kv,)),
+                          prefix + "v_proj.bias": ParamSpec((kv,))})
+        if self.o_bias:
+            specs[prefix + "o_proj.bias"] = ParamSpec((self.hidden,))
+        return specs
 
     def load(self, prefix: str, source: TensorSource) -> None:
         q, kv = self.nh * self.hd, self.nkv * self.hd
@@ -69,6 +80,10 @@ class Attention(Part):
         # both also in the order the few-rows kernel streams them; the rows stay for prompt-sized steps
         self.w_qkv = ops.pack_weight(fused)
         self.w_o = ops.pack_weight(source.get(prefix + "o_proj.weight"))
+        if self.bias:
+            self.b_qkv = torch.cat([source.get(prefix + n + "_proj.bias").float() for n in ("q", "k", "v")]).contiguous()
+        if self.o_bias:
+            self.b_o = source.get(prefix + "o_proj.bias").float().contiguous()
 
     # -- compute --------------------------------------------------------------
     def forward(self, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> torch.Tensor:
@@ -84,13 +99,15 @@ class Attention(Part):
         layout = ops.PAIRS_HALF_SPLIT if self.rotary is not None and self.rotary.pair_layout == "half" else ops.PAIRS_INTERLEAVED
         with section("rope + cache write", nbytes=2 * width * T * (q_dim + 2 * kv_dim)):
             q = ops.rope_kv(qkv, cache.k, cache.v, slots, ctx.positions, inv_freq, self.qk_norm_eps is not None,
-                            self.qk_norm_eps or 1e-6, self.q_temperature, self.nh, self.nkv, self.hd, layout)
+                            self.qk_norm_eps or 1e-6, self.q_temperature, self.nh, self.nkv, self.hd, layout,
+                            bias=self.b_qkv)
         with section("attention", nbytes=lambda: self._keys_held(ctx) * 2 * kv_dim * width + 2 * T * q_dim * width,
                      flops=lambda: 4.0 * self._keys_read(ctx) * q_dim):
             o = ops.attention(q, cache.k, cache.v, g, ctx, self.window_kind, self.window, self.scale, self.nh, self.nkv,
                               self.hd)
         with section("o", nbytes=width * self.hidden * (q_dim + T) + width * T * q_dim, flops=2.0 * T * self.hidden * q_dim):
-            return ops.linear(o, self.w_o, ctx.act_dtype)
+            out = ops.linear(o, self.w_o, ctx.act_dtype)
+            return ops.add_bias(out, self.b_o) if self.b_o is not None else out
 
     def _keys_read(self, ctx: StepContext) -> int:
         """(query, key) pairs of the step: what is computed."""

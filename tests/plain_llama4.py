@@ -115,7 +115,7 @@ def apply_rope_interleaved(x: torch.Tensor, positions: torch.Tensor, inv_freq: t
     x: [T, heads, head_dim]; positions: [T]. The angle is a float32 product, as the
     reference's table builder multiplies in single precision."""
     dt = x.dtype
-    ang = positions.to(torch.float32)[:, None] * inv_freq[None, :]      # [T, hd/2] float32
+    ang = positions.to(torch.float32)[:, None] * inv_freq.to(positions.device)[None, :]      # [T, hd/2] float32
     cos = torch.cos(ang).to(dt)[:, None, :]
     sin = torch.sin(ang).to(dt)[:, None, :]
     x0 = x[..., 0::2]
@@ -186,9 +186,11 @@ def attention_layer(c: dict, W: Dict[str, torch.Tensor], layer: int, n: torch.Te
     p = f"model.layers.{layer}.self_attn."
     nh, nkv, hd = c["num_attention_heads"], c.get("num_key_value_heads", c["num_attention_heads"]), head_dim_of(c)
     T = n.shape[0]
-    q = store(n @ W[p + "q_proj.weight"].T).view(T, nh, hd)
-    k = store(n @ W[p + "k_proj.weight"].T).view(T, nkv, hd)
-    v = store(n @ W[p + "v_proj.weight"].T).view(T, nkv, hd)
+    q, k, v = (store(n @ W[p + f"{name}_proj.weight"].T) for name in "qkv")
+    if c.get("attention_bias", False):       # ForwardPass.cs:1605-1613: biases right after the products
+        q, k, v = (t + W[p + f"{name}_proj.bias"].to(t.dtype) for t, name in zip((q, k, v), "qkv"))
+        v = store(v)                         # values go to the cache as they are
+    q, k, v = q.view(T, nh, hd), k.view(T, nkv, hd), v.view(T, nkv, hd)
     eps = float(c.get("rms_norm_eps", 1e-5))
     if layer_uses_rope(c, layer):
         inv = rope_inv_freq(hd, float(c.get("rope_theta", 500000.0)), c.get("rope_scaling"))
@@ -209,7 +211,10 @@ def attention_layer(c: dict, W: Dict[str, torch.Tensor], layer: int, n: torch.Te
     if kv_in is not None:        # read another layer's keys and values instead of this layer's own
         k, v = kv_in
     o = store(attention(q, k, v, mask)).reshape(T, nh * hd)
-    return store(o @ W[p + "o_proj.weight"].T)
+    out = store(o @ W[p + "o_proj.weight"].T)
+    if c.get("attention_bias", False):       # ForwardPass.cs:893 (the output projection's bias)
+        out = store(out + W[p + "o_proj.bias"].to(out.dtype))
+    return out
 
 
 # ----------------------------------------------------------------------------
@@ -220,9 +225,25 @@ def silu(x: torch.Tensor) -> torch.Tensor:
     return x / (1.0 + torch.exp(-x))
 
 
-def swiglu(n: torch.Tensor, wg: torch.Tensor, wu: torch.Tensor, wd: torch.Tensor, store=_same) -> torch.Tensor:
-    """ForwardPass.cs:2006-2015: down( silu(gate n) * (up n) )."""
-    return store(store(silu(store(n @ wg.T)) * store(n @ wu.T)) @ wd.T)
+def gelu_tanh(x: torch.Tensor) -> torch.Tensor:
+    """SimdKernels.cs:4474-4484 (the scalar form): 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3)))."""
+    return 0.5 * x * (1.0 + torch.tanh(0.7978845608028654 * (x + 0.044715 * x * x * x)))
+
+
+def activation_of(c: dict):
+    """The gated unit's activation by the name config.json gives it (``hidden_act``): SiLU unless the
+    file names the tanh form of GELU."""
+    name = c.get("hidden_act", "silu")
+    if name in ("silu", "swish"):
+        return silu
+    if name in ("gelu_pytorch_tanh", "gelu_tanh"):
+        return gelu_tanh
+    raise ValueError(f"hidden_act {name!r}")
+
+
+def swiglu(n: torch.Tensor, wg: torch.Tensor, wu: torch.Tensor, wd: torch.Tensor, store=_same, act=silu) -> torch.Tensor:
+    """ForwardPass.cs:2006-2015: down( act(gate n) * (up n) ), act = SiLU for this architecture."""
+    return store(store(act(store(n @ wg.T)) * store(n @ wu.T)) @ wd.T)
 
 
 def router_gates(n: torch.Tensor, wr: torch.Tensor) -> torch.Tensor:
@@ -234,10 +255,12 @@ def router_topk(n: torch.Tensor, wr: torch.Tensor, k: int):
     """ForwardPass.cs:2028-2040 and 2132-2150: k picks by gate value, strict > so the lowest
     index wins a tie; weight = that gate value.  No renormalisation of the k weights (the
     reference would renormalise for k > 1, 2156-2162; this engine does not, by decision)."""
-    sig = router_gates(n, wr)                            # [T, E]
+    dev = n.device
+    sig = router_gates(n, wr).cpu()                      # [T, E]; the scan below runs on the host
     T, E = sig.shape
     ids = torch.zeros(T, k, dtype=torch.long)
     wts = torch.zeros(T, k, dtype=sig.dtype)
+    rows = sig.tolist()
     for t in range(T):
         taken: List[int] = []
         for j in range(k):
@@ -245,12 +268,12 @@ def router_topk(n: torch.Tensor, wr: torch.Tensor, k: int):
             for e in range(E):
                 if e in taken:
                     continue
-                if float(sig[t, e]) > bv:
-                    bv, best = float(sig[t, e]), e
+                if rows[t][e] > bv:
+                    bv, best = rows[t][e], e
             taken.append(best)
             ids[t, j] = best
             wts[t, j] = sig[t, best]
-    return ids, wts
+    return ids.to(dev), wts.to(dev)
 
 
 def router_margin(n: torch.Tensor, wr: torch.Tensor, k: int) -> torch.Tensor:
@@ -261,7 +284,7 @@ def router_margin(n: torch.Tensor, wr: torch.Tensor, k: int) -> torch.Tensor:
     r = n @ wr.T
     srt = torch.sort(r, dim=-1, descending=True).values
     if srt.shape[1] <= k:
-        return torch.full((n.shape[0],), float("inf"))
+        return torch.full((n.shape[0],), float("inf"), device=n.device)
     return (srt[:, k - 1] - srt[:, k]) / r.pow(2).mean(dim=-1).sqrt().clamp_min(1e-30)
 
 
@@ -278,7 +301,7 @@ def moe_layer(c: dict, W: Dict[str, torch.Tensor], layer: int, n: torch.Tensor, 
         # implementation's gate values as weights, and record how far each lies below the
         # pick made here, relative to the rms of the token's router logits.
         r = n @ W[p + "router.weight"].T
-        forced = routes[layer].to(torch.long)
+        forced = routes[layer].to(torch.long).to(n.device)
         own = torch.gather(r, 1, ids)
         got = torch.gather(r, 1, forced)
         regret = (own.sort(dim=1).values - got.sort(dim=1).values).abs().max(dim=1).values
@@ -291,8 +314,9 @@ def moe_layer(c: dict, W: Dict[str, torch.Tensor], layer: int, n: torch.Tensor, 
         trace.setdefault("picks", {})[layer] = ids      # the picks this run made (or was given), layer by layer
         m = router_margin(n, W[p + "router.weight"], k)
         trace["router_margin"] = torch.minimum(trace["router_margin"], m) if "router_margin" in trace else m
+    act = activation_of(c)
     out = swiglu(n, W[p + "shared_expert.gate_proj.weight"], W[p + "shared_expert.up_proj.weight"],
-                 W[p + "shared_expert.down_proj.weight"], store)
+                 W[p + "shared_expert.down_proj.weight"], store, act)
     Wg, Wu, Wd = W[p + "experts.gate_proj"], W[p + "experts.up_proj"], W[p + "experts.down_proj"]
     routed = torch.zeros_like(out)
     for e in range(Wg.shape[0]):                 # expert by expert, over the (token, pick) pairs that chose it
@@ -302,13 +326,13 @@ def moe_layer(c: dict, W: Dict[str, torch.Tensor], layer: int, n: torch.Tensor, 
         w = wts[t_idx, j_idx][:, None]
         g = store(n[t_idx] @ Wg[e].T) * w
         u = store(n[t_idx] @ Wu[e].T) * w
-        routed.index_add_(0, t_idx, store(store(silu(g) * u) @ Wd[e].T))
+        routed.index_add_(0, t_idx, store(store(act(g) * u) @ Wd[e].T))
     return store(routed + out)
 
 
 def dense_layer(c: dict, W: Dict[str, torch.Tensor], layer: int, n: torch.Tensor, store=_same) -> torch.Tensor:
     p = f"model.layers.{layer}.feed_forward."
-    return swiglu(n, W[p + "gate_proj.weight"], W[p + "up_proj.weight"], W[p + "down_proj.weight"], store)
+    return swiglu(n, W[p + "gate_proj.weight"], W[p + "up_proj.weight"], W[p + "down_proj.weight"], store, activation_of(c))
 
 
 # ----------------------------------------------------------------------------
@@ -325,8 +349,9 @@ def forward(c: dict, W: Dict[str, torch.Tensor], tokens: Sequence[int], start_po
     replaces the router's picks (see moe_layer)."""
     W = {k: v.to(dtype) if v.is_floating_point() else v for k, v in W.items()}
     eps = float(c.get("rms_norm_eps", 1e-5))
-    ids = torch.tensor(list(tokens), dtype=torch.long)
-    positions = torch.arange(start_pos, start_pos + len(ids))
+    dev = W["model.embed_tokens.weight"].device          # the run follows its weights' device
+    ids = torch.tensor(list(tokens), dtype=torch.long, device=dev)
+    positions = torch.arange(start_pos, start_pos + len(ids), device=dev)
     h = W["model.embed_tokens.weight"][ids]
     for l in range(int(c["num_hidden_layers"])):
         p = f"model.layers.{l}."

@@ -77,7 +77,7 @@ def test_no_rope_layer_interval_fills_the_list():
 
 
 @pytest.mark.parametrize("change,word", [
-    ({"hidden_act": "gelu"}, "hidden_act"), ({"attention_bias": True}, "attention_bias"),
+    ({"hidden_act": "gelu"}, "hidden_act"), ({"hidden_act": "relu"}, "hidden_act"), ({"attention_bias": "yes"}, "attention_bias"),
     ({"layer_types": ["full_attention", "full_attention"]}, "layer_types"),
     ({"attention_chunk_size": None}, "attention_chunk_size"), ({"attention_chunk_size": "8192"}, "attention_chunk_size"),
     ({"rope_parameters": {"rope_theta": 5.0}}, "contradicts"),
@@ -94,6 +94,31 @@ def test_no_rope_layer_interval_fills_the_list():
 def test_keys_that_would_change_the_computation_are_not_passed_over(change, word):
     with pytest.raises(ConfigError, match=word):
         load_config({**TINY_A, **change})
+
+
+def test_activation_and_attention_biases_come_from_the_file():
+    """hidden_act names the gated unit's activation of every feed-forward (the names config.json uses
+    for the two the kernels apply); attention_bias gives the four projections biases, which the
+    model then asks the weight file for."""
+    from sharpinference_amd import ops
+
+    plain = build_model(load_config(TINY_B))
+    assert all(b.ffn.act == ops.ACT_SILU for b in plain.blocks)
+    assert not any(n.endswith(".bias") for n in plain.param_specs())
+    for name in ("gelu_pytorch_tanh", "gelu_tanh"):
+        cfg = load_config({**TINY_B, "hidden_act": name})
+        assert cfg.activation == "gelu_tanh" and cfg.to_dict()["hidden_act"] == name
+        m = build_model(cfg)
+        assert all(b.ffn.act == ops.ACT_GELU_TANH for b in m.blocks)
+        assert all(b.ffn.shared.act == ops.ACT_GELU_TANH for b in m.blocks if hasattr(b.ffn, "shared") and b.ffn.shared)
+    cfg = load_config({**TINY_B, "attention_bias": True})
+    assert load_config(cfg.to_dict()).attention_bias is True
+    specs = build_model(cfg).param_specs()
+    q, kv = TINY_B["num_attention_heads"] * TINY_B["head_dim"], TINY_B["num_key_value_heads"] * TINY_B["head_dim"]
+    for l in range(TINY_B["num_hidden_layers"]):
+        p = f"model.layers.{l}.self_attn."
+        assert specs[p + "q_proj.bias"].shape == (q,) and specs[p + "k_proj.bias"].shape == (kv,)
+        assert specs[p + "v_proj.bias"].shape == (kv,) and specs[p + "o_proj.bias"].shape == (TINY_B["hidden_size"],)
 
 
 def test_unknown_text_keys_are_listed_not_refused():

@@ -771,6 +771,50 @@ def test_rope_kv_kernel_pair_layouts_and_partial_width(hd, rotary_dim, layout, d
         assert float((other - _rotate_plain(x[:, :nh], positions, inv, layout)).abs().max()) > 0.1
 
 
+@pytest.mark.parametrize("nh,nkv,hd", [(3, 1, 48), (6, 3, 32), (5, 5, 128)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rope_kv_kernel_adds_the_projections_biases_first(nh, nkv, hd, dtype):
+    """A bias on q, k and v is added to each token's row before anything else (in float): the result
+    is what the kernel gives for rows that already hold the sum, to the rounding of one more store."""
+    ops = _ops()
+    import plain_llama4 as P
+
+    T, ps, pages = 7, 16, 3
+    qkv = _rand(T, (nh + 2 * nkv) * hd, dtype=dtype, seed=hd)
+    bias = _rand((nh + 2 * nkv) * hd, seed=hd + 1)
+    positions = torch.tensor([0, 1, 5, 17, 31, 100, 4095], dtype=torch.int32)
+    slots = torch.tensor([0, 1, 2, 33, 47, 20, 21], dtype=torch.int32)
+    inv = P.rope_inv_freq(hd, 10000.0, None)
+    kc = torch.zeros(pages, nkv, ps, hd, dtype=dtype, device=DEV)
+    vc = torch.zeros(pages, nkv, hd, ps, dtype=dtype, device=DEV)
+    q = ops.rope_kv(qkv, kc, vc, slots.to(DEV), positions.to(DEV), inv.to(DEV), True, 1e-5, None, nh, nkv, hd, bias=bias)
+    x = (qkv.float().cpu() + bias.cpu()).view(T, nh + 2 * nkv, hd)
+    qr = P.l2_head_norm(P.apply_rope_interleaved(x[:, :nh], positions, inv), 1e-5)
+    kr = P.l2_head_norm(P.apply_rope_interleaved(x[:, nh:nh + nkv], positions, inv), 1e-5)
+    vr = x[:, nh + nkv:]
+    tol = 2e-5 if dtype == torch.float32 else 1e-2
+    assert float((q.float().cpu().view(T, nh, hd) - qr).abs().max()) <= tol * max(1.0, float(qr.abs().max()))
+    kcc, vcc = kc.float().cpu(), vc.float().cpu()
+    for t in range(T):
+        page, off = int(slots[t]) // ps, int(slots[t]) % ps
+        assert float((kcc[page, :, off, :] - kr[t]).abs().max()) <= tol * max(1.0, float(kr.abs().max())), t
+        assert float((vcc[page, :, :, off] - vr[t]).abs().max()) <= tol * max(1.0, float(vr.abs().max())), t
+    # without the bias the queries differ (a kernel that ignored the argument fails)
+    q0 = ops.rope_kv(qkv, kc.clone(), vc.clone(), slots.to(DEV), positions.to(DEV), inv.to(DEV), True, 1e-5, None, nh, nkv, hd)
+    assert float((q0.float() - q.float()).abs().max()) > 0.05
+
+
+@pytest.mark.parametrize("T,N", [(1, 5), (9, 76), (130, 512)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_add_bias_rows(T, N, dtype):
+    ops = _ops()
+    x = _rand(T, N, dtype=dtype, seed=T)
+    b = _rand(N, seed=N)
+    want = (x.float() + b).to(dtype)
+    got = ops.add_bias(x.clone(), b)
+    assert torch.equal(got, want)
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 5, 3), (70, 130, 50), (64, 64, 16), (129, 203, 96)])
 def test_gemm_tiled_is_a_true_float_product_and_batch_invariant(M, N, K):
     ops = _ops()

@@ -32,6 +32,9 @@ CASES = {
                         attention_chunk_size=20)),
     "hd256": ("D", dict(hidden_size=128, num_attention_heads=2, num_key_value_heads=2, head_dim=256, vocab_size=499,
                         intermediate_size=128, num_local_experts=3, num_experts_per_tok=2, attention_chunk_size=56)),
+    # the tanh form of GELU in every feed-forward, and biases on the four attention projections
+    "gelu_bias": ("B", dict(hidden_act="gelu_pytorch_tanh", attention_bias=True, vocab_size=384)),
+    "bias_mfma": ("D", dict(attention_bias=True, vocab_size=500)),
     "hd192": ("D", dict(hidden_size=384, num_attention_heads=2, num_key_value_heads=2, head_dim=192, vocab_size=333,
                         intermediate_size=128, num_local_experts=4, num_experts_per_tok=2, attention_chunk_size=40)),
 }

@@ -118,6 +118,55 @@ def test_gate_vectors_and_silu():
     assert int(ids[0, 0]) == 11 and abs(float(w[0, 0]) - 0.3005) < 1e-3
 
 
+def test_gelu_tanh_is_the_library_routine_and_only_chosen_by_name(tmp_path):
+    """reference: src/SharpInference.Cpu/SimdKernels.cs:4474-4484 (the scalar form) and its tests'
+    zero-input case (tests/SharpInference.Tests.ForwardPass/SimdKernelsGemma4Tests.cs:71-90).  The
+    formula is the library's tanh GELU; it differs from SiLU (a swapped activation fails) and from
+    the erf form; a dense feed-forward with it is the library's."""
+    x = torch.linspace(-3, 3, 97)
+    assert torch.allclose(P.gelu_tanh(x), F.gelu(x, approximate="tanh"), atol=1e-6)
+    assert float(P.gelu_tanh(torch.zeros(1))) == 0.0
+    assert float((P.gelu_tanh(x) - P.silu(x)).abs().max()) > 0.1
+    assert float((P.gelu_tanh(x) - F.gelu(x)).abs().max()) > 1e-4
+    assert P.activation_of({}) is P.silu and P.activation_of({"hidden_act": "gelu_pytorch_tanh"}) is P.gelu_tanh
+    with pytest.raises(ValueError):
+        P.activation_of({"hidden_act": "relu"})
+    n, wg, wu, wd = torch.randn(5, 8), torch.randn(12, 8), torch.randn(12, 8), torch.randn(8, 12)
+    want = (F.gelu(n @ wg.T, approximate="tanh") * (n @ wu.T)) @ wd.T
+    assert torch.allclose(P.swiglu(n, wg, wu, wd, act=P.gelu_tanh), want, atol=1e-5)
+
+
+def test_attention_biases_shift_the_projections(tmp_path):
+    """reference: src/SharpInference.Engine/ForwardPass.cs:1605-1613, 893: biases are added right
+    after their products.  Pinned by what a bias must do: zero biases change nothing; a value bias b_v
+    moves every attention output by exactly W_o b_v's share (softmax weights sum to one), i.e. the layer's
+    output by W_o (b_v repeated per query head); an output bias adds itself."""
+    d = make_model_dir(tmp_path, "A", std=0.1, attention_bias=True)
+    c, W = P.read_config(d), {k: v.float() for k, v in P.load_weights(d).items()}
+    assert c["attention_bias"] is True
+    p = "model.layers.1.self_attn."                  # layer 1 of A has no rotary: v's bias passes straight through
+    n = torch.randn(9, c["hidden_size"])
+    pos = torch.arange(9)
+    zero = dict(W)
+    for name in "qkvo":
+        zero[p + f"{name}_proj.bias"] = torch.zeros_like(W[p + f"{name}_proj.bias"])
+    c0 = {**c, "attention_bias": False}
+    base = P.attention_layer(c0, W, 1, n, pos)
+    assert torch.equal(P.attention_layer(c, zero, 1, n, pos), base)
+    only_v = dict(zero)
+    only_v[p + "v_proj.bias"] = W[p + "v_proj.bias"]
+    nh, nkv, hd = c["num_attention_heads"], c["num_key_value_heads"], P.head_dim_of(c)
+    per_head = W[p + "v_proj.bias"].view(nkv, hd).repeat_interleave(nh // nkv, dim=0).reshape(-1)
+    shift = W[p + "o_proj.weight"] @ per_head
+    assert torch.allclose(P.attention_layer(c, only_v, 1, n, pos), base + shift, atol=1e-5)
+    only_o = dict(zero)
+    only_o[p + "o_proj.bias"] = W[p + "o_proj.bias"]
+    assert torch.allclose(P.attention_layer(c, only_o, 1, n, pos), base + W[p + "o_proj.bias"], atol=1e-6)
+    only_q = dict(zero)
+    only_q[p + "q_proj.bias"] = W[p + "q_proj.bias"] * 30
+    assert not torch.allclose(P.attention_layer(c, only_q, 1, n, pos), base, atol=1e-3)
+
+
 def test_router_ties_and_topk_order():
     n = torch.randn(3, 8)
     ids, w = P.router_topk(n, torch.zeros(5, 8), 2)       # all gates 0.5: lowest indices win
