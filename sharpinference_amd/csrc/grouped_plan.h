@@ -10,8 +10,13 @@
 // and every XCD walks its units one after the other; inside a unit the siblings of one column
 // block are neighbours.  Blocks go to XCDs round-robin by their linear id, so block b is slot
 // b / 8 of XCD b % 8: sibling blocks start together on one XCD and stream the same weight rows at
-// the same pace, and what the first fetches from memory the others find in that XCD's L2.  No
-// block is launched for a sibling that does not exist, except behind an XCD's last unit.
+// the same pace, and what the first fetches from memory the others find in that XCD's L2.
+//
+// The product's blocks stay on their compute units and take slots until none is left: the slots
+// of an XCD's walk are handed out in order by a ticket counter that lies behind the unit lists,
+// first to the blocks of that XCD (block b sits on XCD b % 8), then to blocks of other XCDs that
+// have run out of their own.  So an uneven load is levelled at run time, while the first round of
+// slots, the heaviest units, starts as the plan lays it out.
 //
 // plan (int32), per XCD x at plan + x * plan_stride(G), G groups:
 //   [0]                      units of this XCD
@@ -19,7 +24,7 @@
 #pragma once
 
 constexpr int kPlanXcds = 8;
-constexpr int kPlanTileRows = 192;
+constexpr int kPlanTileRows = 128;
 constexpr int kPlanMaxParts = 16;
 
 __host__ __device__ inline int plan_siblings(int rows) { return (rows + kPlanTileRows - 1) / kPlanTileRows; }
@@ -32,7 +37,12 @@ __host__ __device__ inline int plan_weight(int n_sib) { return n_sib * (kPlanMax
 __host__ __device__ inline int plan_part_first(int part, int parts, int nb) { return (int)((long long)part * nb / parts); }
 __host__ __device__ inline int plan_units_per_xcd_max(int n_groups) { return (kPlanMaxParts * n_groups + kPlanXcds - 1) / kPlanXcds + 1; }
 __host__ __device__ inline int plan_stride(int n_groups) { return 1 + 4 * plan_units_per_xcd_max(n_groups); }
-__host__ __device__ inline int plan_ints(int n_groups) { return kPlanXcds * plan_stride(n_groups); }
+// behind the XCDs' unit lists: one ticket counter per XCD (the next slot of that XCD's walk to hand
+// out) and a count of the blocks that have left; the routing kernel zeroes them with the plan, and
+// the last block of a product to leave zeroes them again for the next product that reads the plan
+constexpr int kPlanCounters = 16;
+__host__ __device__ inline int plan_ints(int n_groups) { return kPlanXcds * plan_stride(n_groups) + kPlanCounters; }
+__host__ __device__ inline int plan_counters_at(int n_groups) { return kPlanXcds * plan_stride(n_groups); }
 // Slots (blocks) an XCD may have to walk, from what the host knows: n_rows rows over n_groups
 // groups, nb column blocks.  Siblings in all: at most ceil(n_rows / tile) + n_groups; an XCD gets
 // an eighth of the (sibling x column block) pairs, give or take one unit.

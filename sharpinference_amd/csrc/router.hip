@@ -339,6 +339,7 @@ __device__ void permute_block(const int* __restrict__ topk_ids, const float* __r
       }
       plan[x * stride] = n;
     }
+    if (threadIdx.x < kPlanCounters) plan[plan_counters_at(n_groups) + threadIdx.x] = 0;
   }
   __syncthreads();
   for (int i = threadIdx.x; i < n_pairs; i += blockDim.x) {

@@ -774,10 +774,13 @@ def route(x: torch.Tensor, wr: torch.Tensor, k: int, gate: int = GATE_SIGMOID, r
     return ids, wts, moe_permute(ids, wts, wr.shape[0], shared_group)
 
 
-def gemm_grouped(x: torch.Tensor, w, rt: Routing, gather: bool, out_dtype: torch.dtype) -> torch.Tensor:
+def gemm_grouped(x: torch.Tensor, w, rt: Routing, gather: bool, out_dtype: torch.dtype, max_blocks: int = 0) -> torch.Tensor:
     """Per-group products for many rows on the matrix cores (bfloat16): the experts, and the
     always-on group if the routing has one (group E of w).  gather: x rows are read through the
-    routing's token list; otherwise x is already in expert-sorted order."""
+    routing's token list; otherwise x is already in expert-sorted order.  The product's blocks
+    stay on their compute units until the work is done; ``max_blocks`` > 0 bounds their number
+    (the units left over are for other work running beside the product).  Products that read
+    one routing must not run at the same time (they share its plan's ticket counters)."""
     w, packed = _unwrap(w)
     _dev(x, w)
     _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_grouped: bfloat16 operands only")
@@ -789,12 +792,12 @@ def gemm_grouped(x: torch.Tensor, w, rt: Routing, gather: bool, out_dtype: torch
     out = torch.empty(rt.n_rows, N, dtype=out_dtype, device=x.device)
     _run("sharpi_gemm_grouped", _ptr(x), x.shape[0], _ptr(w), _ptr(out), _code(out_dtype), rt.n_rows, N, K,
          _ptr(rt.sorted_token) if gather else None, _ptr(rt.offsets), _ptr(rt.plan), rt.n_groups,
-         1 if packed else 0, _stream())
+         1 if packed else 0, int(max_blocks), _stream())
     return out
 
 
 def gemm_grouped_swiglu(x: torch.Tensor, w, rt: Routing, scale: Optional[torch.Tensor], gather: bool = True,
-                        act: int = ACT_SILU) -> torch.Tensor:
+                        act: int = ACT_SILU, max_blocks: int = 0) -> torch.Tensor:
     """Per group, act(s g) * (s u) with (g | u) = x @ w[e]^T rounded to bfloat16, for many rows: the
     grouped product with the activation (ACT_SILU, ACT_GELU_TANH) in its epilogue.  gather: x rows are read through the
     routing's token list (the order inside a group is whatever the routing kernel made it);
@@ -813,7 +816,7 @@ def gemm_grouped_swiglu(x: torch.Tensor, w, rt: Routing, scale: Optional[torch.T
     out = torch.empty(rt.n_rows, N // 2, dtype=torch.bfloat16, device=x.device)
     _run("sharpi_gemm_grouped_swiglu", _ptr(x), x.shape[0], _ptr(w), _ptr(out), rt.n_rows, N, K,
          _ptr(rt.sorted_token) if gather else None, _ptr(rt.offsets), _ptr(rt.plan), rt.n_groups, _ptr(scale), 1 if packed else 0,
-         int(act), _stream())
+         int(act), int(max_blocks), _stream())
     return out
 
 
@@ -921,7 +924,7 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, gro
 
 
 def grouped_swiglu(x: torch.Tensor, w_gate_up, rt: Routing, out_dtype: torch.dtype, scaled: bool = True,
-                   act: int = ACT_SILU) -> torch.Tensor:
+                   act: int = ACT_SILU, max_blocks: int = 0) -> torch.Tensor:
     """The experts' gate|up products of the routed tokens and their activation,
     act(s g) * (s u) with s the pick's weight (``scaled``; otherwise s = 1): [n_rows, I] in
     expert-sorted order.  On the matrix cores the activation is the product's epilogue (the
@@ -933,11 +936,11 @@ def grouped_swiglu(x: torch.Tensor, w_gate_up, rt: Routing, out_dtype: torch.dty
             return gemm_skinny_swiglu(x, w_gate_up, rt.offsets, rt.sorted_token, rt.n_rows, scale,
                                       group_rows=rt.n_tokens, act=act)
         if rt.n_tokens > SKINNY_MAX_ROWS and N % 32 == 0:
-            return gemm_grouped_swiglu(x, w_gate_up, rt, scale, act=act)
+            return gemm_grouped_swiglu(x, w_gate_up, rt, scale, act=act, max_blocks=max_blocks)
     return gated_act(grouped_linear(x, w_gate_up, rt, True, out_dtype), scale, act)
 
 
-def grouped_linear(x: torch.Tensor, w, rt: Routing, gather: bool, out_dtype: torch.dtype) -> torch.Tensor:
+def grouped_linear(x: torch.Tensor, w, rt: Routing, gather: bool, out_dtype: torch.dtype, max_blocks: int = 0) -> torch.Tensor:
     """Per-expert products over the routing's expert-sorted row list: w [E, N, K] (a tensor or a
     PackedWeight); x rows are read through the token list (gather) or are already in sorted order.
     Returns [n_rows, N]."""
@@ -949,7 +952,7 @@ def grouped_linear(x: torch.Tensor, w, rt: Routing, gather: bool, out_dtype: tor
         if rt.n_tokens <= SKINNY_MAX_ROWS:   # no expert has more rows than there are tokens
             return gemm_skinny(x, w, out_dtype, a_rows=a_rows, offsets=rt.offsets, n_rows=rt.n_rows,
                                group_rows=rt.n_tokens)
-        return gemm_grouped(x, w, rt, gather, out_dtype)
+        return gemm_grouped(x, w, rt, gather, out_dtype, max_blocks=max_blocks)
     y = grouped_gemm(x, w, rt.offsets, a_rows, rt.n_rows)
     return y if y.dtype == out_dtype else cast(y, out_dtype)
 

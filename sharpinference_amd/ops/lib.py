@@ -37,8 +37,8 @@ _SIGNATURES = {
     "sharpi_add_rmsnorm_router": [P, P, P, I, P, I, I, F, P, I, P, P, I, I, I, I, P],
     "sharpi_router_topk": [P, I, P, I, P, P, P, I, I, I, I, I, I, P],
     "sharpi_moe_permute": [P, P, P, P, P, P, P, I, I, I, I, I, P],
-    "sharpi_gemm_grouped": [P, I, P, P, I, I, I, I, P, P, P, I, I, P],
-    "sharpi_gemm_grouped_swiglu": [P, I, P, P, I, I, I, P, P, P, I, P, I, I, P],
+    "sharpi_gemm_grouped": [P, I, P, P, I, I, I, I, P, P, P, I, I, I, P],
+    "sharpi_gemm_grouped_swiglu": [P, I, P, P, I, I, I, P, P, P, I, P, I, I, I, P],
     "sharpi_argmax_rows": [P, P, I, I, P],
     "sharpi_sample_rows": [P, P, P, P, P, P, P, P, I, I, P],
     "sharpi_edit_logits": [P, P, P, P, P, P, P, P, I, I, P],

@@ -354,15 +354,16 @@ def test_router_and_permute(T, E, k, H, dtype):
 
 def _check_plan(ops, rt, counts):
     """The plan of the grouped product for many rows: every group with rows is cut into sibling
-    row tiles (as few of at most 192 rows as hold its rows) and its column blocks into parts (2,
-    4, 8 or 16: more the more siblings); every (group, part) unit appears once, on one of the 8
-    XCDs, the heaviest units dealt first so that the XCDs' loads stay level."""
+    row tiles (as few of the library's tile height as hold its rows) and its column blocks into
+    parts (2, 4, 8 or 16: more the more siblings); every (group, part) unit appears once, on one of
+    the 8 XCDs, the heaviest units dealt first so that the XCDs' loads stay level.  Behind the
+    units lie the ticket counters of the product's blocks, zero when the plan is made."""
     G = len(counts)
     tile = ops._lib.grouped_tile_rows()
     plan = rt.plan.cpu().tolist()
     per_xcd = (16 * G + 7) // 8 + 1
     stride = 1 + 4 * per_xcd
-    assert len(plan) == 8 * stride
+    assert len(plan) == 8 * stride + 16 and plan[8 * stride:] == [0] * 16
 
     def parts_of(sibs):
         return 2 if sibs <= 2 else 4 if sibs <= 4 else 8 if sibs <= 8 else 16
@@ -584,6 +585,42 @@ def test_gemm_grouped_swiglu_equals_product_then_activation(T, E, k, I, K):
     ga, up = (gu[:, :I] * s), (gu[:, I:] * s)
     ref = ga / (1 + torch.exp(-ga)) * up
     assert float((ops.gemm_grouped_swiglu(x, w, rt, rt.sorted_w).float().cpu() - ref).abs().max()) <= 3e-2 * float(ref.abs().max() + 1e-6)
+
+
+@pytest.mark.parametrize("T,E,N,K", [(900, 6, 1024, 256), (2100, 16, 2560, 128), (70, 3, 48, 128)])
+def test_gemm_grouped_gives_the_same_bits_however_many_blocks_take_the_work(T, E, N, K):
+    """The many-rows product's blocks stay and take slots from ticket counters that lie behind the
+    plan; the slots of a last, partly filled round are cut by columns.  Every output is one chain
+    over k whoever computes it: any bound on the number of blocks gives the same bits (a single
+    block walks every XCD's slots alone, cut otherwise than 256 blocks cut them), the counters are
+    back at zero after every launch, and the loads are very uneven on purpose."""
+    ops = _ops()
+    x = _rand(T, K, dtype=torch.bfloat16, seed=5)
+    w = _rand(E, N, K, dtype=torch.bfloat16, scale=0.1, seed=6)
+    g = torch.Generator().manual_seed(T)
+    p = torch.tensor([float(2 ** (e % 5)) for e in range(E)])
+    ids = torch.multinomial(p / p.sum(), T, replacement=True, generator=g).to(torch.int32).view(T, 1).to(DEV)
+    rt = ops.moe_permute(ids, torch.ones(T, 1, device=DEV), E)
+    counters = rt.plan[-16:]
+    want = None
+    for form in (w, ops.pack_weight(w, keep_rows=False)):
+        for blocks in (0, 1, 3, 8, 37, 100):
+            got = ops.gemm_grouped(x, form, rt, True, torch.bfloat16, max_blocks=blocks)
+            assert not bool(counters.any()), "the ticket counters were not set back"
+            if want is None:
+                want = got
+                off = rt.offsets.cpu().tolist()
+                st = rt.sorted_token.cpu().long()
+                for e in range(E):
+                    rows = st[off[e]:off[e + 1]]
+                    ref = x.cpu().float()[rows] @ w[e].cpu().float().T
+                    assert float((got[off[e]:off[e + 1]].cpu().float() - ref).abs().max()) <= 2e-2 * float(ref.abs().max() + 1e-6), e
+            assert torch.equal(got, want), blocks
+    if N % 32 == 0:
+        want = ops.gemm_grouped_swiglu(x, w, rt, rt.sorted_w)
+        for blocks in (1, 5, 64):
+            assert torch.equal(ops.gemm_grouped_swiglu(x, w, rt, rt.sorted_w, max_blocks=blocks), want), blocks
+        assert not bool(counters.any())
 
 
 _PREFILL_CASES = [(nh, nkv, hd, kind, window, ps)
