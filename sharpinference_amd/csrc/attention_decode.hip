@@ -227,8 +227,11 @@ __global__ __launch_bounds__(kMergeThreads) void attn_decode_merge_kernel(
   int start = 0;
   if (window_kind == 1) start = (p / window) * window;
   else if (window_kind == 2) start = p - window + 1 > 0 ? p - window + 1 : 0;
-  // (never beyond the runs the workspace holds, whatever the caller's bound was)
-  const int n_runs = min(((p >> 4) - (start >> 4)) / kSplitBlocks + 1, max_splits);
+  // Never beyond the runs the workspace holds, whatever the caller's bound was; but a bound too
+  // small for this token (its nearest keys would be dropped without a trace) gives a row of NaN,
+  // which no caller can take for attention.
+  const int runs_wanted = ((p >> 4) - (start >> 4)) / kSplitBlocks + 1;
+  const int n_runs = min(runs_wanted, max_splits);
   const size_t base = ((size_t)li * nh + h) * max_splits;
 
   float M = -INFINITY;
@@ -266,7 +269,7 @@ __global__ __launch_bounds__(kMergeThreads) void attn_decode_merge_kernel(
   }
   unsigned short b[4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) b[i] = f32_to_bf16(L > 0.f ? o[i] / L : 0.f).bits;
+  for (int i = 0; i < 4; ++i) b[i] = runs_wanted > max_splits ? (unsigned short)0x7fc0 : f32_to_bf16(L > 0.f ? o[i] / L : 0.f).bits;
   uint2 pk;
   pk.x = b[0] | ((unsigned)b[1] << 16);
   pk.y = b[2] | ((unsigned)b[3] << 16);
@@ -295,7 +298,10 @@ static int launch_decode(const void* q, const void* k_cache, const void* v_cache
 // q [T, nh, hd] bf16; caches K [pages, nkv, page_size, hd], V [pages, nkv, hd, page_size] bf16;
 // token_list [n_list] (or null: tokens 0..n_list-1); part_o float [n_list, nh, max_splits, hd];
 // part_ml float [n_list, nh, max_splits, 2]; out [T, nh, hd] bf16 (rows of the listed tokens).
-// max_splits must cover every listed token: ceil over 256-key runs of its visible keys.
+// max_splits must cover every listed token: ((position >> 4) - (first visible key >> 4)) / 16 + 1
+// runs of 256 keys (runs are aligned to absolute positions, so a window that starts inside a run
+// takes one more than its length suggests); ((context - 1) >> 4) / 16 + 1 covers every window of a
+// context.  A token whose runs exceed max_splits gets a row of NaN.
 SHARPI_EXPORT int sharpi_attention_decode(const void* q, const void* k_cache, const void* v_cache,
                                           const int* block_table, const int* entry_of_token, const int* positions,
                                           const int* token_list, float* part_o, float* part_ml, void* out,

@@ -20,6 +20,11 @@ extern "C" {
 // partial results would not fit SHARPI_NOALLOC_SCRATCH_FLOATS.  Calls no hipMalloc / hipFree and
 // no allocating library routine; the caller passes inputs and the output as before.
 //
+// max_splits bounds the 256-key runs of a token: a token at position p whose first visible key is
+// s needs ((p >> 4) - (s >> 4)) / 16 + 1 of them, and ((context - 1) >> 4) / 16 + 1 covers every
+// token of a context whatever its window; a token that needs more than max_splits gets a row of
+// NaN in `out` (never attention over fewer keys than it sees).
+//
 // The first call on a device looks up that device's copy of the array (hipGetSymbolAddress):
 // make it outside a graph capture.  All calls on one GPU share that GPU's array, which keeps
 // the last call's contents; nothing in it has to start at zero (every run that the merge reads

@@ -281,6 +281,13 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
 DECODE_RUN_KEYS = _lib.DECODE_RUN_KEYS   # keys per block of the decode kernel (fixed: sums must not depend on the batch)
 
 
+def decode_max_splits(max_context: int) -> int:
+    """Runs of DECODE_RUN_KEYS keys that cover every token of a context of `max_context` tokens,
+    whatever its window: runs are aligned to absolute positions, so a token at position p whose
+    first visible key is s takes ((p >> 4) - (s >> 4)) // 16 + 1 of them, most for s = 0."""
+    return ((max(1, int(max_context)) - 1) >> 4) // (DECODE_RUN_KEYS // 16) + 1
+
+
 def decode_attention_ok(dtype: torch.dtype, hd: int) -> bool:
     return dtype == torch.bfloat16 and _lib.attention_takes("decode", hd)
 
@@ -306,7 +313,7 @@ def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     if out is None:
         out = torch.empty_like(q)
     _need(out.shape == q.shape and out.dtype == q.dtype, "attention_decode: out must match q")
-    max_splits = ((max(1, int(max_context)) - 1) >> 4) // (DECODE_RUN_KEYS // 16) + 1
+    max_splits = decode_max_splits(max_context)
     part_o = torch.empty(n_list * nh * max_splits * hd, dtype=torch.float32, device=q.device)
     part_ml = torch.empty(n_list * nh * max_splits * 2, dtype=torch.float32, device=q.device)
     _run("sharpi_attention_decode", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), _ptr(entry_of_token),

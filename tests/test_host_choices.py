@@ -25,6 +25,32 @@ def test_few_rows_launch_shapes_follow_the_rows_and_the_compute_units():
     assert ops.skinny_plan(16384, 5120, 4, 17)[0] == 4 and ops.skinny_plan(5120, 8192, 4, 17)[0] == 2
 
 
+def test_the_decode_attention_s_runs_cover_every_window():
+    """The decode attention cuts a token's visible keys into runs of 256, counted from the 16-key
+    block that holds the first visible key, and sizes its workspace for a bound on the contexts.
+    The bound's runs cover every token below it: all keys, chunks, and sliding windows that start
+    inside a 16-key block (a window of 257 keys that starts at key 15 spans two runs)."""
+    from sharpinference_amd import ops
+    from sharpinference_amd.cache.spec import KVSpec, WINDOW_CHUNK, WINDOW_NONE, WINDOW_SLIDING
+
+    run = ops.DECODE_RUN_KEYS
+    assert run % 16 == 0
+    specs = [KVSpec(1, 16, WINDOW_NONE, 0)] + [KVSpec(1, 16, kind, w) for kind in (WINDOW_CHUNK, WINDOW_SLIDING)
+                                                for w in (1, 17, 24, 250, 256, 300, 1000, 4099)]
+    for context in (1, 15, 16, 17, 255, 256, 257, 511, 513, 4096, 4097, 9000):
+        bound = ops.decode_max_splits(context)
+        assert bound == (context - 1) // run + 1            # the runs a context spans from key 0
+        for spec in specs:
+            for p in {0, context // 3, context - 2, context - 1} - {-1}:
+                if p < 0:
+                    continue
+                s = spec.first_visible(p)
+                wanted = ((p >> 4) - (s >> 4)) // (run // 16) + 1     # what the kernels walk (attention_decode.hip)
+                assert (s >> 4) * 16 + wanted * run > p               # ... reaches the token's own key
+                assert (s >> 4) * 16 + (wanted - 1) * run <= p        # ... with no run to spare
+                assert wanted <= bound, (context, spec, p)
+
+
 def test_benchmark_refuses_more_than_one_gpu():
     out = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
     assert out.returncode == 2

@@ -77,6 +77,22 @@ def test_decode_attention_without_allocation_equals_the_workspace_form():
         assert torch.equal(a, b)
 
 
+def test_a_bound_on_the_runs_that_is_too_small_shows_as_nan_not_as_wrong_attention():
+    """A caller of either entry point that passes fewer runs than a token's keys span would lose
+    the keys nearest the query: such a token's row comes back as NaN, the others' rows as they are."""
+    from sharpinference_amd.ops import lib as kernel_lib
+
+    lib = kernel_lib.load()
+    c = _case(4, n_tokens=3, nh=10, nkv=2, hd=128, page_size=16, contexts=[200, 700, 256])
+    good_old, good_new = _both(lib, c)
+    assert torch.equal(good_old, good_new) and torch.isfinite(good_old.float()).all()
+    c["splits"] = 1                       # enough for 256 keys: tokens 0 and 2, not token 1
+    bad_old, bad_new = _both(lib, c)
+    for bad in (bad_old, bad_new):
+        assert torch.isnan(bad[1].float()).all()
+        assert torch.equal(bad[0], good_old[0]) and torch.equal(bad[2], good_old[2])
+
+
 def test_sizes_beyond_the_scratch_array_are_refused():
     from sharpinference_amd.ops import lib as kernel_lib
 
