@@ -116,12 +116,14 @@ def prefill_flops(cfg, T: int, layers: int) -> float:
     return 2.0 * T * lin + attn + 2.0 * cfg.vocab_size * H                 # one row through the head
 
 
-def prefill_bytes(cfg, layers: int) -> float:
-    """Weights a prompt of thousands of tokens has to read once: every expert of every routed layer."""
+def prefill_bytes(cfg, layers: int, experts_used=None) -> float:
+    """Weights a prompt of thousands of tokens has to read once: every expert of every routed layer
+    (or `experts_used` of them a layer, where a prompt does not reach them all)."""
     b = layer_bytes(cfg)
     total = b["head"]
+    used = cfg.num_local_experts if experts_used is None else experts_used
     for l in range(layers):
-        total += b["attn"] + b["norms"] + (b["router"] + b["expert"] * (1 + cfg.num_local_experts) if cfg.is_moe_layer(l) else b["dense"])
+        total += b["attn"] + b["norms"] + (b["router"] + b["expert"] * (1 + used) if cfg.is_moe_layer(l) else b["dense"])
     return total
 
 
@@ -132,7 +134,10 @@ def run_prefill(eng, rid, prompt):
     eng.add_request(rid)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    logits = eng.step([StepEntry(rid, prompt, (len(prompt) - 1,))])
+    logits = None
+    for o in range(0, len(prompt), eng.max_tokens_per_step):     # a prompt longer than a step goes in portions
+        part = prompt[o:o + eng.max_tokens_per_step]
+        logits = eng.step([StepEntry(rid, part, (len(part) - 1,) if o + len(part) == len(prompt) else ())])
     torch.cuda.synchronize()
     return time.perf_counter() - t0, logits
 
@@ -155,7 +160,12 @@ def decode_run(eng, batch: int, steps: int, warmup: int, rng: random.Random, cou
         for r in group:
             eng.add_request(r)
         prompts = [[rng.randrange(vocab) for _ in range(prompt_len)] for _ in group]
-        lg = eng.step([StepEntry(r, p, (prompt_len - 1,)) for r, p in zip(group, prompts)])
+        if prompt_len <= eng.max_tokens_per_step:
+            lg = eng.step([StepEntry(r, p, (prompt_len - 1,)) for r, p in zip(group, prompts)])
+        else:                                                # one prompt at a time, in portions of a step
+            for o in range(0, prompt_len, eng.max_tokens_per_step):
+                part = prompts[0][o:o + eng.max_tokens_per_step]
+                lg = eng.step([StepEntry(group[0], part, (len(part) - 1,) if o + len(part) == prompt_len else ())])
         last += ops.argmax_rows(lg).cpu().tolist()
         log(f"  prefilled {min(i + per_step, batch)}/{batch}")
 
@@ -236,6 +246,92 @@ def profile_report(eng, batch: int, prompt_len: int, rng: random.Random) -> None
         eng.free_request(r)
 
 
+def host_report(eng, prompt_len: int, rng: random.Random, batch: int = 64) -> dict:
+    """What the host does in steps where nothing hides it (no steps launched on end, no choice on
+    the device): a sampled batch (temperature alone; with top-k / top-p / min-p; with the window
+    penalties) and a mixed step (one prompt-sized portion beside the others' decode tokens).
+    Per case: milliseconds inside `Engine.step` (index arrays, launches), milliseconds of the
+    sampler on an idle GPU (packing the rows' settings, two copies, the kernels, the read-back),
+    and the wall time of a whole step.  stderr, and returned for the JSON line."""
+    import torch
+    from sharpinference_amd import SamplingParams
+    from sharpinference_amd.engine import StepEntry
+    from sharpinference_amd.sampling.sampler import penalty_window
+
+    vocab = eng.config.vocab_size
+    batch = min(batch, eng.max_num_seqs)
+    ids = [f"host{i}" for i in range(batch)]
+    history = {}
+    per_step = max(1, eng.max_tokens_per_step // prompt_len)
+    for i in range(0, batch, per_step):
+        group = ids[i:i + per_step]
+        entries = []
+        for r in group:
+            eng.add_request(r)
+            history[r] = [rng.randrange(vocab) for _ in range(prompt_len)]
+            entries.append(StepEntry(r, history[r], ()))
+        eng.step(entries)
+    cases = {
+        "temperature": SamplingParams(temperature=0.8, top_k=0, top_p=1.0, min_p=0.0),
+        "filters": SamplingParams(temperature=0.8, top_k=40, top_p=0.95, min_p=0.05),
+        "penalties": SamplingParams(temperature=0.8, top_k=40, top_p=0.95, min_p=0.05, repetition_penalty=1.1,
+                                    frequency_penalty=0.1, presence_penalty=0.1, penalty_last_n=64),
+    }
+    out = {}
+    tokens = [rng.randrange(vocab) for _ in ids]
+    for name, sp in cases.items():
+        params = [SamplingParams(**{**sp.__dict__, "seed": 100 + i}) for i in range(batch)]
+        t_step = t_sample = t_wall = 0.0
+        n = 6
+        for it in range(n + 2):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            logits = eng.step([StepEntry(r, (t,), (0,)) for r, t in zip(ids, tokens)])
+            t1 = time.perf_counter()
+            hist = [penalty_window(p, history[r][:prompt_len], history[r][prompt_len:]) if p.edits_logits else ()
+                    for p, r in zip(params, ids)]
+            torch.cuda.synchronize()
+            t2 = time.perf_counter()
+            tokens = eng.sampler.sample(logits, params, [it] * batch, hist)
+            t3 = time.perf_counter()
+            for r, t in zip(ids, tokens):
+                history[r].append(t)
+            if it >= 2:
+                t_step += t1 - t0
+                t_sample += t3 - t2
+                t_wall += t3 - t0
+        out[name] = {"step_host_ms": t_step / n * 1e3, "sampler_ms": t_sample / n * 1e3, "step_ms": t_wall / n * 1e3}
+        log(f"host, {batch} sampled rows ({name}): {out[name]['step_host_ms']:.2f} ms inside the step function, "
+            f"{out[name]['sampler_ms']:.2f} ms in the sampler, of a step of {out[name]['step_ms']:.2f} ms")
+    # a mixed step: one request leaves, a new prompt's portion comes in beside the others' decode tokens
+    eng.free_request(ids[-1])
+    portion = min(prompt_len, eng.max_tokens_per_step - (batch - 1))
+    t_step = t_wall = 0.0
+    n = 3
+    for it in range(n + 1):
+        rid = f"hostmix{it}"
+        eng.add_request(rid)
+        entries = [StepEntry(r, (t,), (0,)) for r, t in zip(ids[:-1], tokens[:-1])]
+        entries.append(StepEntry(rid, [rng.randrange(vocab) for _ in range(portion)], (portion - 1,)))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        picked = eng.step(entries, select="argmax")
+        t1 = time.perf_counter()
+        tokens = picked.cpu().tolist()[:batch - 1] + [0]
+        t2 = time.perf_counter()
+        eng.free_request(rid)
+        if it >= 1:
+            t_step += t1 - t0
+            t_wall += t2 - t0
+    out["mixed"] = {"step_host_ms": t_step / n * 1e3, "step_ms": t_wall / n * 1e3, "portion_tokens": portion,
+                    "decode_tokens": batch - 1}
+    log(f"host, mixed step ({portion} prompt tokens beside {batch - 1} decode tokens): {out['mixed']['step_host_ms']:.2f} ms "
+        f"inside the step function (launches run ahead of the GPU), of a step of {out['mixed']['step_ms']:.2f} ms")
+    for r in ids[:-1]:
+        eng.free_request(r)
+    return out
+
+
 def run_maverick8(args) -> int:
     """Eight Maverick-shaped layers: dense feed-forward (16,384) alternating with 128 experts
     top-1 + shared, no rotary scaling, no QK norm; router weights drawn so that router logits are
@@ -278,7 +374,9 @@ def run_maverick8(args) -> int:
                       "expert_ffn": cfg.intermediate_size, "dense_ffn": cfg.intermediate_size_mlp, "vocab": cfg.vocab_size,
                       "prompt_len": P, "generated": steps + warm, "page_size": args.page_size},
            "prefill": {"value": P / pre_s, "tokens": P, "ms": pre_s * 1e3,
-                       "frac": prefill_flops(cfg, P, layers) / pre_s / (PEAK_DENSE_TFLOPS["bf16"] * 1e12)},
+                       "frac": prefill_flops(cfg, P, layers) / pre_s / (PEAK_DENSE_TFLOPS["bf16"] * 1e12),
+                       # with 8 tokens an expert the prompt is a stream of the weights it touches
+                       "hbm_frac": prefill_bytes(cfg, layers, experts_used=len(hist) - hist.count(0)) / pre_s / 1e9 / PEAK_HBM_GBS},
            "roofline": {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": achieved / PEAK_HBM_GBS},
            "expert_load": {"min": min(hist), "median": sorted(hist)[len(hist) // 2], "max": max(hist), "unused": hist.count(0),
                            "distinct_per_decode_step": distinct}}
@@ -435,8 +533,10 @@ def main() -> int:
             log(f"decode b{pb}: {pdt / k * 1e3:.2f} ms/step ({phost:.2f} ms on the host), "
                 f"{points[f'decode_b{pb}']:.1f} tok/s, {gbs:.0f} GB/s "
                 f"({gbs / PEAK_HBM_GBS:.3f} of the roofline; {pdist:.2f} experts per layer)")
+    host_cases = None
     if args.profile:
         profile_report(eng, args.batch, P, rng)
+        host_cases = host_report(eng, P, rng, batch=max_batch)
 
     out = {
         "metric": f"decode tok/s at batch {args.batch} (Scout-shaped, {P:,}-token prompts)",
@@ -463,6 +563,8 @@ def main() -> int:
         "host_ms_per_step": host_ms,
         "points_host_ms_per_step": points_host,
     }
+    if host_cases is not None:
+        out["host_unhidden"] = {k: {a: round(b, 3) for a, b in v.items()} for k, v in host_cases.items()}
     if measured is not None:
         out["measured_peaks"] = {"hbm_gbs": measured["hbm_gbs"], "bf16_tflops": measured["bf16_tflops"],
                                  "roofline_frac_of_measured": achieved / measured["hbm_gbs"]}

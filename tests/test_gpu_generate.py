@@ -107,6 +107,49 @@ def test_temperature_generation_matches_plain(tmp_path):
     assert len({tuple(w) for w in want}) == 4
 
 
+@pytest.mark.parametrize("which,std", [("B", 0.1), ("D", 0.06)])
+def test_temperature_generation_in_bfloat16_token_for_token(tmp_path, which, std):
+    """Sampled generation in bfloat16 (temperature 0.8, fixed seeds) through the entry point, then
+    every drawn token twice over.  (1) The draw itself: the plain sampling function on the ENGINE's
+    own logits of that step (the generation's steps replayed through the step function) and the
+    same uniform u gives the same token.  (2) The logits behind it: against the plain implementation
+    with bfloat16 storage and the engine's own routes, fed the engine's tokens, u must lie in the
+    token's interval of the plain cumulative distribution, widened by what the bound on a bfloat16
+    logit allows (logits off by at most d move every probability by a factor within
+    exp(+-2 d / T), and so any cumulative sum by at most exp(2 d / T) - 1).  With distributions as
+    flat as a random model's, a shift of a thousandth already moves u into a neighbour's interval,
+    so the plain implementation's own draw is the same token for most steps, not for all."""
+    d = make_model_dir(tmp_path, which, std=std)
+    vocab = CONFIGS[which]["vocab_size"]
+    tol_max, _ = H.bounds_of(d)
+    n_new, temp = 24, 0.8
+    same = total = 0
+    for i, (n, seed) in enumerate(((6, 21), (30, 22), (50, 23))):
+        prompt = H.random_tokens(n, vocab, 80 + i)
+        eng = H.make_engine(d, "bfloat16", kv_tokens=256, max_num_seqs=2, max_tokens_per_step=64)
+        out = eng.generate([prompt], max_new_tokens=n_new, temperature=temp, seeds=[seed])[0].token_ids
+        assert len(out) == n_new
+        toks = prompt + out[:-1]
+        got, picks, seen = H.run_cut(eng, "g", toks, [n] + [1] * (n_new - 1), with_routes=True)
+        H.assert_routes_are_the_best(d, picks, seen, f"{which} sampled generation {i}")
+        ref = H.plain_logits_routed(d, toks, dict(zip(H.moe_layers_of(d), picks)))[n - 1:]
+        us = P.uniform_stream(seed, n_new)
+        own = [P.sample(got[n - 1 + j], us[j], temp) for j in range(n_new)]
+        assert sum(a != b for a, b in zip(own, out)) <= 1, f"{which} prompt {i}: the tokens drawn are not the draws from the engine's own logits: {out} vs {own}"
+        for j, tok in enumerate(out):
+            total += 1
+            if P.sample(ref[j], us[j], temp) == tok:
+                same += 1
+                continue
+            rms = float(ref[j].double().pow(2).mean().sqrt())
+            slack = math.expm1(2.0 * tol_max * rms / temp)
+            cdf = torch.cumsum(P.softmax_f32(ref[j].float() * (1.0 / temp)).double(), 0)
+            lo = float(cdf[tok - 1]) if tok > 0 else 0.0
+            assert lo - slack <= us[j] <= float(cdf[tok]) + slack, \
+                f"{which} prompt {i} step {j}: token {tok} drawn at u = {us[j]:.4f}, its plain interval is [{lo:.4f}, {float(cdf[tok]):.4f}] (slack {slack:.4f})"
+    assert same >= total * 3 // 4, f"only {same} of {total} sampled tokens are the plain implementation's own draw"
+
+
 def test_stop_tokens_and_tiny_pool(tmp_path):
     d = make_model_dir(tmp_path, "A", std=0.1)
     c, W = P.read_config(d), P.load_weights(d)

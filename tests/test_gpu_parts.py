@@ -653,6 +653,16 @@ def test_a_stateful_mixer_that_can_be_captured_decodes_from_graphs(graphs):
         assert eng.runner.graph_replays == (10 if graphs else 0)
         whole_a, whole_b = H.run_cut(eng, "wa", a, [30]), H.run_cut(eng, "wb", b, [22])
         assert float((got["a"] - whole_a[19:]).abs().max()) <= 1e-5 and float((got["b"] - whole_b[11:]).abs().max()) <= 1e-5
-        assert float(eng.cache.state[0][:3].abs().max()) >= 0       # (the slots of requests; the scratch slot is the last)
+        # A capture's trial run works on the slot behind the requests' own (it is the only one a
+        # trial may change); requests have left their state in their slots, and the next request
+        # that takes a slot finds it zeroed.
+        scratch = eng.cache.scratch_state_slot
+        assert scratch == 3 and eng.cache.state[0].shape[0] == 4
+        assert bool(eng.cache.state[0][scratch].any()) == graphs
+        assert bool(eng.cache.state[0][:scratch].any())
+        eng.add_request("fresh")
+        slot = eng.cache.requests["fresh"].state_slot
+        assert 0 <= slot < scratch and not bool(eng.cache.state[0][slot].any()) and not bool(eng.cache.state[1][slot].any())
+        eng.free_request("fresh")
     finally:
         unregister_architecture("ToyDecay")
