@@ -5,6 +5,7 @@
 // [start, p] with start = 0 (all keys), floor(p / W) * W (chunk-local) or max(0, p - W + 1)
 // (sliding).  Keys are visited in blocks of 64 dealt round-robin to the block's four waves, so
 // the order of every sum depends on (start, p) alone: not on how the tokens were batched.
+// Values may have another width than keys (vd): q and keys are hd wide, values and the output vd.
 #include "common.h"
 
 constexpr int kAttnWaves = 4;
@@ -15,7 +16,7 @@ __global__ __launch_bounds__(kAttnWaves* kWave) void attn_generic_kernel(
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_table, const int* __restrict__ entry_of_token,
     const int* __restrict__ positions, T* __restrict__ out, int window_kind, int window, float scale, int nh,
-    int nkv, int hd, int page_size, int max_blocks, int num_pages) {
+    int nkv, int hd, int vd, int page_size, int max_blocks, int num_pages) {
   __shared__ float qs[kAttnMaxHd];
   __shared__ float pw[kAttnWaves][kWave];
   __shared__ int vrow[kAttnWaves][kWave];
@@ -82,12 +83,12 @@ __global__ __launch_bounds__(kAttnWaves* kWave) void attn_generic_kernel(
         const int r = vrow[w][j];
         if (r < 0) continue;
         const float pj = pw[w][j];
-        // values are stored transposed inside a page: [page][kv head][hd][page_size]
-        const T* vr = v_cache + (size_t)(r / page_size) * hd * page_size + (r % page_size);
+        // values are stored transposed inside a page: [page][kv head][vd][page_size]
+        const T* vr = v_cache + (size_t)(r / page_size) * vd * page_size + (r % page_size);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int d = lane + i * kWave;
-          if (d < hd) acc[i] = fmaf(pj, to_f32<T>(vr[(size_t)d * page_size]), acc[i]);
+          if (d < vd) acc[i] = fmaf(pj, to_f32<T>(vr[(size_t)d * page_size]), acc[i]);
         }
       }
     }
@@ -101,7 +102,7 @@ __global__ __launch_bounds__(kAttnWaves* kWave) void attn_generic_kernel(
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int d = lane + i * kWave;
-    if (d < hd) acc_s[w][d] = acc[i];
+    if (d < vd) acc_s[w][d] = acc[i];
   }
   __syncthreads();
   float M = m_s[0];
@@ -112,8 +113,8 @@ __global__ __launch_bounds__(kAttnWaves* kWave) void attn_generic_kernel(
     f[i] = m_s[i] > -INFINITY ? expf(m_s[i] - M) : 0.f;
     L += l_s[i] * f[i];
   }
-  T* orow = out + ((size_t)t * nh + h) * hd;
-  for (int d = threadIdx.x; d < hd; d += blockDim.x) {
+  T* orow = out + ((size_t)t * nh + h) * vd;
+  for (int d = threadIdx.x; d < vd; d += blockDim.x) {
     float o = 0.f;
     for (int i = 0; i < kAttnWaves; ++i) o += acc_s[i][d] * f[i];
     orow[d] = from_f32<T>(L > 0.f ? o / L : 0.f);
@@ -123,21 +124,21 @@ __global__ __launch_bounds__(kAttnWaves* kWave) void attn_generic_kernel(
 SHARPI_EXPORT int sharpi_attention_generic(const void* q, const void* k_cache, const void* v_cache, int dtype,
                                            const int* block_table, const int* entry_of_token,
                                            const int* positions, void* out, int window_kind, int window,
-                                           float scale, int n_tokens, int nh, int nkv, int hd, int page_size,
+                                           float scale, int n_tokens, int nh, int nkv, int hd, int vd, int page_size,
                                            int max_blocks, int num_pages, hipStream_t stream) {
   if (n_tokens <= 0) return SHARPI_OK;
-  if (hd <= 0 || hd > kAttnMaxHd || nh <= 0 || nkv <= 0 || nh % nkv != 0 || nh > 65535) return SHARPI_ERR_ARG;
+  if (hd <= 0 || hd > kAttnMaxHd || vd <= 0 || vd > kAttnMaxHd || nh <= 0 || nkv <= 0 || nh % nkv != 0 || nh > 65535) return SHARPI_ERR_ARG;
   if (page_size <= 0 || max_blocks <= 0 || num_pages <= 0) return SHARPI_ERR_ARG;
   if (window_kind < 0 || window_kind > 2 || (window_kind != 0 && window <= 0)) return SHARPI_ERR_ARG;
   dim3 grid(n_tokens, nh), block(kAttnWaves * kWave);
   if (dtype == DT_F32)
     attn_generic_kernel<float><<<grid, block, 0, stream>>>(
         (const float*)q, (const float*)k_cache, (const float*)v_cache, block_table, entry_of_token, positions,
-        (float*)out, window_kind, window, scale, nh, nkv, hd, page_size, max_blocks, num_pages);
+        (float*)out, window_kind, window, scale, nh, nkv, hd, vd, page_size, max_blocks, num_pages);
   else if (dtype == DT_BF16)
     attn_generic_kernel<bf16_t><<<grid, block, 0, stream>>>(
         (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, entry_of_token, positions,
-        (bf16_t*)out, window_kind, window, scale, nh, nkv, hd, page_size, max_blocks, num_pages);
+        (bf16_t*)out, window_kind, window, scale, nh, nkv, hd, vd, page_size, max_blocks, num_pages);
   else
     return SHARPI_ERR_ARG;
   SHARPI_CHECK_LAUNCH();

@@ -3,26 +3,27 @@
 #include "common.h"
 
 // ---------------------------------------------------------------------------
-// embedding gather: out[t, :] = table[ids[t], :]   (out is the float residual stream)
+// embedding gather: out[t, :] = table[ids[t], :] * scale   (out is the float residual stream; the
+// product in float; scale 1 leaves the row as it is)
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ void embed_gather_kernel(const int* __restrict__ ids, const T* __restrict__ table,
-                                    float* __restrict__ out, int hidden) {
+                                    float* __restrict__ out, int hidden, float scale) {
   const int t = blockIdx.x;
   const T* row = table + (size_t)ids[t] * hidden;
   float* o = out + (size_t)t * hidden;
-  for (int i = threadIdx.x; i < hidden; i += blockDim.x) o[i] = to_f32<T>(row[i]);
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) o[i] = to_f32<T>(row[i]) * scale;
 }
 
 SHARPI_EXPORT int sharpi_embed_gather(const int* ids, const void* table, int table_dtype, float* out,
-                                      int n_tokens, int hidden, hipStream_t stream) {
+                                      int n_tokens, int hidden, float scale, hipStream_t stream) {
   if (n_tokens <= 0) return SHARPI_OK;
   if (hidden <= 0) return SHARPI_ERR_ARG;
   dim3 grid(n_tokens), block(256);
   if (table_dtype == DT_F32)
-    embed_gather_kernel<float><<<grid, block, 0, stream>>>(ids, (const float*)table, out, hidden);
+    embed_gather_kernel<float><<<grid, block, 0, stream>>>(ids, (const float*)table, out, hidden, scale);
   else if (table_dtype == DT_BF16)
-    embed_gather_kernel<bf16_t><<<grid, block, 0, stream>>>(ids, (const bf16_t*)table, out, hidden);
+    embed_gather_kernel<bf16_t><<<grid, block, 0, stream>>>(ids, (const bf16_t*)table, out, hidden, scale);
   else
     return SHARPI_ERR_ARG;
   SHARPI_CHECK_LAUNCH();
@@ -426,6 +427,27 @@ SHARPI_EXPORT int sharpi_add_bias(void* x, int dtype, const float* bias, int n_r
   if (dtype == DT_F32) add_bias_kernel<float><<<grid, block, 0, stream>>>((float*)x, bias, n_rows, N);
   else if (dtype == DT_BF16) add_bias_kernel<bf16_t><<<grid, block, 0, stream>>>((bf16_t*)x, bias, n_rows, N);
   else return SHARPI_ERR_ARG;
+  SHARPI_CHECK_LAUNCH();
+  return SHARPI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// logits in place: x <- x * scale, then (cap > 0) x <- cap * tanh(x / cap): the head's scale and the
+// soft cap of architectures that have them.
+// ---------------------------------------------------------------------------
+__global__ void scale_softcap_kernel(float* __restrict__ x, size_t n, float scale, float cap) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    float v = x[i] * scale;
+    if (cap > 0.f) v = tanhf(v / cap) * cap;
+    x[i] = v;
+  }
+}
+
+SHARPI_EXPORT int sharpi_scale_softcap(float* x, long long n, float scale, float cap, hipStream_t stream) {
+  if (n <= 0) return SHARPI_OK;
+  if (!(cap >= 0.f)) return SHARPI_ERR_ARG;
+  const dim3 block(256), grid((unsigned)min((long long)8192, (n + 255) / 256));
+  scale_softcap_kernel<<<grid, block, 0, stream>>>(x, (size_t)n, scale, cap);
   SHARPI_CHECK_LAUNCH();
   return SHARPI_OK;
 }

@@ -1,7 +1,8 @@
 // Position encoding, weightless per-head norm, query temperature and the cache write, one kernel.
 //
-// Input  qkv [T, (nh + 2*nkv) * hd]: q heads, then k heads, then v heads of each token; an optional
-// bias [(nh + 2*nkv) * hd] (float) is added to every token's row first, in float.
+// Input  qkv [T, (nh + nkv) * hd + nkv * vd]: q heads, then k heads (hd wide), then v heads (vd wide,
+// usually hd) of each token; an optional bias of the row's width (float) is added to every
+// token's row first, in float.
 // q head : rotate (if inv_freq) -> norm (if qk_norm) -> * temperature (if temp_tuning) -> q_out
 // k head : rotate (if inv_freq) -> norm (if qk_norm) -> cache K at slot_mapping[t]
 // v head : cache V at slot_mapping[t]
@@ -20,13 +21,15 @@ __global__ void rope_kv_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
                                const int* __restrict__ positions, const float* __restrict__ inv_freq,
                                const float* __restrict__ bias,
                                int qk_norm, float eps, int temp_tuning, float floor_scale, float attn_scale,
-                               int nh, int nkv, int hd, int page_size, int half_split, int rotary_dim) {
+                               int nh, int nkv, int hd, int vd, int page_size, int half_split, int rotary_dim) {
   const int t = blockIdx.x;
   const int head = blockIdx.y;            // 0..nh-1 q, nh..nh+nkv-1 k, then v
   const int lane = threadIdx.x;           // one wave
   const int half = hd >> 1;
-  const T* src = qkv + ((size_t)t * (nh + 2 * nkv) + head) * hd;
-  const float* hb = bias ? bias + (size_t)head * hd : nullptr;
+  const size_t row_width = (size_t)(nh + nkv) * hd + (size_t)nkv * vd;
+  const size_t head_at = head < nh + nkv ? (size_t)head * hd : (size_t)(nh + nkv) * hd + (size_t)(head - nh - nkv) * vd;
+  const T* src = qkv + (size_t)t * row_width + head_at;
+  const float* hb = bias ? bias + head_at : nullptr;
   const int pos = positions[t];
   const bool is_q = head < nh;
   const bool is_k = !is_q && head < nh + nkv;
@@ -35,8 +38,8 @@ __global__ void rope_kv_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
   if (!is_q && !is_k) {  // v: plain copy into the cache
     if (slot < 0) return;
     const int kvh = head - nh - nkv;
-    T* dst = v_cache + ((size_t)(slot / page_size) * nkv + kvh) * hd * page_size + (slot % page_size);
-    for (int d = lane; d < hd; d += kWave)
+    T* dst = v_cache + ((size_t)(slot / page_size) * nkv + kvh) * vd * page_size + (slot % page_size);
+    for (int d = lane; d < vd; d += kWave)
       dst[(size_t)d * page_size] = hb ? from_f32<T>(to_f32<T>(src[d]) + hb[d]) : src[d];
     return;
   }
@@ -214,19 +217,19 @@ __global__ __launch_bounds__(256) void rope_kv_vec_kernel(
 SHARPI_EXPORT int sharpi_rope_kv(const void* qkv, void* q_out, void* k_cache, void* v_cache, int dtype,
                                  const int* slot_mapping, const int* positions, const float* inv_freq,
                                  const float* bias, int qk_norm, float eps, int temp_tuning, float floor_scale, float attn_scale,
-                                 int n_tokens, int nh, int nkv, int hd, int page_size, int pair_layout,
+                                 int n_tokens, int nh, int nkv, int hd, int vd, int page_size, int pair_layout,
                                  int rotary_dim, hipStream_t stream) {
   if (n_tokens <= 0) return SHARPI_OK;
   // pair_layout: 0 = pairs (2i, 2i+1), 1 = pairs (i, i + rotary_dim/2); rotary_dim even, <= hd
   if (pair_layout < 0 || pair_layout > 1) return SHARPI_ERR_ARG;
   if (inv_freq == nullptr) rotary_dim = 0;
   else if (rotary_dim <= 0 || (rotary_dim & 1) || rotary_dim > hd) return SHARPI_ERR_ARG;
-  if (hd <= 0 || (hd & 1) || hd > 512 || nh <= 0 || nkv <= 0 || page_size <= 0) return SHARPI_ERR_ARG;
+  if (hd <= 0 || (hd & 1) || hd > 512 || vd <= 0 || nh <= 0 || nkv <= 0 || page_size <= 0) return SHARPI_ERR_ARG;
   if (nh + 2 * nkv > 65535) return SHARPI_ERR_ARG;
   if (temp_tuning && !(floor_scale > 0.f)) return SHARPI_ERR_ARG;
   dim3 grid(n_tokens, nh + 2 * nkv), block(kWave);
   if (dtype != DT_F32 && dtype != DT_BF16) return SHARPI_ERR_ARG;
-  if ((hd == 32 || hd == 64 || hd == 128 || hd == 256) && pair_layout == 0 && (rotary_dim & 7) == 0) {
+  if ((hd == 32 || hd == 64 || hd == 128 || hd == 256) && vd == hd && pair_layout == 0 && (rotary_dim & 7) == 0) {
     // a few tokens (decode): a token's heads over several blocks, for the compute units' sake;
     // many tokens: one block per token, which then computes its angles once for all heads
     const dim3 vgrid(n_tokens, n_tokens <= 64 ? ceil_div((nh + 2 * nkv) * (hd >> 3), 256) : 1);
@@ -246,13 +249,13 @@ SHARPI_EXPORT int sharpi_rope_kv(const void* qkv, void* q_out, void* k_cache, vo
   if (dtype == DT_F32)
     rope_kv_kernel<float><<<grid, block, 0, stream>>>((const float*)qkv, (float*)q_out, (float*)k_cache,
                                                      (float*)v_cache, slot_mapping, positions, inv_freq, bias, qk_norm,
-                                                     eps, temp_tuning, floor_scale, attn_scale, nh, nkv, hd,
+                                                     eps, temp_tuning, floor_scale, attn_scale, nh, nkv, hd, vd,
                                                      page_size, pair_layout, rotary_dim);
   else if (dtype == DT_BF16)
     rope_kv_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)qkv, (bf16_t*)q_out, (bf16_t*)k_cache,
                                                       (bf16_t*)v_cache, slot_mapping, positions, inv_freq, bias,
                                                       qk_norm, eps, temp_tuning, floor_scale, attn_scale, nh, nkv,
-                                                      hd, page_size, pair_layout, rotary_dim);
+                                                      hd, vd, page_size, pair_layout, rotary_dim);
   else
     return SHARPI_ERR_ARG;
   SHARPI_CHECK_LAUNCH();

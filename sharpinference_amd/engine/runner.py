@@ -60,6 +60,7 @@ class ModelRunner:
             all(t is None for t in cache.state) or bool(safe and safe()))
         self.max_context = int(max_context)
         self._graphs: dict = {}
+        self._graph_pool = None      # one memory pool for every graph of this runner (made with the first capture)
         self._graph_asks: dict = {}
         self.graph_replays = 0
 
@@ -219,7 +220,9 @@ class ModelRunner:
         pieces, info = self._host_arrays(entries, static_blocks=static_blocks)
         if graph is None:
             try:
-                graph = _DecodeGraph(self, pieces, info, bound, select)
+                if self._graph_pool is None:
+                    self._graph_pool = torch.cuda.graph_pool_handle()
+                graph = _DecodeGraph(self, pieces, info, bound, select, pool=self._graph_pool)
             except Exception as e:  # noqa: BLE001 - capture is an optimisation: report once, go on eagerly
                 print(f"[sharpi] decode graph for batch {n}, contexts to {bound} not captured ({type(e).__name__}: {e}); "
                       "running eagerly", file=sys.stderr, flush=True)
@@ -311,7 +314,8 @@ class _DecodeGraph:
     step (block table width, context bound of the decode kernel) are fixed at ``max_context``.
     The logits tensor belongs to the graph: the caller gets a copy."""
 
-    def __init__(self, runner: ModelRunner, pieces, info: dict, max_context: int, select: Optional[str] = None):
+    def __init__(self, runner: ModelRunner, pieces, info: dict, max_context: int, select: Optional[str] = None,
+                 pool=None):
         self.sizes = [p.size for p in pieces]
         total = sum(self.sizes)
         self.host = torch.empty(total, dtype=torch.int32).pin_memory()
@@ -352,7 +356,11 @@ class _DecodeGraph:
         collecting = gc.isenabled()
         gc.disable()
         try:
-            with torch.cuda.graph(self.graph):
+            # One pool for all of a runner's graphs: they are replayed one after the other on one
+            # stream and their results are copied out before the next replay, so what one graph's
+            # intermediate tensors held another's may hold; with a pool each, every shape a served
+            # process meets would keep its own activations and logits for good.
+            with torch.cuda.graph(self.graph, pool=pool):
                 self.logits = runner.model.forward(*args)
         finally:
             if collecting:

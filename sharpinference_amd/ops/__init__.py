@@ -6,6 +6,8 @@ arithmetic runs on the product path except the library matrix product in :func:`
 """
 from __future__ import annotations
 
+import collections
+
 from typing import Optional, Tuple
 
 import torch
@@ -67,8 +69,8 @@ def _run(name: str, *args) -> None:
 
 
 # ---------------------------------------------------------------------------
-def embed_gather(ids: torch.Tensor, table: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out[t] = table[ids[t]] as float32 (the residual stream)."""
+def embed_gather(ids: torch.Tensor, table: torch.Tensor, out: Optional[torch.Tensor] = None, scale: float = 1.0) -> torch.Tensor:
+    """out[t] = table[ids[t]] * scale as float32 (the residual stream)."""
     _dev(ids, table, out)
     _i32(ids, "ids")
     _need(ids.dim() == 1 and table.dim() == 2, "embed_gather: ids [T], table [V, H]")
@@ -76,8 +78,16 @@ def embed_gather(ids: torch.Tensor, table: torch.Tensor, out: Optional[torch.Ten
     if out is None:
         out = torch.empty(T, H, dtype=torch.float32, device=table.device)
     _need(out.shape == (T, H) and out.dtype == torch.float32, "embed_gather: out must be float32 [T, H]")
-    _run("sharpi_embed_gather", _ptr(ids), _ptr(table), _code(table.dtype), _ptr(out), T, H, _stream())
+    _run("sharpi_embed_gather", _ptr(ids), _ptr(table), _code(table.dtype), _ptr(out), T, H, float(scale), _stream())
     return out
+
+
+def scale_softcap(logits: torch.Tensor, scale: float = 1.0, cap: float = 0.0) -> torch.Tensor:
+    """logits (float32, contiguous) in place: x * scale, then cap * tanh(x / cap) if cap > 0."""
+    _dev(logits)
+    _need(logits.dtype == torch.float32 and logits.is_contiguous() and cap >= 0, "scale_softcap: float32 contiguous logits, cap >= 0")
+    _run("sharpi_scale_softcap", _ptr(logits), logits.numel(), float(scale), float(cap), _stream())
+    return logits
 
 
 class ExpertSum:
@@ -213,9 +223,10 @@ def random_fill(out: torch.Tensor, key: int, kind: int, std: float = 0.02, lo: f
 
 
 # ---------------------------------------------------------------------------
-def _cache_shapes_ok(k_cache: torch.Tensor, v_cache: torch.Tensor, nkv: int, hd: int) -> bool:
+def _cache_shapes_ok(k_cache: torch.Tensor, v_cache: torch.Tensor, nkv: int, hd: int, vd: Optional[int] = None) -> bool:
+    """K [pages, nkv, page_size, hd] and V [pages, nkv, vd, page_size] (vd: the values' width, hd unless given)."""
     return (k_cache.dim() == 4 and v_cache.dim() == 4 and k_cache.shape[1] == nkv and k_cache.shape[3] == hd
-            and v_cache.shape == (k_cache.shape[0], nkv, hd, k_cache.shape[2]))
+            and v_cache.shape == (k_cache.shape[0], nkv, vd or hd, k_cache.shape[2]))
 
 
 PAIRS_INTERLEAVED, PAIRS_HALF_SPLIT = 0, 1
@@ -224,8 +235,9 @@ PAIRS_INTERLEAVED, PAIRS_HALF_SPLIT = 0, 1
 def rope_kv(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, slot_mapping: torch.Tensor,
             positions: torch.Tensor, inv_freq: Optional[torch.Tensor], qk_norm: bool, eps: float,
             temperature: Optional[Tuple[float, float]], nh: int, nkv: int, hd: int,
-            pair_layout: int = PAIRS_INTERLEAVED, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Rotate / norm / scale the heads of qkv [T, (nh+2nkv)*hd]; K and V go into the layer's
+            pair_layout: int = PAIRS_INTERLEAVED, bias: Optional[torch.Tensor] = None, vd: Optional[int] = None) -> torch.Tensor:
+    """Rotate / norm / scale the heads of qkv [T, (nh+nkv)*hd + nkv*vd] (vd, the values' width, is hd
+    unless given); K and V go into the layer's
     cache [pages, nkv, page_size, hd] at slot_mapping; returns q [T, nh*hd].  inv_freq [r/2]
     rotates the first r <= hd elements of every head, in pairs (2i, 2i+1) or (i, i + r/2)
     (``pair_layout``); the rest of the head passes through.  ``bias`` (float32, one value per
@@ -233,12 +245,13 @@ def rope_kv(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, slo
     _dev(qkv, k_cache, v_cache, slot_mapping, positions, inv_freq, bias)
     if bias is not None:
         _need(bias.dtype == torch.float32 and bias.shape == (qkv.shape[1],) and bias.is_contiguous(),
-              "rope_kv: bias must be float32 [(nh+2nkv)*hd]")
+              "rope_kv: bias must be float32, one value per column of qkv")
     _i32(slot_mapping, "slot_mapping")
     _i32(positions, "positions")
     T = qkv.shape[0]
-    _need(qkv.dim() == 2 and qkv.shape[1] == (nh + 2 * nkv) * hd, "rope_kv: qkv must be [T, (nh+2nkv)*hd]")
-    _need(_cache_shapes_ok(k_cache, v_cache, nkv, hd), "rope_kv: caches must be K [pages, nkv, page_size, hd], V [pages, nkv, hd, page_size]")
+    vd = int(vd or hd)
+    _need(qkv.dim() == 2 and qkv.shape[1] == (nh + nkv) * hd + nkv * vd, "rope_kv: qkv must be [T, (nh+nkv)*hd + nkv*vd]")
+    _need(_cache_shapes_ok(k_cache, v_cache, nkv, hd, vd), "rope_kv: caches must be K [pages, nkv, page_size, hd], V [pages, nkv, vd, page_size]")
     _need(k_cache.dtype == qkv.dtype and v_cache.dtype == qkv.dtype, "rope_kv: cache dtype differs from qkv's")
     _need(slot_mapping.shape == (T,) and positions.shape == (T,), "rope_kv: slot_mapping / positions must be [T]")
     rotary_dim = 0
@@ -252,29 +265,31 @@ def rope_kv(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, slo
     fs, asc = temperature if temperature is not None else (1.0, 0.0)
     _run("sharpi_rope_kv", _ptr(qkv), _ptr(q_out), _ptr(k_cache), _ptr(v_cache), _code(qkv.dtype),
          _ptr(slot_mapping), _ptr(positions), _ptr(inv_freq), _ptr(bias), 1 if qk_norm else 0, float(eps),
-         1 if temperature is not None else 0, float(fs), float(asc), T, nh, nkv, hd, page_size, int(pair_layout),
+         1 if temperature is not None else 0, float(fs), float(asc), T, nh, nkv, hd, vd, page_size, int(pair_layout),
          rotary_dim, _stream())
     return q_out
 
 
 def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                       entry_of_token: torch.Tensor, positions: torch.Tensor, window_kind: int, window: int,
-                      scale: float, nh: int, nkv: int, hd: int) -> torch.Tensor:
-    """Attention of every token of the batch over its request's pages; float arithmetic."""
+                      scale: float, nh: int, nkv: int, hd: int, vd: Optional[int] = None) -> torch.Tensor:
+    """Attention of every token of the batch over its request's pages; float arithmetic.  Values
+    (and so the output, [T, nh*vd]) may have another width than keys."""
     _dev(q, k_cache, v_cache, block_table, entry_of_token, positions)
     _i32(block_table, "block_table")
     _i32(entry_of_token, "entry_of_token")
     _i32(positions, "positions")
     T = q.shape[0]
+    vd = int(vd or hd)
     _need(q.shape == (T, nh * hd), "attention: q must be [T, nh*hd]")
-    _need(_cache_shapes_ok(k_cache, v_cache, nkv, hd) and k_cache.dtype == q.dtype and v_cache.dtype == q.dtype,
-          "attention: caches must be K [pages, nkv, page_size, hd], V [pages, nkv, hd, page_size] of q's dtype")
+    _need(_cache_shapes_ok(k_cache, v_cache, nkv, hd, vd) and k_cache.dtype == q.dtype and v_cache.dtype == q.dtype,
+          "attention: caches must be K [pages, nkv, page_size, hd], V [pages, nkv, vd, page_size] of q's dtype")
     _need(block_table.dim() == 2, "attention: block_table must be [entries, max_blocks]")
     _need(entry_of_token.shape == (T,) and positions.shape == (T,), "attention: per-token arrays must be [T]")
-    out = torch.empty_like(q)
+    out = torch.empty(T, nh * vd, dtype=q.dtype, device=q.device)
     _run("sharpi_attention_generic", _ptr(q), _ptr(k_cache), _ptr(v_cache), _code(q.dtype), _ptr(block_table),
          _ptr(entry_of_token), _ptr(positions), _ptr(out), int(window_kind), int(window), float(scale), T, nh, nkv,
-         hd, k_cache.shape[2], block_table.shape[1], k_cache.shape[0], _stream())
+         hd, vd, k_cache.shape[2], block_table.shape[1], k_cache.shape[0], _stream())
     return out
 
 
@@ -473,10 +488,23 @@ def skinny_plan(N: int, K: int, row_blocks: int = 1, groups: int = 1, act: bool 
     if row_blocks > 1:
         return (4 if N >= 12288 else 2), 8
     blocks = groups * ((N + 31) // 32)
-    return (1 if not act and COMPUTE_UNITS < blocks < 2 * COMPUTE_UNITS else 2), 8
+    units = compute_units()
+    return (1 if not act and units < blocks < 2 * units else 2), 8
 
 
-COMPUTE_UNITS = 256     # of the GPU this library is written for
+_COMPUTE_UNITS: dict = {}
+
+
+def compute_units(device=None) -> int:
+    """Compute units of the GPU the launches are laid out for: asked of the device once (the
+    MI355X this library is tuned on has 256; so does a host without a GPU, for the tests of the
+    launch shapes).  The shape thresholds of ``skinny_plan`` are measured on that part."""
+    if not torch.cuda.is_available():
+        return 256
+    idx = torch.cuda.current_device() if device is None else torch.device(device).index or 0
+    if idx not in _COMPUTE_UNITS:
+        _COMPUTE_UNITS[idx] = int(torch.cuda.get_device_properties(idx).multi_processor_count)
+    return _COMPUTE_UNITS[idx]
 
 
 def _row_blocks(group_rows: Optional[int]) -> int:
@@ -830,22 +858,26 @@ def gemm_grouped_swiglu(x: torch.Tensor, w, rt: Routing, scale: Optional[torch.T
 # ---------------------------------------------------------------------------
 # plain products of many rows through the grouped kernel (one group: the whole matrix)
 # ---------------------------------------------------------------------------
-_DENSE_ROUTING: dict = {}
+_DENSE_ROUTING: "collections.OrderedDict" = collections.OrderedDict()
+_DENSE_ROUTING_KEPT = 64
 
 
 def _dense_routing(T: int, dev: torch.device) -> Routing:
     """The routing of T rows that all belong to one group: offsets [0, T] and the plan of the
-    grouped product for it, made once per (T, device) by the routing kernel.  Its token list is
-    not used (the routing kernel promises no order inside a group): the products read x row by
-    row (gather off)."""
+    grouped product for it, made by the routing kernel when a row count is first met and kept for
+    the row counts used last (the least recently used one gives way).  Its token list is not used
+    (the routing kernel promises no order inside a group): the products read x row by row
+    (gather off)."""
     key = (T, dev)
     rt = _DENSE_ROUTING.get(key)
     if rt is None:
         _need(not torch.cuda.is_current_stream_capturing(), "a dense routing's first use must not be captured")
-        if len(_DENSE_ROUTING) > 64:
-            _DENSE_ROUTING.clear()
+        while len(_DENSE_ROUTING) >= _DENSE_ROUTING_KEPT:
+            _DENSE_ROUTING.popitem(last=False)
         ids = torch.zeros(T, 1, dtype=torch.int32, device=dev)
         rt = _DENSE_ROUTING[key] = moe_permute(ids, torch.ones(T, 1, dtype=torch.float32, device=dev), 1)
+    else:
+        _DENSE_ROUTING.move_to_end(key)
     return rt
 
 
@@ -913,10 +945,11 @@ def edit_logits(logits: torch.Tensor, row_offsets: torch.Tensor, ids: torch.Tens
 # dispatchers used by the parts
 # ---------------------------------------------------------------------------
 def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, group, ctx, window_kind: int,
-              window: int, scale: float, nh: int, nkv: int, hd: int) -> torch.Tensor:
+              window: int, scale: float, nh: int, nkv: int, hd: int, vd: Optional[int] = None) -> torch.Tensor:
     """Attention of the step's tokens over their requests' pages (`group`: the cache group's
-    block tables, `ctx`: the step)."""
-    if decode_attention_ok(q.dtype, hd) and (prefill_attention_ok(q.dtype, hd) or not ctx.n_prefill_tiles):
+    block tables, `ctx`: the step).  Values of another width than keys (vd) go through the float kernel."""
+    same = vd is None or vd == hd
+    if same and decode_attention_ok(q.dtype, hd) and (prefill_attention_ok(q.dtype, hd) or not ctx.n_prefill_tiles):
         # entries of one token: split-K decode kernel; longer entries: flash kernel, 128 tokens a block
         out = torch.empty_like(q)
         if ctx.n_prefill_tiles:
@@ -927,7 +960,7 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, gro
                              ctx.decode_tokens, group.max_context, window_kind, window, scale, nh, nkv, hd, out=out)
         return out
     return attention_generic(q, k_cache, v_cache, group.block_table, ctx.entry_of_token, ctx.positions, window_kind,
-                             window, scale, nh, nkv, hd)
+                             window, scale, nh, nkv, hd, vd)
 
 
 def grouped_swiglu(x: torch.Tensor, w_gate_up, rt: Routing, out_dtype: torch.dtype, scaled: bool = True,

@@ -17,7 +17,8 @@ I = c_int
 F = c_float
 
 _SIGNATURES = {
-    "sharpi_embed_gather": [P, P, I, P, I, I, P],
+    "sharpi_embed_gather": [P, P, I, P, I, I, F, P],
+    "sharpi_scale_softcap": [P, c_longlong, F, F, P],
     "sharpi_add_rmsnorm": [P, P, I, P, I, P, I, P, I, I, F, I, P, P, P, I, P],
     "sharpi_silu_mul": [P, P, P, I, I, I, I, P],
     "sharpi_moe_combine": [P, P, P, P, P, I, I, I, I, P],
@@ -26,8 +27,8 @@ _SIGNATURES = {
     "sharpi_peak_read": [P, c_longlong, P, P, P],
     "sharpi_peak_mfma": [P, I, I, P],
     "sharpi_random_fill": [P, I, c_longlong, c_ulonglong, I, F, I, I, P],
-    "sharpi_rope_kv": [P, P, P, P, I, P, P, P, P, I, F, I, F, F, I, I, I, I, I, I, I, P],
-    "sharpi_attention_generic": [P, P, P, I, P, P, P, P, I, I, F, I, I, I, I, I, I, I, P],
+    "sharpi_rope_kv": [P, P, P, P, I, P, P, P, P, I, F, I, F, F, I, I, I, I, I, I, I, I, P],
+    "sharpi_attention_generic": [P, P, P, I, P, P, P, P, I, I, F, I, I, I, I, I, I, I, I, P],
     "sharpi_attention_decode": [P, P, P, P, P, P, P, P, P, P, I, I, F, I, I, I, I, I, I, I, I, P],
     "sharpi_attention_prefill": [P, P, P, P, P, P, P, I, I, I, F, I, I, I, I, I, I, P],
     "sharpi_gemm_tiled": [P, P, P, I, I, I, I, I, P, P, I, P],

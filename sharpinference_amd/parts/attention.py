@@ -22,14 +22,16 @@ class Attention(Part):
 
     Everything that differs between layers is an argument: ``rotary`` (None = no position
     encoding; otherwise any object with ``table(device)``, ``pair_layout``, ``rotary_dim`` and
-    ``head_dim``, see parts/position.py), ``qk_norm_eps`` (None = no norm), ``q_temperature`` = (floor_scale, attn_scale)
+    ``head_dim``, see parts/position.py), ``v_head_dim`` (values and a head's output of another width than
+    keys: such layers run the float attention kernel), ``qk_norm_eps`` (None = no norm), ``q_temperature`` = (floor_scale, attn_scale)
     multiplying queries by 1 + attn_scale * ln(floor((pos + 1) / floor_scale) + 1), and the
     window: all keys, the chunk [floor(pos/W)*W, pos], or the last W keys."""
 
     def __init__(self, hidden: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  rotary=None, qk_norm_eps: Optional[float] = None,
                  q_temperature: Optional[Tuple[float, float]] = None, window_kind: int = WINDOW_NONE,
-                 window: int = 0, scale: Optional[float] = None, bias: bool = False, o_bias: Optional[bool] = None):
+                 window: int = 0, scale: Optional[float] = None, bias: bool = False, o_bias: Optional[bool] = None,
+                 v_head_dim: Optional[int] = None):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} heads cannot share {num_kv_heads} kv heads")
         if head_dim % 16 or not 16 <= head_dim <= 256:
@@ -39,6 +41,9 @@ class Attention(Part):
         if rotary is not None and rotary.pair_layout not in ("interleaved", "half"):
             raise ValueError(f"pair layout {rotary.pair_layout!r} is not taken by the rotation kernel")
         self.hidden, self.nh, self.nkv, self.hd = int(hidden), int(num_heads), int(num_kv_heads), int(head_dim)
+        self.vd = int(v_head_dim or head_dim)                    # width of a value (and of a head's output)
+        if not 1 <= self.vd <= 256:
+            raise ValueError(f"v_head_dim {self.vd} is not taken: 1 to 256")
         self.rotary, self.qk_norm_eps, self.q_temperature = rotary, qk_norm_eps, q_temperature
         self.window_kind, self.window = int(window_kind), int(window)
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
@@ -51,28 +56,28 @@ class Attention(Part):
 
     # -- what it needs --------------------------------------------------------
     def cache_spec(self) -> KVSpec:
-        return KVSpec(self.nkv, self.hd, self.window_kind, self.window)
+        return KVSpec(self.nkv, self.hd, self.window_kind, self.window, 0 if self.vd == self.hd else self.vd)
 
     def param_specs(self, prefix: str) -> Dict[str, ParamSpec]:
-        q, kv = self.nh * self.hd, self.nkv * self.hd
+        q, kv, vv, ov = self.nh * self.hd, self.nkv * self.hd, self.nkv * self.vd, self.nh * self.vd
         specs = {
             prefix + "q_proj.weight": ParamSpec((q, self.hidden)),
             prefix + "k_proj.weight": ParamSpec((kv, self.hidden)),
-            prefix + "v_proj.weight": ParamSpec((kv, self.hidden)),
-            prefix + "o_proj.weight": ParamSpec((self.hidden, q)),
+            prefix + "v_proj.weight": ParamSpec((vv, self.hidden)),
+            prefix + "o_proj.weight": ParamSpec((self.hidden, ov)),
         }
         if self.bias:
             specs.update({prefix + "q_proj.bias": ParamSpec((q,)), prefix + "k_proj.bias": ParamSpec((kv,)),
-                          prefix + "v_proj.bias": ParamSpec((kv,))})
+                          prefix + "v_proj.bias": ParamSpec((vv,))})
         if self.o_bias:
             specs[prefix + "o_proj.bias"] = ParamSpec((self.hidden,))
         return specs
 
     def load(self, prefix: str, source: TensorSource) -> None:
-        q, kv = self.nh * self.hd, self.nkv * self.hd
+        q, kv, vv = self.nh * self.hd, self.nkv * self.hd, self.nkv * self.vd
         parts = [source.get(prefix + n + "_proj.weight") for n in ("q", "k", "v")]
         dt = torch.float32 if any(p.dtype == torch.float32 for p in parts) else parts[0].dtype
-        fused = torch.empty(q + 2 * kv, self.hidden, dtype=dt, device=parts[0].device)
+        fused = torch.empty(q + kv + vv, self.hidden, dtype=dt, device=parts[0].device)
         o = 0
         for p in parts:
             fused[o:o + p.shape[0]].copy_(p)
@@ -90,7 +95,7 @@ class Attention(Part):
         g = cache.group
         T = x.shape[0]
         width = 2 if ctx.act_dtype == torch.bfloat16 else 4
-        q_dim, kv_dim = self.nh * self.hd, self.nkv * self.hd
+        q_dim, kv_dim = self.nh * self.hd, self.nkv * (self.hd + self.vd) // 2    # (kv_dim: the mean of a key's and a value's row)
         with section("qkv", nbytes=width * (q_dim + 2 * kv_dim) * (self.hidden + T) + width * T * self.hidden,
                      flops=2.0 * T * self.hidden * (q_dim + 2 * kv_dim)):
             qkv = ops.linear(x, self.w_qkv, ctx.act_dtype)
@@ -100,11 +105,11 @@ class Attention(Part):
         with section("rope + cache write", nbytes=2 * width * T * (q_dim + 2 * kv_dim)):
             q = ops.rope_kv(qkv, cache.k, cache.v, slots, ctx.positions, inv_freq, self.qk_norm_eps is not None,
                             self.qk_norm_eps or 1e-6, self.q_temperature, self.nh, self.nkv, self.hd, layout,
-                            bias=self.b_qkv)
+                            bias=self.b_qkv, vd=self.vd)
         with section("attention", nbytes=lambda: self._keys_held(ctx) * 2 * kv_dim * width + 2 * T * q_dim * width,
                      flops=lambda: 4.0 * self._keys_read(ctx) * q_dim):
             o = ops.attention(q, cache.k, cache.v, g, ctx, self.window_kind, self.window, self.scale, self.nh, self.nkv,
-                              self.hd)
+                              self.hd, self.vd)
         with section("o", nbytes=width * self.hidden * (q_dim + T) + width * T * q_dim, flops=2.0 * T * self.hidden * q_dim):
             out = ops.linear(o, self.w_o, ctx.act_dtype)
             return ops.add_bias(out, self.b_o) if self.b_o is not None else out

@@ -26,19 +26,27 @@ class Run:
 
 
 class DecoderModel(Part):
-    """tokens -> embedding rows (no scaling; reference: src/SharpInference.Engine/ForwardPass.cs:1478-1483)
-    -> blocks in the order of ``schedule`` -> final norm -> logits through the head, which is the
-    embedding table when tied (ForwardPass.cs:1741-1747, 410-413)."""
+    """tokens -> embedding rows (times ``embedding_scale``; 1 for this architecture; reference:
+    src/SharpInference.Engine/ForwardPass.cs:1478-1483) -> blocks in the order of ``schedule`` ->
+    final norm -> logits through the head, which is the embedding table when tied
+    (ForwardPass.cs:1741-1747, 410-413), times ``logit_scale`` and softly capped at
+    ``logit_softcap`` (cap * tanh(x / cap), reference: src/SharpInference.Cpu/SimdKernels.cs:4490-4530)
+    where an architecture has them."""
 
     def __init__(self, vocab_size: int, hidden: int, blocks: Sequence[Part], final_norm: RMSNorm,
                  schedule: Optional[Sequence[Run]] = None, tie_embeddings: bool = False, config=None,
                  layer_prefix: str = "model.layers.", embed_name: str = "model.embed_tokens.weight",
-                 norm_prefix: str = "model.norm.", head_name: str = "lm_head.weight"):
+                 norm_prefix: str = "model.norm.", head_name: str = "lm_head.weight", embedding_scale: float = 1.0,
+                 logit_scale: float = 1.0, logit_softcap: Optional[float] = None):
         self.vocab_size, self.hidden = int(vocab_size), int(hidden)
         self.blocks = list(blocks)
         self.final_norm = final_norm
         self.schedule: List[Run] = list(schedule) if schedule is not None else [Run(i, i) for i in range(len(self.blocks))]
         self.tie_embeddings = bool(tie_embeddings)
+        self.embedding_scale, self.logit_scale = float(embedding_scale), float(logit_scale)
+        self.logit_softcap = float(logit_softcap) if logit_softcap else 0.0
+        if self.logit_softcap < 0:
+            raise ValueError("logit_softcap must be positive (or None)")
         self.config = config
         self.layer_prefix, self.embed_name, self.norm_prefix, self.head_name = layer_prefix, embed_name, norm_prefix, head_name
         self.embed: Optional[torch.Tensor] = None
@@ -108,7 +116,7 @@ class DecoderModel(Part):
         (the reference keeps such a path for all-greedy batches,
         src/SharpInference.Engine/CudaForwardPass.cs:1574-1583)."""
         with section("embed", nbytes=ctx.n_tokens * self.hidden * 6):
-            stream = ResidualStream(ops.embed_gather(ctx.token_ids, self.embed))
+            stream = ResidualStream(ops.embed_gather(ctx.token_ids, self.embed, scale=self.embedding_scale))
         for r in self.schedule:
             c = caches[r.cache]
             if not r.write:
@@ -120,6 +128,8 @@ class DecoderModel(Part):
         m = n.shape[0]
         with section("head", nbytes=2 * self.vocab_size * self.hidden + 4 * m * self.vocab_size, flops=2.0 * m * self.vocab_size * self.hidden):
             logits = ops.linear(n, self.head, torch.float32)
+            if self.logit_scale != 1.0 or self.logit_softcap:
+                ops.scale_softcap(logits, self.logit_scale, self.logit_softcap)
         if select is None:
             return logits
         if select == "argmax":

@@ -714,6 +714,10 @@ def test_silu_mul_and_combine_and_embed(I, dtype):
     table = _rand(50, I, dtype=dtype, seed=6)
     ids = torch.tensor([3, 49, 0, 3], dtype=torch.int32, device=DEV)
     assert torch.equal(ops.embed_gather(ids, table), table.float()[ids.long()])
+    assert torch.equal(ops.embed_gather(ids, table, scale=2.5), table.float()[ids.long()] * 2.5)
+    lg = _rand(3, 77, scale=9.0, seed=7)
+    assert float((ops.scale_softcap(lg.clone(), 0.5, 3.0) - 3.0 * torch.tanh(lg * 0.5 / 3.0)).abs().max()) <= 1e-5
+    assert torch.equal(ops.scale_softcap(lg.clone(), 2.0), lg * 2.0)
 
 
 @pytest.mark.parametrize("nh,nkv,hd", [(4, 2, 16), (6, 3, 32), (5, 5, 48), (40, 8, 128)])

@@ -136,6 +136,60 @@ def test_attention_part_alone(tmp_path, layer, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window_kind,window", [(0, 0), (2, 20)])
+def test_attention_part_with_values_of_another_width_than_keys(dtype, window_kind, window):
+    """A mixer whose values (and heads' outputs) are 24 wide beside keys of 48: its cache holds V
+    [page, kv head, 24, position], the projections take the widths from it, and the result is the
+    library's attention on unrotated, unnormed q and k (softmax(q k^T / sqrt(48)) v per head, kv
+    heads repeated), for a prompt portion beside two decode tokens."""
+    from sharpinference_amd.parts.attention import Attention
+    from sharpinference_amd.parts.base import LayerCache
+
+    H, nh, nkv, hd, vd = 80, 4, 2, 48, 24
+    mixer = Attention(H, nh, nkv, hd, window_kind=window_kind, window=window, v_head_dim=vd)
+    spec = mixer.cache_spec()
+    assert spec.value_dim == vd and spec.head_dim == hd
+    specs = mixer.param_specs("a.")
+    assert specs["a.v_proj.weight"].shape == (nkv * vd, H) and specs["a.o_proj.weight"].shape == (H, nh * vd)
+    g = torch.Generator().manual_seed(3)
+    W = {n: (torch.randn(*sp.shape, generator=g) * 0.2).to(torch.bfloat16).float() for n, sp in specs.items()}
+    mixer.load("a.", _Dict(W, dtype))
+    lens = [37, 30, 45]
+    xs = [torch.randn(L, H, generator=g).to(torch.bfloat16).float() for L in lens]
+    store = P.store_bf16 if dtype == torch.bfloat16 else P._same
+
+    def plain(x):
+        L = x.shape[0]
+        q = store(x @ W["a.q_proj.weight"].T).view(L, nh, hd).transpose(0, 1)
+        k = store(x @ W["a.k_proj.weight"].T).view(L, nkv, hd).transpose(0, 1).repeat_interleave(nh // nkv, 0)
+        v = store(x @ W["a.v_proj.weight"].T).view(L, nkv, vd).transpose(0, 1).repeat_interleave(nh // nkv, 0)
+        pos = torch.arange(L)
+        mask = pos[None, :] <= pos[:, None]
+        if window_kind == 2:
+            mask = mask & (pos[None, :] > pos[:, None] - window)
+        o = torch.nn.functional.scaled_dot_product_attention(q, k, v, attn_mask=mask, scale=hd ** -0.5)
+        return store(store(o.transpose(0, 1).reshape(L, nh * vd)) @ W["a.o_proj.weight"].T)
+
+    want = [plain(x) for x in xs]
+    k = torch.zeros(12, nkv, 16, hd, dtype=dtype, device=DEV)
+    v = torch.zeros(12, nkv, vd, 16, dtype=dtype, device=DEV)
+    done, outs = [0, 0, 0], [[], [], []]
+    for sizes in ([20, 29, 44], [17, 1, 1]):
+        ctx, pages = _ctx([(done[i], sizes[i]) for i in range(3)], dtype=dtype, totals=lens)
+        assert pages <= 12
+        x = torch.cat([xs[i][done[i]:done[i] + sizes[i]] for i in range(3)]).to(dtype).to(DEV)
+        out = mixer.forward(x, ctx, LayerCache(ctx.groups[0], k, v)).float().cpu()
+        o = 0
+        for i in range(3):
+            outs[i].append(out[o:o + sizes[i]])
+            o += sizes[i]
+            done[i] += sizes[i]
+    for i in range(3):
+        tol = 1e-4 if dtype == torch.float32 else 3e-2
+        assert float((torch.cat(outs[i]) - want[i]).abs().max()) <= tol * max(1.0, float(want[i].abs().max())), i
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_feed_forward_parts_alone(tmp_path, dtype):
     from sharpinference_amd import build_model, load_config
     from sharpinference_amd.weights.loader import SafetensorsSource
@@ -283,6 +337,59 @@ def test_schedule_runs_a_layer_twice_and_shares_a_cache(tmp_path):
         H.assert_close_fp32(got, want, "looped schedule")
     finally:
         unregister_architecture("LoopedLlama4ForTest")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_embedding_scale_and_logit_scale_and_cap_are_arguments_of_the_model(tmp_path, dtype):
+    """An architecture that scales its embeddings, scales its logits or caps them softly gives the
+    decoder model three numbers; nothing else changes.  Against the plain functions: the embedding
+    rows times the scale before the first layer, and cap * tanh(scale * logits / cap) behind the head
+    (reference: src/SharpInference.Engine/ForwardPass.cs:1482-1483, src/SharpInference.Cpu/SimdKernels.cs:4490-4530)."""
+    from sharpinference_amd import load_config
+    from sharpinference_amd.engine import Engine
+    from sharpinference_amd.registry import register_architecture, unregister_architecture
+    from sharpinference_amd.config.llama4 import Llama4TextConfig
+    from sharpinference_amd.models.llama4 import build_llama4
+
+    SCALE, LSCALE, CAP = 3.5, 1.5, 2.0
+
+    def build(cfg):
+        m = build_llama4(cfg)
+        m.embedding_scale, m.logit_scale, m.logit_softcap = SCALE, LSCALE, CAP
+        return m
+
+    register_architecture("ScaledLlama4ForTest", Llama4TextConfig, build, replace=True)
+    try:
+        d = make_model_dir(tmp_path, "A", std=0.1)
+        cfg = load_config(d)
+        cfg.architecture = "ScaledLlama4ForTest"
+        import json, os
+        json.dump(cfg.to_dict(), open(os.path.join(d, "config.json"), "w"))
+        eng = Engine(d, dtype=dtype, kv_tokens=256, max_num_seqs=2)
+        toks = H.random_tokens(40, 256, 5)
+        got = H.run_cut(eng, "x", toks, [25, 1, 1, 13])
+        c, W = P.read_config(d), {k: v.float() for k, v in P.load_weights(d).items()}
+        store = P.store_bf16 if dtype == "bfloat16" else P._same
+        eps, pos = c["rms_norm_eps"], torch.arange(40)
+        h = W["model.embed_tokens.weight"][torch.tensor(toks)] * SCALE
+        for lay in range(c["num_hidden_layers"]):
+            p = f"model.layers.{lay}."
+            n = store(P.rms_norm(h, W[p + "input_layernorm.weight"], eps))
+            h = h + P.attention_layer(c, W, lay, n, pos, store)
+            n = store(P.rms_norm(h, W[p + "post_attention_layernorm.weight"], eps))
+            h = h + P.moe_layer(c, W, lay, n, store=store)
+        raw = store(P.rms_norm(h, W["model.norm.weight"], eps)) @ W["lm_head.weight"].T
+        want = CAP * torch.tanh(raw * LSCALE / CAP)
+        assert float(raw.abs().max()) * LSCALE > 0.5 * CAP        # the cap bites
+        if dtype == "float32":
+            H.assert_close_fp32(got, want, "scaled model")
+        else:
+            H.assert_close_bf16(got, want, "scaled model", *H.bounds_of(d))
+        # ... and they do something: the same folder as the plain architecture gives other logits
+        plain_eng = H.make_engine(make_model_dir(tmp_path / "plain", "A", std=0.1), dtype, kv_tokens=256, max_num_seqs=2)
+        assert float((H.run_cut(plain_eng, "y", toks, [40]) - got).abs().max()) > 0.1
+    finally:
+        unregister_architecture("ScaledLlama4ForTest")
 
 
 def test_toy_mixer_with_state_needs_no_change_to_the_framework():
