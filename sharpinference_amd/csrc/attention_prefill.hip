@@ -2,7 +2,10 @@
 // over the paged cache, causal and window masks applied per element.
 //
 // A block owns a tile of up to 128 consecutive tokens of one entry and one query head; each of its
-// four waves takes 32 of the tokens.  The block walks the keys its rows can see in 32-key chunks
+// four waves takes 32 of the tokens (or, for tiles of up to 64 tokens, 16: the keys of a tile are
+// walked one chunk after the other, so a short prompt, whose last tiles alone decide how long the
+// launch takes, is served faster by twice the blocks of half the rows; a row's sums are the same
+// either way).  The block walks the keys its rows can see in 32-key chunks
 // (two 16-key blocks aligned to absolute positions, so a block never straddles a page); a chunk's
 // keys and values are fetched from the cache once, staged in LDS (double-buffered; two chunks
 // are on their way through registers) and read from there by all four waves.  As in the decode kernel everything is transposed:
@@ -10,13 +13,13 @@
 //   O^T[d, q]   += V^T[d, key] * P^T[key, q]    A = V^T block (values are stored transposed
 //                                               inside a page), B = P^T
 // and the S^T accumulator of a lane is the B operand of the second product once exponentiated
-// and split into a bfloat16 pair hi + lo.  In LDS the value columns are permuted so that the
+// and rounded to bfloat16 (the row's sum is taken from the unrounded values).  In LDS the value columns are permuted so that the
 // eight keys a lane needs (4 of each 16-key block) sit side by side; rows and their 16-byte chunks
 // are placed so that reads and stores are free of bank conflicts (see the layouts below).  Softmax
 // state (a reference maximum and the sum per query) is float, kept in base-2 units (scores times
 // log2 e, the hardware's exp2).
-// The keys of a query are always visited in the same blocks, whatever the portion it arrived in,
-// so its sums do not depend on how the prompt was cut.
+// The keys of a query are always visited in the same chunks (pairs of 16-key blocks at absolute
+// positions), whatever the portion or tile it arrived in, so its sums do not depend on how the prompt was cut.
 #include <type_traits>
 
 #include "common.h"
@@ -28,10 +31,12 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 // the head sizes the kernel is compiled for
 #define SHARPI_PREFILL_HEAD_SIZES(X) X(32) X(64) X(96) X(128) X(160) X(192)
 
+#ifndef SHARPI_PREFILL_P_PAIR
+#define SHARPI_PREFILL_P_PAIR 0   // 1: probabilities enter the second product as a bfloat16 pair hi + lo
+#endif
 constexpr int kPreWaves = 4;
-constexpr int kQT = 2;                               // 16-token column tiles per wave
-constexpr int kWaveTokens = 16 * kQT;
-constexpr int kTileTokens = kWaveTokens * kPreWaves; // 128 tokens per block
+constexpr int kMaxQT = 2;                            // most 16-token column tiles per wave
+constexpr int kTileTokens = 16 * kMaxQT * kPreWaves; // 128 tokens per block at most (64 with one column tile a wave)
 constexpr int kVRow = 32;                            // LDS row of the value tile: 32 keys, no pad (chunks swizzled)
 
 // LDS layouts.  The LDS serves a 16-byte read of a wave in four turns of two octets of lanes: one
@@ -59,12 +64,13 @@ constexpr float kLazyMax = 8.0f;                     // how far the row maximum 
 // -inf and its probability 0, and far below any score, so that the first key moves it
 constexpr float kNoMax = -1.0e30f;
 
-template <int HD>
-__global__ __launch_bounds__(kPreWaves* kWave, HD <= 128 ? 2 : 1) void attn_prefill_kernel(
+template <int HD, int kQT>
+__global__ __launch_bounds__(kPreWaves* kWave, HD <= 128 ? (kQT == 1 ? 3 : 2) : 1) void attn_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ block_table, const int* __restrict__ positions, const int* __restrict__ tiles,
     bf16_t* __restrict__ out, int window_kind, int window, float scale, int nh, int nkv, int page_size,
     int max_blocks, int num_pages) {
+  constexpr int kWaveTokens = 16 * kQT;
   constexpr int NJ = HD / 32;
   constexpr int ND = HD / 16;
   constexpr int KPAD = k_row_elems<HD>();
@@ -125,7 +131,11 @@ __global__ __launch_bounds__(kPreWaves* kWave, HD <= 128 ? 2 : 1) void attn_pref
   int first = 0;   // the first key of the tile's first row
   if (window_kind == 1) first = (pos0 / window) * window;
   else if (window_kind == 2) first = pos0 - window + 1 > 0 ? pos0 - window + 1 : 0;
-  const int b_first = first >> 4;
+  // chunks are pairs of 16-key blocks aligned to absolute positions (an even block first): which keys
+  // share a chunk does not depend on the tile.  The block before a window's first, if the pair starts
+  // there, is masked whole; its page may have been given back (the table's -1 reads page 0: finite
+  // values that meet probabilities of zero).
+  const int b_first = (first >> 4) & ~1;
   const int b_last = (pos0 + rows - 1) >> 4;
 
   float m[kQT], l[kQT];
@@ -248,7 +258,10 @@ __global__ __launch_bounds__(kPreWaves* kWave, HD <= 128 ? 2 : 1) void attn_pref
           }
         }
       }
-      bf16x8 pf[kQT], pf_lo[kQT];
+      bf16x8 pf[kQT];
+#if SHARPI_PREFILL_P_PAIR
+      bf16x8 pf_lo[kQT];
+#endif
       // a chunk that every row of the wave sees whole needs no mask
       const bool whole = wave_full && have[1] && ((b + 2) << 4) - 1 <= wave_first_pos && (b << 4) >= wave_last_start;
       // lane holds S^T[key = 16*(b+u) + 4g + i][query row c*16 + r]; scores go to base-2 units
@@ -310,7 +323,9 @@ __global__ __launch_bounds__(kPreWaves* kWave, HD <= 128 ? 2 : 1) void attn_pref
             ls += e;
             const __bf16 hi = (__bf16)e;                                   // round to nearest even
             pf[c][u * 4 + i] = hi;
+#if SHARPI_PREFILL_P_PAIR
             pf_lo[c][u * 4 + i] = (__bf16)(e - (float)hi);
+#endif
           }
         l[c] += ls;
       }
@@ -327,7 +342,9 @@ __global__ __launch_bounds__(kPreWaves* kWave, HD <= 128 ? 2 : 1) void attn_pref
             acc[c][d] *= corr[c];
           }
           acc[c][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[c], acc[c][d], 0, 0, 0);
+#if SHARPI_PREFILL_P_PAIR
           acc[c][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf_lo[c], acc[c][d], 0, 0, 0);
+#endif
         }
       }
     }
@@ -362,29 +379,35 @@ __global__ __launch_bounds__(kPreWaves* kWave, HD <= 128 ? 2 : 1) void attn_pref
 }
 
 // q [T, nh, hd] bf16; caches K [pages, nkv, page_size, hd], V [pages, nkv, hd, page_size] bf16;
-// tiles int32 [n_tiles, 3] = (entry, first token, rows <= 128), tokens of a tile consecutive in
-// one entry; out [T, nh, hd] bf16 (rows of the listed tiles).
+// tiles int32 [n_tiles, 3] = (entry, first token, rows <= tile_tokens), tokens of a tile consecutive
+// in one entry; tile_tokens 128 or 64 (what the caller cut the tiles to: no tile may hold more);
+// out [T, nh, hd] bf16 (rows of the listed tiles).
 SHARPI_EXPORT int sharpi_attention_prefill(const void* q, const void* k_cache, const void* v_cache,
                                            const int* block_table, const int* positions, const int* tiles,
-                                           void* out, int n_tiles, int window_kind, int window, float scale,
-                                           int nh, int nkv, int hd, int page_size, int max_blocks, int num_pages,
-                                           hipStream_t stream) {
+                                           void* out, int n_tiles, int tile_tokens, int window_kind, int window,
+                                           float scale, int nh, int nkv, int hd, int page_size, int max_blocks,
+                                           int num_pages, hipStream_t stream) {
   if (n_tiles <= 0) return SHARPI_OK;
   if (nh <= 0 || nkv <= 0 || nh % nkv != 0 || n_tiles > 65535) return SHARPI_ERR_ARG;
+  if (tile_tokens != kTileTokens && tile_tokens != kTileTokens / 2) return SHARPI_ERR_ARG;
   if (page_size <= 0 || page_size % 16 != 0 || max_blocks <= 0 || num_pages <= 0) return SHARPI_ERR_ARG;
   if (window_kind < 0 || window_kind > 2 || (window_kind != 0 && window <= 0)) return SHARPI_ERR_ARG;
   dim3 grid(nh, n_tiles), block(kPreWaves * kWave);
-#define PRE(HDV)                                                                                              \
-  if (hd == HDV) {                                                                                            \
-    attn_prefill_kernel<HDV><<<grid, block, 0, stream>>>((const bf16_t*)q, (const bf16_t*)k_cache,            \
-                                                        (const bf16_t*)v_cache, block_table, positions, tiles, \
-                                                        (bf16_t*)out, window_kind, window, scale, nh, nkv,     \
-                                                        page_size, max_blocks, num_pages);                    \
-    SHARPI_CHECK_LAUNCH();                                                                                    \
-    return SHARPI_OK;                                                                                         \
+#define PRE_QT(HDV, QTV)                                                                                        \
+  attn_prefill_kernel<HDV, QTV><<<grid, block, 0, stream>>>((const bf16_t*)q, (const bf16_t*)k_cache,               \
+                                                           (const bf16_t*)v_cache, block_table, positions, tiles,  \
+                                                           (bf16_t*)out, window_kind, window, scale, nh, nkv,      \
+                                                           page_size, max_blocks, num_pages)
+#define PRE(HDV)                                  \
+  if (hd == HDV) {                                \
+    if (tile_tokens == kTileTokens) PRE_QT(HDV, 2); \
+    else PRE_QT(HDV, 1);                          \
+    SHARPI_CHECK_LAUNCH();                        \
+    return SHARPI_OK;                             \
   }
   SHARPI_PREFILL_HEAD_SIZES(PRE)
 #undef PRE
+#undef PRE_QT
   return SHARPI_ERR_ARG;  // other head sizes go to the generic kernel
 }
 

@@ -347,9 +347,12 @@ def prefill_attention_ok(dtype: torch.dtype, hd: int) -> bool:
 
 def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                       positions: torch.Tensor, tiles: torch.Tensor, window_kind: int, window: int, scale: float,
-                      nh: int, nkv: int, hd: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Flash attention for the listed tiles: tiles int32 [n, 3] = (entry, first token, rows <= 128),
-    the tokens of a tile consecutive in one entry."""
+                      nh: int, nkv: int, hd: int, out: Optional[torch.Tensor] = None,
+                      tile_tokens: int = PREFILL_TILE_TOKENS) -> torch.Tensor:
+    """Flash attention for the listed tiles: tiles int32 [n, 3] = (entry, first token, rows <=
+    tile_tokens), the tokens of a tile consecutive in one entry.  tile_tokens (128, or 64: blocks of
+    half the rows, for short prompts) is what the caller cut the tiles to; a row's result does not
+    depend on it."""
     _dev(q, k_cache, v_cache, block_table, positions, tiles, out)
     _i32(block_table, "block_table")
     _i32(positions, "positions")
@@ -365,8 +368,8 @@ def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
         out = torch.empty_like(q)
     _need(out.shape == q.shape and out.dtype == q.dtype, "attention_prefill: out must match q")
     _run("sharpi_attention_prefill", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), _ptr(positions),
-         _ptr(tiles), _ptr(out), tiles.shape[0], int(window_kind), int(window), float(scale), nh, nkv, hd,
-         k_cache.shape[2], block_table.shape[1], k_cache.shape[0], _stream())
+         _ptr(tiles), _ptr(out), tiles.shape[0], int(tile_tokens), int(window_kind), int(window), float(scale), nh,
+         nkv, hd, k_cache.shape[2], block_table.shape[1], k_cache.shape[0], _stream())
     return out
 
 
@@ -950,11 +953,11 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, gro
     block tables, `ctx`: the step).  Values of another width than keys (vd) go through the float kernel."""
     same = vd is None or vd == hd
     if same and decode_attention_ok(q.dtype, hd) and (prefill_attention_ok(q.dtype, hd) or not ctx.n_prefill_tiles):
-        # entries of one token: split-K decode kernel; longer entries: flash kernel, 128 tokens a block
+        # entries of one token: split-K decode kernel; longer entries: flash kernel, a tile of tokens a block
         out = torch.empty_like(q)
         if ctx.n_prefill_tiles:
             attention_prefill(q, k_cache, v_cache, group.block_table, ctx.positions, ctx.prefill_tiles, window_kind,
-                              window, scale, nh, nkv, hd, out=out)
+                              window, scale, nh, nkv, hd, out=out, tile_tokens=ctx.prefill_tile_tokens)
         if ctx.n_decode:
             attention_decode(q, k_cache, v_cache, group.block_table, ctx.entry_of_token, ctx.positions,
                              ctx.decode_tokens, group.max_context, window_kind, window, scale, nh, nkv, hd, out=out)

@@ -30,7 +30,7 @@ _SIGNATURES = {
     "sharpi_rope_kv": [P, P, P, P, I, P, P, P, P, I, F, I, F, F, I, I, I, I, I, I, I, I, P],
     "sharpi_attention_generic": [P, P, P, I, P, P, P, P, I, I, F, I, I, I, I, I, I, I, I, P],
     "sharpi_attention_decode": [P, P, P, P, P, P, P, P, P, P, I, I, F, I, I, I, I, I, I, I, I, P],
-    "sharpi_attention_prefill": [P, P, P, P, P, P, P, I, I, I, F, I, I, I, I, I, I, P],
+    "sharpi_attention_prefill": [P, P, P, P, P, P, P, I, I, I, I, F, I, I, I, I, I, I, P],
     "sharpi_gemm_tiled": [P, P, P, I, I, I, I, I, P, P, I, P],
     "sharpi_gemm_skinny": [P, P, P, I, I, I, I, P, P, I, I, I, I, I, P],
     "sharpi_gemm_skinny_swiglu": [P, P, P, I, I, I, P, P, I, P, I, I, I, I, I, P],

@@ -51,11 +51,12 @@ class StepContext:
     groups: List[GroupView]
     act_dtype: torch.dtype
     no_store_slots: Optional[torch.Tensor] = None   # int32 [tokens] of -1: "store nothing" for cache readers
-    # how attention kernels split the batch: entries of one token, and 128-token tiles of the others
+    # how attention kernels split the batch: entries of one token, and tiles of the others' tokens
     n_decode: int = 0
     decode_tokens: Optional[torch.Tensor] = None    # int32 [n_decode] token indices; None = every token
     n_prefill_tiles: int = 0
     prefill_tiles: Optional[torch.Tensor] = None    # int32 [tiles, 3]: (entry, first token, rows)
+    prefill_tile_tokens: int = 128                  # the most rows of a tile (128, or 64 for short prompts)
     # host copies for parts that plan launches
     entry_lens: List[int] = field(default_factory=list)
     entry_starts: List[int] = field(default_factory=list)

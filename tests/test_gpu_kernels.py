@@ -655,6 +655,19 @@ def test_attention_prefill_kernel(nh, nkv, hd, kind, window, ps):
     got = ops.attention_prefill(q.reshape(T, nh * hd).to(DEV), kc.to(DEV), vc.to(DEV), bt.to(DEV),
                                 torch.tensor(positions, dtype=torch.int32, device=DEV),
                                 torch.tensor(tiles, dtype=torch.int32, device=DEV), kind, window, scale, nh, nkv, hd)
+    # tiles of half the rows (what a step with few prompt tokens is cut into): every row keeps its bits
+    half = ops.PREFILL_TILE_TOKENS // 2
+    tiles64 = [(e, t0 + o, min(half, n - o)) for e, t0, n in tiles for o in range(0, n, half)]
+    got64 = ops.attention_prefill(q.reshape(T, nh * hd).to(DEV), kc.to(DEV), vc.to(DEV), bt.to(DEV),
+                                  torch.tensor(positions, dtype=torch.int32, device=DEV),
+                                  torch.tensor(tiles64, dtype=torch.int32, device=DEV), kind, window, scale, nh, nkv, hd,
+                                  tile_tokens=half)
+    assert torch.equal(got64, got)
+    with pytest.raises(Exception):    # a tile size the kernel has no form for is refused
+        ops.attention_prefill(q.reshape(T, nh * hd).to(DEV), kc.to(DEV), vc.to(DEV), bt.to(DEV),
+                              torch.tensor(positions, dtype=torch.int32, device=DEV),
+                              torch.tensor(tiles64, dtype=torch.int32, device=DEV), kind, window, scale, nh, nkv, hd,
+                              tile_tokens=32)
     got = got.float().cpu().view(T, nh, hd)
     err = (got - ref).abs().max(dim=-1).values.max(dim=-1).values
     assert float(err.max()) <= 2e-2, (float(err.max()), int(err.argmax()))
