@@ -19,8 +19,7 @@ import numpy as np
 import torch
 
 from ..cache.manager import CacheError, CacheManager
-from ..ops.lib import PREFILL_TILE_TOKENS
-from ..parts.base import GroupView, LayerCache, StepContext
+from ..parts.base import GroupView, HostStep, LayerCache, StepContext
 
 
 MAX_GRAPH_BATCH = 64   # decode steps of up to this many requests are replayed from a HIP graph (at 64 the host's part of an eager step is still a tenth of the step)
@@ -28,9 +27,7 @@ GRAPH_AT_ONCE = 16     # up to this many requests a graph is captured when its s
 GRAPH_AFTER_ASKS = 4   # shape has been met this often (a graph per width costs capture time and memory of its own)
 MAX_GRAPHS = 48        # graphs kept at a time; beyond, the one replayed longest ago is dropped (and captured again if its shape returns)
 GRAPH_CONTEXT_MIN = 4096   # a graph is captured for a bound on the contexts of its requests: this, or 4, 16, 64 ... times it
-TILE = PREFILL_TILE_TOKENS   # tokens per attention tile of multi-token entries
-SHORT_PROMPT_TOKENS = 1536   # up to so many prompt tokens in a step, tiles of half as many tokens (measured:
-                             # 20-25 % less attention time at 512 and 1,024 tokens, 8 % more at 2,048)
+N_OWN = 7              # index arrays of the step function's own, first in the upload (tokens ... logit rows)
 
 
 class CacheExhausted(CacheError):
@@ -61,6 +58,9 @@ class ModelRunner:
         self.decode_graphs = bool(decode_graphs) and max_context > 0 and (
             all(t is None for t in cache.state) or bool(safe and safe()))
         self.max_context = int(max_context)
+        # what the model's parts want made once a step beside the step's own index arrays (attention: its
+        # kernels' work lists); the step function uploads them and knows nothing of their meaning
+        self.planners = list(getattr(model, "step_planners", list)())
         self._graphs: dict = {}
         self._graph_pool = None      # one memory pool for every graph of this runner (made with the first capture)
         self._graph_asks: dict = {}
@@ -137,20 +137,19 @@ class ModelRunner:
             group_tables.append(bt)
             group_slots.append(sm)
         rows_np = np.asarray(rows, dtype=np.int32)
-        # attention work lists: single-token entries, and tiles of the longer ones
-        dec = [int(cu[i]) for i in range(n) if lens[i] == 1]
-        # (a step with few prompt tokens is cut into tiles of half the rows: its attention launch lasts as
-        # long as its longest tile, and twice the blocks of half the rows walk their keys faster)
-        tile = TILE if sum(L for L in lens if L > 1) > SHORT_PROMPT_TOKENS else TILE // 2
-        tiles = [(i, int(cu[i]) + o, min(tile, lens[i] - o)) for i in range(n) if lens[i] > 1
-                 for o in range(0, lens[i], tile)]
-        dec_np = np.asarray(dec, dtype=np.int32)
-        tiles_np = np.asarray(tiles, dtype=np.int32).reshape(-1)
-        pieces = [token_ids, positions, entry_of, cu, state_slots, np.full(T, -1, dtype=np.int32), rows_np,
-                  dec_np, tiles_np]
+        # what the parts' planners want, then the groups' block tables and slots
+        host = HostStep(n_entries=n, n_tokens=T, lens=lens, starts=starts, cu_tokens=cu)
+        pieces = [token_ids, positions, entry_of, cu, state_slots, np.full(T, -1, dtype=np.int32), rows_np]
+        planned = []                                  # per planner: (number of arrays, host facts)
+        for pl in self.planners:
+            arrays, facts = pl.plan(host)
+            arrays = [np.ascontiguousarray(a, dtype=np.int32).reshape(-1) for a in arrays]
+            planned.append((len(arrays), facts))
+            pieces += arrays
+        n_planned = len(pieces) - N_OWN
         for bt, sm in zip(group_tables, group_slots):
             pieces += [bt.reshape(-1), sm]
-        info = dict(n=n, T=T, lens=lens, starts=starts, n_rows=len(rows), n_dec=len(dec), n_tiles=len(tiles), tile=tile,
+        info = dict(n=n, T=T, lens=lens, starts=starts, n_rows=len(rows), planned=planned, n_planned=n_planned, host=host,
                     max_blocks=[bt.shape[1] for bt in group_tables],
                     max_context=int(positions.max()) + 1 if T else 0)
         return pieces, info
@@ -161,19 +160,21 @@ class ModelRunner:
         for size in sizes:
             views.append(dev[off:off + size])
             off += size
-        d_tok, d_pos, d_ent, d_cu, d_state, d_nostore, d_rows, d_dec, d_tiles = views[:9]
+        d_tok, d_pos, d_ent, d_cu, d_state, d_nostore, d_rows = views[:N_OWN]
         n, T = info["n"], info["T"]
+        first_group = N_OWN + info["n_planned"]
         groups = []
         for g in range(len(self.cache.groups)):
-            bt = views[9 + 2 * g].view(n, info["max_blocks"][g])
-            groups.append(GroupView(bt, views[10 + 2 * g], self.cache.page_size, max_context=info["max_context"]))
+            bt = views[first_group + 2 * g].view(n, info["max_blocks"][g])
+            groups.append(GroupView(bt, views[first_group + 1 + 2 * g], self.cache.page_size, max_context=info["max_context"]))
         ctx = StepContext(n_tokens=T, n_entries=n, token_ids=d_tok, positions=d_pos, entry_of_token=d_ent,
                           cu_tokens=d_cu, state_slots=d_state, groups=groups, act_dtype=self.act_dtype,
                           no_store_slots=d_nostore, entry_lens=info["lens"], entry_starts=info["starts"],
-                          max_entry_len=max(info["lens"]) if info["lens"] else 1, n_decode=info["n_dec"],
-                          decode_tokens=None if info["n_dec"] == T else d_dec, n_prefill_tiles=info["n_tiles"],
-                          prefill_tiles=d_tiles.view(-1, 3) if info["n_tiles"] else None,
-                          prefill_tile_tokens=info["tile"])
+                          max_entry_len=max(info["lens"]) if info["lens"] else 1)
+        at = N_OWN
+        for pl, (count, facts) in zip(self.planners, info["planned"]):
+            pl.attach(ctx, views[at:at + count], facts)
+            at += count
         return ctx, (d_rows if info["n_rows"] else None)
 
     def build_context(self, entries: Sequence[StepEntry]):
@@ -337,8 +338,12 @@ class _DecodeGraph:
         null[4] = np.full_like(pieces[4], runner.cache.scratch_state_slot)   # state: the slot of no request
         null[5] = np.full(n, -1, dtype=np.int32)
         null[6] = np.arange(n, dtype=np.int32)            # logit rows
-        null[7] = np.arange(n, dtype=np.int32)
-        for i in range(9, len(null)):
+        at = N_OWN
+        for pl, (count, _) in zip(runner.planners, info["planned"]):      # the planners' own harmless contents
+            null[at:at + count] = [np.ascontiguousarray(a, dtype=np.int32).reshape(-1)
+                                   for a in pl.null(info["host"], pieces[at:at + count])]
+            at += count
+        for i in range(at, len(null)):                    # block tables and slots
             null[i] = np.full_like(pieces[i], -1)
         self._upload(null)
         ctx, rows = runner._context_from(self.dev, self.sizes, info)

@@ -11,8 +11,9 @@ group, the block tables and the slots where this step's keys and values go.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Dict, List, Optional
+from typing import Dict, List, Optional, Sequence, Tuple
 
+import numpy as np
 import torch
 
 from ..weights.loader import INIT_INT, INIT_NORM_WEIGHT, INIT_NORMAL, ParamSpec, TensorSource  # noqa: F401
@@ -26,6 +27,44 @@ class Part:
 
     def load(self, prefix: str, source: TensorSource) -> None:
         pass
+
+    def step_planners(self) -> Sequence["StepPlanner"]:
+        """The index arrays this part wants made once a step (see :class:`StepPlanner`); none by default."""
+        return ()
+
+
+@dataclass
+class HostStep:
+    """What a step planner sees of a step, on the host: the flat batch's layout."""
+
+    n_entries: int
+    n_tokens: int
+    lens: List[int]                    # tokens of each entry
+    starts: List[int]                  # position of each entry's first token
+    cu_tokens: np.ndarray              # int32 [entries + 1]: entry e's tokens are rows cu[e] .. cu[e + 1]
+
+
+class StepPlanner:
+    """Index arrays that a kind of part needs once a step, made on the host from the batch's layout
+    and uploaded in the step's one copy: the step function knows nothing of what they mean.
+
+    A part returns its planners from ``step_planners()``; planners with the same ``key`` are one
+    (every attention layer shares one set of work lists).  ``plan`` returns int32 arrays and host
+    facts; ``attach`` receives their device views and the facts and puts them where the part's
+    ``forward`` finds them (fields of the context, or ``ctx.extras[key]``).  For a decode step that
+    is replayed from a graph the arrays of a step must have the sizes of every other step of that
+    batch size, and ``null`` gives contents under which a trial run touches no request's data."""
+
+    key: str = ""
+
+    def plan(self, host: HostStep) -> Tuple[List[np.ndarray], dict]:
+        raise NotImplementedError
+
+    def null(self, host: HostStep, arrays: List[np.ndarray]) -> List[np.ndarray]:
+        return [np.zeros_like(a) for a in arrays]
+
+    def attach(self, ctx: "StepContext", views: List[torch.Tensor], facts: dict) -> None:
+        raise NotImplementedError
 
 
 @dataclass
@@ -52,6 +91,7 @@ class StepContext:
     act_dtype: torch.dtype
     no_store_slots: Optional[torch.Tensor] = None   # int32 [tokens] of -1: "store nothing" for cache readers
     # how attention kernels split the batch: entries of one token, and tiles of the others' tokens
+    # (made by the attention parts' planner, parts/attention.py; empty in a model without attention)
     n_decode: int = 0
     decode_tokens: Optional[torch.Tensor] = None    # int32 [n_decode] token indices; None = every token
     n_prefill_tiles: int = 0

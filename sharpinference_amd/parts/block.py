@@ -35,6 +35,12 @@ class PreNormBlock(Part):
         for name, part in self._children():
             part.load(prefix + name, source)
 
+    def step_planners(self):
+        out = []
+        for _, part in self._children():
+            out.extend(getattr(part, "step_planners", tuple)())
+        return out
+
     def cache_spec(self):
         spec = getattr(self.mixer, "cache_spec", None)
         return spec() if spec else None

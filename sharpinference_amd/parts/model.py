@@ -87,6 +87,16 @@ class DecoderModel(Part):
     def decode_graph_safe(self) -> bool:
         return all(getattr(b, "decode_graph_safe", lambda: True)() for b in self.blocks)
 
+    def step_planners(self):
+        """The planners of the parts in the order they first appear, one per key."""
+        out: dict = {}
+        for b in self.blocks:
+            for pl in getattr(b, "step_planners", tuple)():
+                if not pl.key:
+                    raise ValueError(f"{type(pl).__name__}: a step planner needs a key")
+                out.setdefault(pl.key, pl)
+        return list(out.values())
+
     # -- weights ------------------------------------------------------------------
     def param_specs(self, prefix: str = "") -> Dict[str, ParamSpec]:
         out = {self.embed_name: ParamSpec((self.vocab_size, self.hidden))}

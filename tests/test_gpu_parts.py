@@ -773,3 +773,107 @@ def test_a_stateful_mixer_that_can_be_captured_decodes_from_graphs(graphs):
         eng.free_request("fresh")
     finally:
         unregister_architecture("ToyDecay")
+
+
+@pytest.mark.parametrize("graphs", [True, False])
+def test_a_part_declares_the_index_arrays_it_wants_made_once_a_step(graphs, tmp_path):
+    """A mixer asks for index arrays of its own through a step planner (here: the row of each
+    entry's last token); the step function uploads them with its own arrays, in eager steps and
+    in replayed graphs, without knowing what they mean.  A model without attention gets no
+    attention work lists."""
+    import numpy as np
+    from sharpinference_amd.cache.spec import StateSpec
+    from sharpinference_amd.config.base import ModelConfig
+    from sharpinference_amd.engine import Engine
+    from sharpinference_amd.parts.base import Part, StepPlanner
+    from sharpinference_amd.parts.block import PreNormBlock
+    from sharpinference_amd.parts.feedforward import DenseSwiGLU
+    from sharpinference_amd.parts.model import DecoderModel
+    from sharpinference_amd.parts.norm import RMSNorm
+    from sharpinference_amd.registry import register_architecture, unregister_architecture
+
+    @dataclass
+    class ToyConfig(ModelConfig):
+        architecture: str = "ToyLastRow"
+        vocab_size: int = 50
+        max_position_embeddings: int = 256
+
+        @classmethod
+        def from_dict(cls, d):
+            return cls()
+
+        def to_dict(self):
+            return {"architectures": [self.architecture]}
+
+    calls = {"plan": 0, "attach": 0}
+
+    class LastRows(StepPlanner):
+        key = "last_rows"
+
+        def plan(self, host):
+            calls["plan"] += 1
+            return [host.cu_tokens[1:] - 1], {"entries": host.n_entries}
+
+        def null(self, host, arrays):
+            return [np.arange(arrays[0].size, dtype=np.int32)]
+
+        def attach(self, ctx, views, facts):
+            calls["attach"] += 1
+            assert views[0].shape == (facts["entries"],) and views[0].dtype == torch.int32 and views[0].is_cuda
+            ctx.extras["last_rows"] = views[0]
+
+    planner = LastRows()
+
+    class Decay(Part):
+        """out[t] = s[t], s[t] = 0.5 * s[t-1] + x[t]; the state an entry leaves is the row of its last
+        token, found through the planner's list."""
+        graph_safe = True
+
+        def step_planners(self):
+            return (planner,)
+
+        def cache_spec(self):
+            return StateSpec((32,), torch.float32)
+
+        def forward(self, x, ctx, cache):
+            slots = ctx.state_slots.long()
+            s = cache.state.index_select(0, slots)
+            out = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+            o = 0
+            for e, n in enumerate(ctx.entry_lens):
+                cur = s[e]
+                for t in range(n):
+                    cur = 0.5 * cur + x[o + t].float()
+                    out[o + t] = cur
+                o += n
+            cache.state.index_copy_(0, slots, out.index_select(0, ctx.extras["last_rows"].long()))
+            return out.to(x.dtype)
+
+    def build(cfg):
+        blocks = [PreNormBlock(RMSNorm(32, 1e-5), Decay(), RMSNorm(32, 1e-5), DenseSwiGLU(32, 48),
+                               names={"norm1": "n1.", "mixer": "mix.", "norm2": "n2.", "ffn": "ff."}) for _ in range(2)]
+        return DecoderModel(cfg.vocab_size, 32, blocks, RMSNorm(32, 1e-5), config=cfg)
+
+    register_architecture("ToyLastRow", ToyConfig, build, replace=True)
+    try:
+        eng = Engine(config=ToyConfig(), weight_seed=3, dtype="float32", kv_tokens=64, max_num_seqs=3, weight_std=0.3,
+                     decode_graphs=graphs)
+        assert [pl.key for pl in eng.runner.planners] == ["last_rows"]      # one per key, and no attention lists
+        a, b = H.random_tokens(30, 50, 1), H.random_tokens(22, 50, 2)
+        steps = [{"entries": [{"id": "a", "tokens": a[:20], "want": [19]}], "end": []},
+                 {"entries": [{"id": "b", "tokens": b[:12], "want": [11]}, {"id": "a", "tokens": [a[20]], "want": [0]}], "end": []}]
+        steps += [{"entries": [{"id": "a", "tokens": [a[21 + i]], "want": [0]}, {"id": "b", "tokens": [b[12 + i]], "want": [0]}],
+                   "end": []} for i in range(9)]
+        steps[-1]["end"] = ["a", "b"]
+        for i, st in enumerate(steps):
+            st["step"] = i
+        got = H.replay(eng, steps)
+        assert eng.runner.graph_replays == (9 if graphs else 0)
+        assert calls["plan"] >= len(steps) and calls["attach"] >= (3 if graphs else len(steps))
+        whole_a, whole_b = H.run_cut(eng, "wa", a, [30]), H.run_cut(eng, "wb", b[:21], [21])
+        assert float((got["a"] - whole_a[19:]).abs().max()) <= 1e-5 and float((got["b"] - whole_b[11:]).abs().max()) <= 1e-5
+    finally:
+        unregister_architecture("ToyLastRow")
+    # the architecture's own model asks for the attention kernels' work lists, once for all its layers
+    eng = Engine(make_model_dir(tmp_path, "A"), dtype="float32", kv_tokens=128, max_num_seqs=2)
+    assert [pl.key for pl in eng.runner.planners] == ["attention"]
