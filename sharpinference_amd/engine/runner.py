@@ -355,6 +355,11 @@ class _DecodeGraph:
             runner.model.forward(*args)
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
+        # A fresh context for the captured run: what the trial run's parts kept in the context (tensors
+        # they make once a step) was made outside the graph and would never be made again.
+        ctx, rows = runner._context_from(self.dev, self.sizes, info)
+        caches = runner.layer_caches(ctx)
+        args = (ctx, caches, rows, select) if select else (ctx, caches, rows)
         # the captured run also notes where its router picks lie (tensors of the graph's own memory,
         # filled anew by every replay), so that a replayed step can be traced like a launched one
         self.trace: list = []
