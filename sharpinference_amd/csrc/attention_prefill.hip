@@ -13,7 +13,8 @@
 //   O^T[d, q]   += V^T[d, key] * P^T[key, q]    A = V^T block (values are stored transposed
 //                                               inside a page), B = P^T
 // and the S^T accumulator of a lane is the B operand of the second product once exponentiated
-// and rounded to bfloat16 (the row's sum is taken from the unrounded values).  In LDS the value columns are permuted so that the
+// and split into a bfloat16 pair hi + lo (two products: the probabilities keep ~16 bits; the row's
+// sum is taken from the unrounded values).  In LDS the value columns are permuted so that the
 // eight keys a lane needs (4 of each 16-key block) sit side by side; rows and their 16-byte chunks
 // are placed so that reads and stores are free of bank conflicts (see the layouts below).  Softmax
 // state (a reference maximum and the sum per query) is float, kept in base-2 units (scores times
@@ -32,7 +33,11 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 #define SHARPI_PREFILL_HEAD_SIZES(X) X(32) X(64) X(96) X(128) X(160) X(192)
 
 #ifndef SHARPI_PREFILL_P_PAIR
-#define SHARPI_PREFILL_P_PAIR 0   // 1: probabilities enter the second product as a bfloat16 pair hi + lo
+// 1: probabilities enter the second product as a bfloat16 pair hi + lo.  0 (hi alone) is 4 % faster at
+// 2,048 tokens and 10 % at 8,192, but then rounds every probability to 8 bits, which the comparison
+// with a float softmax does not forgive where the softmax is sharp: random mixed traces at a weight
+// scale of 0.08 left the derived bfloat16 bound by up to a quarter in 4 of 60, none with the pair.
+#define SHARPI_PREFILL_P_PAIR 1
 #endif
 constexpr int kPreWaves = 4;
 constexpr int kMaxQT = 2;                            // most 16-token column tiles per wave

@@ -3,6 +3,7 @@ import pytest
 import torch
 
 import helpers as H
+import plain_llama4 as P
 from tiny_configs import CONFIGS, as_other_tools_write_it, make_model_dir, write_other_layout
 
 pytestmark = pytest.mark.gpu
@@ -85,6 +86,31 @@ def test_mixed_batches_with_page_reuse(model_dir, seed):
         for g in eng.cache.groups:
             assert g.pool.total_allocs > g.pool.num_pages, "the pool was large enough to never reuse a page"
             assert g.pool.num_free == g.pool.num_pages
+
+
+@pytest.mark.parametrize("seed,lens,tail,max_live,page_size", [
+    (112, [65, 64, 200, 129, 5, 40, 17, 90], 32, 2, 32), (133, [40, 200, 128, 200, 200, 40], 1, 4, 16),
+    (156, [17, 200, 40, 5, 17, 5, 257, 5], 32, 3, 32)])
+def test_mixed_traces_with_a_sharp_softmax_stay_inside_the_bound(tmp_path, seed, lens, tail, max_live, page_size):
+    """Configuration D at a weight scale of 0.08: scores spread so far that a probability rounded to
+    8 bits before the product with the values shows in the logits (these traces left the bound
+    when the prompt kernel kept only the high half of its probabilities).  In bfloat16 under the
+    engine's picks; in 32-bit under them too, so that a near-tie of two experts is no failure."""
+    d = make_model_dir(tmp_path, "D", std=0.08)
+    vocab = CONFIGS["D"]["vocab_size"]
+    reqs = {f"r{i}": H.random_tokens(n, vocab, 1000 * seed + i) for i, n in enumerate(lens)}
+    steps = H.mixed_trace(reqs, seed, max_live=max_live, tail=tail)
+    held = H.tokens_held(steps, round_to=max(64, page_size))
+    eng = H.make_engine(d, "bfloat16", kv_tokens=held, max_num_seqs=4, page_size=page_size)
+    H.check_trace_against_plain(eng, d, "bfloat16", reqs, steps, f"D 0.08 bfloat16 mixed(seed {seed})")
+    eng = H.make_engine(d, "float32", kv_tokens=held, max_num_seqs=4, page_size=page_size)
+    got, picks, seen = H.replay(eng, steps, with_routes=True)
+    layers = H.moe_layers_of(d)
+    c, W = H._model(d)
+    for rid, toks in reqs.items():
+        H.assert_routes_are_the_best(d, picks[rid], seen[rid], f"request {rid}")
+        ref = P.forward(c, W, list(toks), store=P._same, routes=dict(zip(layers, picks[rid])))
+        H.assert_close_fp32(got[rid], ref, f"D 0.08 float32 mixed(seed {seed}) request {rid}")
 
 
 WIDTHS = [5, 8, 16, 17, 32, 33, 64, 65]   # both sides of every batch size at which a step changes kernels
