@@ -282,8 +282,8 @@ def host_report(eng, prompt_len: int, rng: random.Random, batch: int = 64) -> di
     for name, sp in cases.items():
         params = [SamplingParams(**{**sp.__dict__, "seed": 100 + i}) for i in range(batch)]
         t_step = t_sample = t_wall = 0.0
-        n = 6
-        for it in range(n + 2):
+        n, warm = 6, 5       # (a wide batch's graph is captured when its shape has been met four times: within the warm-up)
+        for it in range(n + warm):
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             logits = eng.step([StepEntry(r, (t,), (0,)) for r, t in zip(ids, tokens)])
@@ -296,7 +296,7 @@ def host_report(eng, prompt_len: int, rng: random.Random, batch: int = 64) -> di
             t3 = time.perf_counter()
             for r, t in zip(ids, tokens):
                 history[r].append(t)
-            if it >= 2:
+            if it >= warm:
                 t_step += t1 - t0
                 t_sample += t3 - t2
                 t_wall += t3 - t0
