@@ -890,7 +890,7 @@ def dense_grouped_ok(M: int, N: int, K: int) -> bool:
 
 def linear_many_rows(x: torch.Tensor, w: PackedWeight, out_dtype: torch.dtype) -> torch.Tensor:
     """x [M, K] @ w^T for many rows against a matrix stored tile by tile, on the matrix cores: the
-    grouped product with the whole matrix as its one group (row tiles of up to 192 rows whose
+    grouped product with the whole matrix as its one group (row tiles of up to 128 rows whose
     blocks share the weight stream through an XCD's L2)."""
     rt = _dense_routing(x.shape[0], x.device)
     return gemm_grouped(x, PackedWeight(w.packed.unsqueeze(0), None), rt, False, out_dtype)
