@@ -247,6 +247,42 @@ def test_a_token_budget_below_the_live_requests_generates_the_same(tmp_path, dty
         assert [r.token_ids for r in wide.generate(prompts, params)] == [r.token_ids for r in want]
 
 
+@pytest.mark.parametrize("seed", [3, 11, 17, 54, 75, 81])
+def test_random_workloads_generate_the_same_batched_as_alone(tmp_path, seed):
+    """Random workloads (2 to 9 requests of random lengths; greedy and sampled rows, top-k on some, a
+    stop token each; random limits on live requests, tokens a step, pages, steps launched on end)
+    in 32-bit: every request gets the tokens and the finish reason it gets alone, nothing is left in
+    the pools.  (In 32-bit a row's logits do not depend on the batch; in bfloat16 they do, within
+    rounding, and a near-tie may flip there.)"""
+    import random
+    from sharpinference_amd import SamplingParams
+    from sharpinference_amd.engine import Engine
+
+    rng = random.Random(seed)
+    which = rng.choice("ABCD")
+    d = make_model_dir(tmp_path, which, std=0.05)
+    vocab = CONFIGS[which]["vocab_size"]
+    n = rng.randint(2, 9)
+    prompts = [H.random_tokens(rng.choice([1, 2, 5, 17, 40, 64, 65, 100, 130]), vocab, seed * 100 + i) for i in range(n)]
+    new = [rng.choice([1, 2, 7, 20, 40]) for _ in range(n)]
+    params = [SamplingParams(temperature=rng.choice([0.0, 0.0, 0.8]), max_new_tokens=m, seed=seed * 7 + i, top_k=rng.choice([0, 5]),
+                             stop_token_ids=(rng.randrange(vocab),)) for i, m in enumerate(new)]
+    seqs, budget, ps, ahead = rng.randint(1, 6), rng.choice([1, 2, 3, 8, 33, 2048]), rng.choice([16, 32]), rng.choice([1, 4])
+    need = max((len(p) + m + ps - 1) // ps * ps for p, m in zip(prompts, new))
+    kv = rng.choice([need, 2 * need, 4 * need])
+    eng = Engine(d, dtype="float32", max_num_seqs=seqs, max_tokens_per_step=budget, kv_tokens=kv, page_size=ps,
+                 decode_run_ahead=ahead)
+    got = eng.generate(prompts, params)
+    eng.cache.check_invariants()
+    assert all(g.pool.num_free == g.pool.num_pages for g in eng.cache.groups)
+    one = Engine(d, dtype="float32", max_num_seqs=1, kv_tokens=need, page_size=ps, decode_run_ahead=1, decode_graphs=False)
+    for i, (p, sp) in enumerate(zip(prompts, params)):
+        ref = one.generate([p], [sp])[0]
+        assert (got[i].token_ids, got[i].finish_reason) == (ref.token_ids, ref.finish_reason), \
+            f"request {i} of {n} (live {seqs}, budget {budget}, page {ps}, ahead {ahead}, pool {kv})"
+        assert len(ref.token_ids) <= new[i]
+
+
 def test_chunks_stream_in_order_and_cancelling_gives_pages_back(tmp_path):
     """The typed chunks of a generation: per prompt one usage chunk first, its tokens in order,
     one stop chunk last; the tokens are those of generate().  A prompt cancelled half-way ends
