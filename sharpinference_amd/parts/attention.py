@@ -14,7 +14,7 @@ from ..cache.spec import KVSpec, WINDOW_CHUNK, WINDOW_NONE, WINDOW_SLIDING  # no
 from .base import HostStep, LayerCache, ParamSpec, Part, StepContext, StepPlanner, TensorSource
 
 SHORT_PROMPT_TOKENS = 1536   # up to so many prompt tokens in a step, tiles of half as many tokens (measured:
-                             # 20-25 % less attention time at 512 and 1,024 tokens, 8 % more at 2,048)
+                             # 20-25 % less attention time from 512 to 1,536 tokens, 6 % more at 2,048)
 
 
 class AttentionWorkLists(StepPlanner):
