@@ -73,3 +73,40 @@ def test_roofline_bytes_count_every_weight_once_and_the_live_cache():
     got = bench.decode_step_bytes(cfg, 48, batch, ctx, distinct)
     assert abs(got - want) / want < 0.01, (got, want)
     json.dumps({"bytes": got})
+
+
+def test_attention_work_lists_cut_a_step_into_decode_tokens_and_tiles():
+    """What the attention parts ask the step function to upload: the tokens of entries of one
+    token, and tiles of the longer entries: 64-token tiles while a step holds few prompt tokens,
+    128-token tiles beyond; every token of a longer entry lies in exactly one tile, tiles do
+    not cross entries."""
+    import numpy as np
+    from sharpinference_amd.parts.attention import SHORT_PROMPT_TOKENS, AttentionWorkLists
+    from sharpinference_amd.parts.base import HostStep
+
+    def plan(lens):
+        cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        host = HostStep(n_entries=len(lens), n_tokens=int(cu[-1]), lens=list(lens), starts=[7 * i for i in range(len(lens))], cu_tokens=cu)
+        (dec, tiles), facts = AttentionWorkLists().plan(host)
+        return cu, dec, tiles.reshape(-1, 3), facts
+
+    cu, dec, tiles, facts = plan([1, 130, 1, 2, 64])
+    assert dec.tolist() == [0, 131] and facts["n_dec"] == 2 and not facts["all_decode"]
+    assert facts["tile"] == 64 and facts["n_tiles"] == len(tiles) == 3 + 1 + 1
+    assert tiles.tolist() == [[1, 1, 64], [1, 65, 64], [1, 129, 2], [3, 132, 2], [4, 134, 64]]
+    cu, dec, tiles, facts = plan([1, 1, 1])
+    assert facts["all_decode"] and facts["n_tiles"] == 0 and tiles.size == 0 and dec.tolist() == [0, 1, 2]
+    for lens in ([SHORT_PROMPT_TOKENS], [SHORT_PROMPT_TOKENS + 1], [700, 1, 900, 300], [4096, 5]):
+        cu, dec, tiles, facts = plan(lens)
+        assert facts["tile"] == (64 if sum(n for n in lens if n > 1) <= SHORT_PROMPT_TOKENS else 128)
+        covered = np.zeros(int(cu[-1]), dtype=np.int32)
+        for e, t0, rows in tiles.tolist():
+            assert 1 <= rows <= facts["tile"] and cu[e] <= t0 and t0 + rows <= cu[e + 1]
+            covered[t0:t0 + rows] += 1
+        want = np.concatenate([np.full(n, 1 if n > 1 else 0) for n in lens])
+        assert covered.tolist() == want.tolist()
+    # under a graph's trial run the lists hold harmless contents of the same sizes
+    host = HostStep(n_entries=3, n_tokens=3, lens=[1, 1, 1], starts=[5, 6, 7], cu_tokens=np.arange(4, dtype=np.int32))
+    arrays, _ = AttentionWorkLists().plan(host)
+    null = AttentionWorkLists().null(host, arrays)
+    assert [a.size for a in null] == [a.size for a in arrays] and null[0].tolist() == [0, 1, 2]
